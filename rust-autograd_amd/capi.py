@@ -1,0 +1,125 @@
+"""ctypes binding of libag_hip.so (the C ABI declared in include/ag_hip.h).
+
+Nothing here computes: it loads the HIP library, declares the prototypes and turns a non-zero
+``ag_status_t`` into a Python exception carrying the library's message.  There is no fallback:
+if the library is missing the import of any operator fails loudly.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libag_hip.so")
+
+c_f = C.c_float
+c_i = C.c_int
+c_ll = C.c_longlong
+c_sz = C.c_size_t
+c_p = C.c_void_p
+
+
+class OpError(RuntimeError):
+    """Mirror of the reference's `op::OpError` (src/op.rs:66-73)."""
+    code = 0
+
+
+class NdArrayError(OpError):
+    code = 1
+
+
+class IncompatibleShape(OpError):
+    code = 2
+
+
+class TypeUnsupported(OpError):
+    code = 3
+
+
+class InvalidDims(OpError):
+    code = 4
+
+
+class OutOfBounds(OpError):
+    code = 5
+
+
+class HipError(OpError):
+    code = 100
+
+
+_ERRORS = {1: NdArrayError, 2: IncompatibleShape, 3: TypeUnsupported, 4: InvalidDims, 5: OutOfBounds}
+
+# name -> (restype, argtypes); kept in the order of include/ag_hip.h
+PROTOTYPES = {
+    "ag_last_error": (C.c_char_p, []),
+    "ag_version": (C.c_char_p, []),
+    "ag_conv_out_size": (c_i, [c_i] * 5),
+    "ag_conv_transpose_out_size": (c_i, [c_i] * 5),
+    "ag_pool_out_size": (c_i, [c_i] * 4),
+    "ag_pool_grad_in_size": (c_i, [c_i] * 4),
+    "ag_im2col_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 12),
+    "ag_col2im_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 14),
+    "ag_gemm_f32": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_f, c_p, c_i, c_ll, c_p, c_i, c_ll, c_f, c_p,
+                          c_i, c_ll, c_i]),
+    "ag_gemm_batchsum_f32_workspace": (c_sz, [c_i] * 4),
+    "ag_gemm_batchsum_f32": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_f, c_p, c_i, c_ll, c_p, c_i, c_ll,
+                                   c_f, c_p, c_i, c_i, c_p, c_sz]),
+    "ag_conv2d_fwd_f32": (c_i, [c_p] * 5 + [c_i] * 10),
+    "ag_conv2d_with_cols_f32": (c_i, [c_p] * 4 + [c_i] * 4),
+    "ag_conv2d_filter_grad_f32_workspace": (c_sz, [c_i] * 4),
+    "ag_conv2d_filter_grad_f32": (c_i, [c_p] * 4 + [c_i] * 4 + [c_p, c_sz]),
+    "ag_conv2d_transpose_f32": (c_i, [c_p] * 5 + [c_i] * 12),
+    "ag_conv2d_transpose_filter_grad_f32": (c_i, [c_p] * 5 + [c_i] * 12 + [c_p, c_sz]),
+    "ag_maxpool2d_fwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
+    "ag_maxpool2d_bwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
+    "ag_maxpool2d_gradgrad_f32": (c_i, [c_p] * 5 + [c_i] * 7),
+    "ag_sum_all_f32_workspace": (c_sz, [c_sz]),
+    "ag_sum_all_f32": (c_i, [c_p, c_p, c_sz, c_p, c_p, c_sz]),
+    "ag_reduce_sum_f32_workspace": (c_sz, [c_p, c_i, c_p, c_i]),
+    "ag_reduce_sum_f32": (c_i, [c_p, c_p, c_p, c_p, c_i, c_p, c_i, c_i, c_p, c_sz]),
+    "ag_broadcast_grad_f32": (c_i, [c_p, c_p, c_p, c_p, c_i, c_p, c_i]),
+    "ag_adam_update_f32": (c_i, [c_p] * 6 + [c_sz] + [c_f] * 4),
+    "ag_relu_f32": (c_i, [c_p, c_p, c_p, c_sz]),
+    "ag_relu_grad_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),
+    "ag_add_bias_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz]),
+    "ag_bias_grad_f32": (c_i, [c_p, c_p, c_p, c_sz, c_sz]),
+    "ag_add_n_f32": (c_i, [c_p, c_p, c_i, c_p, c_sz]),
+    "ag_mul_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),
+    "ag_scale_f32": (c_i, [c_p, c_p, c_f, c_p, c_sz]),
+    "ag_fill_f32": (c_i, [c_p, c_p, c_f, c_sz]),
+    "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
+    "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
+    "ag_gemm_force_config": (None, [c_i]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built (run __graft_entry__.build())."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with rust-autograd_amd/csrc/build.sh "
+                "(there is no CPU fallback)")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(handle, name)  # AttributeError names the missing symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def last_error():
+    return lib().ag_last_error().decode(errors="replace")
+
+
+def check(status):
+    """Raise the exception class that corresponds to a non-zero ag_status_t."""
+    if status == 0:
+        return
+    cls = _ERRORS.get(status, HipError)
+    err = cls(last_error())
+    err.status = status
+    raise err

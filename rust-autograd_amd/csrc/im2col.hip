@@ -1,0 +1,236 @@
+// im2col (gather) and col2im (gather-form scatter-add) for NCHW f32 images.
+//
+// Both are pure data movement bound by HBM: im2col reads |x| and writes kh*kw*|x|-ish bytes,
+// col2im the reverse.  im2col stages the input rows a band of output rows needs in LDS once
+// (zero padding materialised there), then streams kh*kw output planes out of LDS with fully
+// coalesced stores.  col2im assigns one thread per destination pixel and sums the at most
+// kh*kw source values in (ky, kx) ascending order -- the order in which the reference's
+// sequential scatter reaches that pixel (conv_ops/mod.rs:198-219) -- so no atomics are needed
+// and the result is bit-identical for identical input.
+#include "ag_internal.h"
+
+namespace ag {
+
+struct ConvGeom {
+    int C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW;
+};
+
+constexpr int kIm2colThreads = 256;
+constexpr int kIm2colLdsBytes = 32 * 1024;
+
+// One block = one (image, channel) plane x one band of `R` output rows.
+// tile[r][cx] holds x[iy0 + r][cx - pw] (0 outside the image), WL floats per row.
+template <bool VEC4>
+__global__ __launch_bounds__(kIm2colThreads) void im2col_lds_kernel(
+    const float *__restrict__ x, float *__restrict__ cols, ConvGeom g, int R, int bands, int WL)
+{
+    extern __shared__ float tile[];
+    const int tid = threadIdx.x;
+    const int band = blockIdx.x % bands;
+    const long long plane = blockIdx.x / bands;  // b*C + c
+    const int oy0 = band * R;
+    const int rows = min(R, g.OH - oy0);
+    const int iy0 = oy0 * g.sh - g.ph;
+    const int in_rows = (rows - 1) * g.sh + (g.kh - 1) * g.dh + 1;
+    const float *xp = x + plane * (long long)g.H * g.W;
+
+    for (int e = tid; e < in_rows * WL; e += kIm2colThreads) {
+        const int r = e / WL;
+        const int cx = e - r * WL;
+        const int iy = iy0 + r;
+        const int ix = cx - g.pw;
+        float v = 0.f;
+        if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) v = xp[iy * g.W + ix];
+        tile[e] = v;
+    }
+    __syncthreads();
+
+    const long long P = (long long)g.OH * g.OW;
+    const int taps = g.kh * g.kw;
+    float *out = cols + plane * taps * P + (long long)oy0 * g.OW;
+    const int n_out = rows * g.OW;
+
+    if (VEC4) {
+        // OW % 4 == 0: four consecutive outputs share a row and every store is 16-byte aligned.
+        for (int e = tid * 4; e < n_out; e += kIm2colThreads * 4) {
+            const int r = e / g.OW;
+            const int ox = e - r * g.OW;
+            const float *src = tile + (r * g.sh) * WL + ox * g.sw;
+            float *dst = out + e;
+            for (int ky = 0; ky < g.kh; ++ky) {
+                for (int kx = 0; kx < g.kw; ++kx) {
+                    const float *s = src + ky * g.dh * WL + kx * g.dw;
+                    float4 v;
+                    v.x = s[0];
+                    v.y = s[g.sw];
+                    v.z = s[2 * g.sw];
+                    v.w = s[3 * g.sw];
+                    *reinterpret_cast<float4 *>(dst) = v;
+                    dst += P;
+                }
+            }
+        }
+    } else {
+        for (int e = tid; e < n_out; e += kIm2colThreads) {
+            const int r = e / g.OW;
+            const int ox = e - r * g.OW;
+            const float *src = tile + (r * g.sh) * WL + ox * g.sw;
+            float *dst = out + e;
+            for (int ky = 0; ky < g.kh; ++ky) {
+                for (int kx = 0; kx < g.kw; ++kx) {
+                    *dst = src[ky * g.dh * WL + kx * g.dw];
+                    dst += P;
+                }
+            }
+        }
+    }
+}
+
+// Fallback without LDS staging for rows too wide to stage: one thread per output element.
+__global__ __launch_bounds__(256) void im2col_direct_kernel(const float *__restrict__ x,
+                                                            float *__restrict__ cols, ConvGeom g,
+                                                            long long total)
+{
+    const long long P = (long long)g.OH * g.OW;
+    for (long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += gridDim.x * 256LL) {
+        const long long row = i / P;  // (b*C + c)*taps + tap
+        const int p = (int)(i - row * P);
+        const int oy = p / g.OW, ox = p - oy * g.OW;
+        const int taps = g.kh * g.kw;
+        const long long plane = row / taps;
+        const int tap = (int)(row - plane * taps);
+        const int ky = tap / g.kw, kx = tap - ky * g.kw;
+        const int iy = oy * g.sh - g.ph + ky * g.dh;
+        const int ix = ox * g.sw - g.pw + kx * g.dw;
+        float v = 0.f;
+        if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
+            v = x[plane * (long long)g.H * g.W + iy * g.W + ix];
+        cols[i] = v;
+    }
+}
+
+// One thread per destination pixel.  UNIT = stride 1 on both axes (no divisibility tests).
+template <bool UNIT>
+__global__ __launch_bounds__(256) void col2im_gather_kernel(const float *__restrict__ cols,
+                                                            float *__restrict__ gx, ConvGeom g,
+                                                            int chunks)
+{
+    const int chunk = blockIdx.x % chunks;
+    const long long plane = blockIdx.x / chunks;
+    const int HW = g.H * g.W;
+    const int e = chunk * 256 + threadIdx.x;
+    if (e >= HW) return;
+    const int iy = e / g.W, ix = e - iy * g.W;
+    const long long P = (long long)g.OH * g.OW;
+    const float *cp = cols + plane * (long long)(g.kh * g.kw) * P;
+    float acc = 0.f;
+    for (int ky = 0; ky < g.kh; ++ky) {
+        const int ty = iy + g.ph - ky * g.dh;
+        int oy;
+        if (UNIT) {
+            oy = ty;
+        } else {
+            if (ty < 0) break;  // later ky only lowers ty
+            oy = ty / g.sh;
+            if (oy * g.sh != ty) continue;
+        }
+        if ((unsigned)oy >= (unsigned)g.OH) continue;
+        for (int kx = 0; kx < g.kw; ++kx) {
+            const int tx = ix + g.pw - kx * g.dw;
+            int ox;
+            if (UNIT) {
+                ox = tx;
+            } else {
+                if (tx < 0) break;
+                ox = tx / g.sw;
+                if (ox * g.sw != tx) continue;
+            }
+            if ((unsigned)ox >= (unsigned)g.OW) continue;
+            acc += cp[(long long)(ky * g.kw + kx) * P + oy * g.OW + ox];
+        }
+    }
+    gx[plane * HW + e] = acc;
+}
+
+static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int kh, int kw, int ph,
+                              int pw, int sh, int sw, int dh, int dw)
+{
+    AG_REQUIRE(B >= 0 && C >= 0 && H >= 0 && W >= 0, AG_ERR_INVALID_DIMS,
+               "%s: negative extent (B=%d C=%d H=%d W=%d)", who, B, C, H, W);
+    AG_REQUIRE(kh >= 1 && kw >= 1 && sh >= 1 && sw >= 1 && dh >= 1 && dw >= 1 && ph >= 0 && pw >= 0,
+               AG_ERR_INVALID_DIMS,
+               "%s: kernel/stride/dilation must be >= 1 and pad >= 0 (k=%dx%d s=%dx%d d=%dx%d p=%dx%d)",
+               who, kh, kw, sh, sw, dh, dw, ph, pw);
+    return AG_OK;
+}
+
+}  // namespace ag
+
+using namespace ag;
+
+extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *cols, int B, int C,
+                                     int H, int W, int kh, int kw, int ph, int pw, int sh, int sw,
+                                     int dh, int dw)
+{
+    if (ag_status_t s = check_geom("im2col", B, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw)) return s;
+    const int OH = ag_conv_out_size(H, kh, ph, sh, dh);
+    const int OW = ag_conv_out_size(W, kw, pw, sw, dw);
+    AG_REQUIRE(H + 2 * ph >= dh * (kh - 1) + 1 && W + 2 * pw >= dw * (kw - 1) + 1,
+               AG_ERR_INVALID_DIMS, "im2col: kernel extent exceeds the padded image (%dx%d, k=%dx%d d=%dx%d p=%dx%d)",
+               H, W, kh, kw, dh, dw, ph, pw);
+    const long long planes = (long long)B * C;
+    if (planes == 0 || OH <= 0 || OW <= 0) return AG_OK;
+    AG_REQUIRE(x && cols, AG_ERR_INVALID_DIMS, "im2col: null pointer");
+    ConvGeom g{C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW};
+
+    const int WL = (OW - 1) * sw + (kw - 1) * dw + 1;  // staged row length
+    const int rows_min = (kh - 1) * dh + 1;            // input rows for one output row
+    const long long lds_one = (long long)rows_min * WL * 4;
+    if (lds_one <= kIm2colLdsBytes) {
+        // Largest band whose staged rows fit the LDS budget.
+        int R = (int)((kIm2colLdsBytes / 4 / WL - rows_min) / sh + 1);
+        if (R > OH) R = OH;
+        if (R < 1) R = 1;
+        const int bands = (OH + R - 1) / R;
+        const long long blocks = planes * bands;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "im2col: too many tiles (%lld)", blocks);
+        const size_t lds = (size_t)((R - 1) * sh + rows_min) * WL * 4;
+        const bool vec4 = (OW % 4 == 0) && aligned16(cols);
+        if (vec4)
+            hipLaunchKernelGGL(im2col_lds_kernel<true>, dim3((unsigned)blocks), dim3(kIm2colThreads),
+                               lds, as_stream(stream), x, cols, g, R, bands, WL);
+        else
+            hipLaunchKernelGGL(im2col_lds_kernel<false>, dim3((unsigned)blocks),
+                               dim3(kIm2colThreads), lds, as_stream(stream), x, cols, g, R, bands, WL);
+    } else {
+        const long long total = planes * kh * kw * (long long)OH * OW;
+        long long blocks = (total + 255) / 256;
+        if (blocks > 1048576) blocks = 1048576;
+        hipLaunchKernelGGL(im2col_direct_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), x, cols, g, total);
+    }
+    return check_launch("im2col");
+}
+
+extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, float *gx, int B, int C,
+                                     int H, int W, int kh, int kw, int ph, int pw, int sh, int sw,
+                                     int dh, int dw, int OH, int OW)
+{
+    if (ag_status_t s = check_geom("col2im", B, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw)) return s;
+    AG_REQUIRE(OH >= 0 && OW >= 0, AG_ERR_INVALID_DIMS, "col2im: negative output extent (%dx%d)", OH, OW);
+    const long long planes = (long long)B * C;
+    if (planes == 0 || H == 0 || W == 0) return AG_OK;
+    AG_REQUIRE(gx && (cols || OH == 0 || OW == 0), AG_ERR_INVALID_DIMS, "col2im: null pointer");
+    AG_REQUIRE((long long)H * W <= 0x7fffffffLL, AG_ERR_INVALID_DIMS, "col2im: plane too large");
+    ConvGeom g{C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW};
+    const int chunks = (H * W + 255) / 256;
+    const long long blocks = planes * chunks;
+    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "col2im: too many tiles (%lld)", blocks);
+    if (sh == 1 && sw == 1)
+        hipLaunchKernelGGL(col2im_gather_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), cols, gx, g, chunks);
+    else
+        hipLaunchKernelGGL(col2im_gather_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), cols, gx, g, chunks);
+    return check_launch("col2im");
+}

@@ -1,0 +1,596 @@
+"""GPU parity tests: every kernel is called through the C ABI (libag_hip.so) and compared with
+the CPU oracle on the same seeded inputs.
+
+Bars (from the hot path's stated tolerance):
+  * index / data-movement results (im2col, col2im given identical cols, pool output, pool argmax,
+    pool backward, ReLU, broadcasts) are BIT-EXACT;
+  * floating-point results satisfy |got - ref| <= 1e-5 + 1e-4*|ref| element-wise against the f32
+    oracle.  For long, cancelling contractions no f32 algorithm (the reference's BLAS included)
+    meets that bound near zero, so those cases use the conditioning-aware form
+    |got - truth_f64| <= 1e-5 + 1e-4 * (|A|.|B|), where |A|.|B| is the same contraction of
+    absolute values; each such test says so.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+@pytest.fixture(scope="module")
+def K():
+    import __graft_entry__ as entry
+    entry.load_package()
+    from rust_autograd_amd import kernels
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return kernels
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.detach().cpu().numpy()
+
+
+def assert_close(got, ref, what=""):
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    err = np.abs(got - ref)
+    tol = ATOL + RTOL * np.abs(ref)
+    bad = err > tol
+    assert not bad.any(), (f"{what}: {bad.sum()} of {bad.size} elements outside 1e-5 + 1e-4|ref|; "
+                           f"worst err {err.max():.3e} (ref {ref.reshape(-1)[err.argmax()]:.3e})")
+
+
+def assert_close_conditioned(got, truth, absdot, what=""):
+    got, truth, absdot = (np.asarray(a, dtype=np.float64) for a in (got, truth, absdot))
+    err = np.abs(got - truth)
+    tol = ATOL + RTOL * absdot
+    bad = err > tol
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} outside 1e-5 + 1e-4*(|A|.|B|); worst {err.max():.3e}"
+
+
+# =============================================================================== im2col / col2im
+GEOMS = [  # B, C, H, W, kh, kw, pad, stride, dil
+    (2, 2, 3, 3, 2, 2, 0, 1, 1),      # reference unit test geometry
+    (2, 3, 5, 5, 3, 3, 1, 2, 1),
+    (3, 4, 28, 28, 3, 3, 1, 1, 1),    # config 1 / 2 first conv
+    (2, 5, 14, 14, 3, 3, 2, 1, 2),    # config 5 dilated geometry
+    (2, 3, 28, 28, 4, 4, 1, 2, 1),    # config 5 transposed-conv geometry (seen from its output)
+    (1, 2, 9, 7, 2, 3, 1, 3, 1),      # ragged: OW not a multiple of 4
+    (2, 2, 56, 56, 3, 3, 1, 1, 1),    # north-star plane
+    (2, 2, 56, 56, 3, 3, 1, 2, 1),    # north-star stride-2 variant
+    (1, 1, 4, 4, 1, 1, 0, 1, 1),
+    (1, 2, 70, 300, 3, 3, 1, 1, 1),   # several row bands per plane
+    (1, 1, 3, 9000, 3, 3, 1, 1, 1),   # row too wide to stage: direct path
+]
+
+
+def test_im2col_reference_vector(K, orc, golden):
+    g = golden["im2col_batch"]
+    img = np.array(g["x_per_image"], dtype=np.float32).reshape(g["xch"], g["xh"], g["xw"])
+    x = np.stack([img] * g["batch"])
+    say("im2col golden")
+    cols = host(K.im2col(dev(x), g["kh"], g["kw"], g["pad"], g["pad"], g["stride"], g["stride"],
+                         g["dilation"], g["dilation"]))
+    assert cols.reshape(-1).tolist() == [float(v) for v in g["expected"]]
+
+
+@pytest.mark.parametrize("geom", GEOMS)
+def test_im2col_bit_exact(K, orc, rng, geom):
+    B, C, H, W, kh, kw, p, s, d = geom
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    say("im2col", geom)
+    got = host(K.im2col(dev(x), kh, kw, p, p, s, s, d, d))
+    want = orc.im2col(x, kh, kw, p, p, s, s, d, d)
+    assert got.shape == want.shape and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_im2col_unaligned_output_pointer(K, orc, rng):
+    """cols not 16-byte aligned: the scalar store path must give the same bits."""
+    x = rng.standard_normal((1, 2, 8, 8)).astype(np.float32)
+    L = K.capi.lib()
+    buf = torch.zeros(1 + 2 * 9 * 64, dtype=torch.float32, device="cuda")
+    cols = buf[1:]
+    say("im2col unaligned")
+    K.check(L.ag_im2col_f32(K._stream(), K._ptr(dev(x)), K.C.c_void_p(cols.data_ptr()), 1, 2, 8, 8, 3, 3, 1, 1,
+                            1, 1, 1, 1))
+    want = orc.im2col(x, 3, 3, 1, 1, 1, 1, 1, 1)
+    assert np.array_equal(host(cols).reshape(want.shape), want) and host(buf)[0] == 0
+
+
+@pytest.mark.parametrize("geom", GEOMS)
+def test_col2im_bit_exact(K, orc, rng, geom):
+    B, C, H, W, kh, kw, p, s, d = geom
+    OH, OW = orc.conv_out_size(H, kh, p, s, d), orc.conv_out_size(W, kw, p, s, d)
+    cols = rng.standard_normal((B, C * kh * kw, OH * OW)).astype(np.float32)
+    say("col2im", geom)
+    got = host(K.col2im(dev(cols), C, H, W, kh, kw, p, p, s, s, d, d, OH, OW))
+    want = orc.col2im(cols, C, H, W, kh, kw, p, p, s, s, d, d, OH, OW)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_col2im_into_reference_reconstructed_extent(K, orc, rng):
+    """Stride 2 on 56x56: the reference reconstructs 55x55 (conv2d_transpose.rs:55-56); the same
+    columns scattered into 55x55 equal the crop of the 56x56 result."""
+    B, C, H, k, p, s = 2, 3, 56, 3, 1, 2
+    OH = orc.conv_out_size(H, k, p, s, 1)
+    cols = rng.standard_normal((B, C * 9, OH * OH)).astype(np.float32)
+    say("col2im 55 vs 56")
+    small = host(K.col2im(dev(cols), C, 55, 55, k, k, p, p, s, s, 1, 1, OH, OH))
+    full = host(K.col2im(dev(cols), C, 56, 56, k, k, p, p, s, s, 1, 1, OH, OH))
+    assert np.array_equal(small, orc.col2im(cols, C, 55, 55, k, k, p, p, s, s, 1, 1, OH, OH))
+    assert np.array_equal(small, full[:, :, :55, :55])
+
+
+# =============================================================================== GEMM
+def test_matmul_reference_vectors(K, golden):
+    def mk(e, key):
+        return np.ones(e[key + "_ones"], np.float32) if key + "_ones" in e else np.array(e[key], np.float32)
+    for e in golden["matmul"]:
+        say("matmul golden", e["source"])
+        c = host(K.matmul(dev(mk(e, "a")), dev(mk(e, "b")), e["ta"], e["tb"]))
+        assert c.reshape(-1).tolist() == [float(v) for v in e["expected"]]
+    for e in golden["batch_matmul"]:
+        say("batch_matmul golden", e["source"])
+        c = host(K.batch_matmul(dev(mk(e, "a")), dev(mk(e, "b")), e["ta"], e["tb"]))
+        if "expected_fill" in e:
+            assert list(c.shape) == e["expected_shape"] and np.all(c == e["expected_fill"])
+        else:
+            assert np.array_equal(c, np.array(e["expected"], np.float32))
+
+
+GEMM_SHAPES = [(1, 1, 1), (2, 5, 1), (7, 9, 11), (32, 784, 9), (64, 196, 288), (128, 10, 3136), (128, 3136, 10),
+               (3136, 10, 128), (129, 130, 33), (128, 128, 32), (256, 192, 64), (100, 300, 77), (33, 65, 260)]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+def test_gemm_all_layouts(K, orc, rng, shape, ta, tb):
+    m, n, k = shape
+    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+    say("gemm", shape, ta, tb)
+    got = host(K.matmul(dev(a), dev(b), bool(ta), bool(tb)))
+    A = a.T if ta else a
+    Bm = b.T if tb else b
+    truth = A.astype(np.float64) @ Bm.astype(np.float64)
+    assert_close_conditioned(got, truth, np.abs(A).astype(np.float64) @ np.abs(Bm).astype(np.float64), "gemm")
+    if k <= 64:   # short contractions: the plain bound against the f32 oracle holds as well
+        assert_close(got, orc.matmul(a, b, ta, tb), "gemm vs f32 oracle")
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
+def test_gemm_every_tile_configuration(K, rng, cfg):
+    L = K.capi.lib()
+    m, n, k = 200, 333, 130
+    a = rng.random((m, k), dtype=np.float32)
+    b = rng.random((k, n), dtype=np.float32)
+    say("gemm cfg", cfg)
+    L.ag_gemm_force_config(cfg)
+    try:
+        got = host(K.matmul(dev(a), dev(b)))
+        got_t = host(K.matmul(dev(a.T.copy()), dev(b.T.copy()), True, True))
+    finally:
+        L.ag_gemm_force_config(-1)
+    truth = a.astype(np.float64) @ b.astype(np.float64)
+    assert_close(got, truth, "gemm NN")      # positive inputs: no cancellation, plain bound applies
+    assert_close(got_t, truth, "gemm TT")
+
+
+def test_gemm_leading_dims_alpha_beta_batch(K, rng):
+    m, n, k, batch = 45, 70, 52, 3
+    lda, ldb, ldc = k + 4, n + 8, n + 3
+    a = rng.random((batch, m, lda), dtype=np.float32)
+    b = rng.random((batch, k, ldb), dtype=np.float32)
+    c0 = rng.random((batch, m, ldc), dtype=np.float32)
+    cd = dev(c0)
+    say("gemm lda/ldb/ldc alpha beta batch")
+    K.gemm(0, 0, m, n, k, 0.5, dev(a), lda, m * lda, dev(b), ldb, k * ldb, -1.5, cd, ldc, m * ldc, batch)
+    got = host(cd)
+    want = c0.astype(np.float64).copy()
+    want[:, :, :n] = 0.5 * (a[:, :, :k].astype(np.float64) @ b[:, :, :n].astype(np.float64)) - 1.5 * c0[:, :, :n]
+    assert_close(got, want, "strided gemm")
+    assert np.array_equal(got[:, :, n:], c0[:, :, n:]), "padding columns of C were touched"
+
+
+def test_gemm_shared_operand_and_unaligned_pointers(K, rng):
+    """stride 0 shares A across the batch (the conv forward's filter matrix); operands offset by
+    one float take the 32-bit load path."""
+    m, n, k, batch = 32, 50, 27, 4
+    abuf = dev(rng.random(1 + m * k, dtype=np.float32))
+    bbuf = dev(rng.random(1 + batch * k * n, dtype=np.float32))
+    a, b = abuf[1:], bbuf[1:]
+    c = torch.empty(batch, m, n, device="cuda")
+    say("gemm shared A, unaligned")
+    K.gemm(0, 0, m, n, k, 1.0, a, k, 0, b, n, k * n, 0.0, c, n, m * n, batch)
+    A = host(a).reshape(m, k).astype(np.float64)
+    Bm = host(b).reshape(batch, k, n).astype(np.float64)
+    assert_close(host(c), A[None] @ Bm, "shared-A gemm")
+
+
+@pytest.mark.parametrize("batch", [1, 3, 64, 130])
+def test_gemm_batchsum_matches_sequential_accumulation(K, orc, rng, batch):
+    """sum_b A_b * B_b^T: the filter-gradient contraction (conv2d.rs:668-687)."""
+    m, n, k = 40, 72, 196
+    a = rng.standard_normal((batch, m, k)).astype(np.float32)
+    b = rng.standard_normal((batch, n, k)).astype(np.float32)
+    c = torch.empty(m, n, device="cuda")
+    say("gemm_batchsum", batch)
+    K.gemm_batchsum(0, 1, m, n, k, 1.0, dev(a), k, m * k, dev(b), k, n * k, 0.0, c, n, batch)
+    truth = np.einsum("bmk,bnk->mn", a.astype(np.float64), b.astype(np.float64))
+    absdot = np.einsum("bmk,bnk->mn", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
+    assert_close_conditioned(host(c), truth, absdot, "batchsum")
+    # and it is deterministic
+    c2 = torch.empty(m, n, device="cuda")
+    K.gemm_batchsum(0, 1, m, n, k, 1.0, dev(a), k, m * k, dev(b), k, n * k, 0.0, c2, n, batch)
+    assert np.array_equal(host(c), host(c2))
+
+
+def test_gemm_degenerate_k_and_beta(K, rng):
+    c0 = rng.random((5, 6), dtype=np.float32)
+    c = dev(c0)
+    say("gemm K=0")
+    K.gemm(0, 0, 5, 6, 0, 1.0, c, 1, 0, c, 6, 0, 2.0, c, 6, 0, 1)
+    assert np.array_equal(host(c), 2.0 * c0)
+
+
+def test_matmul_shape_errors_follow_reference(K):
+    a = torch.zeros(3, 4, device="cuda")
+    b = torch.zeros(5, 6, device="cuda")
+    with pytest.raises(K.capi.IncompatibleShape, match="not compatible for matrix multiplication"):
+        K.matmul(a, b)
+    with pytest.raises(K.capi.IncompatibleShape, match="Input shapes mismatch"):
+        K.batch_matmul(torch.zeros(2, 3, 4, device="cuda"), torch.zeros(3, 4, 5, device="cuda"))
+    with pytest.raises(K.capi.IncompatibleShape, match="ndim must be >= 2"):
+        K.batch_matmul(torch.zeros(4, device="cuda"), torch.zeros(4, 4, device="cuda"))
+
+
+# =============================================================================== convolution ops
+CONV_CASES = [  # B, C, K, H, W, k, pad, stride, dil
+    (2, 3, 4, 5, 5, 3, 1, 2, 1),       # tests/test_tensor_ops_grad.rs:1473-1493 geometry
+    (4, 1, 32, 28, 28, 3, 1, 1, 1),    # config 1 (4 of its 64 images)
+    (3, 32, 64, 14, 14, 3, 1, 1, 1),   # config 2 second conv
+    (2, 64, 128, 56, 56, 3, 1, 1, 1),  # north star, 2 of 256 images
+    (2, 64, 128, 56, 56, 3, 1, 2, 1),  # north star stride-2 variant
+    (2, 256, 256, 14, 14, 3, 2, 1, 2), # config 5 dilated, 2 of 32 images
+    (2, 5, 7, 9, 11, 2, 0, 1, 1),      # ragged
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_forward_and_gradients(K, orc, rng, case):
+    B, C, Kc, H, W, k, p, s, d = case
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    sc = np.sqrt(6.0 / Kc)                                   # glorot_uniform on [K, C*k*k] (ndarray_ext.rs:335-340)
+    w = rng.uniform(-sc, sc, (Kc, C, k, k)).astype(np.float32)
+    say("conv2d fwd", case)
+    y, cols = K.conv2d(dev(x), dev(w), p, s, d)
+    oy32, ocols = orc.conv2d_fwd(x, w, p, s, d)
+    oy64, _ = orc.conv2d_fwd(x.astype(np.float64), w.astype(np.float64), p, s, d)
+    ay, _ = orc.conv2d_fwd(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), p, s, d)
+    assert np.array_equal(host(cols), ocols), "cols (op output 1) must be bit-exact"
+    assert_close_conditioned(host(y), oy64, ay, "conv2d y")
+    if C * k * k <= 600:
+        assert_close(host(y), oy32, "conv2d y vs f32 oracle")
+
+    gy = rng.standard_normal(oy32.shape).astype(np.float32)
+    say("conv2d filter grad", case)
+    gw = K.conv2d_filter_grad(cols, dev(gy), w.shape)
+    ogw64 = orc.conv2d_filter_grad(ocols.astype(np.float64), gy.astype(np.float64), w.shape)
+    agw = orc.conv2d_filter_grad(np.abs(ocols).astype(np.float64), np.abs(gy).astype(np.float64), w.shape)
+    assert_close_conditioned(host(gw), ogw64, agw, "filter grad")
+
+    say("conv2d input grad", case)
+    gx, gcols = K.conv2d_transpose(dev(gy), dev(w), p, s, d, out_hw=(H, W), return_cols=True)
+    ogx64 = orc.conv2d_transpose(gy.astype(np.float64), w.astype(np.float64), p, s, d, out_hw=(H, W))
+    agx = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, s, d, out_hw=(H, W))
+    assert_close_conditioned(host(gx), ogx64, agx, "input grad")
+    # col2im stage alone is bit-exact on the GPU's own columns
+    OH, OW = oy32.shape[2:]
+    assert np.array_equal(host(gx), orc.col2im(host(gcols), C, H, W, k, k, p, p, s, s, d, d, OH, OW))
+    # the reference's reconstructed size (may be a crop)
+    say("conv2d input grad, reference size", case)
+    gx_ref = host(K.conv2d_transpose(dev(gy), dev(w), p, s, d))
+    rh, rw = gx_ref.shape[2:]
+    assert rh == orc.conv_transpose_out_size(OH, k, p, s, d) and rh <= H
+    assert np.array_equal(gx_ref, host(gx)[:, :, :rh, :rw])
+
+
+def test_conv2d_all_ones_closed_form(K):
+    """Ones input and ones filter: y = C * (number of in-bounds taps); exact integers in f32."""
+    B, C, Kc, H = 2, 64, 128, 56
+    x = torch.ones(B, C, H, H, device="cuda")
+    w = torch.ones(Kc, C, 3, 3, device="cuda")
+    say("conv2d ones")
+    y, _ = K.conv2d(x, w, 1, 1)
+    taps = np.full((H, H), 9.0)
+    taps[0, :] = taps[-1, :] = taps[:, 0] = taps[:, -1] = 6.0
+    taps[0, 0] = taps[0, -1] = taps[-1, 0] = taps[-1, -1] = 4.0
+    assert np.array_equal(host(y), np.broadcast_to(C * taps, (B, Kc, H, H)).astype(np.float32))
+
+
+def test_deconv_reference_vector(K, golden):
+    g = golden["deconv"]
+    say("deconv golden")
+    out = host(K.conv2d_transpose(torch.ones(g["g_shape"], device="cuda"), torch.ones(g["w_shape"], device="cuda"),
+                                  g["pad"], g["stride"]))
+    assert list(out.shape) == g["expected_shape"]
+    assert np.array_equal(out, np.broadcast_to(np.array(g["expected_plane"], np.float32).reshape(3, 3), out.shape))
+
+
+@pytest.mark.parametrize("case", [(2, 3, 2, 4, 4, 2, 0, 1, 1), (2, 128, 64, 14, 14, 4, 1, 2, 1),
+                                  (2, 4, 3, 5, 5, 4, 1, 2, 1)])
+def test_conv2d_transpose_and_filter_grad(K, orc, rng, case):
+    """Public transposed conv (config 5: 128->64, 4x4, stride 2, pad 1, 14x14 -> 28x28)."""
+    B, ych, xch, yh, yw, k, p, s, d = case
+    x = rng.standard_normal((B, ych, yh, yw)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (ych, xch, k, k)).astype(np.float32)
+    say("conv2d_transpose", case)
+    out = K.conv2d_transpose(dev(x), dev(w), p, s, d)
+    o64 = orc.conv2d_transpose(x.astype(np.float64), w.astype(np.float64), p, s, d)
+    oabs = orc.conv2d_transpose(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), p, s, d)
+    assert tuple(out.shape) == o64.shape
+    assert_close_conditioned(host(out), o64, oabs, "conv2d_transpose")
+    assert_close(host(out), orc.conv2d_transpose(x, w, p, s, d), "conv2d_transpose vs f32 oracle")
+    go = rng.standard_normal(o64.shape).astype(np.float32)
+    say("conv2d_transpose filter grad", case)
+    gw = K.conv2d_transpose_filter_grad(dev(x), dev(go), w.shape, p, s, d)
+    g64 = orc.conv2d_transpose_filter_grad(x.astype(np.float64), go.astype(np.float64), w.shape, p, s, d)
+    gabs = orc.conv2d_transpose_filter_grad(np.abs(x).astype(np.float64), np.abs(go).astype(np.float64), w.shape, p, s, d)
+    assert_close_conditioned(host(gw), g64, gabs, "conv2d_transpose filter grad")
+
+
+def test_conv2d_errors_follow_reference(K):
+    x = torch.zeros(1, 3, 8, 8, device="cuda")
+    with pytest.raises(K.capi.IncompatibleShape, match=r"conv2d: filter must be 4D"):
+        K.conv2d(x, torch.zeros(4, 3, 3, device="cuda"), 1, 1)
+    with pytest.raises(K.capi.IncompatibleShape, match=r"input channel dim \(3\) must match filter's second dim \(2\)"):
+        K.conv2d(x, torch.zeros(4, 2, 3, 3, device="cuda"), 1, 1)
+    with pytest.raises(K.capi.TypeUnsupported):
+        K.conv2d(x.double(), torch.zeros(4, 3, 3, 3, device="cuda"), 1, 1)
+
+
+# =============================================================================== max pooling
+def test_max_pool_reference_vector(K, golden):
+    g = golden["max_pool"]
+    x = np.array(g["x"], dtype=np.float32).reshape(g["batch"], g["ch"], g["xh"], g["xw"])
+    say("max_pool golden")
+    y, am, il = K.max_pool2d(dev(x), g["size"], g["pad"], g["stride"])
+    assert host(y).reshape(-1).tolist() == [float(v) for v in g["expected_output"]]
+    assert host(am).reshape(-1).tolist() == [float(v) for v in g["expected_argmax"]]
+    assert host(il).reshape(-1).tolist() == g["expected_argmax"]
+
+
+POOL_CASES = [(2, 3, 6, 6, 2, 2), (2, 3, 7, 9, 3, 2), (1, 2, 8, 8, 3, 1), (3, 32, 28, 28, 2, 2),
+              (2, 16, 56, 56, 3, 2), (1, 1, 5, 7, 2, 3), (1, 3, 33, 65, 3, 2)]
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
+    B, C, H, W, size, stride = case
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    x[0, 0, :2, :4] = 0.5                                       # ties: first element must win
+    say("max_pool fwd", case)
+    y, am, il = K.max_pool2d(dev(x), size, 0, stride)
+    oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, stride)
+    assert np.array_equal(host(y), oy)
+    assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32)), "argmax must be bit-exact"
+    assert np.array_equal(host(il), oil)
+    gy = rng.standard_normal(oy.shape).astype(np.float32)
+    ogx, skipped = orc.maxpool2d_bwd(gy, oam, x.shape)
+    assert skipped == 0
+    say("max_pool bwd (f32 argmax)", case)
+    gx_f = host(K.max_pool2d_grad(dev(gy), am, None, x.shape, size, 0, stride))
+    say("max_pool bwd (int32 index)", case)
+    gx_i = host(K.max_pool2d_grad(dev(gy), am, il, x.shape, size, 0, stride))
+    assert np.array_equal(gx_f.view(np.uint32), ogx.view(np.uint32))
+    assert np.array_equal(gx_i.view(np.uint32), ogx.view(np.uint32))
+    ggx = rng.standard_normal(x.shape).astype(np.float32)
+    say("max_pool gradgrad", case)
+    for idx in (None, il):
+        ggy = host(K.max_pool2d_grad_grad(dev(ggx), am, idx, size, 0, stride))
+        assert np.array_equal(ggy, orc.maxpool2d_gradgrad(ggx, oam, oy.shape))
+
+
+def test_max_pool_nan_window_and_pad_error(K, orc):
+    x = np.zeros((1, 2, 4, 4), dtype=np.float32)
+    x[0, 1] = np.nan
+    say("max_pool NaN")
+    y, am, il = K.max_pool2d(dev(x), 2, 0, 2)
+    oy, oam, oil = orc.maxpool2d_fwd(x, 2, 0, 2)
+    assert np.array_equal(host(y), oy) and np.array_equal(host(am), oam) and np.array_equal(host(il), oil)
+    with pytest.raises(K.capi.InvalidDims, match="pad must be 0"):
+        K.max_pool2d(dev(x), 2, 1, 2)
+
+
+def test_max_pool_above_2_pow_24_elements(K, orc, rng):
+    """33.5 M elements: the f32 argmax is the rounded offset (bit-exact with the reference's
+    encoding), the int32 plane index is exact, the backward refuses the f32 indices and is
+    bit-exact with the exact-index oracle."""
+    B, C, H, W = 2, 64, 512, 512
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    say("max_pool 2^25 fwd")
+    y, am, il = K.max_pool2d(dev(x), 2, 0, 2)
+    oy, oam, oil = orc.maxpool2d_fwd(x, 2, 0, 2)
+    assert np.array_equal(host(y), oy)
+    assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32))
+    assert np.array_equal(host(il), oil)
+    gy = rng.standard_normal(oy.shape).astype(np.float32)
+    with pytest.raises(K.capi.InvalidDims, match="2\\^24"):
+        K.max_pool2d_grad(dev(gy), am, None, x.shape, 2, 0, 2)
+    say("max_pool 2^25 bwd")
+    gx = host(K.max_pool2d_grad(dev(gy), am, il, x.shape, 2, 0, 2))
+    assert np.array_equal(gx, orc.maxpool2d_bwd_local(gy, oil, x.shape))
+
+
+# =============================================================================== reductions
+def test_reduce_mean_reference_value(K, golden):
+    g = golden["reduce_mean"]
+    say("reduce_mean golden")
+    out = host(K.reduce_mean(dev(np.array(g["x"], np.float32)), g["axes"], g["keep_dims"]))
+    assert out.shape == () and float(out) == g["expected"]
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 64, 1000, 4099, 1 << 20, (1 << 22) + 3])
+def test_sum_all(K, orc, rng, n):
+    x = rng.random(n, dtype=np.float32)
+    say("sum_all", n)
+    got = float(host(K.sum_all(dev(x)))) if n else float(host(K.sum_all(torch.zeros(0, device="cuda"))))
+    assert_close(got, float(x.astype(np.float64).sum()), "sum_all vs f64")
+    assert_close(got, float(orc.sum_all(x)), "sum_all vs f32 oracle")
+
+
+def test_sum_all_exact_on_integers(K):
+    n = 4099
+    say("sum_all arange")
+    assert float(host(K.sum_all(torch.arange(1, n + 1, device="cuda", dtype=torch.float32)))) == n * (n + 1) // 2
+
+
+@pytest.mark.parametrize("axes", [[0], [1], [2], [3], [0, 2], [1, 3], [0, 1, 2, 3], [-1], [3, 0], []])
+@pytest.mark.parametrize("keep", [False, True])
+def test_reduce_sum_and_mean(K, orc, rng, axes, keep):
+    x = rng.standard_normal((3, 4, 5, 6)).astype(np.float32)
+    say("reduce", axes, keep)
+    for mean in (False, True):
+        got = host(K.reduce_sum(dev(x), axes, keep, mean))
+        want = orc.reduce_sum(x, axes, keep, mean)
+        assert got.shape == want.shape
+        ax = tuple(a % 4 for a in axes)
+        cond = np.abs(x).astype(np.float64).sum(axis=ax, keepdims=keep) / (np.prod([x.shape[a] for a in ax]) if mean and ax else 1)
+        truth = (x.astype(np.float64).mean(axis=ax, keepdims=keep) if mean and ax
+                 else x.astype(np.float64).sum(axis=ax, keepdims=keep))
+        assert_close_conditioned(got, truth, cond, "reduce")
+        if 3 not in ax:   # no innermost-axis fold: same sequential order as the reference => same bits
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_reduce_mean_config2_loss_shape(K, orc, rng):
+    x = rng.random((128, 1), dtype=np.float32)
+    say("reduce_mean [128,1] over axis 0")
+    got = host(K.reduce_mean(dev(x), [0]))
+    assert got.shape == (1,) and np.array_equal(got, orc.reduce_mean(x, [0]))
+
+
+def test_reduce_large_rows_and_columns(K, rng):
+    x = rng.random((2048, 1024), dtype=np.float32)
+    say("reduce [2048,1024]")
+    assert_close(host(K.reduce_sum(dev(x), [1])), x.astype(np.float64).sum(1), "row sums")
+    assert_close(host(K.reduce_sum(dev(x), [0])), x.astype(np.float64).sum(0), "column sums")
+
+
+def test_broadcast_grad(K, orc, rng):
+    gy = rng.standard_normal((3, 1, 5, 1)).astype(np.float32)
+    say("broadcast_grad")
+    assert np.array_equal(host(K.broadcast_grad(dev(gy), (3, 4, 5, 6), [1, 3])), np.broadcast_to(gy, (3, 4, 5, 6)))
+    s = host(K.broadcast_grad(dev(np.array(2.5, np.float32)), (64, 32, 14, 14), [0, 1, 2, 3]))
+    assert s.shape == (64, 32, 14, 14) and np.all(s == 2.5)
+
+
+# =============================================================================== Adam
+@pytest.mark.parametrize("n", [1, 10, 288, 18432, 31360, 100003])
+def test_adam_matches_oracle_over_steps(K, orc, rng, n):
+    p = rng.standard_normal(n).astype(np.float32)
+    m, v, t = np.zeros(n, np.float32), np.zeros(n, np.float32), np.array([1.0], np.float32)
+    pd, md, vd, td = dev(p), dev(m), dev(v), dev(t)
+    say("adam", n)
+    for step in range(4):
+        g = rng.standard_normal(n).astype(np.float32)
+        orc.adam(p, g, m, v, t)
+        K.adam_update(pd, dev(g), md, vd, td)
+    assert host(td)[0] == t[0] == 5.0
+    # m and v involve no transcendental: bit-exact; p goes through powf (device vs host libm)
+    assert np.array_equal(host(md).view(np.uint32), m.view(np.uint32))
+    assert np.array_equal(host(vd).view(np.uint32), v.view(np.uint32))
+    assert_close(host(pd), p, "adam param")
+
+
+def test_adam_first_step_closed_form(K, rng):
+    n = 5000
+    g = rng.standard_normal(n).astype(np.float32)
+    p0 = rng.standard_normal(n).astype(np.float32)
+    pd = dev(p0)
+    say("adam closed form")
+    K.adam_update(pd, dev(g), dev(np.zeros(n, np.float32)), dev(np.zeros(n, np.float32)),
+                  dev(np.array([1.0], np.float32)))
+    want = p0.astype(np.float64) - 1e-3 * g.astype(np.float64) / (np.abs(g.astype(np.float64)) + 1e-8)
+    assert_close(host(pd), want, "adam step 1")
+
+
+# =============================================================================== glue
+def test_relu_bias_addn_mul_fill(K, orc, rng):
+    x = rng.standard_normal((37, 10)).astype(np.float32)
+    gy = rng.standard_normal((37, 10)).astype(np.float32)
+    say("glue")
+    assert np.array_equal(host(K.relu(dev(x))), orc.relu(x))
+    assert np.array_equal(host(K.relu_grad(dev(x), dev(gy))), orc.relu_grad(x, gy))
+    b = rng.standard_normal((1, 10)).astype(np.float32)
+    assert np.array_equal(host(K.add_bias(dev(x), dev(b))), orc.add_bias(x, b.reshape(-1)))
+    assert np.array_equal(host(K.bias_grad(dev(gy))), orc.reduce_sum(gy, [0], keep_dims=True))
+    xs = [rng.standard_normal(1001).astype(np.float32) for _ in range(5)]
+    assert np.array_equal(host(K.add_n([dev(a) for a in xs])), orc.add_n(xs))
+    assert np.array_equal(host(K.mul(dev(x), dev(gy))), x * gy)
+    assert np.array_equal(host(K.scale(dev(x), 0.25)), x * np.float32(0.25))
+    assert np.all(host(K.fill((3, 5), 1.5)) == 1.5)
+
+
+def test_sparse_softmax_cross_entropy(K, orc, rng):
+    logits = (rng.standard_normal((128, 10)) * 3).astype(np.float32)
+    labels = rng.integers(0, 10, size=(128, 1)).astype(np.float32)
+    say("xent")
+    loss, lsm = K.sparse_softmax_cross_entropy(dev(logits), dev(labels))
+    oloss, olsm = orc.sparse_softmax_xent(logits, labels)
+    assert tuple(loss.shape) == (128, 1)
+    assert_close(host(loss), oloss, "xent loss")
+    assert_close(host(lsm), olsm, "log softmax")
+    gy = rng.standard_normal((128, 1)).astype(np.float32)
+    gx = K.sparse_softmax_cross_entropy_grad(lsm, dev(labels), dev(gy))
+    assert_close(host(gx), orc.sparse_softmax_xent_grad(olsm, labels, gy), "xent grad")
+    with pytest.raises(K.capi.IncompatibleShape, match="ndim is not 2"):
+        K.sparse_softmax_cross_entropy(dev(logits.reshape(-1)), dev(labels))
+
+
+# =============================================================================== end-to-end config 1
+def test_config1_conv_block_forward_backward(K, orc, rng):
+    """conv(1->32, 3x3, pad 1) -> ReLU -> max_pool 2x2/2 -> sum; grads w.r.t. x and w."""
+    B = 64
+    x = rng.random((B, 1, 28, 28), dtype=np.float32)
+    sc = np.sqrt(6.0 / 32)
+    w = rng.uniform(-sc, sc, (32, 1, 3, 3)).astype(np.float32)
+    say("config 1")
+    y, cols = K.conv2d(dev(x), dev(w), 1, 1)
+    r = K.relu(y)
+    p, am, il = K.max_pool2d(r, 2, 0, 2)
+    loss = K.sum_all(p)
+    gp = K.broadcast_grad(K.fill((), 1.0), tuple(p.shape), [0, 1, 2, 3])
+    gr = K.max_pool2d_grad(gp, am, None, tuple(r.shape), 2, 0, 2)
+    gyd = K.relu_grad(y, gr)
+    gw = K.conv2d_filter_grad(cols, gyd, w.shape)
+    gx = K.conv2d_transpose(gyd, dev(w), 1, 1)
+
+    oy, ocols = orc.conv2d_fwd(x, w, 1, 1, 1)
+    assert_close(host(y), oy, "y")
+    # ReLU masks and pooling choices are discrete: a last-bit difference in y next to zero would
+    # move a whole gradient, so the stages after the conv are checked on the GPU's own y.
+    oy = host(y)
+    orl = orc.relu(oy)
+    op, oam, _ = orc.maxpool2d_fwd(orl, 2, 0, 2)
+    ogr, _ = orc.maxpool2d_bwd(np.ones_like(op), oam, orl.shape)
+    ogy = orc.relu_grad(oy, ogr)
+    assert_close(host(p), op, "pooled")
+    assert_close(float(host(loss)), float(orc.sum_all(op)), "loss")
+    assert_close(host(gw), orc.conv2d_filter_grad(ocols, ogy, w.shape), "gw")
+    assert_close(host(gx), orc.conv2d_transpose(ogy, w, 1, 1, 1), "gx")
+    assert tuple(gx.shape) == x.shape
