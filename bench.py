@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+A "step" is one conv2d forward + backward over one synthetic batch at the headline shape
+(B=256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, f32):
+
+    forward      im2col(x) -> cols ;  y   = W . cols            (Conv2D)
+    filter grad  gW = sum_b gy_b . cols_b^T                      (Conv2DFilterGrad)
+    input grad   gcols = W^T . gy ;  gx = col2im(gcols)          (Conv2DTranspose)
+
+Inputs are resident in HBM before the timed region.  Every kernel launch inside the timed steps
+is bracketed by events on the launch stream, so the per-kernel figures and the roofline object
+come from the same K steps as `value`.  The CPU baseline (the oracle's restatement of the
+reference path with OpenBLAS, timed on this machine's host cores on a bounded sample of the same
+workload) is reported beside it; it is a baseline, not a target.
+
+Prints ONE JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+
+# headline workload
+B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=B, help="images per step (headline: 256)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
+    ap.add_argument("--cpu-images", type=int, default=32, help="images in the CPU baseline sample")
+    return ap.parse_args()
+
+
+class Timer:
+    """Accumulates event-bracketed durations per kernel name on the current stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pending = []
+        self.enabled = False
+
+    def run(self, name, fn):
+        if not self.enabled:
+            return fn()
+        a = self.torch.cuda.Event(enable_timing=True)
+        b = self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn()
+        b.record()
+        self.pending.append((name, a, b))
+        return out
+
+    def totals(self):
+        self.torch.cuda.synchronize()
+        tot, cnt = {}, {}
+        for name, a, b in self.pending:
+            tot[name] = tot.get(name, 0.0) + a.elapsed_time(b)
+            cnt[name] = cnt.get(name, 0) + 1
+        return {k: tot[k] / cnt[k] for k in tot}
+
+
+def time_events(torch, fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = []
+    for _ in range(iters):
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return ts[len(ts) // 2]
+
+
+def cpu_baseline(images):
+    """conv2d fwd+bwd of the oracle (reference restatement + OpenBLAS) on `images` images."""
+    import numpy as np
+    from oracle import pyoracle as orc
+
+    orc.build()
+    blas = orc.load_openblas()
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        cores = min(cores, int(env))
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((images, C, H, W), dtype=np.float32)
+    s = np.sqrt(6.0 / K)
+    w = rng.uniform(-s, s, (K, C, KH, KH)).astype(np.float32)
+    gy = rng.standard_normal((images, K, H, W), dtype=np.float32)
+
+    def step():
+        # batch-parallel stages (rayon in the reference): one BLAS thread per image task
+        orc.blas_set_threads(1)
+        y, cols = orc.conv2d_fwd(x, w, PAD, STRIDE, DIL, threads=cores)
+        gx = orc.conv2d_transpose(gy, w, PAD, STRIDE, DIL, out_hw=(H, W), threads=cores)
+        # image-sequential filter gradient: parallelism only inside BLAS
+        orc.blas_set_threads(cores)
+        gw = orc.conv2d_filter_grad(cols, gy, w.shape)
+        return y, gx, gw
+
+    step()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        step()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > 8.0 or reps >= 20:
+            break
+    return {
+        "value": round(images * reps / dt, 2), "unit": "images/s", "cores": cores, "kind": "port",
+        "sample": f"{images} of {B} images of the same conv2d fwd+bwd workload, {reps} repetitions, "
+                  f"BLAS: {blas or 'none (built-in loops, not OpenBLAS)'}",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as entry
+    entry.load_package()
+    from rust_autograd_amd import capi, kernels as Kn
+
+    capi.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    Bn = args.batch
+    OH = Kn.conv_out_size(H, KH, PAD, STRIDE, DIL)
+    P, CK = OH * OH, C * KH * KH
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(1234)
+    x = torch.randn(Bn, C, H, W, device=dev, generator=g)
+    s = (6.0 / K) ** 0.5
+    w = (torch.rand(K, C, KH, KH, device=dev, generator=g) * 2 - 1) * s
+    gy = torch.randn(Bn, K, OH, OH, device=dev, generator=g)
+    cols = torch.empty(Bn, CK, P, device=dev)
+    y = torch.empty(Bn, K, OH, OH, device=dev)
+    gcols = torch.empty(Bn, CK, P, device=dev)
+    gx = torch.empty(Bn, C, H, W, device=dev)
+    gw = torch.empty(K, C, KH, KH, device=dev)
+    L = capi.lib()
+    ws = torch.empty(max(16, L.ag_conv2d_filter_grad_f32_workspace(Bn, CK, P, K)), dtype=torch.uint8, device=dev)
+    st, ptr, chk = Kn._stream, Kn._ptr, capi.check
+    T = Timer(torch)
+
+    def step():
+        T.run("im2col", lambda: chk(L.ag_im2col_f32(st(), ptr(x), ptr(cols), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
+                                                    STRIDE, DIL, DIL)))
+        T.run("gemm_fwd", lambda: chk(L.ag_gemm_f32(st(), 0, 0, K, P, CK, 1.0, ptr(w), CK, 0, ptr(cols), P, CK * P,
+                                                    0.0, ptr(y), P, K * P, Bn)))
+        T.run("gemm_filter_grad", lambda: chk(L.ag_gemm_batchsum_f32(st(), 0, 1, K, CK, P, 1.0, ptr(gy), P, K * P,
+                                                                     ptr(cols), P, CK * P, 0.0, ptr(gw), CK, Bn,
+                                                                     ptr(ws), ws.numel())))
+        T.run("gemm_input_grad", lambda: chk(L.ag_gemm_f32(st(), 1, 0, CK, P, K, 1.0, ptr(w), CK, 0, ptr(gy), P,
+                                                           K * P, 0.0, ptr(gcols), P, CK * P, Bn)))
+        T.run("col2im", lambda: chk(L.ag_col2im_f32(st(), ptr(gcols), ptr(gx), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
+                                                    STRIDE, DIL, DIL, OH, OH)))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    T.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+    per = T.totals()
+
+    gemm_flop = 2.0 * K * P * CK * Bn            # identical for the three contractions
+    col_bytes = 4.0 * (Bn * C * H * W + Bn * CK * P)
+    kernels = {}
+    for name in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"):
+        tf = gemm_flop / (per[name] * 1e-3) / 1e12
+        kernels[name] = {"ms": round(per[name], 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    for name in ("im2col", "col2im"):
+        gbs = col_bytes / (per[name] * 1e-3) / 1e9
+        kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+    gemm_ms = sum(per[n] for n in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"))
+    gemm_tf = 3 * gemm_flop / (gemm_ms * 1e-3) / 1e12
+    dominant = max(("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"), key=lambda n: per[n])
+    dom_tf = gemm_flop / (per[dominant] * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(dom_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                "gemm_phase_TFLOP/s": round(gemm_tf, 2),
+                "gemm_phase_frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+
+    if not args.no_micro:
+        kernels.update(micro(torch, Kn, capi, dev))
+
+    out = {
+        "metric": "conv2d fwd+bwd images/sec (B256 64->128 @56x56, 3x3 f32)",
+        "value": round(Bn / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"C4 conv2d fwd+bwd: x [{Bn},{C},{H},{W}] N(0,1), w [{K},{C},{KH},{KH}] glorot-uniform, "
+                               f"stride {STRIDE} pad {PAD}; im2col + 3 fp32-MFMA GEMMs + col2im per step"},
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_images)
+    print(json.dumps(out))
+
+
+def micro(torch, Kn, capi, dev):
+    """Per-kernel microbenchmarks at the shapes of the other configurations (median of 10)."""
+    res = {}
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+
+    # max_pool2d 3x3 stride 2 on the conv output [256,128,56,56], forward and argmax backward
+    x = torch.randn(256, 128, 56, 56, device=dev, generator=g)
+    y, am, il = Kn.max_pool2d(x, 3, 0, 2)
+    gy = torch.randn_like(y)
+    by = 4.0 * (x.numel() + 2 * y.numel())
+    ms = time_events(torch, lambda: Kn.max_pool2d(x, 3, 0, 2), 10)
+    res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), 10)
+    res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del x, y, am, il, gy
+
+    # reduce_sum (to scalar) and Adam on 2^26 elements
+    n = 1 << 26
+    a = torch.randn(n, device=dev, generator=g)
+    ms = time_events(torch, lambda: Kn.sum_all(a), 10)
+    res["sum_all_2^26"] = {"ms": round(ms, 4), "GB/s": round(4.0 * n / ms / 1e6, 1), "frac_hbm": round(4.0 * n / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    p, m, v = torch.randn(n, device=dev, generator=g), torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+    t = torch.ones(1, device=dev)
+    ms = time_events(torch, lambda: Kn.adam_update(p, a, m, v, t), 10)
+    res["adam_2^26"] = {"ms": round(ms, 4), "GB/s": round(28.0 * n / ms / 1e6, 1), "frac_hbm": round(28.0 * n / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del a, p, m, v
+
+    # dense contractions of config 3
+    A = torch.randn(4096, 4096, device=dev, generator=g)
+    Bm = torch.randn(4096, 4096, device=dev, generator=g)
+    for name, ta, tb in (("matmul_4096_NN", False, False), ("matmul_4096_NT", False, True), ("matmul_4096_TN", True, False)):
+        ms = time_events(torch, lambda: Kn.matmul(A, Bm, ta, tb), 10)
+        tf = 2.0 * 4096 ** 3 / ms / 1e9
+        res[name] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    del A, Bm
+    A = torch.randn(64, 512, 512, device=dev, generator=g)
+    Bm = torch.randn(64, 512, 512, device=dev, generator=g)
+    ms = time_events(torch, lambda: Kn.batch_matmul(A, Bm), 10)
+    tf = 2.0 * 64 * 512 ** 3 / ms / 1e9
+    res["batch_matmul_64x512"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    return res
+
+
+if __name__ == "__main__":
+    main()

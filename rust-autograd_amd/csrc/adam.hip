@@ -1,7 +1,7 @@
 // Fused Adam update: one pass over param / grad / m / v (28 bytes of HBM traffic per element)
 // instead of the reference's seven array passes and two temporaries
 // (gradient_descent_ops/adam.rs:11-58).  The arithmetic keeps the reference's operation order
-// and uses explicitly rounded multiplies and adds so that no fused multiply-add changes it.
+// with contraction into fused multiply-adds switched off, so m and v match it bit for bit.
 #include "ag_internal.h"
 
 namespace ag {
@@ -13,14 +13,15 @@ struct AdamCoef {
 __device__ inline void adam_one(float &p, float g, float &m, float &v, float c1, float c2, float rm,
                                 float rv, const AdamCoef &k)
 {
-    // m = m*b1 + (1-b1)*g                         adam.rs:16-23
-    m = __fadd_rn(__fmul_rn(m, k.b1), __fmul_rn(c1, g));
-    // v = v*b2 + ((1-b2)*g)*g                     adam.rs:26-33
-    v = __fadd_rn(__fmul_rn(v, k.b2), __fmul_rn(__fmul_rn(c2, g), g));
-    const float vh = __fmul_rn(v, rv);           // v * (1/(1-b2^t))            adam.rs:38-39
-    float mh = __fmul_rn(m, rm);                 // m * (1/(1-b1^t))            adam.rs:40-41
-    mh = __fdiv_rn(mh, __fadd_rn(__fsqrt_rn(vh), k.eps));  //                   adam.rs:44
-    p = __fsub_rn(p, __fmul_rn(k.alpha, mh));    //                             adam.rs:49-50
+// Every multiply and add below is rounded on its own, as in the reference (no fused multiply-add);
+// this file is also compiled with -ffp-contract=off.
+#pragma clang fp contract(off)
+    m = m * k.b1 + c1 * g;               // adam.rs:16-23
+    v = v * k.b2 + c2 * g * g;           // adam.rs:26-33   ((1-b2)*g)*g
+    const float vh = v * rv;             // adam.rs:38-39   v * (1/(1-b2^t))
+    float mh = m * rm;                   // adam.rs:40-41   m * (1/(1-b1^t))
+    mh = mh / (sqrtf(vh) + k.eps);       // adam.rs:44      correctly rounded sqrt and divide
+    p = p - k.alpha * mh;                // adam.rs:49-50
 }
 
 __global__ __launch_bounds__(256) void adam_kernel(float *__restrict__ p, const float *__restrict__ g,

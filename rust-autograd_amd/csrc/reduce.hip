@@ -5,8 +5,9 @@
 // step, and writes one partial; one block then folds the partials in index order.  Axis
 // reductions are applied one axis at a time from the last listed axis to the first, exactly as
 // the reference does (reduction_ops.rs:74-89).  With trailing elements after the folded axis
-// (inner > 1) each thread owns one output and adds along the axis sequentially, which is the
-// reference's own order; a reduction of the innermost axis uses one wave per row instead.
+// (inner > 1), or a short folded axis, each thread owns one output and adds along the axis
+// sequentially, which is the reference's own order (bit-identical sums); a long innermost axis
+// uses one wave per row instead (tolerance-level agreement).
 #include "ag_internal.h"
 
 namespace ag {
@@ -14,6 +15,7 @@ namespace ag {
 constexpr int kSumBlocks = 2048;  // stage-1 partials (fixed: result does not depend on the device)
 constexpr int kSumThreads = 256;
 constexpr int kMaxRank = 8;
+constexpr size_t kSeqRowLimit = 256;  // innermost folds up to this length are added sequentially
 
 __device__ inline float wave_sum(float v)
 {
@@ -254,7 +256,9 @@ extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, flo
         const size_t len = (size_t)dims[ax[a]];
         float *dst = (a == 0) ? out : buf[(n_axes - 1 - a) & 1];
         const int sc = (a == 0) ? do_scale : 0;
-        if (inner == 1)
+        // Short innermost folds stay sequential per output (the reference's order, bit-identical);
+        // long rows take one wave each.
+        if (inner == 1 && len > kSeqRowLimit)
             hipLaunchKernelGGL(fold_last_axis_kernel, dim3(grid_for(outer, 4)), dim3(256), 0, st, cur, dst,
                                outer, len, scale, sc);
         else
