@@ -236,8 +236,12 @@ ag_status_t ag_sparse_softmax_xent_grad_f32(ag_stream_t stream, const float *log
                                             size_t rows, size_t classes);
 
 /* Experiment hook, not part of the operator surface: force GEMM tile configuration `cfg`
- * (0..3; -1 restores the automatic choice) for later calls in this process. */
+ * (-1 restores the automatic choice) for later calls in this process. */
 void ag_gemm_force_config(int cfg);
+/* Experiment hook: force the split count of accumulated-batch GEMMs (0 = automatic). */
+void ag_gemm_force_splits(int splits);
+/* Experiment hook: blocks per CU of the persistent GEMM grid (0 = as many as stay resident). */
+void ag_gemm_force_grid(int blocks_per_cu);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -89,6 +89,8 @@ PROTOTYPES = {
     "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_gemm_force_config": (None, [c_i]),
+    "ag_gemm_force_splits": (None, [c_i]),
+    "ag_gemm_force_grid": (None, [c_i]),
 }
 
 _lib = None

@@ -24,38 +24,48 @@ __device__ inline void adam_one(float &p, float g, float &m, float &v, float c1,
     p = p - k.alpha * mh;                // adam.rs:49-50
 }
 
+// One 128-bit quad per thread (no loop: the grid covers the array, which measured fastest for a
+// streaming read-modify-write); the two bias-correction factors are computed by one lane per
+// block and shared through LDS.  The last partial quad is handled by the final thread.
 __global__ __launch_bounds__(256) void adam_kernel(float *__restrict__ p, const float *__restrict__ g,
                                                    float *__restrict__ m, float *__restrict__ v,
                                                    const float *__restrict__ t, size_t n, AdamCoef k,
                                                    int vec)
 {
-    const float tv = t[0];
+    __shared__ float corr[2];
+    if (threadIdx.x == 0) {
+        const float tv = t[0];
+        corr[0] = 1.0f / (1.0f - powf(k.b1, tv));  // adam.rs:40
+        corr[1] = 1.0f / (1.0f - powf(k.b2, tv));  // adam.rs:38
+    }
+    __syncthreads();
+    const float rm = corr[0], rv = corr[1];
     const float c1 = 1.0f - k.b1, c2 = 1.0f - k.b2;
-    const float rv = 1.0f / (1.0f - powf(k.b2, tv));
-    const float rm = 1.0f / (1.0f - powf(k.b1, tv));
-    const size_t tid = blockIdx.x * 256ull + threadIdx.x;
-    const size_t nthreads = gridDim.x * 256ull;
-    size_t done = 0;
+    const size_t i = blockIdx.x * 256ull + threadIdx.x;
     if (vec) {
         const size_t n4 = n / 4;
-        float4 *p4 = reinterpret_cast<float4 *>(p);
-        const float4 *g4 = reinterpret_cast<const float4 *>(g);
-        float4 *m4 = reinterpret_cast<float4 *>(m);
-        float4 *v4 = reinterpret_cast<float4 *>(v);
-        for (size_t i = tid; i < n4; i += nthreads) {
-            float4 pp = p4[i], mm = m4[i], vv = v4[i];
-            const float4 gg = g4[i];
+        if (i < n4) {
+            float4 pp = ld_stream(reinterpret_cast<const float4 *>(p) + i);
+            float4 mm = ld_stream(reinterpret_cast<const float4 *>(m) + i);
+            float4 vv = ld_stream(reinterpret_cast<const float4 *>(v) + i);
+            const float4 gg = ld_stream(reinterpret_cast<const float4 *>(g) + i);
             adam_one(pp.x, gg.x, mm.x, vv.x, c1, c2, rm, rv, k);
             adam_one(pp.y, gg.y, mm.y, vv.y, c1, c2, rm, rv, k);
             adam_one(pp.z, gg.z, mm.z, vv.z, c1, c2, rm, rv, k);
             adam_one(pp.w, gg.w, mm.w, vv.w, c1, c2, rm, rv, k);
-            p4[i] = pp;
-            m4[i] = mm;
-            v4[i] = vv;
+            st_stream(reinterpret_cast<float4 *>(p) + i, pp);
+            st_stream(reinterpret_cast<float4 *>(m) + i, mm);
+            st_stream(reinterpret_cast<float4 *>(v) + i, vv);
+        } else if (i == n4) {
+            for (size_t e = n4 * 4; e < n; ++e) {
+                float pp = p[e], mm = m[e], vv = v[e];
+                adam_one(pp, g[e], mm, vv, c1, c2, rm, rv, k);
+                p[e] = pp;
+                m[e] = mm;
+                v[e] = vv;
+            }
         }
-        done = n4 * 4;
-    }
-    for (size_t i = done + tid; i < n; i += nthreads) {
+    } else if (i < n) {
         float pp = p[i], mm = m[i], vv = v[i];
         adam_one(pp, g[i], mm, vv, c1, c2, rm, rv, k);
         p[i] = pp;
@@ -80,9 +90,9 @@ extern "C" ag_status_t ag_adam_update_f32(ag_stream_t stream, float *param, cons
     hipStream_t st = as_stream(stream);
     if (n > 0) {
         const int vec = aligned16(param) && aligned16(grad) && aligned16(m) && aligned16(v);
-        size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
-        if (blocks < 1) blocks = 1;
-        if (blocks > 8192) blocks = 8192;
+        const size_t items = vec ? n / 4 + 1 : n;  // +1: the thread that finishes a partial quad
+        const size_t blocks = (items + 255) / 256;
+        AG_REQUIRE(blocks <= (size_t)kMaxGridX, AG_ERR_INVALID_DIMS, "adam: too many elements (%zu)", n);
         hipLaunchKernelGGL(adam_kernel, dim3((unsigned)blocks), dim3(256), 0, st, param, grad, m, v, t, n,
                            AdamCoef{alpha, eps, b1, b2}, vec);
     }

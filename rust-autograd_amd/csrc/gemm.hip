@@ -22,6 +22,8 @@
 // writes a partial result that a second fixed-order kernel folds, keeping the result
 // deterministic.  Block ids are permuted so that each XCD (which has its own L2) works on a
 // contiguous range of tiles / images.
+#include <type_traits>
+
 #include "ag_internal.h"
 
 namespace ag {
@@ -60,194 +62,332 @@ __device__ inline unsigned xcd_remap(unsigned id, unsigned total)
 
 template <int LT, int ROWS, int BK, int NT>
 struct TileLoader {
-    static constexpr int QUADS = BK / 4;
-    static constexpr int PASSES = ROWS * BK / (4 * NT);
-    static_assert(ROWS * BK % (4 * NT) == 0 && PASSES >= 1, "tile does not divide over the block");
-    // k-contiguous mapping
-    static constexpr int RPP = NT / QUADS;  // rows per pass
-    // mn-contiguous mapping
-    static constexpr int GROUPS = NT / ROWS > 0 ? NT / ROWS : 1;
-    static_assert(LT != LMN || (NT % ROWS == 0 && QUADS % GROUPS == 0), "mn-contiguous mapping needs NT % ROWS == 0");
-    static_assert(LT == LMN || (NT % QUADS == 0 && ROWS % RPP == 0), "k-contiguous mapping needs ROWS % (NT/(BK/4)) == 0");
+    static constexpr int QUADS = BK / 4;                 // 4-float groups along k per row
+    static constexpr int PASSES = ROWS * QUADS / NT;     // (row, quad) items per thread
+    static_assert(ROWS * QUADS % NT == 0 && PASSES >= 1, "tile does not divide over the block");
+    static_assert(NT % QUADS == 0, "threads per row must divide the block");
 
-    // Fetch this thread's share of the tile whose first row is row0 and first k is k0.
-    // `base` already points at the right batch.  Out-of-range rows and k read as zero.
-    __device__ static inline void load(const float *__restrict__ base, long long ld, int row0, int rows,
-                                       int k0, int K, int tid, float4 (&r)[PASSES])
+    // Item `it` = ps*NT + tid of this thread.  k-contiguous operands walk the quads of a row with
+    // consecutive lanes (128-bit loads along k); mn-contiguous operands walk the rows with
+    // consecutive lanes (coalesced 32-bit loads, four k per lane).
+    __device__ static inline void item(int it, int &row, int &quad)
     {
         if (LT == LMN) {
-            const int idx = tid % ROWS, grp = tid / ROWS;
-            const bool row_ok = row0 + idx < rows;
-            const float *p = base + row0 + idx;
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int k = k0 + (ps * GROUPS + grp) * 4;
-                float4 v;
-                v.x = (row_ok && k + 0 < K) ? p[(long long)(k + 0) * ld] : 0.f;
-                v.y = (row_ok && k + 1 < K) ? p[(long long)(k + 1) * ld] : 0.f;
-                v.z = (row_ok && k + 2 < K) ? p[(long long)(k + 2) * ld] : 0.f;
-                v.w = (row_ok && k + 3 < K) ? p[(long long)(k + 3) * ld] : 0.f;
-                r[ps] = v;
-            }
+            row = it % ROWS;
+            quad = it / ROWS;
         } else {
-            const int rr = tid / QUADS, kq = (tid % QUADS) * 4;
-            const int k = k0 + kq;
+            row = it / QUADS;
+            quad = it % QUADS;
+        }
+    }
+
+    int off[PASSES];   // element offset of this thread's items from the tile origin (row clamped)
+
+    // Offsets are 32-bit (the host checks the operand slice fits) and fixed for the whole k loop:
+    // the tile origin moves as a wave-uniform pointer.
+    __device__ inline void init(int ld, int row0, int rows, int tid)
+    {
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int row = row0 + ps * RPP + rr;
-                const float *p = base + (long long)row * ld + k;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (row < rows) {
-                    if (LT == LK_VEC) {
-                        if (k < K) v = *reinterpret_cast<const float4 *>(p);  // K % 4 == 0 here
-                    } else {
-                        if (k + 0 < K) v.x = p[0];
-                        if (k + 1 < K) v.y = p[1];
-                        if (k + 2 < K) v.z = p[2];
-                        if (k + 3 < K) v.w = p[3];
-                    }
-                }
-                r[ps] = v;
+        for (int ps = 0; ps < PASSES; ++ps) {
+            int rr, q;
+            item(ps * NT + tid, rr, q);
+            const int row = row0 + rr;
+            const int rc = row < rows ? row : rows - 1;
+            off[ps] = (LT == LMN) ? q * 4 * ld + rc : rc * ld + q * 4;
+        }
+    }
+
+    // Distance between the origins of consecutive k tiles.
+    __device__ static inline long long k_step(int ld) { return (LT == LMN) ? (long long)BK * ld : BK; }
+
+    // Interior k tile: `origin` = operand + k0 (k-contiguous) or + k0*ld (mn-contiguous).
+    __device__ inline void load(const float *__restrict__ origin, int ld, float4 (&r)[PASSES]) const
+    {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const float *p = origin + off[ps];
+            if (LT == LMN) {
+                r[ps] = make_float4(p[0], p[ld], p[2 * ld], p[3 * ld]);
+            } else if (LT == LK_VEC) {
+                r[ps] = *reinterpret_cast<const float4 *>(p);
+            } else {
+                r[ps] = make_float4(p[0], p[1], p[2], p[3]);
             }
+        }
+    }
+
+    // Last k tile when K is not a multiple of BK: `krem` (1..BK-1) valid k remain; the rest reads
+    // as zero (addresses are clamped, values selected).
+    __device__ inline void load_tail(const float *__restrict__ origin, int ld, int krem, int tid,
+                                     float4 (&r)[PASSES]) const
+    {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            int rr, q;
+            item(ps * NT + tid, rr, q);
+            const long long kstride = (LT == LMN) ? ld : 1;
+            const float *p = origin + off[ps] - (long long)q * 4 * kstride;   // k = 0 of this row
+            float v[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int k = q * 4 + jj;
+                const float x = p[(long long)min(k, krem - 1) * kstride];
+                v[jj] = k < krem ? x : 0.f;
+            }
+            r[ps] = make_float4(v[0], v[1], v[2], v[3]);
         }
     }
 
     __device__ static inline void store(float *__restrict__ lds, int ldk, int tid, const float4 (&r)[PASSES])
     {
-        if (LT == LMN) {
-            const int idx = tid % ROWS, grp = tid / ROWS;
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps)
-                *reinterpret_cast<float4 *>(lds + idx * ldk + (ps * GROUPS + grp) * 4) = r[ps];
-        } else {
-            const int rr = tid / QUADS, kq = (tid % QUADS) * 4;
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps)
-                *reinterpret_cast<float4 *>(lds + (ps * RPP + rr) * ldk + kq) = r[ps];
+        for (int ps = 0; ps < PASSES; ++ps) {
+            int rr, q;
+            item(ps * NT + tid, rr, q);
+            *reinterpret_cast<float4 *>(lds + rr * ldk + q * 4) = r[ps];
         }
     }
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int LA, int LB>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void gemm_mfma_kernel(GemmParams p)
+template <int BM, int BN, int BK, int WM, int WN, int OCC, int STAGES, int LA, int LB>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_kernel(GemmParams p)
 {
+    static_assert(STAGES == 2 || STAGES == 3, "LDS ring of two or three tiles");
+    constexpr int KK = BK / 8;
     constexpr int WAVES_N = BN / WN;
     constexpr int NT = (BM / WM) * (BN / WN) * 64;
     constexpr int LDK = BK + 4;
     constexpr int MI = WM / 32, NI = WN / 32;
-    static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 8 == 0, "tile shape");
+    static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape (BK/8 must be even)");
     using LoadA = TileLoader<LA, BM, BK, NT>;
     using LoadB = TileLoader<LB, BN, BK, NT>;
 
-    __shared__ __attribute__((aligned(16))) float lds[2][(BM + BN) * LDK];
+    __shared__ __attribute__((aligned(16))) float lds[STAGES][(BM + BN) * LDK];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-    const unsigned lb = xcd_remap(blockIdx.x, p.total_blocks);
+    const unsigned total = p.total_blocks;  // work items = tiles x independent batches x splits
     const unsigned tiles = (unsigned)(p.tiles_m * p.tiles_n);
-    const unsigned z = lb / tiles, t_in = lb % tiles;
-    const int tile_m = t_in % p.tiles_m, tile_n = t_in / p.tiles_m;
-    const int bz = z / p.splits, sp = z % p.splits;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int kb0 = sp * p.kb_per_split;
-    const int kb1 = min(p.kbatch, kb0 + p.kb_per_split);
-
-    const float *Ab = p.A + (long long)bz * p.sA;
-    const float *Bb = p.B + (long long)bz * p.sB;
-
-    f32x16 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
     const int kt_per = (p.K + BK - 1) / BK;
-    const int n_tiles = (kb1 - kb0) * kt_per;
+    const int krem = p.K - (kt_per - 1) * BK;  // k in the last tile of a batch
+    const bool ktail = krem != BK;
+    const int lda = (int)p.lda, ldb = (int)p.ldb;
 
+    // A work item is one output tile of one batch / split.  The block walks items
+    // blockIdx.x, blockIdx.x + gridDim.x, ... as ONE stream of k tiles: fetching runs
+    // STAGES-1 tiles ahead of the MFMAs and crosses item boundaries, so the loads of the next
+    // item are in flight while the current one finishes and is written out.
+    struct Item {
+        int m0, n0, bz, sp, kb0, nt;
+    };
+    auto decode = [&](unsigned w) {
+        const unsigned lb = xcd_remap(w, total);
+        const unsigned z = lb / tiles, t_in = lb % tiles;
+        Item it;
+        it.m0 = (int)(t_in % p.tiles_m) * BM;
+        it.n0 = (int)(t_in / p.tiles_m) * BN;
+        it.bz = (int)(z / p.splits);
+        it.sp = (int)(z % p.splits);
+        it.kb0 = it.sp * p.kb_per_split;
+        it.nt = (min(p.kbatch, it.kb0 + p.kb_per_split) - it.kb0) * kt_per;
+        return it;
+    };
+
+    // ---- fetch stream ----
+    unsigned fw = blockIdx.x;
+    bool f_valid = fw < total;
+    if (!f_valid) return;
+    LoadA ldr_a;
+    LoadB ldr_b;
+    const float *fA = nullptr, *fB = nullptr;
+    int fkb = 0, fkt = 0, f_left = 0;
+    auto f_begin = [&]() {
+        const Item it = decode(fw);
+        ldr_a.init(lda, it.m0, p.M, tid);
+        ldr_b.init(ldb, it.n0, p.N, tid);
+        fA = p.A + (long long)it.bz * p.sA;
+        fB = p.B + (long long)it.bz * p.sB;
+        fkb = it.kb0;
+        fkt = 0;
+        f_left = it.nt;
+    };
     float4 ra[LoadA::PASSES], rb[LoadB::PASSES];
-
-    if (n_tiles > 0) {
-        LoadA::load(Ab + (long long)kb0 * p.sAk, p.lda, m0, p.M, 0, p.K, tid, ra);
-        LoadB::load(Bb + (long long)kb0 * p.sBk, p.ldb, n0, p.N, 0, p.K, tid, rb);
-        LoadA::store(lds[0], LDK, tid, ra);
-        LoadB::store(lds[0] + BM * LDK, LDK, tid, rb);
-    }
-    __syncthreads();
-
-    int kb = kb0, kt = 0;
-    for (int t = 0; t < n_tiles; ++t) {
-        const int cur = t & 1;
-        // advance to the next (accumulated batch, k tile) and start fetching it
-        if (++kt == kt_per) { kt = 0; ++kb; }
-        const bool more = t + 1 < n_tiles;
-        if (more) {
-            LoadA::load(Ab + (long long)kb * p.sAk, p.lda, m0, p.M, kt * BK, p.K, tid, ra);
-            LoadB::load(Bb + (long long)kb * p.sBk, p.ldb, n0, p.N, kt * BK, p.K, tid, rb);
+    // Rows beyond M (or N) are fetched from a clamped, valid address and left as they are: they
+    // only feed output rows (columns) that are never written.
+    // Loads of the next tile of the stream.  TAIL: K is not a multiple of BK.
+    auto fetch_issue = [&](auto tail_tag) {
+        const float *oa = fA + (long long)fkb * p.sAk + fkt * LoadA::k_step(lda);
+        const float *ob = fB + (long long)fkb * p.sBk + fkt * LoadB::k_step(ldb);
+        if (decltype(tail_tag)::value && fkt == kt_per - 1) {
+            ldr_a.load_tail(oa, lda, krem, tid, ra);
+            ldr_b.load_tail(ob, ldb, krem, tid, rb);
+        } else {
+            ldr_a.load(oa, lda, ra);
+            ldr_b.load(ob, ldb, rb);
         }
+    };
+    // Move the fetch stream to the following tile (possibly of the next work item).
+    // At the end of the stream the position stays on the last tile, which is a valid address for
+    // the (discarded) loads issued after it.
+    auto fetch_advance = [&]() {
+        if (--f_left == 0) {
+            fw += gridDim.x;
+            f_valid = fw < total;
+            if (f_valid) f_begin();
+        } else if (++fkt == kt_per) {
+            fkt = 0;
+            ++fkb;
+        }
+    };
+    auto stage = [&](int buf) {
+        LoadA::store(lds[buf], LDK, tid, ra);
+        LoadB::store(lds[buf] + BM * LDK, LDK, tid, rb);
+    };
 
-        const float *As = lds[cur] + (wm * WM + (lane & 31)) * LDK + (lane >> 5) * 4;
-        const float *Bs = lds[cur] + BM * LDK + (wn * WN + (lane & 31)) * LDK + (lane >> 5) * 4;
+    // ---- compute stream ----
+    f32x16 acc[MI][NI];
+    auto zero_acc = [&]() {
 #pragma unroll
-        for (int kk = 0; kk < BK / 8; ++kk) {
-            float4 af[MI], bf[NI];
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const float4 *>(As + i * 32 * LDK + kk * 8);
+            for (int j = 0; j < NI; ++j)
 #pragma unroll
-            for (int j = 0; j < NI; ++j) bf[j] = *reinterpret_cast<const float4 *>(Bs + j * 32 * LDK + kk * 8);
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
+    // Fragment reads: one 128-bit LDS read per 32-row block gives four MFMA k steps.
+    const int frag_off = (lane & 31) * LDK + (lane >> 5) * 4;
+    auto read_frags = [&](int buf, int kk, float4 (&af)[MI], float4 (&bf)[NI]) {
+        const float *As = lds[buf] + wm * WM * LDK + frag_off + kk * 8;
+        const float *Bs = lds[buf] + (BM + wn * WN) * LDK + frag_off + kk * 8;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const float4 *>(As + i * 32 * LDK);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) bf[j] = *reinterpret_cast<const float4 *>(Bs + j * 32 * LDK);
+    };
+    auto mfma_frags = [&](const float4 (&af)[MI], const float4 (&bf)[NI]) {
+        // k step outermost: consecutive MFMAs write different accumulators
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].z, bf[j].z, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].w, bf[j].w, acc[i][j], 0, 0, 0);
+                    const float a = s4 == 0 ? af[i].x : s4 == 1 ? af[i].y : s4 == 2 ? af[i].z : af[i].w;
+                    const float b = s4 == 0 ? bf[j].x : s4 == 1 ? bf[j].y : s4 == 2 ? bf[j].z : bf[j].w;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i][j], 0, 0, 0);
+                }
+    };
+    // Accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4 and column l%32 of its
+    // 32x32 block.
+    auto write_out = [&](const Item &it) {
+        float *Cb;
+        long long ldc;
+        float alpha, beta;
+        if (p.splits > 1) {
+            Cb = p.C + (long long)it.bz * p.sC + (long long)it.sp * p.sCsplit;
+            ldc = p.N;
+            alpha = 1.f;
+            beta = 0.f;
+        } else {
+            Cb = p.C + (long long)it.bz * p.sC;
+            ldc = p.ldc;
+            alpha = p.alpha;
+            beta = p.beta;
+        }
+        const bool full = it.m0 + BM <= p.M && it.n0 + BN <= p.N;
+        const int row_base = it.m0 + wm * WM + 4 * (lane >> 5);
+        const int col_base = it.n0 + wn * WN + (lane & 31);
+        if (full && beta == 0.f) {
+            // interior tile, overwrite: straight stores
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    float *dst = Cb + (long long)(row_base + i * 32) * ldc + col_base + j * 32;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        dst[(long long)(8 * (v / 4) + (v % 4)) * ldc] = alpha * acc[i][j][v];
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    const int col = col_base + j * 32;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
+                        if (row < p.M && col < p.N) {
+                            float *dst = Cb + (long long)row * ldc + col;
+                            const float r = alpha * acc[i][j][v];
+                            *dst = beta == 0.f ? r : r + beta * *dst;
+                        }
+                    }
                 }
         }
+    };
 
-        if (more) {
-            LoadA::store(lds[cur ^ 1], LDK, tid, ra);
-            LoadB::store(lds[cur ^ 1] + BM * LDK, LDK, tid, rb);
-        }
+    auto run = [&](auto tail_tag) {
+        // Prologue: the first STAGES-1 tiles of the stream go to LDS.
+        f_begin();
+#pragma unroll
+        for (int st = 0; st < STAGES - 1; ++st)
+            if (f_valid) {
+                fetch_issue(tail_tag);
+                fetch_advance();
+                stage(st);
+            }
         __syncthreads();
-    }
 
-    // Epilogue.  Accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4 and column
-    // l%32 of its 32x32 block.
-    float *Cb;
-    long long ldc;
-    float alpha, beta;
-    if (p.splits > 1) {
-        Cb = p.C + (long long)bz * p.sC + (long long)sp * p.sCsplit;
-        ldc = p.N;
-        alpha = 1.f;
-        beta = 0.f;
-    } else {
-        Cb = p.C + (long long)bz * p.sC;
-        ldc = p.ldc;
-        alpha = p.alpha;
-        beta = p.beta;
-    }
+        unsigned cw = blockIdx.x;
+        Item ci = decode(cw);
+        int c_left = ci.nt;
+        zero_acc();
+        float4 af[2][MI], bf[2][NI];
+        read_frags(0, 0, af[0], bf[0]);
+
+        int cur = 0;                       // ring slot of the tile being multiplied
+        int fill = (STAGES - 1) % STAGES;  // ring slot the tile being fetched goes to
+        while (true) {
+            const bool more = f_valid;
+            if (more) fetch_issue(tail_tag);  // global loads fly during this tile's MFMAs
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int col = n0 + wn * WN + j * 32 + (lane & 31);
-            if (col >= p.N) continue;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (row < p.M) {
-                    float *dst = Cb + (long long)row * ldc + col;
-                    const float r = alpha * acc[i][j][v];
-                    *dst = beta == 0.f ? r : r + beta * *dst;
-                }
+            for (int kk = 0; kk < KK; ++kk) {
+                if (kk + 1 < KK) read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+                mfma_frags(af[kk & 1], bf[kk & 1]);
+            }
+            if (more) {
+                fetch_advance();
+                stage(fill);
+            }
+            const bool item_done = --c_left == 0;
+            const bool last = item_done && cw + gridDim.x >= total;  // nothing follows in the stream
+            const int nxt = cur + 1 == STAGES ? 0 : cur + 1;
+            if (STAGES == 3) {
+                // The next tile was completed before the previous barrier: start reading it now.
+                if (!last) read_frags(nxt, 0, af[0], bf[0]);
+                __syncthreads();
+            } else {
+                __syncthreads();
+                if (!last) read_frags(nxt, 0, af[0], bf[0]);
+            }
+            cur = nxt;
+            fill = fill + 1 == STAGES ? 0 : fill + 1;
+
+            if (item_done) {
+                write_out(ci);
+                if (last) break;
+                cw += gridDim.x;
+                ci = decode(cw);
+                c_left = ci.nt;
+                zero_acc();
             }
         }
+    };
+    if (ktail) run(std::true_type{});
+    else run(std::false_type{});
 }
 
 // C[m][n] = alpha * sum_s partial[s][m][n] + beta * C[m][n], s ascending.
@@ -275,14 +415,44 @@ struct TileCfg {
     int bm, bn;
 };
 
-template <int BM, int BN, int BK, int WM, int WN>
+// Resident blocks per CU of one kernel instantiation, and the CU count (both cached).
+static int num_cus()
+{
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+template <typename Kern>
+static int resident_blocks(Kern kern, int threads, int fallback)
+{
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = fallback;
+    return n;
+}
+
+static int g_grid_scale = 0;  // experiment hook: blocks per CU of the persistent grid (0 = resident count)
+
+template <int BM, int BN, int BK, int WM, int WN, int OCC, int STAGES>
 static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
 {
     constexpr int NT = (BM / WM) * (BN / WN) * 64;
-    const dim3 grid(p.total_blocks), block(NT);
+    const dim3 block(NT);
 #define AG_GEMM_CASE(LA_, LB_)                                                                        \
     if (la == LA_ && lb == LB_) {                                                                     \
-        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, WM, WN, LA_, LB_>), grid, block, 0, st, p);  \
+        auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, OCC, STAGES, LA_, LB_>;                      \
+        static const int per_cu = resident_blocks(kern, NT, OCC);                                     \
+        /* persistent grid: every resident slot gets one block, which walks the items */             \
+        long long g = (long long)num_cus() * (g_grid_scale > 0 ? g_grid_scale : per_cu);              \
+        if (g > p.total_blocks) g = p.total_blocks;                                                   \
+        hipLaunchKernelGGL(kern, dim3((unsigned)g), block, 0, st, p);                                 \
         return;                                                                                       \
     }
     AG_GEMM_CASE(LK_VEC, LK_VEC)
@@ -299,44 +469,60 @@ static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
 
 static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
 
-// Tile configurations, largest first.  {BM, BN}; all use BK = 32... except where noted in launch().
-static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+// Tile configurations {BM, BN}; see launch() for BK, the wave tile and the occupancy target.
+static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
+                                {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
+                                {128, 128}, {192, 128}, {128, 64}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
     switch (cfg) {
-        case 0: launch_cfg<128, 128, 32, 64, 64>(st, la, lb, p); break;
-        case 1: launch_cfg<128, 64, 32, 64, 32>(st, la, lb, p); break;
-        case 2: launch_cfg<64, 128, 32, 32, 64>(st, la, lb, p); break;
-        default: launch_cfg<64, 64, 32, 32, 32>(st, la, lb, p); break;
+        //                 BM   BN  BK  WM   WN OCC STAGES
+        case 0: launch_cfg<128, 128, 32, 64, 64, 2, 2>(st, la, lb, p); break;
+        case 1: launch_cfg<128, 64, 32, 64, 32, 2, 2>(st, la, lb, p); break;
+        case 2: launch_cfg<64, 128, 32, 32, 64, 2, 2>(st, la, lb, p); break;
+        case 3: launch_cfg<64, 64, 32, 32, 32, 2, 2>(st, la, lb, p); break;
+        case 4: launch_cfg<128, 128, 16, 64, 64, 3, 2>(st, la, lb, p); break;
+        case 5: launch_cfg<192, 128, 16, 96, 64, 2, 2>(st, la, lb, p); break;
+        case 6: launch_cfg<256, 128, 16, 128, 64, 2, 2>(st, la, lb, p); break;
+        case 7: launch_cfg<128, 256, 16, 64, 128, 2, 2>(st, la, lb, p); break;
+        case 8: launch_cfg<64, 64, 16, 32, 32, 4, 2>(st, la, lb, p); break;
+        case 9: launch_cfg<128, 64, 16, 64, 32, 3, 2>(st, la, lb, p); break;
+        case 10: launch_cfg<128, 128, 16, 64, 64, 2, 3>(st, la, lb, p); break;
+        case 11: launch_cfg<192, 128, 16, 96, 64, 2, 3>(st, la, lb, p); break;
+        default: launch_cfg<128, 64, 16, 64, 32, 3, 3>(st, la, lb, p); break;
     }
 }
 
 static long long cdiv(long long a, long long b) { return (a + b - 1) / b; }
 
-// Pick the configuration with the least padded work, preferring larger tiles on ties, but do
-// not starve the 256 CUs: small problems take smaller tiles.
-static int choose_cfg(int M, int N, long long zcount)
+// Tile choice.  The block-tile shape comes first: least padded output area, larger tiles on ties
+// (they re-read operands less).  Contractions with few k tiles per output tile, and the
+// accumulated-batch GEMMs, take the BK = 16 family with a three-tile LDS ring (3-4 blocks stay
+// resident per CU, which hides the per-tile staging); long contractions take BK = 32.
+// Problems too small to give every CU a block fall back to 64 x 64 tiles.
+static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate)
 {
     if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg;
-    int best = kNumCfgs - 1;
-    double best_cost = 1e300;
-    for (int c = 0; c < kNumCfgs; ++c) {
-        const long long tm = cdiv(M, kCfgs[c].bm), tn = cdiv(N, kCfgs[c].bn);
-        const double blocks = (double)tm * tn * zcount;
-        const double tile_work = (double)kCfgs[c].bm * kCfgs[c].bn;
-        // waves of 512 resident blocks (2 per CU); partial waves cost a full one
-        const double slots = 512.0;
-        const double waves = blocks <= slots ? 1.0 : blocks / slots;
-        // smaller tiles re-read operands more: penalise them slightly
-        const double eff = (c == 0) ? 1.0 : (c == 3 ? 1.25 : 1.1);
-        const double cost = waves * tile_work * eff;
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = c;
+    static const int short_k[] = {11, 10, 12, 8};  // 192x128, 128x128, 128x64, 64x64 (BK 16)
+    static const int long_k[] = {0, 1, 2, 3};      // 128x128, 128x64, 64x128, 64x64 (BK 32)
+    const bool use_short = accumulate || K <= 1024;
+    const int *cand = use_short ? short_k : long_k;
+    int best = cand[3];
+    double best_area = 1e300;
+    long long best_blocks = 0;
+    for (int c = 0; c < 4; ++c) {
+        const TileCfg &t = kCfgs[cand[c]];
+        const long long tm = cdiv(M, t.bm), tn = cdiv(N, t.bn);
+        const double area = (double)tm * t.bm * tn * t.bn;
+        if (area < best_area * 0.97) {  // needs a >3 % saving to beat a larger tile
+            best_area = area;
+            best = cand[c];
+            best_blocks = tm * tn * zcount;
         }
     }
+    if (best_blocks < 256) best = cand[3];
     return best;
 }
 
@@ -395,6 +581,12 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         return check_launch(who);
     }
     AG_REQUIRE(c.A && c.B, AG_ERR_INVALID_DIMS, "%s: null operand", who);
+    // tile offsets inside one operand slice are 32-bit
+    const long long a_span = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
+    const long long b_span = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
+    AG_REQUIRE(a_span < 0x7fffffffLL && b_span < 0x7fffffffLL, AG_ERR_INVALID_DIMS,
+               "%s: an operand slice spans %lld elements; at most 2^31-1 supported", who,
+               a_span > b_span ? a_span : b_span);
 
     GemmParams p;
     p.A = c.A; p.B = c.B; p.C = c.C;
@@ -409,7 +601,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.alpha = c.alpha; p.beta = c.beta;
     p.sCsplit = (long long)c.M * c.N;
 
-    const int cfg = choose_cfg(c.M, c.N, (long long)c.batch * p.splits);
+    const int cfg = choose_cfg(c.M, c.N, c.K, (long long)c.batch * p.splits, c.kbatch > 1);
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(c.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * c.batch * p.splits;
@@ -439,12 +631,15 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     return AG_OK;
 }
 
+static int g_force_splits = 0;  // experiment hook, see ag_gemm_force_splits
+
 // Number of splits for an accumulated-batch GEMM: enough blocks for a few waves over the chip.
-static int choose_splits(int M, int N, int kbatch)
+static int choose_splits(int M, int N, int K, int kbatch)
 {
-    const int cfg = choose_cfg(M, N, kbatch);  // tile choice as if every image were a block
+    if (g_force_splits > 0) return g_force_splits < kbatch ? g_force_splits : kbatch;
+    const int cfg = choose_cfg(M, N, K, kbatch, true);  // tile choice as if every image were a block
     const long long tiles = cdiv(M, kCfgs[cfg].bm) * cdiv(N, kCfgs[cfg].bn);
-    long long want = cdiv(2048, tiles);
+    long long want = cdiv(4096, tiles);
     if (want > kbatch) want = kbatch;
     if (want < 1) want = 1;
     // make the splits even
@@ -457,8 +652,14 @@ static int choose_splits(int M, int N, int kbatch)
 using namespace ag;
 
 // Experiment hook (not part of the operator surface): force tile configuration `cfg`
-// (0..3, -1 = automatic) for subsequent GEMM calls of this process.
+// (-1 = automatic) for subsequent GEMM calls of this process.
 extern "C" void ag_gemm_force_config(int cfg) { g_force_cfg = cfg; }
+
+// Experiment hook: force the number of splits of accumulated-batch GEMMs (0 = automatic).
+extern "C" void ag_gemm_force_splits(int splits) { g_force_splits = splits; }
+
+// Experiment hook: blocks per CU of the persistent GEMM grid (0 = as many as stay resident).
+extern "C" void ag_gemm_force_grid(int blocks_per_cu) { g_grid_scale = blocks_per_cu; }
 
 extern "C" ag_status_t ag_gemm_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K,
                                    float alpha, const float *A, int lda, long long strideA, const float *B,
@@ -472,9 +673,8 @@ extern "C" ag_status_t ag_gemm_f32(ag_stream_t stream, int transA, int transB, i
 
 extern "C" size_t ag_gemm_batchsum_f32_workspace(int M, int N, int K, int batch)
 {
-    (void)K;
     if (M <= 0 || N <= 0 || batch <= 0) return 16;
-    const int splits = choose_splits(M, N, batch);
+    const int splits = choose_splits(M, N, K, batch);
     return splits > 1 ? sizeof(float) * (size_t)splits * M * N : 16;
 }
 
@@ -484,6 +684,6 @@ extern "C" ag_status_t ag_gemm_batchsum_f32(ag_stream_t stream, int transA, int 
                                             int ldc, int batch, void *ws, size_t ws_bytes)
 {
     GemmCall c{transA, transB, M, N, K, alpha, beta, A, lda, 0, strideA, B, ldb, 0, strideB, C, ldc, 0, 1, batch};
-    const int splits = (M > 0 && N > 0 && batch > 0) ? choose_splits(M, N, batch) : 1;
+    const int splits = (M > 0 && N > 0 && batch > 0) ? choose_splits(M, N, K, batch) : 1;
     return run_gemm(as_stream(stream), "gemm_batchsum", c, ws, ws_bytes, splits);
 }

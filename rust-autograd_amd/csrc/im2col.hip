@@ -20,7 +20,7 @@ constexpr int kIm2colLdsBytes = 32 * 1024;
 
 // One block = one (image, channel) plane x one band of `R` output rows.
 // tile[r][cx] holds x[iy0 + r][cx - pw] (0 outside the image), WL floats per row.
-template <bool VEC4>
+template <bool VEC4, bool STREAM>
 __global__ __launch_bounds__(kIm2colThreads) void im2col_lds_kernel(
     const float *__restrict__ x, float *__restrict__ cols, ConvGeom g, int R, int bands, int WL)
 {
@@ -65,7 +65,8 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_lds_kernel(
                     v.y = s[g.sw];
                     v.z = s[2 * g.sw];
                     v.w = s[3 * g.sw];
-                    *reinterpret_cast<float4 *>(dst) = v;
+                    if (STREAM) st_stream(reinterpret_cast<float4 *>(dst), v);
+                    else *reinterpret_cast<float4 *>(dst) = v;
                     dst += P;
                 }
             }
@@ -78,7 +79,8 @@ __global__ __launch_bounds__(kIm2colThreads) void im2col_lds_kernel(
             float *dst = out + e;
             for (int ky = 0; ky < g.kh; ++ky) {
                 for (int kx = 0; kx < g.kw; ++kx) {
-                    *dst = src[ky * g.dh * WL + kx * g.dw];
+                    if (STREAM) st_stream(dst, src[ky * g.dh * WL + kx * g.dw]);
+                    else *dst = src[ky * g.dh * WL + kx * g.dw];
                     dst += P;
                 }
             }
@@ -109,8 +111,7 @@ __global__ __launch_bounds__(256) void im2col_direct_kernel(const float *__restr
     }
 }
 
-// One thread per destination pixel.  UNIT = stride 1 on both axes (no divisibility tests).
-template <bool UNIT>
+// One thread per destination pixel (any stride / dilation).
 __global__ __launch_bounds__(256) void col2im_gather_kernel(const float *__restrict__ cols,
                                                             float *__restrict__ gx, ConvGeom g,
                                                             int chunks)
@@ -126,30 +127,69 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(const float *__restr
     float acc = 0.f;
     for (int ky = 0; ky < g.kh; ++ky) {
         const int ty = iy + g.ph - ky * g.dh;
-        int oy;
-        if (UNIT) {
-            oy = ty;
-        } else {
-            if (ty < 0) break;  // later ky only lowers ty
-            oy = ty / g.sh;
-            if (oy * g.sh != ty) continue;
-        }
-        if ((unsigned)oy >= (unsigned)g.OH) continue;
+        if (ty < 0) break;  // later ky only lowers ty
+        const int oy = ty / g.sh;
+        if (oy * g.sh != ty || oy >= g.OH) continue;
         for (int kx = 0; kx < g.kw; ++kx) {
             const int tx = ix + g.pw - kx * g.dw;
-            int ox;
-            if (UNIT) {
-                ox = tx;
-            } else {
-                if (tx < 0) break;
-                ox = tx / g.sw;
-                if (ox * g.sw != tx) continue;
-            }
-            if ((unsigned)ox >= (unsigned)g.OW) continue;
+            if (tx < 0) break;
+            const int ox = tx / g.sw;
+            if (ox * g.sw != tx || ox >= g.OW) continue;
             acc += cp[(long long)(ky * g.kw + kx) * P + oy * g.OW + ox];
         }
     }
     gx[plane * HW + e] = acc;
+}
+
+// 16 bytes that are only 4-byte aligned (the hardware handles the misalignment).
+struct __attribute__((packed, aligned(4))) Float4U {
+    float x, y, z, w;
+};
+
+// Stride 1, W % 4 == 0: one thread per four consecutive destination pixels of a row.  Each of
+// the kh*kw taps is one (generally misaligned) 128-bit load from its plane of the columns; the
+// four sums keep the (ky, kx) ascending order of the reference.  Groups that touch the left or
+// right border take per-pixel loads.
+template <int KH, int KW>  // 0 = run-time extents
+__global__ __launch_bounds__(256) void col2im_unit_vec4_kernel(const float *__restrict__ cols,
+                                                               float *__restrict__ gx, ConvGeom g,
+                                                               long long groups)
+{
+    const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
+    const int W4 = g.W >> 2;
+    const long long P = (long long)g.OH * g.OW;
+    const long long taps_stride = (long long)(kh * kw) * P;
+    for (long long gi = blockIdx.x * 256LL + threadIdx.x; gi < groups; gi += gridDim.x * 256LL) {
+        const long long row = gi / W4;  // (plane, iy)
+        const int ix0 = (int)(gi - row * W4) * 4;
+        const long long plane = row / g.H;
+        const int iy = (int)(row - plane * g.H);
+        const float *cp = cols + plane * taps_stride;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+        for (int ky = 0; ky < kh; ++ky) {
+            const int oy = iy + g.ph - ky * g.dh;
+            if ((unsigned)oy >= (unsigned)g.OH) continue;
+#pragma unroll
+            for (int kx = 0; kx < kw; ++kx) {
+                const int ox0 = ix0 + g.pw - kx * g.dw;
+                const float *src = cp + (long long)(ky * kw + kx) * P + (long long)oy * g.OW + ox0;
+                if (ox0 >= 0 && ox0 + 3 < g.OW) {
+                    const Float4U v = *reinterpret_cast<const Float4U *>(src);  // read once, misaligned
+                    a0 += v.x;
+                    a1 += v.y;
+                    a2 += v.z;
+                    a3 += v.w;
+                } else {
+                    if ((unsigned)(ox0 + 0) < (unsigned)g.OW) a0 += src[0];
+                    if ((unsigned)(ox0 + 1) < (unsigned)g.OW) a1 += src[1];
+                    if ((unsigned)(ox0 + 2) < (unsigned)g.OW) a2 += src[2];
+                    if ((unsigned)(ox0 + 3) < (unsigned)g.OW) a3 += src[3];
+                }
+            }
+        }
+        st_stream(reinterpret_cast<float4 *>(gx + gi * 4), make_float4(a0, a1, a2, a3));
+    }
 }
 
 static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int kh, int kw, int ph,
@@ -187,8 +227,13 @@ extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *
     const int rows_min = (kh - 1) * dh + 1;            // input rows for one output row
     const long long lds_one = (long long)rows_min * WL * 4;
     if (lds_one <= kIm2colLdsBytes) {
-        // Largest band whose staged rows fit the LDS budget.
+        // Band height: many small blocks keep more independent store streams in flight than a
+        // few long-running ones, but every band re-stages (kh-1)*dh halo rows, which costs more
+        // the larger the stride.  Aim at 448*sh*sw outputs per tap and block (8 rows of 56 at
+        // stride 1 measured best inside the conv step), capped by the LDS budget.
         int R = (int)((kIm2colLdsBytes / 4 / WL - rows_min) / sh + 1);
+        const int want = (448 * sh * sw + OW - 1) / OW;
+        if (R > want) R = want;
         if (R > OH) R = OH;
         if (R < 1) R = 1;
         const int bands = (OH + R - 1) / R;
@@ -196,12 +241,15 @@ extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "im2col: too many tiles (%lld)", blocks);
         const size_t lds = (size_t)((R - 1) * sh + rows_min) * WL * 4;
         const bool vec4 = (OW % 4 == 0) && aligned16(cols);
-        if (vec4)
-            hipLaunchKernelGGL(im2col_lds_kernel<true>, dim3((unsigned)blocks), dim3(kIm2colThreads),
-                               lds, as_stream(stream), x, cols, g, R, bands, WL);
-        else
-            hipLaunchKernelGGL(im2col_lds_kernel<false>, dim3((unsigned)blocks),
-                               dim3(kIm2colThreads), lds, as_stream(stream), x, cols, g, R, bands, WL);
+        const bool strm = true;  // streaming stores: cols is far larger than the caches
+#define AG_IM2COL_LAUNCH(V, S)                                                                           \
+    hipLaunchKernelGGL((im2col_lds_kernel<V, S>), dim3((unsigned)blocks), dim3(kIm2colThreads), lds,      \
+                       as_stream(stream), x, cols, g, R, bands, WL)
+        if (vec4 && strm) AG_IM2COL_LAUNCH(true, true);
+        else if (vec4) AG_IM2COL_LAUNCH(true, false);
+        else if (strm) AG_IM2COL_LAUNCH(false, true);
+        else AG_IM2COL_LAUNCH(false, false);
+#undef AG_IM2COL_LAUNCH
     } else {
         const long long total = planes * kh * kw * (long long)OH * OW;
         long long blocks = (total + 255) / 256;
@@ -223,14 +271,22 @@ extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, floa
     AG_REQUIRE(gx && (cols || OH == 0 || OW == 0), AG_ERR_INVALID_DIMS, "col2im: null pointer");
     AG_REQUIRE((long long)H * W <= 0x7fffffffLL, AG_ERR_INVALID_DIMS, "col2im: plane too large");
     ConvGeom g{C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW};
-    const int chunks = (H * W + 255) / 256;
-    const long long blocks = planes * chunks;
-    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "col2im: too many tiles (%lld)", blocks);
-    if (sh == 1 && sw == 1)
-        hipLaunchKernelGGL(col2im_gather_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), cols, gx, g, chunks);
-    else
-        hipLaunchKernelGGL(col2im_gather_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), cols, gx, g, chunks);
+    if (sh == 1 && sw == 1 && W % 4 == 0 && aligned16(gx)) {
+        const long long groups = planes * H * (W / 4);
+        long long blocks = (groups + 255) / 256;
+        if (blocks > 262144) blocks = 262144;
+        if (kh == 3 && kw == 3)
+            hipLaunchKernelGGL((col2im_unit_vec4_kernel<3, 3>), dim3((unsigned)blocks), dim3(256), 0,
+                               as_stream(stream), cols, gx, g, groups);
+        else
+            hipLaunchKernelGGL((col2im_unit_vec4_kernel<0, 0>), dim3((unsigned)blocks), dim3(256), 0,
+                               as_stream(stream), cols, gx, g, groups);
+    } else {
+        const int chunks = (H * W + 255) / 256;
+        const long long blocks = planes * chunks;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "col2im: too many tiles (%lld)", blocks);
+        hipLaunchKernelGGL(col2im_gather_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cols,
+                           gx, g, chunks);
+    }
     return check_launch("col2im");
 }

@@ -82,6 +82,118 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restric
     gx[flat] = acc;
 }
 
+constexpr int kPoolLdsBytes = 32 * 1024;
+
+// LDS-staged forward: one block per (plane, band of R output rows).  The input rows the band
+// needs are copied to LDS with coalesced loads (each input byte is fetched once), then every
+// thread scans its windows out of LDS.
+__global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__restrict__ x,
+                                                              float *__restrict__ y,
+                                                              float *__restrict__ argmax,
+                                                              int32_t *__restrict__ idx_local,
+                                                              PoolGeom g, int R, int bands, int vec)
+{
+    extern __shared__ float tile[];
+    const int band = blockIdx.x % bands;
+    const long long plane = blockIdx.x / bands;
+    const int oy0 = band * R;
+    const int rows = min(R, g.OH - oy0);
+    const int iy0 = oy0 * g.stride;
+    const int in_rows = (rows - 1) * g.stride + g.size;
+    const long long base = plane * (long long)g.H * g.W;
+    const float *xp = x + base + (long long)iy0 * g.W;
+    const int n_in = in_rows * g.W;
+    if (vec) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(xp);
+        float4 *t4 = reinterpret_cast<float4 *>(tile);
+        for (int e = threadIdx.x; e < n_in / 4; e += 256) t4[e] = ld_stream(x4 + e);
+    } else {
+        for (int e = threadIdx.x; e < n_in; e += 256) tile[e] = xp[e];
+    }
+    __syncthreads();
+    const long long obase = plane * (long long)g.OH * g.OW + (long long)oy0 * g.OW;
+    for (int o = threadIdx.x; o < rows * g.OW; o += 256) {
+        const int r = o / g.OW, ox = o - r * g.OW;
+        const float *w0 = tile + (r * g.stride) * g.W + ox * g.stride;
+        float best = -FLT_MAX;
+        int best_local = -1;
+        for (int dy = 0; dy < g.size; ++dy)
+            for (int dx = 0; dx < g.size; ++dx) {
+                const float v = w0[dy * g.W + dx];
+                if (v > best) {
+                    best = v;
+                    best_local = (iy0 + r * g.stride + dy) * g.W + ox * g.stride + dx;
+                }
+            }
+        st_stream(y + obase + o, best);
+        const unsigned long long flat = best_local >= 0 ? (unsigned long long)(base + best_local) : 0ull;
+        st_stream(argmax + obase + o, (float)flat);
+        if (idx_local) st_stream(idx_local + obase + o, best_local);
+    }
+}
+
+// LDS-staged backward: one block per (plane, band of IR input rows).  The upstream gradient and
+// the selection indices of every window that can touch the band are staged in LDS; each thread
+// then produces four consecutive pixels (one 128-bit store), visiting candidate windows in
+// ascending (oy, ox) order.
+template <bool EXACT>
+__global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__restrict__ gy,
+                                                              const float *__restrict__ argmax,
+                                                              const int32_t *__restrict__ idx_local,
+                                                              float *__restrict__ gx, PoolGeom g,
+                                                              int IR, int bands, int max_orows)
+{
+    extern __shared__ float smem[];
+    float *s_gy = smem;
+    int *s_idx = reinterpret_cast<int *>(smem + max_orows * g.OW);
+    const int band = blockIdx.x % bands;
+    const long long plane = blockIdx.x / bands;
+    const int iy0 = band * IR;
+    const int rows = min(IR, g.H - iy0);
+    const int iy1 = iy0 + rows - 1;
+    // output rows whose window intersects [iy0, iy1]
+    const int o_lo = iy0 < g.size ? 0 : (iy0 - g.size + g.stride) / g.stride;
+    const int o_hi = min(iy1 / g.stride, g.OH - 1);
+    const int n_o = max(0, o_hi - o_lo + 1) * g.OW;
+    const long long obase = plane * (long long)g.OH * g.OW + (long long)o_lo * g.OW;
+    const long long xbase = plane * (long long)g.H * g.W;
+    for (int e = threadIdx.x; e < n_o; e += 256) {
+        s_gy[e] = gy[obase + e];
+        if (EXACT) {
+            s_idx[e] = idx_local[obase + e];
+        } else {
+            // whole-tensor offset -> plane-local (exact below 2^24 elements); other planes never match
+            const long long a = (long long)argmax[obase + e] - xbase;
+            s_idx[e] = (a >= 0 && a < (long long)g.H * g.W) ? (int)a : -1;
+        }
+    }
+    __syncthreads();
+    const int W4 = g.W >> 2;
+    for (int q = threadIdx.x; q < rows * W4; q += 256) {
+        const int r = q / W4, ix0 = (q - r * W4) * 4;
+        const int iy = iy0 + r;
+        const int oy_lo = iy < g.size ? 0 : (iy - g.size + g.stride) / g.stride;
+        const int oy_hi = min(iy / g.stride, g.OH - 1);
+        float out[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int ix = ix0 + k;
+            const int ox_lo = ix < g.size ? 0 : (ix - g.size + g.stride) / g.stride;
+            const int ox_hi = min(ix / g.stride, g.OW - 1);
+            const int me = iy * g.W + ix;
+            float acc = 0.f;
+            for (int oy = oy_lo; oy <= oy_hi; ++oy)
+                for (int ox = ox_lo; ox <= ox_hi; ++ox) {
+                    const int o = (oy - o_lo) * g.OW + ox;
+                    if (s_idx[o] == me) acc += s_gy[o];
+                }
+            out[k] = acc;
+        }
+        st_stream(reinterpret_cast<float4 *>(gx + xbase + (long long)iy * g.W + ix0),
+                  make_float4(out[0], out[1], out[2], out[3]));
+    }
+}
+
 template <bool EXACT>
 __global__ __launch_bounds__(256) void maxpool_gradgrad_kernel(const float *__restrict__ ggx,
                                                                const float *__restrict__ argmax,
@@ -134,11 +246,26 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
     if ((long long)B * C == 0) return AG_OK;
     if (ag_status_t s = pool_geom("max_pool2d", B, C, H, W, size, pad, stride, &g)) return s;
     AG_REQUIRE(x && y && argmax, AG_ERR_INVALID_DIMS, "max_pool2d: null pointer");
-    const int chunks = (g.OH * g.OW + 255) / 256;
-    const long long blocks = (long long)B * C * chunks;
-    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
-    hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), x,
-                       y, argmax, idx_local, g, chunks);
+    if (g.OH <= 0 || g.OW <= 0) return AG_OK;
+    const long long row_bytes = (long long)W * 4;
+    if (row_bytes * size <= kPoolLdsBytes) {
+        // rows of output per band so that the staged input rows fit the LDS budget
+        int R = (int)((kPoolLdsBytes / row_bytes - size) / stride + 1);
+        if (R > g.OH) R = g.OH;
+        const int bands = (g.OH + R - 1) / R;
+        const long long blocks = (long long)B * C * bands;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
+        const size_t lds = (size_t)((R - 1) * stride + size) * row_bytes;
+        const int vec = (W % 4 == 0) && aligned16(x);
+        hipLaunchKernelGGL(maxpool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), lds, as_stream(stream), x,
+                           y, argmax, idx_local, g, R, bands, vec);
+    } else {
+        const int chunks = (g.OH * g.OW + 255) / 256;
+        const long long blocks = (long long)B * C * chunks;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
+        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), x, y,
+                           argmax, idx_local, g, chunks);
+    }
     return check_launch("max_pool2d");
 }
 
@@ -153,6 +280,29 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
     AG_REQUIRE(idx_local || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
                "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the int32 plane-local indices",
                (long long)B * C * H * W);
+    // LDS-staged path: W % 4 == 0 (128-bit stores) and the windows of a band fit the budget
+    const long long orow_bytes = (long long)g.OW * 8;  // gy + index per output
+    if (W % 4 == 0 && aligned16(gx) && g.OH > 0 && g.OW > 0 &&
+        orow_bytes * ((size + stride - 1) / stride + 1) <= kPoolLdsBytes) {
+        // IR input rows touch at most IR/stride + size/stride + 2 output rows
+        const int budget_rows = (int)(kPoolLdsBytes / orow_bytes);
+        int IR = (budget_rows - (size + stride - 1) / stride - 2) * stride;
+        if (IR < 1) IR = 1;
+        if (IR > H) IR = H;
+        const int bands = (H + IR - 1) / IR;
+        int max_orows = (IR - 1) / stride + (size + stride - 1) / stride + 2;
+        if (max_orows > g.OH) max_orows = g.OH;
+        const long long blocks = (long long)B * C * bands;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);
+        const size_t lds = (size_t)max_orows * orow_bytes;
+        if (idx_local)
+            hipLaunchKernelGGL(maxpool_bwd_lds_kernel<true>, dim3((unsigned)blocks), dim3(256), lds,
+                               as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows);
+        else
+            hipLaunchKernelGGL(maxpool_bwd_lds_kernel<false>, dim3((unsigned)blocks), dim3(256), lds,
+                               as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows);
+        return check_launch("max_pool2d_grad");
+    }
     const int chunks = (H * W + 255) / 256;
     const long long blocks = (long long)B * C * chunks;
     AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);

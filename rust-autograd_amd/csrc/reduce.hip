@@ -49,7 +49,17 @@ __global__ __launch_bounds__(kSumThreads) void sum_stage1_kernel(const float *__
     if (vec) {
         const size_t n4 = n / 4;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
-        for (size_t i = tid; i < n4; i += nthreads) {
+        size_t i = tid;
+        // four independent 128-bit loads in flight per thread
+        for (; i + 3 * nthreads < n4; i += 4 * nthreads) {
+            const float4 v0 = ld_stream(x4 + i), v1 = ld_stream(x4 + i + nthreads), v2 = ld_stream(x4 + i + 2 * nthreads),
+                         v3 = ld_stream(x4 + i + 3 * nthreads);
+            a0 += (v0.x + v1.x) + (v2.x + v3.x);
+            a1 += (v0.y + v1.y) + (v2.y + v3.y);
+            a2 += (v0.z + v1.z) + (v2.z + v3.z);
+            a3 += (v0.w + v1.w) + (v2.w + v3.w);
+        }
+        for (; i < n4; i += nthreads) {
             const float4 v = x4[i];
             a0 += v.x;
             a1 += v.y;

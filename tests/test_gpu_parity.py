@@ -172,7 +172,7 @@ def test_gemm_all_layouts(K, orc, rng, shape, ta, tb):
         assert_close(got, orc.matmul(a, b, ta, tb), "gemm vs f32 oracle")
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
+@pytest.mark.parametrize("cfg", list(range(13)))
 def test_gemm_every_tile_configuration(K, rng, cfg):
     L = K.capi.lib()
     m, n, k = 200, 333, 130
