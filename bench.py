@@ -32,6 +32,19 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 # headline workload
 B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 
+# HBM bytes per launch at the headline shape, measured with two rocprofv3 --pmc passes over this
+# script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
+# reads for the --pmc-calibration copy kernel (1 GiB in, 1 GiB out): FETCH_SIZE reads 0.5 of the
+# true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
+KIB = 1024.0
+TRAFFIC_BYTES = {
+    "gemm_fwd": (920481.0 * 2.0 + 401408.0) * KIB,
+    "gemm_filter_grad": (1157507.4 * 2.0 + 73728.0) * KIB,
+    "gemm_input_grad": (291922.1 * 2.0 + 1806336.0) * KIB,
+    "im2col": (124964.5 * 2.0 + 1806336.2) * KIB,
+    "col2im": (920882.1 * 2.0 + 200704.0) * KIB,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -42,6 +55,10 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
     ap.add_argument("--cpu-images", type=int, default=32, help="images in the CPU baseline sample")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also launch one plain copy kernel (ag_scale_f32 by 1.0) over 2^28 floats, "
+                         "so that a rocprofv3 --pmc run of this command holds a kernel of known traffic "
+                         "(1 GiB read, 1 GiB written) to scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -182,6 +199,13 @@ def main():
         T.run("col2im", lambda: chk(L.ag_col2im_f32(st(), ptr(gcols), ptr(gx), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
                                                     STRIDE, DIL, DIL, OH, OH)))
 
+    if args.pmc_calibration:
+        src = torch.ones(1 << 28, device=dev)
+        dst = torch.empty_like(src)
+        chk(L.ag_scale_f32(st(), ptr(src), 1.0, ptr(dst), src.numel()))
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -203,12 +227,16 @@ def main():
     for name in ("im2col", "col2im"):
         gbs = col_bytes / (per[name] * 1e-3) / 1e9
         kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+    if Bn == B:
+        for name in kernels:
+            kernels[name]["traffic_bytes"] = round(TRAFFIC_BYTES[name])
     gemm_ms = sum(per[n] for n in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"))
     gemm_tf = 3 * gemm_flop / (gemm_ms * 1e-3) / 1e12
     dominant = max(("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"), key=lambda n: per[n])
     dom_tf = gemm_flop / (per[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(dom_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4),
+                "traffic": round(TRAFFIC_BYTES[dominant]) if Bn == B else None,
                 "gemm_phase_TFLOP/s": round(gemm_tf, 2),
                 "gemm_phase_frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)}
 

@@ -192,6 +192,56 @@ __global__ __launch_bounds__(256) void col2im_unit_vec4_kernel(const float *__re
     }
 }
 
+// Stride 2 on both axes: one thread per 2x2 block of destination pixels.  Every tap (ky, kx)
+// feeds exactly one pixel of the block (the one whose offset has the right parity), so a thread
+// reads each of the kh*kw planes once, at consecutive positions for consecutive threads, and no
+// lane idles on a divisibility test.  Taps are visited in (ky, kx) ascending order, so each
+// pixel still receives its terms in the reference's order.
+__global__ __launch_bounds__(256) void col2im_stride2_kernel(const float *__restrict__ cols,
+                                                             float *__restrict__ gx, ConvGeom g,
+                                                             long long nblk)
+{
+    const int BW = (g.W + 1) >> 1, BH = (g.H + 1) >> 1;
+    const long long P = (long long)g.OH * g.OW;
+    for (long long gi = blockIdx.x * 256LL + threadIdx.x; gi < nblk; gi += gridDim.x * 256LL) {
+        const long long rowi = gi / BW;  // (plane, by)
+        const int bx = (int)(gi - rowi * BW);
+        const long long plane = rowi / BH;
+        const int by = (int)(rowi - plane * BH);
+        const float *cp = cols + plane * (long long)(g.kh * g.kw) * P;
+        float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            const int ry = (ky * g.dh - g.ph) & 1;  // parity of the row this tap feeds
+            const int ty = 2 * by + ry + g.ph - ky * g.dh;
+            const int oy = ty >> 1;
+            const bool vy = ty >= 0 && oy < g.OH;
+            for (int kx = 0; kx < g.kw; ++kx) {
+                const int rx = (kx * g.dw - g.pw) & 1;
+                const int tx = 2 * bx + rx + g.pw - kx * g.dw;
+                const int ox = tx >> 1;
+                if (vy && tx >= 0 && ox < g.OW) {
+                    const float v = cp[(long long)(ky * g.kw + kx) * P + (long long)oy * g.OW + ox];
+                    if (ry == 0) {
+                        if (rx == 0) a00 += v;
+                        else a01 += v;
+                    } else {
+                        if (rx == 0) a10 += v;
+                        else a11 += v;
+                    }
+                }
+            }
+        }
+        float *dst = gx + plane * (long long)g.H * g.W + (long long)(2 * by) * g.W + 2 * bx;
+        const bool c1 = 2 * bx + 1 < g.W, r1 = 2 * by + 1 < g.H;
+        dst[0] = a00;
+        if (c1) dst[1] = a01;
+        if (r1) {
+            dst[g.W] = a10;
+            if (c1) dst[g.W + 1] = a11;
+        }
+    }
+}
+
 static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int kh, int kw, int ph,
                               int pw, int sh, int sw, int dh, int dw)
 {
@@ -281,6 +331,12 @@ extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, floa
         else
             hipLaunchKernelGGL((col2im_unit_vec4_kernel<0, 0>), dim3((unsigned)blocks), dim3(256), 0,
                                as_stream(stream), cols, gx, g, groups);
+    } else if (sh == 2 && sw == 2) {
+        const long long nblk = planes * ((H + 1) / 2) * ((W + 1) / 2);
+        long long blocks = (nblk + 255) / 256;
+        if (blocks > 1048576) blocks = 1048576;
+        hipLaunchKernelGGL(col2im_stride2_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cols,
+                           gx, g, nblk);
     } else {
         const int chunks = (H * W + 255) / 256;
         const long long blocks = planes * chunks;

@@ -87,6 +87,7 @@ constexpr int kPoolLdsBytes = 32 * 1024;
 // LDS-staged forward: one block per (plane, band of R output rows).  The input rows the band
 // needs are copied to LDS with coalesced loads (each input byte is fetched once), then every
 // thread scans its windows out of LDS.
+template <int SIZE, int STRIDE>  // 0 = run-time window / stride
 __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__restrict__ x,
                                                               float *__restrict__ y,
                                                               float *__restrict__ argmax,
@@ -94,12 +95,13 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
                                                               PoolGeom g, int R, int bands, int vec)
 {
     extern __shared__ float tile[];
+    const int size = SIZE ? SIZE : g.size, stride = STRIDE ? STRIDE : g.stride;
     const int band = blockIdx.x % bands;
     const long long plane = blockIdx.x / bands;
     const int oy0 = band * R;
     const int rows = min(R, g.OH - oy0);
-    const int iy0 = oy0 * g.stride;
-    const int in_rows = (rows - 1) * g.stride + g.size;
+    const int iy0 = oy0 * stride;
+    const int in_rows = (rows - 1) * stride + size;
     const long long base = plane * (long long)g.H * g.W;
     const float *xp = x + base + (long long)iy0 * g.W;
     const int n_in = in_rows * g.W;
@@ -114,15 +116,17 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
     const long long obase = plane * (long long)g.OH * g.OW + (long long)oy0 * g.OW;
     for (int o = threadIdx.x; o < rows * g.OW; o += 256) {
         const int r = o / g.OW, ox = o - r * g.OW;
-        const float *w0 = tile + (r * g.stride) * g.W + ox * g.stride;
+        const float *w0 = tile + (r * stride) * g.W + ox * stride;
         float best = -FLT_MAX;
         int best_local = -1;
-        for (int dy = 0; dy < g.size; ++dy)
-            for (int dx = 0; dx < g.size; ++dx) {
+#pragma unroll
+        for (int dy = 0; dy < size; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < size; ++dx) {
                 const float v = w0[dy * g.W + dx];
                 if (v > best) {
                     best = v;
-                    best_local = (iy0 + r * g.stride + dy) * g.W + ox * g.stride + dx;
+                    best_local = (iy0 + r * stride + dy) * g.W + ox * stride + dx;
                 }
             }
         st_stream(y + obase + o, best);
@@ -136,7 +140,7 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
 // the selection indices of every window that can touch the band are staged in LDS; each thread
 // then produces four consecutive pixels (one 128-bit store), visiting candidate windows in
 // ascending (oy, ox) order.
-template <bool EXACT>
+template <bool EXACT, int SIZE, int STRIDE>  // SIZE/STRIDE 0 = run-time
 __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__restrict__ gy,
                                                               const float *__restrict__ argmax,
                                                               const int32_t *__restrict__ idx_local,
@@ -146,21 +150,22 @@ __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__res
     extern __shared__ float smem[];
     float *s_gy = smem;
     int *s_idx = reinterpret_cast<int *>(smem + max_orows * g.OW);
+    const int size = SIZE ? SIZE : g.size, stride = STRIDE ? STRIDE : g.stride;
     const int band = blockIdx.x % bands;
     const long long plane = blockIdx.x / bands;
     const int iy0 = band * IR;
     const int rows = min(IR, g.H - iy0);
     const int iy1 = iy0 + rows - 1;
     // output rows whose window intersects [iy0, iy1]
-    const int o_lo = iy0 < g.size ? 0 : (iy0 - g.size + g.stride) / g.stride;
-    const int o_hi = min(iy1 / g.stride, g.OH - 1);
+    const int o_lo = iy0 < size ? 0 : (iy0 - size + stride) / stride;
+    const int o_hi = min(iy1 / stride, g.OH - 1);
     const int n_o = max(0, o_hi - o_lo + 1) * g.OW;
     const long long obase = plane * (long long)g.OH * g.OW + (long long)o_lo * g.OW;
     const long long xbase = plane * (long long)g.H * g.W;
     for (int e = threadIdx.x; e < n_o; e += 256) {
-        s_gy[e] = gy[obase + e];
+        s_gy[e] = ld_stream(gy + obase + e);
         if (EXACT) {
-            s_idx[e] = idx_local[obase + e];
+            s_idx[e] = ld_stream(idx_local + obase + e);
         } else {
             // whole-tensor offset -> plane-local (exact below 2^24 elements); other planes never match
             const long long a = (long long)argmax[obase + e] - xbase;
@@ -168,25 +173,42 @@ __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__res
         }
     }
     __syncthreads();
+    // A pixel lies in at most CAND windows per axis; they are visited in ascending order.
+    constexpr int CAND = (SIZE && STRIDE) ? (SIZE + STRIDE - 1) / STRIDE : 0;
     const int W4 = g.W >> 2;
     for (int q = threadIdx.x; q < rows * W4; q += 256) {
         const int r = q / W4, ix0 = (q - r * W4) * 4;
         const int iy = iy0 + r;
-        const int oy_lo = iy < g.size ? 0 : (iy - g.size + g.stride) / g.stride;
-        const int oy_hi = min(iy / g.stride, g.OH - 1);
+        const int oy_lo = iy < size ? 0 : (iy - size + stride) / stride;
+        const int oy_hi = min(iy / stride, g.OH - 1);
         float out[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int ix = ix0 + k;
-            const int ox_lo = ix < g.size ? 0 : (ix - g.size + g.stride) / g.stride;
-            const int ox_hi = min(ix / g.stride, g.OW - 1);
+            const int ox_lo = ix < size ? 0 : (ix - size + stride) / stride;
+            const int ox_hi = min(ix / stride, g.OW - 1);
             const int me = iy * g.W + ix;
             float acc = 0.f;
-            for (int oy = oy_lo; oy <= oy_hi; ++oy)
-                for (int ox = ox_lo; ox <= ox_hi; ++ox) {
-                    const int o = (oy - o_lo) * g.OW + ox;
-                    if (s_idx[o] == me) acc += s_gy[o];
+            if (CAND) {
+#pragma unroll
+                for (int a = CAND - 1; a >= 0; --a) {
+                    const int oy = iy / stride - a;
+                    if (oy < oy_lo || oy > oy_hi) continue;
+#pragma unroll
+                    for (int b = CAND - 1; b >= 0; --b) {
+                        const int ox = ix / stride - b;
+                        if (ox < ox_lo || ox > ox_hi) continue;
+                        const int o = (oy - o_lo) * g.OW + ox;
+                        if (s_idx[o] == me) acc += s_gy[o];
+                    }
                 }
+            } else {
+                for (int oy = oy_lo; oy <= oy_hi; ++oy)
+                    for (int ox = ox_lo; ox <= ox_hi; ++ox) {
+                        const int o = (oy - o_lo) * g.OW + ox;
+                        if (s_idx[o] == me) acc += s_gy[o];
+                    }
+            }
             out[k] = acc;
         }
         st_stream(reinterpret_cast<float4 *>(gx + xbase + (long long)iy * g.W + ix0),
@@ -257,8 +279,13 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
         const size_t lds = (size_t)((R - 1) * stride + size) * row_bytes;
         const int vec = (W % 4 == 0) && aligned16(x);
-        hipLaunchKernelGGL(maxpool_fwd_lds_kernel, dim3((unsigned)blocks), dim3(256), lds, as_stream(stream), x,
-                           y, argmax, idx_local, g, R, bands, vec);
+#define AG_POOL_FWD(SZ, ST)                                                                                   \
+    hipLaunchKernelGGL((maxpool_fwd_lds_kernel<SZ, ST>), dim3((unsigned)blocks), dim3(256), lds, as_stream(stream), \
+                       x, y, argmax, idx_local, g, R, bands, vec)
+        if (size == 3 && stride == 2) AG_POOL_FWD(3, 2);
+        else if (size == 2 && stride == 2) AG_POOL_FWD(2, 2);
+        else AG_POOL_FWD(0, 0);
+#undef AG_POOL_FWD
     } else {
         const int chunks = (g.OH * g.OW + 255) / 256;
         const long long blocks = (long long)B * C * chunks;
@@ -295,12 +322,20 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
         const long long blocks = (long long)B * C * bands;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);
         const size_t lds = (size_t)max_orows * orow_bytes;
-        if (idx_local)
-            hipLaunchKernelGGL(maxpool_bwd_lds_kernel<true>, dim3((unsigned)blocks), dim3(256), lds,
-                               as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows);
-        else
-            hipLaunchKernelGGL(maxpool_bwd_lds_kernel<false>, dim3((unsigned)blocks), dim3(256), lds,
-                               as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows);
+#define AG_POOL_BWD(EX, SZ, ST)                                                                               \
+    hipLaunchKernelGGL((maxpool_bwd_lds_kernel<EX, SZ, ST>), dim3((unsigned)blocks), dim3(256), lds,               \
+                       as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows)
+        const bool s32 = size == 3 && stride == 2, s22 = size == 2 && stride == 2;
+        if (idx_local) {
+            if (s32) AG_POOL_BWD(true, 3, 2);
+            else if (s22) AG_POOL_BWD(true, 2, 2);
+            else AG_POOL_BWD(true, 0, 0);
+        } else {
+            if (s32) AG_POOL_BWD(false, 3, 2);
+            else if (s22) AG_POOL_BWD(false, 2, 2);
+            else AG_POOL_BWD(false, 0, 0);
+        }
+#undef AG_POOL_BWD
         return check_launch("max_pool2d_grad");
     }
     const int chunks = (H * W + 255) / 256;

@@ -100,6 +100,34 @@ __global__ __launch_bounds__(256) void fold_axis_seq_kernel(const float *__restr
     }
 }
 
+// Long axis, few outputs: x [outer][len][inner] -> part [outer][splits][inner]; split s adds rows
+// [s*chunk, min(len, (s+1)*chunk)) sequentially.  A second fold_axis_seq_kernel over the `splits`
+// axis finishes the sum (fixed order, deterministic; rounding differs from one long chain).
+__global__ __launch_bounds__(256) void fold_axis_split_kernel(const float *__restrict__ x,
+                                                              float *__restrict__ part, size_t outer,
+                                                              size_t len, size_t inner, size_t splits,
+                                                              size_t chunk)
+{
+    const size_t total = outer * splits * inner;
+    for (size_t t = blockIdx.x * 256ull + threadIdx.x; t < total; t += gridDim.x * 256ull) {
+        const size_t i = t % inner, os = t / inner;
+        const size_t sp = os % splits, o = os / splits;
+        const size_t r0 = sp * chunk, r1 = min(len, r0 + chunk);
+        const float *p = x + (o * len + r0) * inner + i;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        size_t r = r0;
+        for (; r + 3 < r1; r += 4) {  // four independent loads in flight
+            a0 += p[0];
+            a1 += p[inner];
+            a2 += p[2 * inner];
+            a3 += p[3 * inner];
+            p += 4 * inner;
+        }
+        for (; r < r1; ++r, p += inner) a0 += p[0];
+        part[t] = (a0 + a1) + (a2 + a3);
+    }
+}
+
 // x [rows][len] -> out [rows]: one wave per row, lanes stride the row, shuffle fold.
 __global__ __launch_bounds__(256) void fold_last_axis_kernel(const float *__restrict__ x,
                                                              float *__restrict__ out, size_t rows,
@@ -145,6 +173,19 @@ __global__ __launch_bounds__(256) void broadcast_kernel(const float *__restrict_
         }
         gx[flat] = gy[src];
     }
+}
+
+// Split a long fold with few outputs so that the whole chip takes part.  Returns the number of
+// splits (1 = no split) and the rows per split.
+static size_t fold_splits(size_t outer, size_t len, size_t inner, size_t *chunk)
+{
+    *chunk = len;
+    if (inner <= 1 || len < 1024 || outer * inner >= 262144) return 1;
+    size_t want = 1048576 / (outer * inner);  // aim at ~1 M threads
+    if (want > len / 64) want = len / 64;
+    if (want < 2) return 1;
+    *chunk = (len + want - 1) / want;
+    return (len + *chunk - 1) / *chunk;
 }
 
 static unsigned grid_for(size_t work_items, int per_block)
@@ -206,15 +247,53 @@ extern "C" ag_status_t ag_sum_all_f32(ag_stream_t stream, const float *x, size_t
     return check_launch("sum_all");
 }
 
+// Workspace layout: two ping-pong buffers for the intermediate results of multi-axis reductions
+// (each as large as the result of the first fold) followed by the partials of a split fold.
+static void reduce_ws_layout(const int *shape, int rank, const int *sorted_axes, int n_axes, size_t *pingpong,
+                             size_t *split_floats)
+{
+    *pingpong = 0;
+    *split_floats = 0;
+    if (n_axes <= 0 || rank <= 0) return;
+    size_t total = 1;
+    int dims[kMaxRank];
+    for (int i = 0; i < rank; ++i) {
+        dims[i] = shape[i];
+        total *= (size_t)shape[i];
+    }
+    if (n_axes > 1) {
+        const int last = sorted_axes[n_axes - 1];
+        size_t first = shape[last] ? total / (size_t)shape[last] : 0;
+        if (first < 1) first = 1;
+        *pingpong = (first + 3) & ~(size_t)3;
+    }
+    for (int a = n_axes - 1; a >= 0; --a) {
+        size_t outer = 1, inner = 1, chunk;
+        for (int i = 0; i < sorted_axes[a]; ++i) outer *= (size_t)dims[i];
+        for (int i = sorted_axes[a] + 1; i < rank; ++i) inner *= (size_t)dims[i];
+        const size_t sp = fold_splits(outer, (size_t)dims[sorted_axes[a]], inner, &chunk);
+        if (sp > 1 && sp * outer * inner > *split_floats) *split_floats = sp * outer * inner;
+        dims[sorted_axes[a]] = 1;
+    }
+}
+
 extern "C" size_t ag_reduce_sum_f32_workspace(const int *shape, int rank, const int *axes, int n_axes)
 {
-    // Two ping-pong buffers, each as large as the result of the first fold.
-    if (n_axes <= 1 || rank <= 0) return 16;
-    int last = axes[0];
-    for (int i = 1; i < n_axes; ++i) last = axes[i] > last ? axes[i] : last;
-    size_t total = 1;
-    for (int i = 0; i < rank; ++i) total *= (size_t)(i == last ? 1 : shape[i]);
-    return 2 * sizeof(float) * (total ? total : 1) + 32;
+    int ax[kMaxRank];
+    if (rank < 0 || rank > kMaxRank || n_axes < 0 || n_axes > rank) return 16;
+    for (int i = 0; i < n_axes; ++i) {
+        if (axes[i] < 0 || axes[i] >= rank) return 16;
+        ax[i] = axes[i];
+    }
+    for (int i = 1; i < n_axes; ++i)
+        for (int j = i; j > 0 && ax[j - 1] > ax[j]; --j) {
+            const int t = ax[j];
+            ax[j] = ax[j - 1];
+            ax[j - 1] = t;
+        }
+    size_t pp, sf;
+    reduce_ws_layout(shape, rank, ax, n_axes, &pp, &sf);
+    return sizeof(float) * (2 * pp + sf) + 32;
 }
 
 extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, float *out,
@@ -248,32 +327,36 @@ extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, flo
                            1.f, 0);
         return check_launch("reduce_sum");
     }
-    const size_t need = ag_reduce_sum_f32_workspace(shape, rank, ax, n_axes);
-    AG_REQUIRE(n_axes == 1 || (ws && ws_bytes >= need), AG_ERR_INVALID_DIMS,
+    size_t pp, sf;
+    reduce_ws_layout(shape, rank, ax, n_axes, &pp, &sf);
+    const size_t need = sizeof(float) * (2 * pp + sf);
+    AG_REQUIRE(need == 0 || (ws && ws_bytes >= need), AG_ERR_INVALID_DIMS,
                "reduce_sum: workspace of %zu bytes needed, %zu given", need, ws_bytes);
-    float *buf[2] = {nullptr, nullptr};
-    if (n_axes > 1) {
-        size_t first = total / (size_t)(shape[ax[n_axes - 1]] ? shape[ax[n_axes - 1]] : 1);
-        if (first < 1) first = 1;
-        buf[0] = static_cast<float *>(ws);
-        buf[1] = buf[0] + ((first + 3) & ~(size_t)3);
-    }
+    float *buf[2] = {static_cast<float *>(ws), static_cast<float *>(ws) + pp};
+    float *part = static_cast<float *>(ws) + 2 * pp;
     const float *cur = x;
     for (int a = n_axes - 1; a >= 0; --a) {
-        size_t outer = 1, inner = 1;
+        size_t outer = 1, inner = 1, chunk;
         for (int i = 0; i < ax[a]; ++i) outer *= (size_t)dims[i];
         for (int i = ax[a] + 1; i < rank; ++i) inner *= (size_t)dims[i];
         const size_t len = (size_t)dims[ax[a]];
         float *dst = (a == 0) ? out : buf[(n_axes - 1 - a) & 1];
         const int sc = (a == 0) ? do_scale : 0;
+        const size_t sp = fold_splits(outer, len, inner, &chunk);
         // Short innermost folds stay sequential per output (the reference's order, bit-identical);
-        // long rows take one wave each.
-        if (inner == 1 && len > kSeqRowLimit)
+        // long rows take one wave each; long folds with few outputs are split over the chip.
+        if (inner == 1 && len > kSeqRowLimit) {
             hipLaunchKernelGGL(fold_last_axis_kernel, dim3(grid_for(outer, 4)), dim3(256), 0, st, cur, dst,
                                outer, len, scale, sc);
-        else
-            hipLaunchKernelGGL(fold_axis_seq_kernel, dim3(grid_for(outer * inner, 256)), dim3(256), 0, st,
-                               cur, dst, outer, len, inner, scale, sc);
+        } else if (sp > 1) {
+            hipLaunchKernelGGL(fold_axis_split_kernel, dim3(grid_for(outer * sp * inner, 256)), dim3(256), 0, st,
+                               cur, part, outer, len, inner, sp, chunk);
+            hipLaunchKernelGGL(fold_axis_seq_kernel, dim3(grid_for(outer * inner, 256)), dim3(256), 0, st, part,
+                               dst, outer, sp, inner, scale, sc);
+        } else {
+            hipLaunchKernelGGL(fold_axis_seq_kernel, dim3(grid_for(outer * inner, 256)), dim3(256), 0, st, cur,
+                               dst, outer, len, inner, scale, sc);
+        }
         dims[ax[a]] = 1;
         cur = dst;
     }
