@@ -223,6 +223,9 @@ ag_status_t ag_add_n_f32(ag_stream_t stream, const float *const *xs, int count, 
 /* Same-shape MulOp (binary_ops.rs:209-237) and scalar scaling. */
 ag_status_t ag_mul_f32(ag_stream_t stream, const float *a, const float *b, float *out, size_t n);
 ag_status_t ag_scale_f32(ag_stream_t stream, const float *a, float s, float *out, size_t n);
+/* Division by a scalar, out = a / s: the `broadcast / reduction_len` of ReduceMean::grad
+ * (reduction_ops.rs:231-234).  out may alias a. */
+ag_status_t ag_div_scalar_f32(ag_stream_t stream, const float *a, float s, float *out, size_t n);
 /* Fill with a constant (zeros / ones / scalar, const_gen_ops.rs:16-90). */
 ag_status_t ag_fill_f32(ag_stream_t stream, float *out, float value, size_t n);
 /* SparseSoftmaxCrossEntropy::compute (xent_ops.rs:63-115): logits [rows,classes], labels [rows]

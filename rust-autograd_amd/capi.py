@@ -85,6 +85,7 @@ PROTOTYPES = {
     "ag_add_n_f32": (c_i, [c_p, c_p, c_i, c_p, c_sz]),
     "ag_mul_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),
     "ag_scale_f32": (c_i, [c_p, c_p, c_f, c_p, c_sz]),
+    "ag_div_scalar_f32": (c_i, [c_p, c_p, c_f, c_p, c_sz]),
     "ag_fill_f32": (c_i, [c_p, c_p, c_f, c_sz]),
     "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),

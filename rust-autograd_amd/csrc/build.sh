@@ -19,3 +19,12 @@ done
 for p in "${pids[@]}"; do wait "$p"; done
 /opt/rocm/bin/hipcc --offload-arch=gfx950 -shared -fPIC -o "$out" "$here"/obj/*.o
 echo "built $out"
+
+# Host-side operator layer (C++ mirror of the reference's Op / graph / optimizer code); links the
+# kernel library next to it.
+host_out="$here/../libag_host.so"
+/opt/rocm/bin/hipcc -O2 -std=c++17 -fPIC -fvisibility=hidden -Wall -I"$here/../../include" -I"$here/host" -I/opt/rocm/include \
+    -x c++ "$here/host/runtime.cpp" "$here/host/ops.cpp" "$here/host/gradient.cpp" "$here/host/capi_host.cpp" \
+    -D__HIP_PLATFORM_AMD__ -shared -o "$host_out" -L"$here/.." -lag_hip -L/opt/rocm/lib -lamdhip64 \
+    -Wl,-rpath,'$ORIGIN' -Wl,-rpath,/opt/rocm/lib
+echo "built $host_out"

@@ -78,6 +78,12 @@ __global__ __launch_bounds__(256) void scale_kernel(const float *__restrict__ a,
     AG_EW_LOOP(i, n) out[i] = a[i] * s;
 }
 
+__global__ __launch_bounds__(256) void div_scalar_kernel(const float *__restrict__ a, float s,
+                                                         float *__restrict__ out, size_t n)
+{
+    AG_EW_LOOP(i, n) out[i] = a[i] / s;
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(float *__restrict__ out, float v, size_t n)
 {
     AG_EW_LOOP(i, n) out[i] = v;
@@ -192,6 +198,12 @@ extern "C" ag_status_t ag_scale_f32(ag_stream_t stream, const float *a, float s,
 {
     AG_REQUIRE(n == 0 || (a && out), AG_ERR_INVALID_DIMS, "scale: null pointer");
     AG_EW_ENTRY("scale", scale_kernel, n, a, s, out, n);
+}
+
+extern "C" ag_status_t ag_div_scalar_f32(ag_stream_t stream, const float *a, float s, float *out, size_t n)
+{
+    AG_REQUIRE(n == 0 || (a && out), AG_ERR_INVALID_DIMS, "div: null pointer");
+    AG_EW_ENTRY("div", div_scalar_kernel, n, a, s, out, n);
 }
 
 extern "C" ag_status_t ag_fill_f32(ag_stream_t stream, float *out, float value, size_t n)

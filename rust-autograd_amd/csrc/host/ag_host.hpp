@@ -1,0 +1,333 @@
+// Host-side mirror of rust-autograd's operator interface for the GPU path.
+//
+// The reference is Rust; this is its C++ counterpart for the same path: `Op` with
+// `compute(ComputeContext&)` / `grad(GradientContext&)` (src/op.rs:90-101), a lazy `Graph` of
+// `Tensor` handles built with `TensorBuilder` (src/tensor.rs:609-803), reverse-mode `grad()`
+// (src/gradient.rs:20-247, src/tensor_ops/mod.rs:94-114), the evaluator (src/evaluation.rs:
+// 251-363), `VariableEnvironment` (src/variable.rs) and the `Adam` optimizer
+// (src/optimizers/adam.rs).  Arrays live in device memory; every op's numerics is one or more
+// calls into the C ABI of libag_hip.so.  Only what the conv / matmul / pool / reduce / Adam path
+// and its immediate neighbours need is here; it is not a port of the crate.
+#pragma once
+#include <stdexcept>
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <optional>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace ag {
+namespace host {
+
+// ---------------------------------------------------------------------------------------------
+// errors                                                                        src/op.rs:66-73
+// ---------------------------------------------------------------------------------------------
+enum class ErrorKind { None = 0, NdArrayError = 1, IncompatibleShape = 2, TypeUnsupported = 3, InvalidDims = 4,
+                       OutOfBounds = 5, Hip = 100 };
+
+struct OpError {
+    ErrorKind kind = ErrorKind::None;
+    std::string message;
+    bool ok() const { return kind == ErrorKind::None; }
+    static OpError none() { return OpError{}; }
+    static OpError make(ErrorKind k, std::string m) { return OpError{k, std::move(m)}; }
+};
+
+// Misuse of the API ("Bad op impl: ..." panics of the reference) is reported by throwing this.
+struct Panic : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+// ---------------------------------------------------------------------------------------------
+// device arrays
+// ---------------------------------------------------------------------------------------------
+using Shape = std::vector<int64_t>;
+
+struct DeviceBlock;  // one allocation of the caching arena
+
+// Contiguous row-major f32 array in device memory.  Copies share the block (cheap views);
+// `deep_copy()` allocates.  A default-constructed array has rank 0 and no storage.
+class NdArray {
+  public:
+    NdArray() = default;
+    static NdArray empty(const Shape &shape);
+    static NdArray zeros(const Shape &shape);
+    static NdArray filled(const Shape &shape, float value);
+    static NdArray from_host(const Shape &shape, const float *data);
+    static NdArray scalar(float v) { return filled({}, v); }
+
+    const Shape &shape() const { return shape_; }
+    int ndim() const { return (int)shape_.size(); }
+    size_t len() const;
+    float *ptr() const;
+    bool defined() const { return block_ != nullptr; }
+    NdArray reshaped(const Shape &shape) const;  // same storage, new extents (len must match)
+    NdArray deep_copy() const;
+    std::vector<float> to_host() const;  // synchronises the stream
+
+  private:
+    Shape shape_;
+    std::shared_ptr<DeviceBlock> block_;
+};
+
+void *current_stream();  // hipStream_t used by every op (the null stream)
+void synchronize();
+
+// ---------------------------------------------------------------------------------------------
+// graph                                                        src/tensor.rs, src/graph.rs
+// ---------------------------------------------------------------------------------------------
+class Graph;
+class Op;
+class Context;
+using TensorID = int;
+using VariableID = int;
+
+struct Tensor {  // a (graph, id) handle, like the reference's Tensor<'graph, F>
+    Graph *graph = nullptr;
+    TensorID id = -1;
+    bool valid() const { return graph && id >= 0; }
+};
+
+struct IncomingTensor {  // src/tensor.rs:542-550
+    TensorID id;
+    bool allow_mut;
+    int array_selector;
+};
+
+struct TensorInternal {  // src/tensor.rs:408-441
+    TensorID id = -1;
+    std::unique_ptr<Op> op;
+    std::vector<IncomingTensor> incoming_nodes;
+    int topo_rank = 0;
+    std::string placeholder_name;  // empty = not a placeholder
+    bool is_placeholder = false;
+    bool is_differentiable = true;
+    std::optional<std::vector<IncomingTensor>> backprop_inputs;
+    std::optional<Shape> known_shape;  // -1 = unknown extent
+    VariableID variable_id = -1;
+
+    bool is_source() const { return incoming_nodes.empty(); }
+    bool is_variable() const { return variable_id >= 0; }
+    const std::vector<IncomingTensor> &get_backprop_inputs() const
+    {
+        return backprop_inputs ? *backprop_inputs : incoming_nodes;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Op and its contexts                                                     src/op.rs:90-434
+// ---------------------------------------------------------------------------------------------
+class ComputeContext {
+  public:
+    enum class InputKind { NonVariable, RdOnlyVariable, RdWrVariable };
+    struct Input {
+        NdArray array;
+        InputKind kind;
+        bool taken = false;
+    };
+    explicit ComputeContext(std::vector<Input> xs) : xs_(std::move(xs)) {}
+
+    // Each input may be grabbed once; variable inputs registered with allow_mut must be grabbed
+    // with input_mut (src/op.rs:206-259).
+    NdArray input(size_t i);
+    NdArray input_mut(size_t i);
+    size_t num_inputs() const { return xs_.size(); }
+
+    void append_output(NdArray y) { ys_.push_back(std::move(y)); }
+    // A view of an input: copied first when any input is a variable (src/op.rs:273-287).
+    void append_output_view(const NdArray &y);
+    void append_empty_output() { ys_.push_back(NdArray::zeros({})); }  // src/op.rs:290-294
+
+    std::vector<NdArray> &outputs() { return ys_; }
+    void *stream() const { return current_stream(); }
+
+  private:
+    std::vector<Input> xs_;
+    std::vector<NdArray> ys_;
+};
+
+class GradientContext {
+  public:
+    GradientContext(Tensor gy, Tensor y, Graph *g) : gy_(gy), y_(y), graph_(g) {}
+    Tensor output_grad() const { return gy_; }
+    Tensor output() const { return y_; }
+    Tensor input(size_t i) const;
+    std::vector<Tensor> inputs() const;
+    size_t num_inputs() const;
+    Graph *graph() const { return graph_; }
+    void append_input_grad(std::optional<Tensor> gx) { gxs_.push_back(gx); }
+    std::vector<std::optional<Tensor>> &input_grads() { return gxs_; }
+
+  private:
+    Tensor gy_, y_;
+    Graph *graph_;
+    std::vector<std::optional<Tensor>> gxs_;
+};
+
+class Op {
+  public:
+    virtual ~Op() = default;
+    virtual const char *name() const = 0;
+    virtual OpError compute(ComputeContext &ctx) const = 0;
+    virtual void grad(GradientContext &ctx) const = 0;
+};
+
+class TensorBuilder {  // src/tensor.rs:609-803
+  public:
+    explicit TensorBuilder(Graph *g) : graph_(g) {}
+    TensorBuilder &append_input(Tensor t, bool allow_mut) { return append_input_with_selector(t, allow_mut, 0); }
+    TensorBuilder &append_input_with_selector(Tensor t, bool allow_mut, int selector);
+    TensorBuilder &append_backprop_input(Tensor t);
+    TensorBuilder &set_differentiable(bool d) { differentiable_ = d; return *this; }
+    TensorBuilder &set_variable(VariableID v) { variable_id_ = v; return *this; }
+    TensorBuilder &set_placeholder_name(std::string n) { placeholder_ = std::move(n); is_placeholder_ = true; return *this; }
+    TensorBuilder &set_known_shape(const Shape &s) { known_shape_ = s; return *this; }
+    Tensor build(std::unique_ptr<Op> op);
+
+  private:
+    Graph *graph_;
+    std::vector<IncomingTensor> in_nodes_;
+    std::optional<std::vector<IncomingTensor>> backprop_inputs_;
+    bool differentiable_ = true;
+    VariableID variable_id_ = -1;
+    std::string placeholder_;
+    bool is_placeholder_ = false;
+    std::optional<Shape> known_shape_;
+};
+
+// ---------------------------------------------------------------------------------------------
+// variables                                                              src/variable.rs
+// ---------------------------------------------------------------------------------------------
+class VariableEnvironment {
+  public:
+    // `namespace_id` "" is the default namespace.  Names are unique inside a namespace.
+    VariableID set(const std::string &namespace_id, const std::string &name, NdArray array);
+    VariableID set_anonymous(NdArray array);
+    std::optional<VariableID> find(const std::string &namespace_id, const std::string &name) const;
+    NdArray &array(VariableID id);
+    size_t size() const { return arrays_.size(); }
+    std::vector<std::pair<std::string, VariableID>> names_in(const std::string &namespace_id) const;
+
+    // Runs `f` with a fresh graph bound to this environment (src/variable.rs:670-683).
+    void run(const std::function<void(Context &)> &f);
+
+  private:
+    std::vector<NdArray> arrays_;
+    std::map<std::string, VariableID> name_to_id_;  // "namespace\x01name", src/variable.rs:225-229
+};
+
+struct EvalResult {
+    OpError error;  // error.ok() => array holds the value
+    NdArray array;
+};
+
+class Graph {
+  public:
+    TensorBuilder builder() { return TensorBuilder(this); }
+    TensorInternal &node(TensorID id) { return *nodes_.at((size_t)id); }
+    const TensorInternal &node(TensorID id) const { return *nodes_.at((size_t)id); }
+    size_t num_nodes() const { return nodes_.size(); }
+    Tensor tensor(TensorID id) { return Tensor{this, id}; }
+    TensorID install(std::unique_ptr<TensorInternal> n);  // src/graph.rs:27-47 (node-count guards)
+
+  private:
+    std::vector<std::unique_ptr<TensorInternal>> nodes_;
+};
+
+class Evaluator;
+
+class Context : public Graph {  // src/graph.rs Context: graph + variable environment
+  public:
+    explicit Context(VariableEnvironment *env) : env_(env) {}
+    VariableEnvironment &env() { return *env_; }
+    Tensor variable(VariableID id);                                              // src/graph.rs variable_by_id
+    Tensor variable(const std::string &name, const std::string &namespace_id = "");
+    Tensor placeholder(const std::string &name, const Shape &shape);             // src/graph.rs:178-199
+    Evaluator evaluator();
+    // Graph::eval (src/evaluation.rs:251-363)
+    std::vector<EvalResult> eval(const std::vector<Tensor> &tensors,
+                                 const std::vector<std::pair<std::string, NdArray>> &feeds);
+
+  private:
+    VariableEnvironment *env_;
+    std::unordered_map<VariableID, TensorID> var_nodes_;
+};
+
+class Evaluator {  // src/evaluation.rs:100-181
+  public:
+    explicit Evaluator(Context *c) : ctx_(c) {}
+    Evaluator &push(Tensor t) { targets_.push_back(t); return *this; }
+    Evaluator &extend(const std::vector<Tensor> &ts) { targets_.insert(targets_.end(), ts.begin(), ts.end()); return *this; }
+    Evaluator &feed(const std::string &name, NdArray value) { feeds_.emplace_back(name, std::move(value)); return *this; }
+    std::vector<EvalResult> run() { return ctx_->eval(targets_, feeds_); }
+
+  private:
+    Context *ctx_;
+    std::vector<Tensor> targets_;
+    std::vector<std::pair<std::string, NdArray>> feeds_;
+};
+
+// ---------------------------------------------------------------------------------------------
+// tensor_ops: the functional API for this path                   src/tensor_ops/mod.rs
+// ---------------------------------------------------------------------------------------------
+namespace tensor_ops {
+Tensor conv2d(Tensor x, Tensor w, int pad, int stride);                                   // :2733
+Tensor dilated_conv2d(Tensor x, Tensor w, int pad, int stride, int dilate);               // :2763
+Tensor conv2d_transpose(Tensor x, Tensor w, int pad, int stride);                         // :2799
+Tensor dilated_conv2d_transpose(Tensor x, Tensor w, int pad, int stride, int dilate);     // :2834
+Tensor max_pool2d(Tensor x, int pool_size, int pad, int stride);                          // :2869
+Tensor matmul(Tensor a, Tensor b);                                                        // :1870
+Tensor batch_matmul(Tensor a, Tensor b);                                                  // :2007
+Tensor batch_matmul_t(Tensor a, Tensor b, bool trans_a, bool trans_b);                    // :1967
+Tensor reduce_sum(Tensor x, const std::vector<int> &axes, bool keep_dims);                // :1195
+Tensor reduce_mean(Tensor x, const std::vector<int> &axes, bool keep_dims);               // :1227
+Tensor sum_all(Tensor x);                                                                 // :1149
+Tensor relu(Tensor x);
+Tensor add(Tensor a, Tensor b);   // same shape, or b = [1, cols] / [cols] broadcast over the rows of a 2-D a
+Tensor mul(Tensor a, Tensor b);   // same shape
+Tensor add_n(const std::vector<Tensor> &xs);                                              // :831
+Tensor nth_tensor(Tensor x, int n);                                                       // :545
+Tensor reshape(Tensor x, const Shape &shape);  // one extent may be -1
+Tensor sparse_softmax_cross_entropy(Tensor logits, Tensor labels);
+Tensor scalar(float v, Graph *g);
+Tensor zeros_like(Tensor x);      // zeros(shape(x)): what grad() returns for a non-differentiable x
+Tensor stop_gradient(Tensor x);
+std::vector<Tensor> grad(const std::vector<Tensor> &ys, const std::vector<Tensor> &xs);   // :94
+}  // namespace tensor_ops
+
+// ---------------------------------------------------------------------------------------------
+// optimizers                                        src/optimizers/mod.rs, src/optimizers/adam.rs
+// ---------------------------------------------------------------------------------------------
+namespace optimizers {
+// (variables, gradients) of every variable of `namespace_id` the losses depend on (mod.rs:21-46).
+std::pair<std::vector<Tensor>, std::vector<Tensor>> grad_helper(const std::vector<Tensor> &losses, Context &ctx,
+                                                                const std::string &namespace_id = "");
+
+class Adam {
+  public:
+    // Allocates m, v (zeros) and t (= 1) for every listed variable in `adam_namespace_id`
+    // under the names "<id>m", "<id>v", "<id>t" (adam.rs:75-112).
+    Adam(float alpha, float eps, float b1, float b2, const std::vector<VariableID> &vars, VariableEnvironment &env,
+         std::string adam_namespace_id);
+    static Adam with_defaults(const std::vector<VariableID> &vars, VariableEnvironment &env,
+                              std::string adam_namespace_id)
+    {
+        return Adam(0.001f, 1e-08f, 0.9f, 0.999f, vars, env, std::move(adam_namespace_id));
+    }
+    std::vector<Tensor> compute_updates(const std::vector<Tensor> &params, const std::vector<Tensor> &grads,
+                                        Context &ctx) const;                                     // adam.rs:116-153
+    void update(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, Context &ctx,
+                const std::vector<std::pair<std::string, NdArray>> &feeds) const;                // mod.rs:66-85
+    Tensor get_update_op(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, Context &ctx) const;
+
+  private:
+    float alpha_, eps_, b1_, b2_;
+    std::string ns_;
+};
+}  // namespace optimizers
+
+}  // namespace host
+}  // namespace ag

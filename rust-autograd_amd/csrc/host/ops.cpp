@@ -1,0 +1,1047 @@
+// Operators of the conv / matmul / pool / reduce / Adam path as `Op` implementations whose
+// `compute` calls the C ABI of libag_hip.so and whose `grad` builds the same gradient sub-graphs
+// as the reference.  Citations are to the reference's src/tensor_ops/.
+#include <algorithm>
+#include <sstream>
+
+#include "ag_hip.h"
+#include "ag_host.hpp"
+
+namespace ag {
+namespace host {
+
+namespace {
+
+std::string shape_str(const Shape &s)
+{
+    std::ostringstream os;
+    os << "[";
+    for (size_t i = 0; i < s.size(); ++i) os << (i ? ", " : "") << s[i];
+    os << "]";
+    return os.str();
+}
+
+// Status of a C-ABI call -> OpError (1..5 are the OpError variants, src/op.rs:66-73).
+OpError from_status(ag_status_t st)
+{
+    if (st == AG_OK) return OpError::none();
+    const ErrorKind k = (st >= 1 && st <= 5) ? static_cast<ErrorKind>(st) : ErrorKind::Hip;
+    return OpError::make(k, ag_last_error());
+}
+
+NdArray workspace(size_t bytes) { return NdArray::empty({(int64_t)((bytes + 3) / 4 + 4)}); }
+
+Tensor build(Graph *g, std::initializer_list<Tensor> inputs, std::unique_ptr<Op> op)
+{
+    TensorBuilder b = g->builder();
+    for (const Tensor &t : inputs) b.append_input(t, false);
+    return b.build(std::move(op));
+}
+
+// ------------------------------------------------------------------------------------------
+// Identity (selector for multi-output ops)                     activation_ops.rs:169-181
+// ------------------------------------------------------------------------------------------
+struct Identity : Op {
+    const char *name() const override { return "Identity"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        ctx.append_output_view(ctx.input(0));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override { ctx.append_input_grad(ctx.output_grad()); }
+};
+
+struct StopGradient : Op {  // gradient_ops.rs
+    const char *name() const override { return "StopGradient"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        ctx.append_output_view(ctx.input(0));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override { ctx.append_input_grad(std::nullopt); }
+};
+
+struct ScalarOp : Op {  // const_gen_ops.rs Scalar
+    float value;
+    explicit ScalarOp(float v) : value(v) {}
+    const char *name() const override { return "Scalar"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        ctx.append_output(NdArray::scalar(value));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override { (void)ctx; }
+};
+
+// zeros(shape(x)) with the shape read from x's array.
+struct ZerosLike : Op {
+    const char *name() const override { return "Zeros"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        ctx.append_output(NdArray::zeros(ctx.input(0).shape()));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override { ctx.append_input_grad(std::nullopt); }
+};
+
+// ------------------------------------------------------------------------------------------
+// convolution                                   conv_ops/conv2d.rs, conv_ops/conv2d_transpose.rs
+// ------------------------------------------------------------------------------------------
+struct Conv2D;
+struct Conv2DTranspose;
+struct Conv2DFilterGrad;
+struct Conv2DWithCols;
+struct Conv2DTransposeFilterGrad;
+
+struct ConvHyper {
+    int pad, stride, dilation;
+};
+
+struct Conv2DTransposeFilterGrad : Op, ConvHyper {  // conv2d_transpose.rs:433-480
+    explicit Conv2DTransposeFilterGrad(ConvHyper h) : ConvHyper(h) {}
+    const char *name() const override { return "Conv2DTransposeFilterGrad"; }
+    OpError compute(ComputeContext &ctx) const override;
+    void grad(GradientContext &ctx) const override;
+};
+
+struct Conv2DTranspose : Op, ConvHyper {  // conv2d_transpose.rs:249-301
+    // Inputs (gy, w) as in the reference, which reconstructs the output extent from gy
+    // (conv2d_transpose.rs:55-56).  An optional third input supplies the extent instead (only its
+    // shape is read): Conv2D::grad passes the convolution's input there, so the input gradient
+    // has the input's size even when (H + 2p - k_eff) is not a multiple of the stride.
+    explicit Conv2DTranspose(ConvHyper h) : ConvHyper(h) {}
+    const char *name() const override { return "Conv2DTranspose"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), w = ctx.input(1);
+        int out_h = -1, out_w = -1;
+        if (ctx.num_inputs() > 2) {
+            const NdArray like = ctx.input(2);
+            if (like.ndim() == 4) {
+                out_h = (int)like.shape()[2];
+                out_w = (int)like.shape()[3];
+            }
+        }
+        if (gy.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "conv2d_transpose: Input must be 4D (got " + shape_str(gy.shape()) + ")");
+        if (w.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "conv2d_transpose: Filter must be 4D (got " + shape_str(w.shape()) + ")");
+        const int B = (int)gy.shape()[0], ych = (int)gy.shape()[1], yh = (int)gy.shape()[2], yw = (int)gy.shape()[3];
+        const int xch = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
+        if (ych != w.shape()[0])
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "conv2d_transpose: Number of input channels (" + std::to_string(ych) +
+                                     ") must match second filter dim (" + std::to_string(w.shape()[0]) + ")");
+        const int xh = out_h >= 0 ? out_h : ag_conv_transpose_out_size(yh, kh, pad, stride, dilation);
+        const int xw = out_w >= 0 ? out_w : ag_conv_transpose_out_size(yw, kw, pad, stride, dilation);
+        if (xh < 0 || xw < 0)
+            return OpError::make(ErrorKind::IncompatibleShape, "conv2d_transpose: negative output extent");
+        NdArray gx = NdArray::empty({B, xch, xh, xw});
+        NdArray gcols = NdArray::empty({B, (int64_t)xch * kh * kw, (int64_t)yh * yw});
+        const OpError e = from_status(ag_conv2d_transpose_f32(ctx.stream(), gy.ptr(), w.ptr(), gx.ptr(), gcols.ptr(), B,
+                                                              ych, yh, yw, xch, kh, kw, pad, stride, dilation, xh, xw));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override;
+};
+
+struct Conv2DFilterGrad : Op, ConvHyper {  // conv2d.rs:736-776
+    explicit Conv2DFilterGrad(ConvHyper h) : ConvHyper(h) {}
+    const char *name() const override { return "Conv2DFilterGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray cols = ctx.input(0), gy = ctx.input(1), w = ctx.input(2);  // must be columns
+        const int B = (int)gy.shape()[0], K = (int)gy.shape()[1], P = (int)(gy.shape()[2] * gy.shape()[3]);
+        const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
+        NdArray gw = NdArray::empty(w.shape());
+        const size_t nb = ag_conv2d_filter_grad_f32_workspace(B, CK, P, K);
+        NdArray ws = workspace(nb);
+        const OpError e = from_status(
+            ag_conv2d_filter_grad_f32(ctx.stream(), cols.ptr(), gy.ptr(), gw.ptr(), B, CK, P, K, ws.ptr(), ws.len() * 4));
+        if (!e.ok()) return e;
+        ctx.append_output(gw);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override;
+};
+
+struct Conv2DWithCols : Op, ConvHyper {  // conv2d.rs:589-629
+    explicit Conv2DWithCols(ConvHyper h) : ConvHyper(h) {}
+    const char *name() const override { return "Conv2DWithCols"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray cols = ctx.input(0), w = ctx.input(1);
+        // cols carries [B, C*kh*kw, OH, OW] here (the reference labels it [B,C,kw,kh,OH,OW], conv2d.rs:484)
+        const int B = (int)cols.shape()[0], K = (int)w.shape()[0];
+        const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
+        const int OH = (int)cols.shape()[cols.ndim() - 2], OW = (int)cols.shape()[cols.ndim() - 1];
+        NdArray y = NdArray::empty({B, K, OH, OW});
+        const OpError e = from_status(ag_conv2d_with_cols_f32(ctx.stream(), cols.ptr(), w.ptr(), y.ptr(), B, CK, OH * OW, K));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override;
+};
+
+struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
+    explicit Conv2D(ConvHyper h) : ConvHyper(h) {}
+    const char *name() const override { return "Conv2D"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0), w = ctx.input(1);
+        // conv2d_extract_params, conv2d.rs:349-404
+        if (x.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape, "conv2d: lhs input must be 4D (got " + shape_str(x.shape()) + ")");
+        if (w.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape, "conv2d: filter must be 4D (got " + shape_str(w.shape()) + ")");
+        if (x.shape()[1] != w.shape()[1])
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "conv2d: input channel dim (" + std::to_string(x.shape()[1]) +
+                                     ") must match filter's second dim (" + std::to_string(w.shape()[1]) + ")");
+        const int B = (int)x.shape()[0], C = (int)x.shape()[1], H = (int)x.shape()[2], W = (int)x.shape()[3];
+        const int K = (int)w.shape()[0], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
+        const int OH = ag_conv_out_size(H, kh, pad, stride, dilation), OW = ag_conv_out_size(W, kw, pad, stride, dilation);
+        if (OH <= 0 || OW <= 0)
+            return OpError::make(ErrorKind::IncompatibleShape, "conv2d: filter extent exceeds the padded input");
+        NdArray y = NdArray::empty({B, K, OH, OW});
+        NdArray cols = NdArray::empty({B, (int64_t)C * kh * kw, OH, OW});
+        const OpError e = from_status(ag_conv2d_fwd_f32(ctx.stream(), x.ptr(), w.ptr(), y.ptr(), cols.ptr(), B, C, H, W, K, kh,
+                                                        kw, pad, stride, dilation));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        ctx.append_output(cols);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        Graph *g = ctx.graph();
+        const Tensor gy = ctx.output_grad(), y = ctx.output(), x = ctx.input(0), w = ctx.input(1);
+        const Tensor gx = build(g, {gy, w, tensor_ops::stop_gradient(x)},
+                                std::make_unique<Conv2DTranspose>(ConvHyper{pad, stride, dilation}));
+        const Tensor cols = tensor_ops::nth_tensor(y, 1);
+        const Tensor gw = g->builder()
+                              .append_input(cols, false)
+                              .append_input(gy, false)
+                              .append_input(w, false)
+                              .append_backprop_input(x)
+                              .append_backprop_input(gy)
+                              .build(std::make_unique<Conv2DFilterGrad>(ConvHyper{pad, stride, dilation}));
+        ctx.append_input_grad(gx);
+        ctx.append_input_grad(gw);
+    }
+};
+
+void Conv2DWithCols::grad(GradientContext &ctx) const
+{
+    Graph *g = ctx.graph();
+    const Tensor cols = ctx.input(0), w = ctx.input(1), y = ctx.output(), gy = ctx.output_grad();
+    const Tensor gx = build(g, {gy, w}, std::make_unique<Conv2DTranspose>(ConvHyper{pad, stride, dilation}));
+    const Tensor x0 = g->tensor(g->node(y.id).get_backprop_inputs()[0].id);
+    const Tensor gw = g->builder()
+                          .append_input(cols, false)
+                          .append_input(gy, false)
+                          .append_input(w, false)
+                          .append_backprop_input(x0)
+                          .append_backprop_input(gy)
+                          .build(std::make_unique<Conv2DFilterGrad>(ConvHyper{pad, stride, dilation}));
+    ctx.append_input_grad(gx);
+    ctx.append_input_grad(gw);
+}
+
+void Conv2DFilterGrad::grad(GradientContext &ctx) const
+{
+    // conv2d.rs:746-775: two gradients for the two back-prop inputs (x, gy)
+    Graph *g = ctx.graph();
+    const Tensor cols = ctx.input(0), gy = ctx.input(1), ggw = ctx.output_grad(), y = ctx.output();
+    const Tensor gx = build(g, {gy, ggw}, std::make_unique<Conv2DTranspose>(ConvHyper{pad, stride, dilation}));
+    const Tensor x0 = g->tensor(g->node(y.id).get_backprop_inputs()[0].id);
+    const Tensor ggy = g->builder()
+                           .append_input(cols, false)
+                           .append_input(ggw, false)
+                           .append_backprop_input(x0)
+                           .append_backprop_input(ggw)
+                           .build(std::make_unique<Conv2DWithCols>(ConvHyper{pad, stride, dilation}));
+    ctx.append_input_grad(gx);
+    ctx.append_input_grad(ggy);
+}
+
+void Conv2DTranspose::grad(GradientContext &ctx) const
+{
+    // conv2d_transpose.rs:274-300
+    Graph *g = ctx.graph();
+    const Tensor x = ctx.input(0), w = ctx.input(1), gy = ctx.output_grad();
+    const Tensor gx = build(g, {gy, w}, std::make_unique<Conv2D>(ConvHyper{pad, stride, dilation}));
+    const Tensor gw = build(g, {gy, x, tensor_ops::stop_gradient(w)},
+                            std::make_unique<Conv2DTransposeFilterGrad>(ConvHyper{pad, stride, dilation}));
+    ctx.append_input_grad(gx);
+    ctx.append_input_grad(gw);
+    if (ctx.num_inputs() > 2) ctx.append_input_grad(std::nullopt);  // the extent-only input
+}
+
+OpError Conv2DTransposeFilterGrad::compute(ComputeContext &ctx) const
+{
+    const NdArray gy = ctx.input(0), x = ctx.input(1), w = ctx.input(2);
+    const int B = (int)x.shape()[0], ych = (int)x.shape()[1], yh = (int)x.shape()[2], yw = (int)x.shape()[3];
+    const int xch = (int)gy.shape()[1], H = (int)gy.shape()[2], W = (int)gy.shape()[3];
+    const int kh = (int)w.shape()[2], kw = (int)w.shape()[3];
+    NdArray gw = NdArray::empty(w.shape());
+    NdArray gycols = NdArray::empty({B, (int64_t)xch * kh * kw, (int64_t)yh * yw});
+    const size_t nb = ag_conv2d_filter_grad_f32_workspace(B, xch * kh * kw, yh * yw, ych);
+    NdArray ws = workspace(nb);
+    const OpError e = from_status(ag_conv2d_transpose_filter_grad_f32(ctx.stream(), x.ptr(), gy.ptr(), gw.ptr(), gycols.ptr(),
+                                                                      B, ych, yh, yw, xch, H, W, kh, kw, pad, stride, dilation,
+                                                                      ws.ptr(), ws.len() * 4));
+    if (!e.ok()) return e;
+    ctx.append_output(gw);
+    return OpError::none();
+}
+
+void Conv2DTransposeFilterGrad::grad(GradientContext &ctx) const
+{
+    // conv2d_transpose.rs:453-479
+    Graph *g = ctx.graph();
+    const Tensor gy = ctx.input(0), gw = ctx.output_grad(), x = ctx.input(1);
+    const Tensor ggy = build(g, {x, gw}, std::make_unique<Conv2DTranspose>(ConvHyper{pad, stride, dilation}));
+    const Tensor ggx = build(g, {gy, gw}, std::make_unique<Conv2D>(ConvHyper{pad, stride, dilation}));
+    ctx.append_input_grad(ggy);
+    ctx.append_input_grad(ggx);
+    ctx.append_input_grad(std::nullopt);
+}
+
+// ------------------------------------------------------------------------------------------
+// max pooling                                                       conv_ops/max_pool2d.rs
+// ------------------------------------------------------------------------------------------
+struct PoolHyper {
+    int pad, stride, size;
+};
+
+// Outputs of MaxPool2D: [0] y, [1] argmax as f32 (the reference's encoding), [2] exact plane-local
+// int32 indices (bit pattern stored in an f32 array; an addition of this implementation that the
+// backward uses so it stays exact above 2^24 elements).
+struct MaxPool2DGradGrad : Op, PoolHyper {  // max_pool2d.rs:297-337
+    explicit MaxPool2DGradGrad(PoolHyper h) : PoolHyper(h) {}
+    const char *name() const override { return "MaxPool2DGradGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray ggx = ctx.input(0), argmax = ctx.input(1), idx = ctx.input(2);
+        const int B = (int)ggx.shape()[0], C = (int)ggx.shape()[1], H = (int)ggx.shape()[2], W = (int)ggx.shape()[3];
+        NdArray ggy = NdArray::empty(argmax.shape());
+        const OpError e = from_status(ag_maxpool2d_gradgrad_f32(ctx.stream(), ggx.ptr(), argmax.ptr(),
+                                                                reinterpret_cast<const int32_t *>(idx.ptr()), ggy.ptr(), B, C,
+                                                                H, W, size, pad, stride));
+        if (!e.ok()) return e;
+        ctx.append_output(ggy);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct MaxPool2DGrad : Op, PoolHyper {  // max_pool2d.rs:245-295
+    // Inputs (gy, argmax, exact indices[, x]).  Without the optional last input the input extent
+    // is reconstructed like the reference (max_pool2d.rs:263-264); MaxPool2D::grad passes x so
+    // that the gradient has x's size (the reference's reconstruction is too small whenever
+    // (H - size) is not a multiple of the stride, and it then writes out of bounds).
+    explicit MaxPool2DGrad(PoolHyper h) : PoolHyper(h) {}
+    const char *name() const override { return "MaxPool2DGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), argmax = ctx.input(1), idx = ctx.input(2);
+        int in_h = -1, in_w = -1;
+        if (ctx.num_inputs() > 3) {
+            const NdArray like = ctx.input(3);
+            if (like.ndim() == 4) {
+                in_h = (int)like.shape()[2];
+                in_w = (int)like.shape()[3];
+            }
+        }
+        const int B = (int)gy.shape()[0], C = (int)gy.shape()[1], yh = (int)gy.shape()[2], yw = (int)gy.shape()[3];
+        const int xh = in_h >= 0 ? in_h : ag_pool_grad_in_size(yh, size, pad, stride);
+        const int xw = in_w >= 0 ? in_w : ag_pool_grad_in_size(yw, size, pad, stride);
+        NdArray gx = NdArray::empty({B, C, xh, xw});
+        const OpError e = from_status(ag_maxpool2d_bwd_f32(ctx.stream(), gy.ptr(), argmax.ptr(),
+                                                           reinterpret_cast<const int32_t *>(idx.ptr()), gx.ptr(), B, C, xh, xw,
+                                                           size, pad, stride));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor ggx = ctx.output_grad(), argmax = ctx.input(1), idx = ctx.input(2);
+        const Tensor ggy = build(ctx.graph(), {ggx, argmax, idx}, std::make_unique<MaxPool2DGradGrad>(PoolHyper{pad, stride, size}));
+        ctx.append_input_grad(ggy);
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+        if (ctx.num_inputs() > 3) ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct MaxPool2D : Op, PoolHyper {  // max_pool2d.rs:166-243
+    explicit MaxPool2D(PoolHyper h) : PoolHyper(h) {}
+    const char *name() const override { return "MaxPool2D"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0);
+        if (x.ndim() != 4) return OpError::make(ErrorKind::IncompatibleShape, "max_pool2d: input must be 4D (got " + shape_str(x.shape()) + ")");
+        const int B = (int)x.shape()[0], C = (int)x.shape()[1], H = (int)x.shape()[2], W = (int)x.shape()[3];
+        const int OH = ag_pool_out_size(H, size, pad, stride), OW = ag_pool_out_size(W, size, pad, stride);
+        const Shape ys{B, C, std::max(OH, 0), std::max(OW, 0)};
+        NdArray y = NdArray::empty(ys), argmax = NdArray::empty(ys), idx = NdArray::empty(ys);
+        const OpError e = from_status(ag_maxpool2d_fwd_f32(ctx.stream(), x.ptr(), y.ptr(), argmax.ptr(),
+                                                           reinterpret_cast<int32_t *>(idx.ptr()), B, C, H, W, size, pad, stride));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        ctx.append_output(argmax);
+        ctx.append_output(idx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        // max_pool2d.rs:229-242, with the input extent taken from x instead of being reconstructed
+        const Tensor gy = ctx.output_grad(), y = ctx.output();
+        const Tensor indices = tensor_ops::nth_tensor(y, 1), exact = tensor_ops::nth_tensor(y, 2);
+        const Tensor gx = build(ctx.graph(), {gy, indices, exact, tensor_ops::stop_gradient(ctx.input(0))},
+                                std::make_unique<MaxPool2DGrad>(PoolHyper{pad, stride, size}));
+        ctx.append_input_grad(gx);
+    }
+};
+
+// ------------------------------------------------------------------------------------------
+// MatMul / BatchMatMul                                                     dot_ops.rs:554-718
+// ------------------------------------------------------------------------------------------
+struct MatMul : Op {
+    bool transpose_a, transpose_b;
+    MatMul(bool ta, bool tb) : transpose_a(ta), transpose_b(tb) {}
+    const char *name() const override { return "MatMul"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray a = ctx.input(0), b = ctx.input(1);
+        if (a.ndim() != 2) throw Panic("lhs input for MatMul must be 2D");  // `expect` panics, dot_ops.rs:566-573
+        if (b.ndim() != 2) throw Panic("rhs input for MatMul must be 2D");
+        const int64_t m = transpose_a ? a.shape()[1] : a.shape()[0], k = transpose_a ? a.shape()[0] : a.shape()[1];
+        const int64_t k2 = transpose_b ? b.shape()[1] : b.shape()[0], n = transpose_b ? b.shape()[0] : b.shape()[1];
+        if (k != k2)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "ndarray: inputs " + std::to_string(m) + " \xc3\x97 " + std::to_string(k) + " and " +
+                                     std::to_string(k2) + " \xc3\x97 " + std::to_string(n) +
+                                     " are not compatible for matrix multiplication");
+        NdArray c = NdArray::empty({m, n});
+        const OpError e = from_status(ag_gemm_f32(ctx.stream(), transpose_a, transpose_b, (int)m, (int)n, (int)k, 1.f, a.ptr(),
+                                                  (int)std::max<int64_t>(a.shape()[1], 1), 0, b.ptr(),
+                                                  (int)std::max<int64_t>(b.shape()[1], 1), 0, 0.f, c.ptr(),
+                                                  (int)std::max<int64_t>(n, 1), 0, 1));
+        if (!e.ok()) return e;
+        ctx.append_output(c);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        // dot_ops.rs:608-628
+        const Tensor gy = ctx.output_grad();
+        ctx.append_input_grad(build(ctx.graph(), {gy, ctx.input(1)}, std::make_unique<MatMul>(false, true)));
+        ctx.append_input_grad(build(ctx.graph(), {ctx.input(0), gy}, std::make_unique<MatMul>(true, false)));
+    }
+};
+
+struct BatchMatMul : Op {
+    bool transpose_a, transpose_b;
+    BatchMatMul(bool ta, bool tb) : transpose_a(ta), transpose_b(tb) {}
+    const char *name() const override { return "BatchMatMul"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x0 = ctx.input(0), x1 = ctx.input(1);
+        const int r0 = x0.ndim(), r1 = x1.ndim();
+        if (r0 < 2)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "BatchMatMul: Left-hand-side input's ndim must be >= 2, actual: " + std::to_string(r0));
+        if (r1 < 2)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "BatchMatMul: Right-hand-side input's ndim must be >= 2, actual: " + std::to_string(r1));
+        Shape s0 = x0.shape(), s1 = x1.shape();
+        if (transpose_a) std::swap(s0[r0 - 2], s0[r0 - 1]);
+        if (transpose_b) std::swap(s1[r1 - 2], s1[r1 - 1]);
+        if (r0 != r1 || !std::equal(s0.begin(), s0.end() - 2, s1.begin()) || s0[r0 - 1] != s1[r1 - 2])
+            return OpError::make(ErrorKind::IncompatibleShape, "Input shapes mismatch: " + shape_str(s0) + " vs " + shape_str(s1));
+        const int64_t m = s0[r0 - 2], k = s0[r0 - 1], n = s1[r1 - 1];
+        int64_t batch = 1;
+        for (int i = 0; i < r0 - 2; ++i) batch *= s0[i];
+        Shape out(s0.begin(), s0.end() - 2);
+        out.push_back(m);
+        out.push_back(n);
+        NdArray c = NdArray::empty(out);
+        const int64_t lda = x0.shape()[r0 - 1], ldb = x1.shape()[r1 - 1];
+        const OpError e = from_status(ag_gemm_f32(ctx.stream(), transpose_a, transpose_b, (int)m, (int)n, (int)k, 1.f, x0.ptr(),
+                                                  (int)std::max<int64_t>(lda, 1), x0.shape()[r0 - 2] * lda, x1.ptr(),
+                                                  (int)std::max<int64_t>(ldb, 1), x1.shape()[r1 - 2] * ldb, 0.f, c.ptr(),
+                                                  (int)std::max<int64_t>(n, 1), m * n, (int)batch));
+        if (!e.ok()) return e;
+        ctx.append_output(c);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        // dot_ops.rs:697-717
+        const Tensor gy = ctx.output_grad();
+        ctx.append_input_grad(build(ctx.graph(), {gy, ctx.input(1)}, std::make_unique<BatchMatMul>(false, true)));
+        ctx.append_input_grad(build(ctx.graph(), {ctx.input(0), gy}, std::make_unique<BatchMatMul>(true, false)));
+    }
+};
+
+// ------------------------------------------------------------------------------------------
+// reductions                                                               reduction_ops.rs
+// ------------------------------------------------------------------------------------------
+std::vector<int> normalize_axes(const std::vector<int> &axes, int rank)
+{
+    std::vector<int> r;
+    for (int a : axes) r.push_back(a < 0 ? a + rank : a);
+    return r;
+}
+
+// ReduceGradCommon (:459-512): broadcast gy back to the shape of x.  The reference passes
+// shape(x) as a tensor; here x itself is the second input and only its extents are read.
+struct ReduceGradCommon : Op {
+    std::vector<int> axes;
+    float divide_by_len;  // != 0: additionally divide by the reduced length (ReduceMean::grad, :217-238)
+    ReduceGradCommon(std::vector<int> a, bool mean) : axes(std::move(a)), divide_by_len(mean ? 1.f : 0.f) {}
+    const char *name() const override { return "ReduceGradCommon"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), x = ctx.input(1);
+        const int rank = x.ndim();
+        std::vector<int> shape(x.shape().begin(), x.shape().end());
+        const std::vector<int> ax = normalize_axes(axes, rank);
+        NdArray gx = NdArray::empty(x.shape());
+        OpError e = from_status(ag_broadcast_grad_f32(ctx.stream(), gy.ptr(), gx.ptr(), shape.data(), rank, ax.data(), (int)ax.size()));
+        if (!e.ok()) return e;
+        if (divide_by_len != 0.f) {
+            float len = 1.f;  // reduce_prod of the gathered extents, as f32
+            for (int a : ax) len *= (float)shape[(size_t)a];
+            e = from_status(ag_div_scalar_f32(ctx.stream(), gx.ptr(), len, gx.ptr(), gx.len()));
+            if (!e.ok()) return e;
+        }
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        // the gradient of a broadcast is the matching sum (:498-511)
+        Tensor s = tensor_ops::reduce_sum(ctx.output_grad(), axes, true);
+        ctx.append_input_grad(s);
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct ReduceSum : Op {
+    std::vector<int> axes;
+    bool keep_dims, mean;
+    ReduceSum(std::vector<int> a, bool k, bool m) : axes(std::move(a)), keep_dims(k), mean(m) {}
+    const char *name() const override { return mean ? "ReduceMean" : "ReduceSum"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0);
+        const int rank = x.ndim();
+        std::vector<int> ax = normalize_axes(axes, rank);
+        for (int a : ax)
+            if (a < 0 || a >= rank) return OpError::make(ErrorKind::OutOfBounds, "reduce: axis out of range");
+        if (rank == 0 || ax.empty()) {  // the reference returns a view of x (:63-70, :192-195)
+            ctx.append_output_view(x);
+            return OpError::none();
+        }
+        std::vector<int> shape(x.shape().begin(), x.shape().end());
+        Shape out;
+        for (int i = 0; i < rank; ++i) {
+            const bool red = std::find(ax.begin(), ax.end(), i) != ax.end();
+            if (!red) out.push_back(shape[(size_t)i]);
+            else if (keep_dims) out.push_back(1);
+        }
+        NdArray y = NdArray::empty(out);
+        const size_t nb = ag_reduce_sum_f32_workspace(shape.data(), rank, ax.data(), (int)ax.size());
+        NdArray ws = workspace(nb);
+        const OpError e = from_status(ag_reduce_sum_f32(ctx.stream(), x.ptr(), y.ptr(), shape.data(), rank, ax.data(),
+                                                        (int)ax.size(), mean ? 1 : 0, ws.ptr(), ws.len() * 4));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor gx = build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceGradCommon>(axes, mean));
+        ctx.append_input_grad(gx);
+    }
+};
+
+struct ReduceSumToScalarGrad;
+
+struct ReduceSumToScalar : Op {  // :123-137
+    const char *name() const override { return "ReduceSumToScalar"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0);
+        NdArray out = NdArray::empty({});
+        NdArray ws = workspace(ag_sum_all_f32_workspace(x.len()));
+        const OpError e = from_status(ag_sum_all_f32(ctx.stream(), x.ptr(), x.len(), out.ptr(), ws.ptr(), ws.len() * 4));
+        if (!e.ok()) return e;
+        ctx.append_output(out);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override;
+};
+
+struct ReduceSumToScalarGrad : Op {  // :139-159; input 1 is x (for its extents) instead of shape(x)
+    const char *name() const override { return "ReduceSumToScalarGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), x = ctx.input(1);
+        const int rank = x.ndim();
+        std::vector<int> shape(x.shape().begin(), x.shape().end()), ax((size_t)rank);
+        for (int i = 0; i < rank; ++i) ax[(size_t)i] = i;
+        NdArray gx = NdArray::empty(x.shape());
+        const OpError e = from_status(ag_broadcast_grad_f32(ctx.stream(), gy.ptr(), gx.ptr(), shape.data(), rank, ax.data(), rank));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(build(ctx.graph(), {ctx.output_grad()}, std::make_unique<ReduceSumToScalar>()));
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+void ReduceSumToScalar::grad(GradientContext &ctx) const
+{
+    ctx.append_input_grad(build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceSumToScalarGrad>()));
+}
+
+// ------------------------------------------------------------------------------------------
+// elementwise and loss glue
+// ------------------------------------------------------------------------------------------
+struct ReLUGrad : Op {  // greater(x, 0) * gy as one kernel (activation_ops.rs:161-166)
+    const char *name() const override { return "ReLUGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0), gy = ctx.input(1);
+        if (x.shape() != gy.shape()) return OpError::make(ErrorKind::IncompatibleShape, "relu grad: shapes differ");
+        NdArray gx = NdArray::empty(x.shape());
+        const OpError e = from_status(ag_relu_grad_f32(ctx.stream(), x.ptr(), gy.ptr(), gx.ptr(), x.len()));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        // second order: d/dgy (mask * gy) = mask * ggx; the mask itself has zero gradient
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(build(ctx.graph(), {ctx.input(0), ctx.output_grad()}, std::make_unique<ReLUGrad>()));
+    }
+};
+
+struct ReLU : Op {  // activation_ops.rs:154-167
+    const char *name() const override { return "ReLU"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0);
+        NdArray y = NdArray::empty(x.shape());
+        const OpError e = from_status(ag_relu_f32(ctx.stream(), x.ptr(), y.ptr(), x.len()));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(build(ctx.graph(), {ctx.input(0), ctx.output_grad()}, std::make_unique<ReLUGrad>()));
+    }
+};
+
+// MaybeReduceSum (binary_ops.rs:39-105): reduce gy to the shape of the operand it belongs to.
+// Input 1 is that operand (only its extents are read).
+// True when `b` is `a` without its leading axis, or with a leading axis of extent 1: the bias
+// shapes of the reference's examples ([1, classes] on [batch, classes], [1, C, H, W] on NCHW).
+static bool broadcasts_over_rows(const Shape &a, const Shape &b)
+{
+    if (a.empty() || a[0] == 0) return false;
+    if (b.size() == a.size()) return b[0] == 1 && std::equal(a.begin() + 1, a.end(), b.begin() + 1);
+    return b.size() + 1 == a.size() && std::equal(a.begin() + 1, a.end(), b.begin());
+}
+
+struct MaybeReduceSum : Op {
+    const char *name() const override { return "MaybeReduceSum"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), x = ctx.input(1);
+        if (gy.shape() == x.shape()) {
+            ctx.append_output_view(gy);
+            return OpError::none();
+        }
+        if (broadcasts_over_rows(gy.shape(), x.shape())) {
+            NdArray out = NdArray::empty(x.shape());
+            const size_t rows = (size_t)gy.shape()[0];
+            const OpError e = from_status(ag_bias_grad_f32(ctx.stream(), gy.ptr(), out.ptr(), rows, gy.len() / rows));
+            if (!e.ok()) return e;
+            ctx.append_output(out);
+            return OpError::none();
+        }
+        return OpError::make(ErrorKind::IncompatibleShape,
+                             "MaybeReduceSum: cannot reduce " + shape_str(gy.shape()) + " to " + shape_str(x.shape()));
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct AddOp : Op {  // binary_ops.rs:147-166, 304-346
+    const char *name() const override { return "AddOp"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray a = ctx.input(0), b = ctx.input(1);
+        NdArray y = NdArray::empty(a.shape());
+        OpError e;
+        if (a.shape() == b.shape()) {
+            const float *xs[2] = {a.ptr(), b.ptr()};
+            e = from_status(ag_add_n_f32(ctx.stream(), xs, 2, y.ptr(), a.len()));
+        } else if (broadcasts_over_rows(a.shape(), b.shape())) {
+            const size_t rows = (size_t)a.shape()[0];
+            e = from_status(ag_add_bias_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), rows, a.len() / rows));
+        } else {
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "AddOp: unsupported broadcast " + shape_str(a.shape()) + " + " + shape_str(b.shape()));
+        }
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor gy = ctx.output_grad();
+        ctx.append_input_grad(build(ctx.graph(), {gy, ctx.input(0)}, std::make_unique<MaybeReduceSum>()));
+        ctx.append_input_grad(build(ctx.graph(), {gy, ctx.input(1)}, std::make_unique<MaybeReduceSum>()));
+    }
+};
+
+struct MulOp : Op {  // binary_ops.rs:209-237 (same-shape operands)
+    const char *name() const override { return "MulOp"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray a = ctx.input(0), b = ctx.input(1);
+        if (a.shape() != b.shape())
+            return OpError::make(ErrorKind::IncompatibleShape, "MulOp: shapes " + shape_str(a.shape()) + " and " + shape_str(b.shape()) + " differ");
+        NdArray y = NdArray::empty(a.shape());
+        const OpError e = from_status(ag_mul_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), a.len()));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor gy = ctx.output_grad();
+        ctx.append_input_grad(tensor_ops::mul(gy, ctx.input(1)));
+        ctx.append_input_grad(tensor_ops::mul(gy, ctx.input(0)));
+    }
+};
+
+struct AddN : Op {  // array_ops.rs:503-535
+    const char *name() const override { return "AddN"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const size_t n = ctx.num_inputs();
+        if (n == 0) throw Panic("add_n: no inputs");
+        std::vector<NdArray> xs;
+        for (size_t i = 0; i < n; ++i) xs.push_back(ctx.input(i));
+        if (n == 1) {
+            ctx.append_output_view(xs[0]);
+            return OpError::none();
+        }
+        for (size_t i = 1; i < n; ++i)
+            if (xs[i].shape() != xs[0].shape()) return OpError::make(ErrorKind::IncompatibleShape, "add_n: shapes differ");
+        NdArray acc = NdArray::empty(xs[0].shape());
+        // ((x0 + x1) + x2) + ... in groups of at most 8 operands per launch
+        size_t done = 0;
+        bool have_acc = false;
+        while (done < n) {
+            const float *ptrs[8];
+            int cnt = 0;
+            if (have_acc) ptrs[cnt++] = acc.ptr();
+            while (cnt < 8 && done < n) ptrs[cnt++] = xs[done++].ptr();
+            const OpError e = from_status(ag_add_n_f32(ctx.stream(), ptrs, cnt, acc.ptr(), acc.len()));
+            if (!e.ok()) return e;
+            have_acc = true;
+        }
+        ctx.append_output(acc);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        for (size_t i = 0; i < ctx.num_inputs(); ++i) ctx.append_input_grad(ctx.output_grad());
+    }
+};
+
+struct ReshapeLike : Op {  // gradient of Reshape: back to the extents of input 1
+    const char *name() const override { return "Reshape"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray gy = ctx.input(0), x = ctx.input(1);
+        if (gy.len() != x.len()) return OpError::make(ErrorKind::IncompatibleShape, "reshape: element counts differ");
+        ctx.append_output_view(gy.reshaped(x.shape()));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct Reshape : Op {  // array_ops.rs:183-239: a view when the input is contiguous (always, here)
+    Shape target;
+    explicit Reshape(Shape s) : target(std::move(s)) {}
+    const char *name() const override { return "Reshape"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0);
+        Shape s = target;
+        int64_t known = 1;
+        int unknown = -1;
+        for (size_t i = 0; i < s.size(); ++i) {
+            if (s[i] == -1) {
+                if (unknown >= 0) return OpError::make(ErrorKind::IncompatibleShape, "reshape: more than one -1 in " + shape_str(target));
+                unknown = (int)i;
+            } else {
+                known *= s[i];
+            }
+        }
+        if (unknown >= 0) {
+            if (known == 0 || x.len() % (size_t)known) return OpError::make(ErrorKind::IncompatibleShape, "reshape: cannot infer -1");
+            s[(size_t)unknown] = (int64_t)(x.len() / (size_t)known);
+        }
+        size_t n = 1;
+        for (int64_t d : s) n *= (size_t)d;
+        if (n != x.len())
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "reshape: cannot reshape " + shape_str(x.shape()) + " into " + shape_str(target));
+        ctx.append_output_view(x.reshaped(s));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReshapeLike>()));
+    }
+};
+
+struct SparseSoftmaxCrossEntropyGrad : Op {  // xent_ops.rs:139-158
+    const char *name() const override { return "SparseSoftmaxCrossEntropyGrad"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray lsm = ctx.input(0), t = ctx.input(1), gy = ctx.input(2);
+        NdArray gx = NdArray::empty(lsm.shape());
+        const OpError e = from_status(ag_sparse_softmax_xent_grad_f32(ctx.stream(), lsm.ptr(), t.ptr(), gy.ptr(), gx.ptr(),
+                                                                      (size_t)lsm.shape()[0], (size_t)lsm.shape()[1]));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        ctx.append_input_grad(std::nullopt);
+        ctx.append_input_grad(std::nullopt);
+    }
+};
+
+struct SparseSoftmaxCrossEntropy : Op {  // xent_ops.rs:63-137
+    const char *name() const override { return "SparseSoftmaxCrossEntropy"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0), t = ctx.input(1);
+        if (x.ndim() != 2)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "SparseSoftmaxCrossEntropy: given first argument's ndim is not 2: shape=" + shape_str(x.shape()));
+        if (!(t.ndim() == 1 || (t.ndim() == 2 && t.shape()[1] == 1)))
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "SparseSoftmaxCrossEntropy: second argument's shape must be (batch_size, 1) or (batch_size,). given shape=" +
+                                     shape_str(t.shape()));
+        if (t.len() != (size_t)x.shape()[0]) throw Panic("Batch size mismatch: inputs vs labels");
+        NdArray loss = NdArray::empty({x.shape()[0], 1}), lsm = NdArray::empty(x.shape());
+        const OpError e = from_status(ag_sparse_softmax_xent_f32(ctx.stream(), x.ptr(), t.ptr(), loss.ptr(), lsm.ptr(),
+                                                                 (size_t)x.shape()[0], (size_t)x.shape()[1]));
+        if (!e.ok()) return e;
+        ctx.append_output(loss);
+        ctx.append_output(lsm);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor t = ctx.input(1), gy = ctx.output_grad();
+        const Tensor log_x = tensor_ops::nth_tensor(ctx.output(), 1);
+        ctx.append_input_grad(build(ctx.graph(), {log_x, t, gy}, std::make_unique<SparseSoftmaxCrossEntropyGrad>()));
+        ctx.append_input_grad(std::nullopt);  // the reference builds a label gradient "that won't be used in most cases"
+    }
+};
+
+// ------------------------------------------------------------------------------------------
+// AdamOp                                                  gradient_descent_ops/adam.rs:3-67
+// ------------------------------------------------------------------------------------------
+struct AdamOp : Op {
+    float alpha, eps, b1, b2;
+    AdamOp(float a, float e, float x, float y) : alpha(a), eps(e), b1(x), b2(y) {}
+    const char *name() const override { return "AdamOp"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        NdArray t = ctx.input_mut(4);
+        const NdArray g = ctx.input(1);
+        NdArray m = ctx.input_mut(2), v = ctx.input_mut(3), p = ctx.input_mut(0);
+        if (g.len() != p.len() || m.len() != p.len() || v.len() != p.len())
+            return OpError::make(ErrorKind::IncompatibleShape, "AdamOp: parameter, gradient and moment shapes differ");
+        const OpError e = from_status(ag_adam_update_f32(ctx.stream(), p.ptr(), g.ptr(), m.ptr(), v.ptr(), t.ptr(), p.len(), alpha, eps, b1, b2));
+        if (!e.ok()) return e;
+        ctx.append_empty_output();
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        for (int i = 0; i < 5; ++i) ctx.append_input_grad(std::nullopt);
+    }
+};
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// tensor_ops                                                          src/tensor_ops/mod.rs
+// ---------------------------------------------------------------------------------------------
+namespace tensor_ops {
+
+Tensor nth_tensor(Tensor x, int n)
+{
+    return x.graph->builder().append_input_with_selector(x, false, n).build(std::make_unique<Identity>());
+}
+
+Tensor dilated_conv2d(Tensor x, Tensor w, int pad, int stride, int dilate)
+{
+    return build(x.graph, {x, w}, std::make_unique<Conv2D>(ConvHyper{pad, stride, dilate}));
+}
+Tensor conv2d(Tensor x, Tensor w, int pad, int stride) { return dilated_conv2d(x, w, pad, stride, 1); }
+
+Tensor dilated_conv2d_transpose(Tensor x, Tensor w, int pad, int stride, int dilate)
+{
+    return build(x.graph, {x, w}, std::make_unique<Conv2DTranspose>(ConvHyper{pad, stride, dilate}));
+}
+Tensor conv2d_transpose(Tensor x, Tensor w, int pad, int stride) { return dilated_conv2d_transpose(x, w, pad, stride, 1); }
+
+Tensor max_pool2d(Tensor x, int pool_size, int pad, int stride)
+{
+    return build(x.graph, {x}, std::make_unique<MaxPool2D>(PoolHyper{pad, stride, pool_size}));
+}
+
+Tensor matmul(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<MatMul>(false, false)); }
+Tensor batch_matmul_t(Tensor a, Tensor b, bool ta, bool tb) { return build(a.graph, {a, b}, std::make_unique<BatchMatMul>(ta, tb)); }
+Tensor batch_matmul(Tensor a, Tensor b) { return batch_matmul_t(a, b, false, false); }
+
+Tensor reduce_sum(Tensor x, const std::vector<int> &axes, bool keep_dims)
+{
+    return build(x.graph, {x}, std::make_unique<ReduceSum>(axes, keep_dims, false));
+}
+Tensor reduce_mean(Tensor x, const std::vector<int> &axes, bool keep_dims)
+{
+    return build(x.graph, {x}, std::make_unique<ReduceSum>(axes, keep_dims, true));
+}
+Tensor sum_all(Tensor x) { return build(x.graph, {x}, std::make_unique<ReduceSumToScalar>()); }
+Tensor relu(Tensor x) { return build(x.graph, {x}, std::make_unique<ReLU>()); }
+Tensor add(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<AddOp>()); }
+Tensor mul(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<MulOp>()); }
+
+Tensor add_n(const std::vector<Tensor> &xs)
+{
+    if (xs.empty()) throw Panic("add_n: no inputs");
+    if (xs.size() == 1) return xs[0];  // mod.rs:831-847
+    TensorBuilder b = xs[0].graph->builder();
+    for (const Tensor &t : xs) b.append_input(t, false);
+    return b.build(std::make_unique<AddN>());
+}
+
+Tensor reshape(Tensor x, const Shape &shape) { return build(x.graph, {x}, std::make_unique<Reshape>(shape)); }
+
+Tensor sparse_softmax_cross_entropy(Tensor logits, Tensor labels)
+{
+    return build(logits.graph, {logits, labels}, std::make_unique<SparseSoftmaxCrossEntropy>());
+}
+
+Tensor scalar(float v, Graph *g) { return g->builder().build(std::make_unique<ScalarOp>(v)); }
+
+Tensor zeros_like(Tensor x)
+{
+    return x.graph->builder().append_input(x, false).set_differentiable(false).build(std::make_unique<ZerosLike>());
+}
+
+Tensor stop_gradient(Tensor x)
+{
+    return x.graph->builder().append_input(x, false).set_differentiable(false).build(std::make_unique<StopGradient>());
+}
+
+}  // namespace tensor_ops
+
+// ---------------------------------------------------------------------------------------------
+// Adam                                                              src/optimizers/adam.rs
+// ---------------------------------------------------------------------------------------------
+namespace optimizers {
+
+Adam::Adam(float alpha, float eps, float b1, float b2, const std::vector<VariableID> &vars, VariableEnvironment &env,
+           std::string adam_namespace_id)
+    : alpha_(alpha), eps_(eps), b1_(b1), b2_(b2), ns_(std::move(adam_namespace_id))
+{
+    for (VariableID vid : vars) {
+        const Shape shape = env.array(vid).shape();
+        env.set(ns_, std::to_string(vid) + "m", NdArray::zeros(shape));
+        env.set(ns_, std::to_string(vid) + "v", NdArray::zeros(shape));
+        env.set(ns_, std::to_string(vid) + "t", NdArray::scalar(1.f));
+    }
+}
+
+std::vector<Tensor> Adam::compute_updates(const std::vector<Tensor> &params, const std::vector<Tensor> &grads,
+                                          Context &ctx) const
+{
+    if (params.size() != grads.size()) throw Panic("assertion failed: num_params == grads.len()");
+    std::vector<Tensor> ret;
+    for (size_t i = 0; i < params.size(); ++i) {
+        const VariableID vid = ctx.node(params[i].id).variable_id;
+        if (vid < 0) throw Panic("Got non-variable tensor");
+        const Tensor m = ctx.variable(std::to_string(vid) + "m", ns_);
+        const Tensor v = ctx.variable(std::to_string(vid) + "v", ns_);
+        const Tensor t = ctx.variable(std::to_string(vid) + "t", ns_);
+        ret.push_back(ctx.builder()
+                          .append_input(params[i], true)
+                          .append_input(grads[i], false)
+                          .append_input(m, true)
+                          .append_input(v, true)
+                          .append_input(t, true)
+                          .build(std::make_unique<AdamOp>(alpha_, eps_, b1_, b2_)));
+    }
+    return ret;
+}
+
+void Adam::update(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, Context &ctx,
+                  const std::vector<std::pair<std::string, NdArray>> &feeds) const
+{
+    const std::vector<Tensor> ops = compute_updates(params, grads, ctx);
+    for (const EvalResult &r : ctx.eval(ops, feeds))
+        if (!r.error.ok()) throw Panic("called `Result::unwrap()` on an `Err` value: " + r.error.message);
+}
+
+Tensor Adam::get_update_op(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, Context &ctx) const
+{
+    return tensor_ops::add_n(compute_updates(params, grads, ctx));
+}
+
+}  // namespace optimizers
+
+}  // namespace host
+}  // namespace ag

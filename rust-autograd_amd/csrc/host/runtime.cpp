@@ -1,0 +1,445 @@
+// Device arrays, graph construction, the evaluator and the variable environment.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <mutex>
+#include <stdexcept>
+
+#include "ag_hip.h"
+#include "ag_host.hpp"
+
+namespace ag {
+namespace host {
+
+// ---------------------------------------------------------------------------------------------
+// caching device arena: freed blocks are kept in per-size free lists, so a training loop that
+// rebuilds its graph every step (as the reference does, src/variable.rs:670-683) stops calling
+// hipMalloc after the first step.
+// ---------------------------------------------------------------------------------------------
+struct DeviceBlock {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    ~DeviceBlock();
+};
+
+namespace {
+struct Arena {
+    std::mutex mu;
+    std::multimap<size_t, void *> free_blocks;
+    ~Arena()
+    {
+        for (auto &kv : free_blocks) (void)hipFree(kv.second);
+    }
+    static size_t round_up(size_t bytes)
+    {
+        const size_t q = bytes < (1u << 20) ? 256 : (1u << 16);
+        return (bytes + q - 1) / q * q;
+    }
+    void *take(size_t bytes)
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        auto it = free_blocks.lower_bound(bytes);
+        if (it != free_blocks.end() && it->first <= bytes + bytes / 8) {
+            void *p = it->second;
+            free_blocks.erase(it);
+            return p;
+        }
+        return nullptr;
+    }
+    void give(size_t bytes, void *p)
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        free_blocks.emplace(bytes, p);
+    }
+};
+Arena &arena()
+{
+    static Arena a;
+    return a;
+}
+void check(hipError_t e, const char *what)
+{
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+std::shared_ptr<DeviceBlock> allocate(size_t bytes)
+{
+    auto blk = std::make_shared<DeviceBlock>();
+    blk->bytes = Arena::round_up(bytes ? bytes : 4);
+    blk->ptr = arena().take(blk->bytes);
+    if (!blk->ptr) check(hipMalloc(&blk->ptr, blk->bytes), "hipMalloc");
+    return blk;
+}
+size_t product(const Shape &s)
+{
+    size_t n = 1;
+    for (int64_t d : s) n *= (size_t)d;
+    return n;
+}
+}  // namespace
+
+DeviceBlock::~DeviceBlock()
+{
+    if (ptr) arena().give(bytes, ptr);
+}
+
+void *current_stream() { return nullptr; }  // the null stream: every op is ordered on it
+
+void synchronize() { check(hipStreamSynchronize(nullptr), "hipStreamSynchronize"); }
+
+size_t NdArray::len() const { return product(shape_); }
+
+float *NdArray::ptr() const { return block_ ? static_cast<float *>(block_->ptr) : nullptr; }
+
+NdArray NdArray::empty(const Shape &shape)
+{
+    for (int64_t d : shape)
+        if (d < 0) throw Panic("NdArray: negative extent");
+    NdArray a;
+    a.shape_ = shape;
+    a.block_ = allocate(product(shape) * sizeof(float));
+    return a;
+}
+
+NdArray NdArray::filled(const Shape &shape, float value)
+{
+    NdArray a = empty(shape);
+    if (ag_fill_f32(current_stream(), a.ptr(), value, a.len()) != AG_OK) throw std::runtime_error(ag_last_error());
+    return a;
+}
+
+NdArray NdArray::zeros(const Shape &shape) { return filled(shape, 0.f); }
+
+NdArray NdArray::from_host(const Shape &shape, const float *data)
+{
+    NdArray a = empty(shape);
+    if (a.len())
+        check(hipMemcpyAsync(a.ptr(), data, a.len() * sizeof(float), hipMemcpyHostToDevice,
+                             static_cast<hipStream_t>(current_stream())),
+              "hipMemcpy H2D");
+    synchronize();  // the host buffer may be reused by the caller
+    return a;
+}
+
+NdArray NdArray::reshaped(const Shape &shape) const
+{
+    if (product(shape) != len()) throw Panic("NdArray::reshaped: element count differs");
+    NdArray a = *this;
+    a.shape_ = shape;
+    return a;
+}
+
+NdArray NdArray::deep_copy() const
+{
+    NdArray a = empty(shape_);
+    if (len())
+        check(hipMemcpyAsync(a.ptr(), ptr(), len() * sizeof(float), hipMemcpyDeviceToDevice,
+                             static_cast<hipStream_t>(current_stream())),
+              "hipMemcpy D2D");
+    return a;
+}
+
+std::vector<float> NdArray::to_host() const
+{
+    std::vector<float> out(len());
+    if (len())
+        check(hipMemcpyAsync(out.data(), ptr(), len() * sizeof(float), hipMemcpyDeviceToHost,
+                             static_cast<hipStream_t>(current_stream())),
+              "hipMemcpy D2H");
+    synchronize();
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------
+// ComputeContext / GradientContext                                        src/op.rs:186-434
+// ---------------------------------------------------------------------------------------------
+NdArray ComputeContext::input(size_t i)
+{
+    if (i >= xs_.size()) throw Panic("Bad op impl: input index out of range.");
+    Input &x = xs_[i];
+    if (x.kind == InputKind::RdWrVariable)
+        throw Panic("Bad op impl: cannot perform mutable borrowing for input(" + std::to_string(i) +
+                    "). Use input_mut() instead.");
+    if (x.taken)
+        throw Panic("Bad op impl: input(" + std::to_string(i) + ")/input_mut(" + std::to_string(i) +
+                    ") cannot be called twice");
+    x.taken = true;
+    return x.array;
+}
+
+NdArray ComputeContext::input_mut(size_t i)
+{
+    if (i >= xs_.size()) throw Panic("Bad op impl: " + std::to_string(i) + "'s input doesn't exist.");
+    Input &x = xs_[i];
+    if (x.kind != InputKind::RdWrVariable)
+        throw Panic("Bad op impl: cannot perform mutable borrowing for input(" + std::to_string(i) + ")");
+    if (x.taken)
+        throw Panic("Bad op impl: input(" + std::to_string(i) + ")/input_mut(" + std::to_string(i) +
+                    ") cannot be called twice");
+    x.taken = true;
+    return x.array;
+}
+
+void ComputeContext::append_output_view(const NdArray &y)
+{
+    bool contains_variable_input = false;
+    for (const Input &x : xs_) contains_variable_input |= x.kind != InputKind::NonVariable;
+    ys_.push_back(contains_variable_input ? y.deep_copy() : y);
+}
+
+Tensor GradientContext::input(size_t i) const
+{
+    const TensorInternal &n = graph_->node(y_.id);
+    if (i >= n.incoming_nodes.size()) throw Panic("bad Op::grad impl");
+    return graph_->tensor(n.incoming_nodes[i].id);
+}
+
+std::vector<Tensor> GradientContext::inputs() const
+{
+    std::vector<Tensor> r;
+    for (const IncomingTensor &in : graph_->node(y_.id).incoming_nodes) r.push_back(graph_->tensor(in.id));
+    return r;
+}
+
+size_t GradientContext::num_inputs() const { return graph_->node(y_.id).incoming_nodes.size(); }
+
+// ---------------------------------------------------------------------------------------------
+// graph building                                            src/tensor.rs:609-803, src/graph.rs
+// ---------------------------------------------------------------------------------------------
+TensorID Graph::install(std::unique_ptr<TensorInternal> n)
+{
+    const size_t count = nodes_.size();
+    if (count == 50000)  // src/graph.rs:30-36
+        std::fprintf(stderr, "Current graph size is 50,000! Graph should be reset regularly.\n");
+    if (count > 500000) throw Panic("Maximum graph size exceeded: 500,000. Use Graph::clear and so on.");
+    n->id = (TensorID)count;
+    nodes_.push_back(std::move(n));
+    return (TensorID)count;
+}
+
+TensorBuilder &TensorBuilder::append_input_with_selector(Tensor t, bool allow_mut, int selector)
+{
+    if (t.graph != graph_) throw Panic("Detected tensors belonging to different graphs");
+    in_nodes_.push_back(IncomingTensor{t.id, allow_mut, selector});
+    return *this;
+}
+
+TensorBuilder &TensorBuilder::append_backprop_input(Tensor t)
+{
+    if (t.graph != graph_) throw Panic("Detected tensors belonging to different graphs");
+    if (!backprop_inputs_) backprop_inputs_.emplace();
+    backprop_inputs_->push_back(IncomingTensor{t.id, false, 0});
+    return *this;
+}
+
+Tensor TensorBuilder::build(std::unique_ptr<Op> op)
+{
+    int rank = 0;
+    for (const IncomingTensor &in : in_nodes_) rank = std::max(rank, graph_->node(in.id).topo_rank + 1);
+    auto n = std::make_unique<TensorInternal>();
+    n->op = std::move(op);
+    n->incoming_nodes = std::move(in_nodes_);
+    n->topo_rank = rank;
+    n->placeholder_name = std::move(placeholder_);
+    n->is_placeholder = is_placeholder_;
+    n->is_differentiable = differentiable_;
+    n->backprop_inputs = std::move(backprop_inputs_);
+    n->known_shape = std::move(known_shape_);
+    n->variable_id = variable_id_;
+    const TensorID id = graph_->install(std::move(n));
+    return Tensor{graph_, id};
+}
+
+// ---------------------------------------------------------------------------------------------
+// source ops                                               src/tensor_ops/basic_source_ops.rs
+// ---------------------------------------------------------------------------------------------
+namespace {
+struct SourceOp : Op {
+    const char *label;
+    explicit SourceOp(const char *l) : label(l) {}
+    const char *name() const override { return label; }
+    OpError compute(ComputeContext &) const override
+    {
+        throw Panic(std::string(label) + ": source nodes are never computed");
+    }
+    void grad(GradientContext &) const override {}
+};
+}  // namespace
+
+Tensor Context::variable(VariableID id)
+{
+    if (id < 0 || (size_t)id >= env_->size()) throw Panic("variable array not found");
+    auto it = var_nodes_.find(id);
+    if (it != var_nodes_.end()) return tensor(it->second);
+    Tensor t = builder().set_variable(id).build(std::make_unique<SourceOp>("Variable"));
+    var_nodes_[id] = t.id;
+    return t;
+}
+
+Tensor Context::variable(const std::string &name, const std::string &namespace_id)
+{
+    auto id = env_->find(namespace_id, name);
+    if (!id) throw Panic("variable array not found in namespace '" + namespace_id + "': " + name);
+    return variable(*id);
+}
+
+Tensor Context::placeholder(const std::string &name, const Shape &shape)
+{
+    for (int64_t d : shape)
+        if (d == 0 || d < -1) throw Panic("Given shape contains invalid dim size(s)");  // src/tensor.rs KnownShape::new
+    return builder().set_placeholder_name(name).set_known_shape(shape).build(std::make_unique<SourceOp>("Placeholder"));
+}
+
+Evaluator Context::evaluator() { return Evaluator(this); }
+
+// ---------------------------------------------------------------------------------------------
+// evaluator                                                      src/evaluation.rs:183-363
+// ---------------------------------------------------------------------------------------------
+namespace {
+struct StorageEntry {
+    OpError error;
+    std::vector<NdArray> outputs;
+};
+
+const NdArray *find_placeholder(const std::vector<std::pair<std::string, NdArray>> &feeds, const TensorInternal &n)
+{
+    // src/evaluation.rs:225-249: the feed must exist and match the placeholder's known shape
+    for (const auto &f : feeds)
+        if (f.first == n.placeholder_name) {
+            if (n.known_shape) {
+                const Shape &ks = *n.known_shape;
+                bool ok = ks.size() == f.second.shape().size();
+                for (size_t i = 0; ok && i < ks.size(); ++i) ok = ks[i] <= 0 || ks[i] == f.second.shape()[i];
+                if (!ok) throw Panic("Shape error: placeholder '" + n.placeholder_name + "' was fed an array of another shape");
+            }
+            return &f.second;
+        }
+    throw Panic("Placeholder unfilled: " + n.placeholder_name);
+}
+}  // namespace
+
+std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
+                                      const std::vector<std::pair<std::string, NdArray>> &feeds)
+{
+    std::unordered_map<TensorID, StorageEntry> storage;  // every output lives until eval returns
+    auto would_not_visit = [&](const TensorInternal &n) {
+        return n.is_placeholder || n.is_variable() || storage.count(n.id) != 0;
+    };
+    std::vector<std::pair<TensorID, bool>> dfs;
+    for (const Tensor &t : tensors) {
+        if (t.graph != this) throw Panic("Detected tensors belonging to different graphs");
+        dfs.emplace_back(t.id, false);
+    }
+    while (!dfs.empty()) {
+        const auto [id, should_visit] = dfs.back();
+        dfs.pop_back();
+        const TensorInternal &n = node(id);
+        if (should_visit) {
+            if (would_not_visit(n)) continue;
+            std::vector<ComputeContext::Input> inputs;
+            OpError status;
+            for (const IncomingTensor &in : n.incoming_nodes) {
+                const TensorInternal &src = node(in.id);
+                if (src.is_placeholder) {
+                    inputs.push_back({*find_placeholder(feeds, src), ComputeContext::InputKind::NonVariable});
+                } else if (src.is_variable()) {
+                    inputs.push_back({env_->array(src.variable_id), in.allow_mut ? ComputeContext::InputKind::RdWrVariable
+                                                                                 : ComputeContext::InputKind::RdOnlyVariable});
+                } else {
+                    const StorageEntry &e = storage.at(in.id);
+                    if (!e.error.ok()) {
+                        status = e.error;
+                        break;
+                    }
+                    if ((size_t)in.array_selector >= e.outputs.size())
+                        throw Panic("Bad op impl: output selector out of range");
+                    inputs.push_back({e.outputs[(size_t)in.array_selector], ComputeContext::InputKind::NonVariable});
+                }
+            }
+            StorageEntry entry;
+            if (status.ok()) {
+                ComputeContext cc(std::move(inputs));
+                status = n.op->compute(cc);
+                if (status.ok()) {
+                    if (cc.outputs().empty()) throw Panic("Bad op implementation: empty return value");
+                    entry.outputs = std::move(cc.outputs());
+                }
+            }
+            entry.error = status;
+            storage.emplace(id, std::move(entry));
+        } else {
+            dfs.emplace_back(id, true);
+            for (const IncomingTensor &in : n.incoming_nodes)
+                if (!would_not_visit(node(in.id))) dfs.emplace_back(in.id, false);
+        }
+    }
+    std::vector<EvalResult> ret;
+    for (const Tensor &t : tensors) {
+        const TensorInternal &n = node(t.id);
+        EvalResult r;
+        if (n.is_variable()) {
+            r.array = env_->array(n.variable_id).deep_copy();
+        } else if (n.is_placeholder) {
+            r.array = find_placeholder(feeds, n)->deep_copy();
+        } else {
+            const StorageEntry &e = storage.at(t.id);
+            r.error = e.error;
+            if (e.error.ok()) r.array = e.outputs.at(0);
+        }
+        ret.push_back(std::move(r));
+    }
+    return ret;
+}
+
+// ---------------------------------------------------------------------------------------------
+// variable environment                                                    src/variable.rs
+// ---------------------------------------------------------------------------------------------
+static std::string full_name(const std::string &ns, const std::string &name) { return ns + '\x01' + name; }
+
+VariableID VariableEnvironment::set(const std::string &namespace_id, const std::string &name, NdArray array)
+{
+    const std::string key = full_name(namespace_id, name);
+    if (name_to_id_.count(key)) throw Panic("Bad variable name: " + name + " is already registered");
+    const VariableID id = (VariableID)arrays_.size();
+    arrays_.push_back(std::move(array));
+    name_to_id_[key] = id;
+    return id;
+}
+
+VariableID VariableEnvironment::set_anonymous(NdArray array)
+{
+    arrays_.push_back(std::move(array));
+    return (VariableID)arrays_.size() - 1;
+}
+
+std::optional<VariableID> VariableEnvironment::find(const std::string &namespace_id, const std::string &name) const
+{
+    auto it = name_to_id_.find(full_name(namespace_id, name));
+    if (it == name_to_id_.end()) return std::nullopt;
+    return it->second;
+}
+
+NdArray &VariableEnvironment::array(VariableID id)
+{
+    if (id < 0 || (size_t)id >= arrays_.size()) throw Panic("variable array not found");
+    return arrays_[(size_t)id];
+}
+
+std::vector<std::pair<std::string, VariableID>> VariableEnvironment::names_in(const std::string &namespace_id) const
+{
+    std::vector<std::pair<std::string, VariableID>> r;
+    const std::string prefix = namespace_id + '\x01';
+    for (const auto &kv : name_to_id_)
+        if (kv.first.compare(0, prefix.size(), prefix) == 0) r.emplace_back(kv.first.substr(prefix.size()), kv.second);
+    std::sort(r.begin(), r.end(), [](const auto &a, const auto &b) { return a.second < b.second; });
+    return r;
+}
+
+void VariableEnvironment::run(const std::function<void(Context &)> &f)
+{
+    Context ctx(this);
+    f(ctx);
+}
+
+}  // namespace host
+}  // namespace ag

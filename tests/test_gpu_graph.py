@@ -1,0 +1,424 @@
+"""GPU tests of the host operator layer: the graphs the reference's examples and tests build
+(conv block, small CNN with Adam, matmul / batch_matmul, transposed and dilated convolutions,
+second-order gradients) are built through libag_host.so, evaluated on the GPU and compared with the
+CPU oracle run stage by stage on the same inputs.
+
+Tolerance for floating point: |got - want| <= 1e-5 + 1e-4 * |want| (contractions are scaled by the
+magnitude of their operands instead, as in test_gpu_parity.py); integer-valued results
+(argmax-driven scatter positions, shapes, the Adam step counter) must be exact.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(f"[graph] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def G():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from __graft_entry__ import load_package
+
+    load_package()
+    import rust_autograd_amd.graph as graph
+
+    graph.lib()
+    return graph
+
+
+def assert_close(got, want, what, rtol=1e-4, atol=1e-5, scale=None):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
+    bound = atol + rtol * (np.abs(want) if scale is None else scale)
+    err = np.abs(got - want)
+    bad = err > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} outside tolerance, worst {float((err / bound).max()):.2f}x"
+
+
+def glorot(rng, shape):
+    fan_in = int(np.prod(shape[1:]))
+    fan_out = shape[0] * int(np.prod(shape[2:])) if len(shape) > 2 else shape[0]
+    if len(shape) == 2:
+        fan_in, fan_out = shape
+    sc = np.sqrt(6.0 / (fan_in + fan_out))
+    return rng.uniform(-sc, sc, shape).astype(np.float32)
+
+
+# ------------------------------------------------------------------------------- config 1
+def test_config1_through_the_graph(G, orc, rng):
+    B = 64
+    xv = rng.random((B, 1, 28, 28), dtype=np.float32)
+    wv = glorot(rng, (32, 1, 3, 3))
+    env = G.VariableEnvironment()
+    wid = env.set("w", wv)
+    c = env.context()
+    x = c.placeholder("x", [-1, 1, 28, 28])
+    w = c.variable(wid)
+    y = c.conv2d(x, w, 1, 1)
+    p = c.max_pool2d(c.relu(y), 2, 0, 2)
+    loss = c.reduce_sum(p, [0, 1, 2, 3])
+    gx, gw = c.grad([loss], [x, w])
+    say("config 1 eval")
+    yv, pv, lv, gxv, gwv = c.eval([y, p, loss, gx, gw], {"x": xv})
+
+    oy, ocols = orc.conv2d_fwd(xv, wv, 1, 1, 1)
+    assert_close(yv, oy, "y")
+    orl = orc.relu(yv)  # discrete stages are checked on the GPU's own conv output
+    op, oam, _ = orc.maxpool2d_fwd(orl, 2, 0, 2)
+    assert np.array_equal(pv, op)
+    assert_close(lv, orc.reduce_sum(op, [0, 1, 2, 3]), "loss")
+    ogr, _ = orc.maxpool2d_bwd(np.ones_like(op), oam, orl.shape)
+    ogy = orc.relu_grad(yv, ogr)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, ogy, wv.shape), "gw", scale=np.abs(gwv).max())
+    assert_close(gxv, orc.conv2d_transpose(ogy, wv, 1, 1, 1), "gx")
+    assert gxv.shape == xv.shape and gwv.shape == wv.shape
+
+
+# ------------------------------------------------------------------------------- config 2
+class OracleCNN:
+    """The small CNN of examples/cnn_mnist.rs, forward and backward, stage by stage on the oracle."""
+
+    def __init__(self, orc, params):
+        self.o = orc
+        self.p = {k: v.copy() for k, v in params.items()}
+
+    def step_grads(self, x, labels):
+        o, p = self.o, self.p
+        y1, cols1 = o.conv2d_fwd(x, p["w1"], 1, 1, 1)
+        z1 = o.add_bias(y1.reshape(y1.shape[0], -1), p["b1"].reshape(-1)).reshape(y1.shape)
+        r1 = o.relu(z1)
+        p1, am1, _ = o.maxpool2d_fwd(r1, 2, 0, 2)
+        y2, cols2 = o.conv2d_fwd(p1, p["w2"], 1, 1, 1)
+        z2 = o.add_bias(y2.reshape(y2.shape[0], -1), p["b2"].reshape(-1)).reshape(y2.shape)
+        r2 = o.relu(z2)
+        p2, am2, _ = o.maxpool2d_fwd(r2, 2, 0, 2)
+        flat = p2.reshape(p2.shape[0], -1)
+        logits = o.add_bias(o.matmul(flat, p["w3"]), p["b3"].reshape(-1))
+        per_row, lsm = o.sparse_softmax_xent(logits, labels)
+        loss = o.reduce_mean(per_row, [0])
+        n = per_row.shape[0]
+        g_rows = np.full((n, 1), np.float32(1.0) / np.float32(n), dtype=np.float32)
+        g_logits = o.sparse_softmax_xent_grad(lsm, labels, g_rows)
+        g = {}
+        g["b3"] = g_logits.sum(axis=0, dtype=np.float64).astype(np.float32).reshape(p["b3"].shape)
+        g["w3"] = o.matmul(flat, g_logits, ta=True)
+        g_flat = o.matmul(g_logits, p["w3"], tb=True)
+        g_r2, _ = o.maxpool2d_bwd(g_flat.reshape(p2.shape), am2, r2.shape)
+        g_z2 = o.relu_grad(z2, g_r2)
+        g["b2"] = g_z2.sum(axis=0, dtype=np.float64).astype(np.float32).reshape(p["b2"].shape)
+        g["w2"] = o.conv2d_filter_grad(cols2, g_z2, p["w2"].shape)
+        g_p1 = o.conv2d_transpose(g_z2, p["w2"], 1, 1, 1)
+        g_r1, _ = o.maxpool2d_bwd(g_p1, am1, r1.shape)
+        g_z1 = o.relu_grad(z1, g_r1)
+        g["b1"] = g_z1.sum(axis=0, dtype=np.float64).astype(np.float32).reshape(p["b1"].shape)
+        g["w1"] = o.conv2d_filter_grad(cols1, g_z1, p["w1"].shape)
+        return loss, logits, g
+
+
+def cnn_params(rng):
+    return {
+        "w1": glorot(rng, (32, 1, 3, 3)),
+        "w2": glorot(rng, (64, 32, 3, 3)),
+        "w3": glorot(rng, (64 * 7 * 7, 10)),
+        "b1": np.zeros((1, 32, 28, 28), np.float32),
+        "b2": np.zeros((1, 64, 14, 14), np.float32),
+        "b3": np.zeros((1, 10), np.float32),
+    }
+
+
+def build_cnn(G, env, c):
+    v = {k: c.variable(k) for k in ("w1", "w2", "w3", "b1", "b2", "b3")}
+    x = c.placeholder("x", [-1, 1, 28, 28])
+    t = c.placeholder("y", [-1, 1])
+    z1 = c.relu(c.conv2d(x, v["w1"], 1, 1) + v["b1"])
+    z2 = c.max_pool2d(z1, 2, 0, 2)
+    z3 = c.relu(c.conv2d(z2, v["w2"], 1, 1) + v["b2"])
+    z4 = c.max_pool2d(z3, 2, 0, 2)
+    z5 = c.reshape(z4, [-1, 64 * 7 * 7])
+    logits = c.matmul(z5, v["w3"]) + v["b3"]
+    loss = c.sparse_softmax_cross_entropy(logits, t)
+    return v, logits, loss
+
+
+def test_config2_training_steps_with_adam(G, orc, rng):
+    B = 128
+    params = cnn_params(rng)
+    env = G.VariableEnvironment()
+    ids = {k: env.set(k, a) for k, a in params.items()}
+    names = ["w1", "w2", "w3", "b1", "b2", "b3"]
+    adam = G.Adam(env, [ids[k] for k in names], alpha=1e-3)
+    ref = OracleCNN(orc, params)
+    m = {k: np.zeros_like(a) for k, a in params.items()}
+    vv = {k: np.zeros_like(a) for k, a in params.items()}
+    tt = {k: np.ones(1, np.float32) for k in params}
+    solid_so_far = {k: np.ones(a.shape, bool) for k, a in params.items()}
+
+    for step in range(3):
+        xv = rng.random((B, 1, 28, 28), dtype=np.float32)
+        lab = rng.integers(0, 10, (B, 1)).astype(np.float32)
+        c = env.context()  # a fresh graph per step, as `env.run(|ctx| ...)` in the example's loop
+        v, logits, loss = build_cnn(G, env, c)
+        mean_loss = c.reduce_mean(loss, [0], False)
+        grads = c.grad([mean_loss], [v[k] for k in names])
+        say(f"config 2 step {step}: grads")
+        out = c.eval([mean_loss, logits] + grads, {"x": xv, "y": lab})
+        oloss, ologits, og = ref.step_grads(xv, lab)
+        assert_close(out[1], ologits, f"logits step {step}", scale=1.0)
+        assert_close(out[0], oloss, f"loss step {step}")
+        for k, gv in zip(names, out[2:]):
+            scale = np.abs(og[k]).max()
+            assert_close(gv, og[k], f"grad {k} step {step}", scale=scale, atol=1e-7)
+        say(f"config 2 step {step}: update")
+        adam.update([v[k] for k in names], grads, c, {"x": xv, "y": lab})
+        for k in names:
+            orc.adam(ref.p[k], og[k], m[k], vv[k], tt[k], alpha=1e-3)
+            # The update's size is alpha whatever the gradient's, so compare on that scale; where
+            # the gradient is a near-total cancellation its relative error, and with it the
+            # update's, is unbounded: those elements only have to stay within the step size.
+            got, want = env.array(ids[k]), ref.p[k]
+            solid_so_far[k] &= np.abs(og[k]) >= 1e-3 * np.abs(og[k]).max()
+            solid = solid_so_far[k]
+            assert_close(got[solid], want[solid], f"param {k} after step {step}", scale=1e-3, rtol=2e-3, atol=1e-7)
+            assert np.abs(got - want).max() <= 2.1e-3 * (step + 1)
+    # optimizer state lives in the environment under the optimizer's namespace (adam.rs:66-89)
+    for k in names:
+        tid = env.find(f"{ids[k]}t", "adam")
+        assert tid is not None and env.array(tid).reshape(-1)[0] == 4.0
+        assert env.find(f"{ids[k]}m", "adam") is not None and env.find(f"{ids[k]}v", "adam") is not None
+
+
+def test_grad_helper_returns_every_variable_of_the_namespace(G, rng):
+    env = G.VariableEnvironment()
+    env.set("a", rng.random((4, 3), dtype=np.float32))
+    env.set("b", rng.random((1, 3), dtype=np.float32))
+    c = env.context()
+    x = c.placeholder("x", [-1, 4])
+    loss = c.sum_all(c.matmul(x, c.variable("a")) + c.variable("b"))
+    vs, gs = c.grad_helper([loss])
+    assert len(vs) == 2 and len(gs) == 2
+    xv = rng.random((5, 4), dtype=np.float32)
+    ga, gb = c.eval(gs, {"x": xv})
+    got = {tuple(ga.shape): ga, tuple(gb.shape): gb}
+    assert_close(got[(4, 3)], np.repeat(xv.sum(axis=0)[:, None], 3, axis=1), "d/da")
+    assert_close(got[(1, 3)], np.full((1, 3), 5.0), "d/db")
+
+
+# ------------------------------------------------------------------------------- config 3 (reduced)
+@pytest.mark.parametrize("shape", [((96, 200), (200, 72)), ((1, 17), (17, 1))])
+def test_matmul_and_its_gradients(G, orc, rng, shape):
+    av, bv = (rng.standard_normal(s).astype(np.float32) for s in shape)
+    env = G.VariableEnvironment()
+    c = env.context()
+    a, b = c.placeholder("a", list(shape[0])), c.placeholder("b", list(shape[1]))
+    z = c.matmul(a, b)
+    ga, gb = c.grad([c.sum_all(z)], [a, b])
+    say(f"matmul {shape}")
+    zv, gav, gbv = c.eval([z, ga, gb], {"a": av, "b": bv})
+    k = shape[0][1]
+    assert_close(zv, orc.matmul(av, bv), "z", scale=np.sqrt(k))
+    ones = np.ones_like(zv)
+    assert_close(gav, orc.matmul(ones, bv, tb=True), "ga", scale=np.abs(bv).sum(axis=1)[None, :] + 0 * gav)
+    assert_close(gbv, orc.matmul(av, ones, ta=True), "gb", scale=np.abs(av).sum(axis=0)[:, None] + 0 * gbv)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_batch_matmul_and_its_gradients(G, orc, rng, ta, tb):
+    Bt, M, K, N = 6, 40, 56, 24
+    av = rng.standard_normal((Bt, K, M) if ta else (Bt, M, K)).astype(np.float32)
+    bv = rng.standard_normal((Bt, N, K) if tb else (Bt, K, N)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    a, b = c.placeholder("a", list(av.shape)), c.placeholder("b", list(bv.shape))
+    z = c.batch_matmul(a, b, ta, tb)
+    ga, gb = c.grad([c.sum_all(z)], [a, b])
+    say(f"batch_matmul ta={ta} tb={tb}")
+    zv, gav, gbv = c.eval([z, ga, gb], {"a": av, "b": bv})
+    assert_close(zv, orc.batch_matmul(av, bv, ta, tb), "z", scale=np.sqrt(K))
+    # BatchMatMul::grad builds batch_matmul(gy, b^T) and batch_matmul(a^T, gy) whatever the op's own
+    # transpose flags are (dot_ops.rs:697-717), so like the reference the gradients are those of
+    # sum(z) only for untransposed operands; with a flag set they are shape errors or differently
+    # shaped products, exactly as there.
+    ones = np.ones_like(zv)
+    for got, args, what in ((gav, (ones, bv, False, True), "ga"), (gbv, (av, ones, True, False), "gb")):
+        try:
+            want = orc.batch_matmul(*args)
+        except Exception:
+            assert isinstance(got, G.OpError), what
+            continue
+        assert_close(got, want, what, scale=np.sqrt(max(M, N)), rtol=2e-4)
+    if not ta and not tb:
+        gA = np.repeat(bv.astype(np.float64).sum(axis=2)[:, None, :], M, axis=1)
+        gB = np.repeat(av.astype(np.float64).sum(axis=1)[:, :, None], N, axis=2)
+        assert_close(gav, gA, "ga analytic", scale=np.sqrt(N), rtol=2e-4)
+        assert_close(gbv, gB, "gb analytic", scale=np.sqrt(M), rtol=2e-4)
+
+
+# ------------------------------------------------------------------------------- configs 4 / 5 (reduced)
+@pytest.mark.parametrize("H,pad,stride,dil,k", [(14, 1, 1, 1, 3), (16, 1, 2, 1, 3), (14, 2, 1, 2, 3), (15, 0, 2, 1, 2)])
+def test_conv2d_gradients_every_geometry(G, orc, rng, H, pad, stride, dil, k):
+    B, Cin, Cout = 3, 5, 7
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = glorot(rng, (Cout, Cin, k, k))
+    env = G.VariableEnvironment()
+    c = env.context()
+    x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+    y = c.dilated_conv2d(x, w, pad, stride, dil)
+    gyv = None
+    gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+    say(f"conv grads H={H} pad={pad} stride={stride} dil={dil} k={k}")
+    yv, gxv, gwv = c.eval([y, gx, gw], {"x": xv, "w": wv})
+    oy, ocols = orc.conv2d_fwd(xv, wv, pad, stride, dil)
+    assert_close(yv, oy, "y", scale=1.0)
+    gyv = (2 * yv).astype(np.float32)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    # the gradient has x's own extent, also where the transposed-convolution size formula would
+    # come out one short (stride 2 on an even extent)
+    assert gxv.shape == xv.shape
+    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, stride, dil, out_hw=(H, H)), "gx", scale=np.abs(gxv).max(), rtol=2e-4)
+
+
+def test_conv2d_transpose_upsampling_and_gradients(G, orc, rng):
+    B, Cin, Cout, H = 4, 12, 6, 7
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = rng.uniform(-0.1, 0.1, (Cin, Cout, 4, 4)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+    y = c.conv2d_transpose(x, w, 1, 2)
+    gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+    say("conv2d_transpose 4x4 stride 2")
+    yv, gxv, gwv = c.eval([y, gx, gw], {"x": xv, "w": wv})
+    assert yv.shape == (B, Cout, 14, 14)
+    assert_close(yv, orc.conv2d_transpose(xv, wv, 1, 2, 1), "y", scale=1.0)
+    gyv = (2 * yv).astype(np.float32)
+    # d/dx of a transposed convolution is the forward convolution of gy with the same filter
+    ogx, _ = orc.conv2d_fwd(gyv, wv, 1, 2, 1)
+    assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max(), rtol=2e-4)
+    assert_close(gwv, orc.conv2d_transpose_filter_grad(xv, gyv, wv.shape, 1, 2, 1), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+
+
+def test_max_pool_gradient_and_second_order(G, orc, rng):
+    xv = rng.standard_normal((2, 3, 9, 9)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x = c.placeholder("x", list(xv.shape))
+    y = c.max_pool2d(x, 3, 0, 2)
+    (gx,) = c.grad([c.sum_all(c.mul(y, y))], [x])
+    (ggx,) = c.grad([c.sum_all(c.mul(gx, gx))], [x])  # runs MaxPool2DGradGrad (max_pool2d.rs:297-337)
+    say("max pool second order")
+    yv, gxv, ggxv = c.eval([y, gx, ggx], {"x": xv})
+    oy, oam, _ = orc.maxpool2d_fwd(xv, 3, 0, 2)
+    assert np.array_equal(yv, oy)
+    ogx, _ = orc.maxpool2d_bwd((2 * oy).astype(np.float32), oam, xv.shape)
+    assert np.array_equal(gxv, ogx)
+    assert ggxv.shape == xv.shape and np.isfinite(ggxv).all()
+
+
+def test_second_order_conv_filter_grad_wrt_input(G, orc, rng):
+    # sum over the filter gradient of sum(conv(x, w)) is linear in x: its gradient is the
+    # transposed convolution of an all-ones gy with an all-ones filter.
+    xv = rng.standard_normal((2, 3, 8, 8)).astype(np.float32)
+    wv = glorot(rng, (4, 3, 3, 3))
+    env = G.VariableEnvironment()
+    c = env.context()
+    x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+    y = c.conv2d(x, w, 1, 1)
+    (gw,) = c.grad([c.sum_all(y)], [w])
+    (ggx,) = c.grad([c.sum_all(gw)], [x])
+    say("second order conv")
+    gwv, ggxv = c.eval([gw, ggx], {"x": xv, "w": wv})
+    _, ocols = orc.conv2d_fwd(xv, wv, 1, 1, 1)
+    ones_gy = np.ones((2, 4, 8, 8), np.float32)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, ones_gy, wv.shape), "gw", scale=np.abs(gwv).max())
+    assert_close(ggxv, orc.conv2d_transpose(ones_gy, np.ones_like(wv), 1, 1, 1), "ggx")
+
+
+@pytest.mark.parametrize("axes,keep", [([0], False), ([1], True), ([0, 2], False), ([-1], False)])
+def test_reduce_ops_and_gradients(G, orc, rng, axes, keep):
+    xv = rng.standard_normal((6, 5, 4)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x = c.placeholder("x", list(xv.shape))
+    s, m = c.reduce_sum(x, axes, keep), c.reduce_mean(x, axes, keep)
+    (gs,) = c.grad([c.sum_all(c.mul(s, s))], [x])
+    (gm,) = c.grad([c.sum_all(m)], [x])
+    sv, mv, gsv, gmv = c.eval([s, m, gs, gm], {"x": xv})
+    assert np.array_equal(sv, orc.reduce_sum(xv, axes, keep))
+    assert np.array_equal(mv, orc.reduce_mean(xv, axes, keep))
+    ax = [a % 3 for a in axes]
+    assert_close(gsv, np.broadcast_to(2 * xv.sum(axis=tuple(ax), keepdims=True), xv.shape), "d sum^2", atol=1e-4)
+    count = int(np.prod([xv.shape[a] for a in ax]))
+    assert_close(gmv, np.full(xv.shape, 1.0 / count), "d mean")
+
+
+def test_finite_difference_check_of_a_conv_block(G, rng):
+    # the reference's own way of testing gradients (src/test_helper.rs:11-94): central differences
+    xv = rng.standard_normal((1, 2, 6, 6)).astype(np.float32)
+    wv = rng.standard_normal((3, 2, 3, 3)).astype(np.float32)
+    env = G.VariableEnvironment()
+    wid = env.set("w", wv)
+    c = env.context()
+    x = c.placeholder("x", list(xv.shape))
+    loss = c.sum_all(c.mul(c.conv2d(x, c.variable(wid), 1, 1), c.conv2d(x, c.variable(wid), 1, 1)))
+    (gw,) = c.grad([loss], [c.variable(wid)])
+    gwv = c.eval([gw], {"x": xv})[0]
+    eps = 1e-2
+    for idx in [(0, 0, 0, 0), (2, 1, 1, 1), (1, 0, 2, 1)]:
+        vals = []
+        for sgn in (+1, -1):
+            wp = wv.copy()
+            wp[idx] += sgn * eps
+            env2 = G.VariableEnvironment()
+            w2 = env2.set("w", wp)
+            c2 = env2.context()
+            x2 = c2.placeholder("x", list(xv.shape))
+            y2 = c2.conv2d(x2, c2.variable(w2), 1, 1)
+            vals.append(float(c2.eval([c2.sum_all(c2.mul(y2, y2))], {"x": xv})[0]))
+        numeric = (vals[0] - vals[1]) / (2 * eps)
+        assert abs(numeric - gwv[idx]) <= 2e-2 * max(1.0, abs(numeric)), (idx, numeric, gwv[idx])
+
+
+# ------------------------------------------------------------------------------- error behaviour
+def test_op_errors_come_back_as_results_and_misuse_panics(G, rng):
+    env = G.VariableEnvironment()
+    c = env.context()
+    a, b = c.placeholder("a", [-1, -1]), c.placeholder("b", [-1, -1])
+    z = c.matmul(a, b)
+    ok = c.relu(a)
+    av, bv = rng.random((3, 4), dtype=np.float32), rng.random((5, 2), dtype=np.float32)
+    r = c.eval([z, ok], {"a": av, "b": bv})
+    # evaluation.rs:341-360: a failed op yields Err for that tensor, the others still evaluate
+    assert isinstance(r[0], G.OpError) and r[0].kind == "IncompatibleShape"
+    assert np.array_equal(r[1], av)
+    with pytest.raises(G.Panic, match="[Pp]laceholder"):
+        c.eval([z], {"a": av})
+    x4 = c.placeholder("x4", [-1, 3, 8, 8])
+    w4 = c.placeholder("w4", [4, 2, 3, 3])
+    r = c.eval([c.conv2d(x4, w4, 1, 1)], {"x4": rng.random((1, 3, 8, 8), dtype=np.float32),
+                                         "w4": rng.random((4, 2, 3, 3), dtype=np.float32)})
+    assert isinstance(r[0], G.OpError)
+
+
+def test_variables_are_shared_between_contexts_and_updated_in_place(G, orc, rng):
+    env = G.VariableEnvironment()
+    wv = rng.random((8, 8), dtype=np.float32) + 2.0
+    wid = env.set("w", wv)
+    adam = G.Adam(env, [wid], alpha=0.5)
+    p, m, v, t = wv.copy(), np.zeros_like(wv), np.zeros_like(wv), np.ones(1, np.float32)
+    for step in range(2):
+        c = env.context()
+        w = c.variable(wid)
+        (g,) = c.grad([c.sum_all(c.mul(w, w))], [w])
+        adam.update([w], [g], c)
+        orc.adam(p, (p + p).astype(np.float32), m, v, t, alpha=0.5)
+        assert_close(env.array(wid), p, f"Adam step {step}")
+    # with a constant-sign gradient Adam moves every element by about alpha per step
+    assert np.abs(env.array(wid) - (wv - 1.0)).max() < 0.05
