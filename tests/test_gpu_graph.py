@@ -283,6 +283,12 @@ def test_conv2d_gradients_every_geometry(G, orc, rng, H, pad, stride, dil, k):
     # come out one short (stride 2 on an even extent)
     assert gxv.shape == xv.shape
     assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, stride, dil, out_hw=(H, H)), "gx", scale=np.abs(gxv).max(), rtol=2e-4)
+    # what the reference itself returns (extent rebuilt from gy, conv2d_transpose.rs:55-56) is the
+    # top-left crop of that gradient
+    ref_like = orc.conv2d_transpose(gyv, wv, pad, stride, dil)
+    h = ref_like.shape[2]
+    assert h <= H
+    assert_close(gxv[:, :, :h, :h], ref_like, "gx crop", scale=np.abs(gxv).max(), rtol=2e-4)
 
 
 def test_conv2d_transpose_upsampling_and_gradients(G, orc, rng):
