@@ -3,7 +3,7 @@
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 out="$here/../libag_hip.so"
-srcs=(common.hip im2col.hip gemm.hip conv.hip pool.hip reduce.hip adam.hip elementwise.hip)
+srcs=(common.hip im2col.hip gemm.hip gemm_dl.hip conv.hip pool.hip reduce.hip adam.hip elementwise.hip)
 flags=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -fvisibility=hidden
        -Xclang -target-feature -Xclang -packed-fp32-ops
        -I"$here/../../include" -I"$here" -Wall -Wno-unused-function "$@")
@@ -13,6 +13,8 @@ for s in "${srcs[@]}"; do
   extra=()
   # adam.hip must keep the reference's separately rounded multiplies and adds
   [ "$s" = adam.hip ] && extra=(-ffp-contract=off)
+  # keep the MFMA accumulators in ordinary VGPRs (no copies to and from AGPRs around the epilogue)
+  [ "$s" = gemm_dl.hip ] && extra=(-Wno-inline-asm -Wno-pass-failed)
   /opt/rocm/bin/hipcc "${flags[@]}" "${extra[@]}" -c "$here/$s" -o "$here/obj/${s%.hip}.o" &
   pids+=($!)
 done

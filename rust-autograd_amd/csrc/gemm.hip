@@ -24,41 +24,9 @@
 // contiguous range of tiles / images.
 #include <type_traits>
 
-#include "ag_internal.h"
+#include "gemm_shared.h"
 
 namespace ag {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-enum { LK_VEC = 0, LK_SCALAR = 1, LMN = 2 };
-
-struct GemmParams {
-    const float *A;
-    const float *B;
-    float *C;
-    int M, N, K;
-    long long lda, ldb, ldc;
-    long long sA, sB, sC;  // stride between independent batches
-    long long sAk, sBk;    // stride between accumulated batches
-    int kbatch;            // accumulated batches (>= 1)
-    int kb_per_split;
-    int splits;
-    long long sCsplit;     // stride between the partial outputs of consecutive splits
-    float alpha, beta;
-    int tiles_m, tiles_n;
-    unsigned total_blocks;
-};
-
-constexpr int kXcds = 8;
-
-// Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
-// contiguous slice of the logical block range instead.
-__device__ inline unsigned xcd_remap(unsigned id, unsigned total)
-{
-    const unsigned per = total / kXcds, rem = total % kXcds;
-    const unsigned xcd = id % kXcds, pos = id / kXcds;
-    return xcd * per + (xcd < rem ? xcd : rem) + pos;
-}
 
 template <int LT, int ROWS, int BK, int NT>
 struct TileLoader {
@@ -472,9 +440,9 @@ static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
 // Tile configurations {BM, BN}; see launch() for BK, the wave tile and the occupancy target.
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
                                 {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
-                                {128, 128}, {192, 128}, {128, 64}};
+                                {128, 128}, {192, 128}, {128, 64},
+                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
-
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
     switch (cfg) {
@@ -498,13 +466,33 @@ static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 static long long cdiv(long long a, long long b) { return (a + b - 1) / b; }
 
 // Tile choice.  The block-tile shape comes first: least padded output area, larger tiles on ties
-// (they re-read operands less).  Contractions with few k tiles per output tile, and the
-// accumulated-batch GEMMs, take the BK = 16 family with a three-tile LDS ring (3-4 blocks stay
-// resident per CU, which hides the per-tile staging); long contractions take BK = 32.
-// Problems too small to give every CU a block fall back to 64 x 64 tiles.
-static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate)
+// (they re-read operands less).  Problems the direct-to-LDS kernel accepts (`direct`) choose among
+// its five tiles; the eight-wave tiles keep the matrix pipe about 8 % busier than the four-wave
+// 128 x 128 tile, which is weighed against their padding.  Otherwise: contractions with few k
+// tiles per output tile, and the accumulated-batch GEMMs, take the BK = 16 family with a
+// three-tile LDS ring, long contractions take BK = 32.  Problems too small to give every CU a
+// block fall back to 64 x 64 tiles of the register-staged kernel.
+static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bool direct)
 {
     if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg;
+    if (direct) {
+        static const int dl[] = {14, 15, 16, 17, 13};  // 128x256, 256x128, 192x128, 128x192, 128x128
+        static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.92};
+        int best = -1;
+        double best_cost = 1e300;
+        long long best_blocks = 0;
+        for (int c = 0; c < 5; ++c) {
+            const TileCfg &t = kCfgs[dl[c]];
+            const long long tm = cdiv(M, t.bm), tn = cdiv(N, t.bn);
+            const double cost = (double)tm * t.bm * tn * t.bn / eff[c];
+            if (cost < best_cost * 0.995) {
+                best_cost = cost;
+                best = dl[c];
+                best_blocks = tm * tn * zcount;
+            }
+        }
+        if (best_blocks >= 256) return best;
+    }
     static const int short_k[] = {11, 10, 12, 8};  // 192x128, 128x128, 128x64, 64x64 (BK 16)
     static const int long_k[] = {0, 1, 2, 3};      // 128x128, 128x64, 64x128, 64x64 (BK 32)
     const bool use_short = accumulate || K <= 1024;
@@ -544,6 +532,19 @@ struct GemmCall {
     long long ldc, sC;
     int batch, kbatch;
 };
+
+static bool direct_ok(const GemmCall &c)
+{
+    auto mult4 = [](long long v) { return v % 4 == 0; };
+    if (c.K % 32 != 0 || !aligned16(c.A) || !aligned16(c.B)) return false;
+    if (!mult4(c.lda) || !mult4(c.ldb) || !mult4(c.sA) || !mult4(c.sB) || !mult4(c.sAk) || !mult4(c.sBk)) return false;
+    if (c.transA && (c.M % 4 != 0 || c.M < 4)) return false;   // A is m-contiguous
+    if (!c.transB && (c.N % 4 != 0 || c.N < 4)) return false;  // B is n-contiguous
+    // byte offsets inside one operand slice are unsigned 32-bit
+    const long long a_span = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
+    const long long b_span = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
+    return a_span < (1LL << 30) && b_span < (1LL << 30);
+}
 
 static ag_status_t validate(const char *who, const GemmCall &c)
 {
@@ -601,7 +602,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.alpha = c.alpha; p.beta = c.beta;
     p.sCsplit = (long long)c.M * c.N;
 
-    const int cfg = choose_cfg(c.M, c.N, c.K, (long long)c.batch * p.splits, c.kbatch > 1);
+    int cfg = choose_cfg(c.M, c.N, c.K, (long long)c.batch * p.splits, c.kbatch > 1, direct_ok(c));
+    if (cfg >= kFirstDirectCfg && !direct_ok(c)) cfg = 0;  // a forced configuration that cannot run
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(c.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * c.batch * p.splits;
@@ -619,7 +621,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     // A is k-contiguous when not transposed; B is k-contiguous when transposed.
     const int la = loader_kind(!c.transA, c.A, c.lda, c.K, c.sA, c.sAk);
     const int lb = loader_kind(c.transB != 0, c.B, c.ldb, c.K, c.sB, c.sBk);
-    launch(st, cfg, la, lb, p);
+    if (cfg >= kFirstDirectCfg) launch_direct(st, cfg, !c.transA, c.transB != 0, p, num_cus(), g_grid_scale);
+    else launch(st, cfg, la, lb, p);
     if (ag_status_t s = check_launch(who)) return s;
     if (p.splits > 1) {
         const long long total = (long long)c.M * c.N;
@@ -637,7 +640,8 @@ static int g_force_splits = 0;  // experiment hook, see ag_gemm_force_splits
 static int choose_splits(int M, int N, int K, int kbatch)
 {
     if (g_force_splits > 0) return g_force_splits < kbatch ? g_force_splits : kbatch;
-    const int cfg = choose_cfg(M, N, K, kbatch, true);  // tile choice as if every image were a block
+    // tile choice as if every image were a block; the alignment of the operands is not known here
+    const int cfg = choose_cfg(M, N, K, kbatch, true, K % 32 == 0);
     const long long tiles = cdiv(M, kCfgs[cfg].bm) * cdiv(N, kCfgs[cfg].bn);
     long long want = cdiv(4096, tiles);
     if (want > kbatch) want = kbatch;

@@ -1,0 +1,443 @@
+// fp32 GEMM on the matrix cores with operand tiles loaded from global memory straight into LDS.
+#include <type_traits>
+
+#include "gemm_shared.h"
+
+namespace ag {
+
+// ---------------------------------------------------------------------------------------------
+// Direct-to-LDS variant.  gfx950 can load 16 bytes per lane from global memory straight into LDS
+// (global_load_lds_dwordx4): lane l of a wave deposits its 16 bytes at LDS base + 16*l, whatever
+// global address it fetched.  Operand tiles therefore never pass through registers; the layout
+// in LDS is made conflict-free by choosing WHICH 16-byte chunk each lane fetches (an XOR swizzle
+// on the global side) instead of by padding.  BK = 32.
+//
+//   k-contiguous operand (rows x 32 k):  row r, chunk c (4 k) lives at chunk position
+//       r*8 + (c ^ f(r)),  f(r) = (r & 7) ^ ((r >> 3) & 1);
+//     a lane reads four consecutive k of its row with one 128-bit LDS read.
+//   m/n-contiguous operand (32 k x rows): element (k, n) lives at k*rows + (n ^ (32 * ((k>>2)&1)));
+//     a lane reads one k of its column per MFMA step with 32-bit LDS reads (the two half-waves
+//     read k and k+4, which the swizzle puts 128 bytes apart).
+//
+// The ring has STAGES slots; loads run STAGES-1 k tiles ahead of the MFMAs.  Each k tile has one
+// barrier, in its middle: before it a wave waits (vmcnt) until the NEXT tile's loads have
+// landed, after it the slot of the PREVIOUS tile is free for the loads issued next.  The loads
+// and the wait are inline assembly because the compiler would otherwise put a full vmcnt(0)
+// in front of every LDS read that follows an LDS-writing load; vmcnt counts loads and stores in
+// issue order, so "at most n outstanding" identifies which tiles have landed.
+// Requirements (checked on the host, else the register-staged kernel above runs): K % 32 == 0,
+// 16-byte aligned operands, leading dimensions and batch strides multiples of 4, and for an
+// m/n-contiguous operand an extent that is a multiple of 4.
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) float lds_float_t;
+
+// One wave-level 1 KiB load: lane l fetches 16 bytes at base + byte_off and they land at LDS byte
+// address lds_wave_base + LDS_IMM + 16*l.  (m0 carries the LDS address; a write to m0 needs one
+// wait state before the load that uses it.)
+template <int LDS_IMM>
+__device__ inline void dma16(const float *base, unsigned byte_off, unsigned lds_wave_base)
+{
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_wave_base), "v"(byte_off), "s"(base), "n"(LDS_IMM)
+                 : "m0", "scc");
+}
+
+template <int N>
+__device__ inline void wait_loads_then_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+
+// Swizzle of a k-contiguous tile: which 16-byte chunk position of row r holds chunk c.
+template <int BK>
+__device__ inline int kc_swizzle(int r)
+{
+    return BK == 32 ? ((r & 7) ^ ((r >> 3) & 1)) : (((r >> 1) ^ (r >> 3)) & 3);
+}
+
+template <bool KC, int ROWS, int BK, int NW>
+struct DirectTile {
+    static constexpr int CPR = KC ? BK / 4 : ROWS / 4;  // 16-byte chunks per LDS row
+    static constexpr int INSTR = ROWS * BK / 4 / 64;    // wave-level 1 KiB loads per tile
+    static constexpr int PER_WAVE = INSTR / NW;
+    static_assert(INSTR % NW == 0 && PER_WAVE >= 1, "tile does not divide over the waves");
+    static_assert(KC || ROWS % 64 == 0, "m/n-contiguous tiles are swizzled in 64-element groups");
+
+    unsigned off[PER_WAVE];  // byte offset of this lane's chunk from the k-tile origin
+
+    __device__ inline void init(int ld, int row0, int rows, int wave, int lane)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int pos = (i * NW + wave) * 64 + lane;  // chunk position in the LDS tile
+            if (KC) {
+                const int r = pos / CPR, c = (pos % CPR) ^ kc_swizzle<BK>(r);
+                const int row = min(row0 + r, rows - 1);
+                off[i] = (unsigned)(row * ld + c * 4) * 4u;
+            } else {
+                const int k = pos / CPR, cn = (pos % CPR) ^ (((k >> 2) & 1) * 8);
+                const int n = min(row0 + cn * 4, rows - 4);
+                off[i] = (unsigned)(k * ld + n) * 4u;
+            }
+        }
+    }
+    __device__ static inline long long k_step(int ld) { return KC ? BK : (long long)BK * ld; }
+
+    // Load number `i` (a constant after unrolling) of this wave.
+    __device__ inline void issue_one(int i, const float *origin, unsigned lds_wave_base) const
+    {
+        if (i == 0 && 0 < PER_WAVE) dma16<0 * NW * 1024>(origin, off[0], lds_wave_base);
+        if (i == 1 && 1 < PER_WAVE) dma16<1 * NW * 1024>(origin, off[1 < PER_WAVE ? 1 : 0], lds_wave_base);
+        if (i == 2 && 2 < PER_WAVE) dma16<2 * NW * 1024>(origin, off[2 < PER_WAVE ? 2 : 0], lds_wave_base);
+        if (i == 3 && 3 < PER_WAVE) dma16<3 * NW * 1024>(origin, off[3 < PER_WAVE ? 3 : 0], lds_wave_base);
+        if (i == 4 && 4 < PER_WAVE) dma16<4 * NW * 1024>(origin, off[4 < PER_WAVE ? 4 : 0], lds_wave_base);
+        if (i == 5 && 5 < PER_WAVE) dma16<5 * NW * 1024>(origin, off[5 < PER_WAVE ? 5 : 0], lds_wave_base);
+        if (i == 6 && 6 < PER_WAVE) dma16<6 * NW * 1024>(origin, off[6 < PER_WAVE ? 6 : 0], lds_wave_base);
+        if (i == 7 && 7 < PER_WAVE) dma16<7 * NW * 1024>(origin, off[7 < PER_WAVE ? 7 : 0], lds_wave_base);
+    }
+
+    // lds_wave_base: LDS byte address of the tile + 1024 * wave.
+    template <int I0, int I1>
+    __device__ inline void issue(const float *origin, unsigned lds_wave_base) const
+    {
+        // the LDS immediate must be a constant expression: unrolled by hand
+        if (I0 <= 0 && 0 < I1 && 0 < PER_WAVE) dma16<0 * NW * 1024>(origin, off[0], lds_wave_base);
+        if (I0 <= 1 && 1 < I1 && 1 < PER_WAVE) dma16<1 * NW * 1024>(origin, off[1 < PER_WAVE ? 1 : 0], lds_wave_base);
+        if (I0 <= 2 && 2 < I1 && 2 < PER_WAVE) dma16<2 * NW * 1024>(origin, off[2 < PER_WAVE ? 2 : 0], lds_wave_base);
+        if (I0 <= 3 && 3 < I1 && 3 < PER_WAVE) dma16<3 * NW * 1024>(origin, off[3 < PER_WAVE ? 3 : 0], lds_wave_base);
+        if (I0 <= 4 && 4 < I1 && 4 < PER_WAVE) dma16<4 * NW * 1024>(origin, off[4 < PER_WAVE ? 4 : 0], lds_wave_base);
+        if (I0 <= 5 && 5 < I1 && 5 < PER_WAVE) dma16<5 * NW * 1024>(origin, off[5 < PER_WAVE ? 5 : 0], lds_wave_base);
+        if (I0 <= 6 && 6 < I1 && 6 < PER_WAVE) dma16<6 * NW * 1024>(origin, off[6 < PER_WAVE ? 6 : 0], lds_wave_base);
+        if (I0 <= 7 && 7 < I1 && 7 < PER_WAVE) dma16<7 * NW * 1024>(origin, off[7 < PER_WAVE ? 7 : 0], lds_wave_base);
+        static_assert(PER_WAVE <= 8, "at most eight loads per wave and operand");
+    }
+};
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
+{
+    static_assert(STAGES >= 3 && STAGES <= 8, "ring of three to eight tiles");
+    static_assert(BK == 16 || BK == 32, "k tile");
+    constexpr int KK = BK / 8;  // groups of four MFMA k steps per tile
+    constexpr int WAVES_N = BN / WN;
+    constexpr int NW = (BM / WM) * (BN / WN);
+    constexpr int MI = WM / 32, NI = WN / 32;
+    constexpr int TILE = (BM + BN) * BK;  // floats per ring slot
+    using LoadA = DirectTile<KA, BM, BK, NW>;
+    using LoadB = DirectTile<KB, BN, BK, NW>;
+    constexpr int L = LoadA::PER_WAVE + LoadB::PER_WAVE;  // loads per wave per k tile
+    constexpr int STORES = MI * NI * 16;                  // epilogue stores per wave
+    constexpr int STEADY = (STAGES - 3) * L;              // loads that may stay in flight at a tile's barrier
+    constexpr int AFTER_EPILOGUE = STEADY + STORES > 63 ? 63 : STEADY + STORES;
+    static_assert((STAGES - 2) * L <= 63, "vmcnt range");
+
+    __shared__ __attribute__((aligned(1024))) float lds[STAGES * TILE];
+    const unsigned lds_base = (unsigned)(size_t)(lds_float_t *)lds;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l31 = lane & 31, half = lane >> 5;
+    const unsigned lds_wave = lds_base + (unsigned)wave * 1024u;
+
+    const unsigned total = p.total_blocks;
+    const unsigned tiles = (unsigned)(p.tiles_m * p.tiles_n);
+    const int kt_per = p.K / BK;
+    const int lda = (int)p.lda, ldb = (int)p.ldb;
+    // pointer steps of the fetch stream: to the next k tile, and from the last k tile of one
+    // accumulated batch to the first of the next
+    const long long step_a = LoadA::k_step(lda), step_b = LoadB::k_step(ldb);
+    const long long wrap_a = p.sAk - (kt_per - 1) * step_a, wrap_b = p.sBk - (kt_per - 1) * step_b;
+
+    struct Item {
+        int m0, n0, bz, sp, kb0, nt;
+    };
+    auto decode = [&](unsigned w) {
+        const unsigned lb = xcd_remap(w, total);
+        const unsigned z = lb / tiles, t_in = lb % tiles;
+        Item it;
+        it.m0 = (int)(t_in % p.tiles_m) * BM;
+        it.n0 = (int)(t_in / p.tiles_m) * BN;
+        it.bz = (int)(z / p.splits);
+        it.sp = (int)(z % p.splits);
+        it.kb0 = it.sp * p.kb_per_split;
+        it.nt = (min(p.kbatch, it.kb0 + p.kb_per_split) - it.kb0) * kt_per;
+        return it;
+    };
+
+    // ---- fetch stream ----
+    unsigned fw = blockIdx.x;
+    bool f_valid = fw < total;
+    if (!f_valid) return;
+    LoadA ldr_a;
+    LoadB ldr_b;
+    const float *pa = nullptr, *pb = nullptr;  // origin of the next k tile to fetch
+    int fkt = 0, f_left = 0;
+    auto f_begin = [&]() {
+        const Item it = decode(fw);
+        ldr_a.init(lda, it.m0, p.M, wave, lane);
+        ldr_b.init(ldb, it.n0, p.N, wave, lane);
+        pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
+        pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
+        fkt = 0;
+        f_left = it.nt;
+    };
+    auto fetch_advance = [&]() {
+        if (--f_left == 0) {
+            fw += gridDim.x;
+            f_valid = fw < total;
+            if (f_valid) f_begin();
+        } else if (++fkt == kt_per) {
+            fkt = 0;
+            pa += wrap_a;
+            pb += wrap_b;
+        } else {
+            pa += step_a;
+            pb += step_b;
+        }
+    };
+    // ---- compute stream ----
+    f32x16 acc[MI][NI];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
+    // Per-lane float indices of the fragments inside a ring slot.
+    int a_idx[KA ? KK : MI], b_idx[KB ? KK : NI];
+    {
+        const int x = half ^ kc_swizzle<BK>(l31);
+        if (KA) {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) a_idx[kk] = (wm * WM + l31) * BK + (((kk << 1) ^ x) << 2);
+        } else {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) a_idx[i] = half * 4 * BM + ((wm * WM + i * 32 + l31) ^ (half << 5));
+        }
+        if (KB) {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) b_idx[kk] = BM * BK + (wn * WN + l31) * BK + (((kk << 1) ^ x) << 2);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) b_idx[j] = BM * BK + half * 4 * BN + ((wn * WN + j * 32 + l31) ^ (half << 5));
+        }
+    }
+    struct Frag {
+        float v[4];
+    };
+    auto read_frags = [&](const float *S, int kk, Frag (&af)[MI], Frag (&bf)[NI]) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            if (KA) {
+                const float4 t = *reinterpret_cast<const float4 *>(S + a_idx[kk] + i * 32 * BK);
+                af[i].v[0] = t.x; af[i].v[1] = t.y; af[i].v[2] = t.z; af[i].v[3] = t.w;
+            } else {
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) af[i].v[s4] = S[a_idx[i] + (kk * 8 + s4) * BM];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            if (KB) {
+                const float4 t = *reinterpret_cast<const float4 *>(S + b_idx[kk] + j * 32 * BK);
+                bf[j].v[0] = t.x; bf[j].v[1] = t.y; bf[j].v[2] = t.z; bf[j].v[3] = t.w;
+            } else {
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) bf[j].v[s4] = S[b_idx[j] + (kk * 8 + s4) * BN];
+            }
+        }
+    };
+    auto mfma_frags = [&](const Frag (&af)[MI], const Frag (&bf)[NI]) {
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].v[s4], bf[j].v[s4], acc[i][j], 0, 0, 0);
+    };
+    // Returns true when exactly STORES store instructions were issued (interior tile, overwrite).
+    auto write_out = [&](const Item &it) -> bool {
+        float *Cb;
+        long long ldc;
+        float alpha, beta;
+        if (p.splits > 1) {
+            Cb = p.C + (long long)it.bz * p.sC + (long long)it.sp * p.sCsplit;
+            ldc = p.N;
+            alpha = 1.f;
+            beta = 0.f;
+        } else {
+            Cb = p.C + (long long)it.bz * p.sC;
+            ldc = p.ldc;
+            alpha = p.alpha;
+            beta = p.beta;
+        }
+        const bool full = it.m0 + BM <= p.M && it.n0 + BN <= p.N;
+        const int row_base = it.m0 + wm * WM + 4 * half;
+        const int col_base = it.n0 + wn * WN + l31;
+        if (full && beta == 0.f) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    float *dst = Cb + (long long)(row_base + i * 32) * ldc + col_base + j * 32;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        dst[(long long)(8 * (v / 4) + (v % 4)) * ldc] = alpha * acc[i][j][v];
+                }
+            return true;
+        } else {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    const int col = col_base + j * 32;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
+                        if (row < p.M && col < p.N) {
+                            float *dst = Cb + (long long)row * ldc + col;
+                            const float r = alpha * acc[i][j][v];
+                            *dst = beta == 0.f ? r : r + beta * *dst;
+                        }
+                    }
+                }
+        }
+        return false;
+    };
+
+    Frag af[2][MI], bf[2][NI];
+    unsigned fill_addr = lds_wave;  // LDS byte address (this wave's share) of the slot being filled
+    auto second_half = [&](const bool fetching, const float *cur, const float *nxt, bool last) {
+        constexpr int NM = (KK - KK / 2) * 4 * MI * NI;  // MFMAs in this half
+#ifdef AG_DL_SPACING
+        constexpr int SPACING = AG_DL_SPACING;
+#else
+        constexpr int SPACING = NM / L;                   // MFMAs between two loads
+#endif
+        static_assert(SPACING >= 1, "more loads than MFMAs");
+#pragma unroll
+        for (int kk = KK / 2; kk < KK; ++kk) {
+            if (kk + 1 < KK) read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+            else if (!last) read_frags(nxt, 0, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kk & 1][i].v[s4], bf[kk & 1][j].v[s4],
+                                                                         acc[i][j], 0, 0, 0);
+                        const int m = (((kk - KK / 2) * 4 + s4) * MI + i) * NI + j;
+                        const int load = m / SPACING;
+                        if (m % SPACING == SPACING - 1 && load < L && fetching) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (load < LoadA::PER_WAVE) ldr_a.issue_one(load, pa, fill_addr);
+                            else ldr_b.issue_one(load - LoadA::PER_WAVE, pb, fill_addr + BM * BK * 4u);
+                            if (load == L - 1) fetch_advance();
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Prologue: tiles 0 .. STAGES-2 of the stream.
+    f_begin();
+    bool all_issued = true;  // did the last attempt to issue a tile find one?
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) {
+        all_issued = f_valid;
+        if (f_valid) {
+            ldr_a.template issue<0, 8>(pa, fill_addr);
+            ldr_b.template issue<0, 8>(pb, fill_addr + BM * BK * 4u);
+            fetch_advance();
+        }
+        fill_addr += TILE * 4u;
+    }
+    if (all_issued) wait_loads_then_barrier<(STAGES - 2) * L>();
+    else wait_loads_then_barrier<0>();
+
+    unsigned cw = blockIdx.x;
+    Item ci = decode(cw);
+    const float *cur = lds;  // ring slot being multiplied
+    const float *const ring_end = lds + STAGES * TILE;
+    read_frags(cur, 0, af[0], bf[0]);
+
+    bool after_epilogue = false;
+    while (true) {  // work items of this block
+        zero_acc();
+        int c_left = ci.nt;
+        const bool last_item = cw + gridDim.x >= total;
+        do {  // k tiles of the item: the accumulators are touched by MFMAs only
+            const bool last = c_left == 1 && last_item;  // nothing follows in the stream
+            const float *nxt = cur + TILE == ring_end ? lds : cur + TILE;
+
+            // first half of the tile's k range
+#pragma unroll
+            for (int kk = 0; kk < KK / 2; ++kk) {
+                read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);  // all fragment reads of the next group go out first
+                mfma_frags(af[kk & 1], bf[kk & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // The next tile must have landed; tiles further ahead may still be in flight.
+            if (!all_issued) wait_loads_then_barrier<0>();
+            else if (after_epilogue) wait_loads_then_barrier<AFTER_EPILOGUE>();
+            else wait_loads_then_barrier<STEADY>();
+            after_epilogue = false;
+            all_issued = f_valid;
+            // Every wave has left the previous tile's slot.  Its loads are issued one at a time
+            // between the MFMAs of the rest of this tile: a clump of loads would leave the matrix
+            // pipe idle while the wave issues them, and all waves of the block would queue at the
+            // address unit right after the barrier.
+            second_half(all_issued, cur, nxt, last);
+            fill_addr = fill_addr + TILE * 4u == lds_wave + STAGES * TILE * 4u ? lds_wave : fill_addr + TILE * 4u;
+            cur = nxt;
+        } while (--c_left != 0);
+        const bool counted = write_out(ci);
+        if (last_item) break;
+        after_epilogue = counted;
+        cw += gridDim.x;
+        ci = decode(cw);
+    }
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES>
+static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu)
+{
+    constexpr int NT = (BM / WM) * (BN / WN) * 64;
+#define AG_GEMM_DL_CASE(KA_, KB_)                                                                     \
+    if (ka == KA_ && kb == KB_) {                                                                     \
+        auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_>;                                 \
+        long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \
+        if (g > p.total_blocks) g = p.total_blocks;                                                   \
+        hipLaunchKernelGGL(kern, dim3((unsigned)g), dim3(NT), 0, st, p);                              \
+        return;                                                                                       \
+    }
+    AG_GEMM_DL_CASE(true, true)
+    AG_GEMM_DL_CASE(true, false)
+    AG_GEMM_DL_CASE(false, true)
+    AG_GEMM_DL_CASE(false, false)
+#undef AG_GEMM_DL_CASE
+}
+
+void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu)
+{
+    switch (cfg) {
+        //                BM   BN  BK   WM  WN STAGES
+        case 13: launch_dl<128, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 14: launch_dl<128, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 15: launch_dl<256, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        default: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+    }
+}
+
+}  // namespace ag

@@ -1,0 +1,45 @@
+// Declarations shared by the two GEMM translation units (register-staged kernel and host
+// dispatch in gemm.hip, direct-to-LDS kernel in gemm_dl.hip).
+#pragma once
+#include "ag_internal.h"
+
+namespace ag {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+enum { LK_VEC = 0, LK_SCALAR = 1, LMN = 2 };
+
+struct GemmParams {
+    const float *A;
+    const float *B;
+    float *C;
+    int M, N, K;
+    long long lda, ldb, ldc;
+    long long sA, sB, sC;  // stride between independent batches
+    long long sAk, sBk;    // stride between accumulated batches
+    int kbatch;            // accumulated batches (>= 1)
+    int kb_per_split;
+    int splits;
+    long long sCsplit;     // stride between the partial outputs of consecutive splits
+    float alpha, beta;
+    int tiles_m, tiles_n;
+    unsigned total_blocks;
+};
+
+constexpr int kXcds = 8;
+
+// Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
+// contiguous slice of the logical block range instead.
+__device__ inline unsigned xcd_remap(unsigned id, unsigned total)
+{
+    const unsigned per = total / kXcds, rem = total % kXcds;
+    const unsigned xcd = id % kXcds, pos = id / kXcds;
+    return xcd * per + (xcd < rem ? xcd : rem) + pos;
+}
+
+// Launches direct-to-LDS configuration `cfg` (kFirstDirectCfg ..); `ka` / `kb`: the operand is
+// k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
+constexpr int kFirstDirectCfg = 13;
+void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
+
+}  // namespace ag

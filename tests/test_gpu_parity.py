@@ -190,6 +190,51 @@ def test_gemm_every_tile_configuration(K, rng, cfg):
     assert_close(got_t, truth, "gemm TT")
 
 
+DIRECT_CFGS = list(range(13, 18))  # operand tiles loaded from global memory straight into LDS
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("cfg", DIRECT_CFGS)
+def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb):
+    """K a multiple of 32, aligned operands: ragged M / N edges, a K of one and of several tiles,
+    and a batch large enough that every persistent block walks more than one output tile."""
+    L = K.capi.lib()
+    for (m, n, k, batch) in ((200, 332, 32, 1), (200, 332, 160, 3), (256, 384, 64, 80), (64, 64, 96, 5)):
+        a = rng.random((batch, k, m) if ta else (batch, m, k), dtype=np.float32)
+        b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
+        say("gemm direct cfg", cfg, ta, tb, m, n, k, batch)
+        c = dev(np.zeros((batch, m, n), np.float32))
+        L.ag_gemm_force_config(cfg)
+        try:
+            K.gemm(ta, tb, m, n, k, 1.0, dev(a), a.shape[2], a.shape[1] * a.shape[2], dev(b), b.shape[2],
+                   b.shape[1] * b.shape[2], 0.0, c, n, m * n, batch)
+        finally:
+            L.ag_gemm_force_config(-1)
+        A = a.transpose(0, 2, 1) if ta else a
+        Bm = b.transpose(0, 2, 1) if tb else b
+        truth = A.astype(np.float64) @ Bm.astype(np.float64)
+        assert_close(host(c), truth, f"direct gemm {m}x{n}x{k}x{batch}")
+
+
+@pytest.mark.parametrize("cfg", DIRECT_CFGS)
+def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg):
+    """The filter-gradient form (sum over images, split into a workspace and folded) and the
+    alpha / beta epilogue."""
+    L = K.capi.lib()
+    kf, ck, pp, imgs = 128, 288, 192, 37
+    gy = rng.random((imgs, kf, pp), dtype=np.float32)
+    cols = rng.random((imgs, ck, pp), dtype=np.float32)
+    c0 = rng.random((kf, ck), dtype=np.float32)
+    say("gemm direct batchsum cfg", cfg)
+    L.ag_gemm_force_config(cfg)
+    try:
+        got = host(K.gemm_batchsum(0, 1, kf, ck, pp, 0.5, dev(gy), pp, kf * pp, dev(cols), pp, ck * pp, 2.0, dev(c0), ck, imgs))
+    finally:
+        L.ag_gemm_force_config(-1)
+    want = 0.5 * np.einsum("bkp,bcp->kc", gy.astype(np.float64), cols.astype(np.float64)) + 2.0 * c0
+    assert_close(got, want, "direct batchsum")
+
+
 def test_gemm_leading_dims_alpha_beta_batch(K, rng):
     m, n, k, batch = 45, 70, 52, 3
     lda, ldb, ldc = k + 4, n + 8, n + 3
