@@ -192,6 +192,88 @@ __global__ __launch_bounds__(256) void col2im_unit_vec4_kernel(const float *__re
     }
 }
 
+// Stride 1, dilation 1 along x, output as wide as the input (W == OW, W % 4 == 0, W <= 256): the
+// "same"-size convolutions.  LPR lanes (a power of two >= W/4) share one destination row, each
+// owning four consecutive pixels.  Every tap plane is read with ALIGNED 128-bit streaming loads
+// at the lane's own four columns; the horizontal shift of the tap (pw - kx, between -3 and 3) is
+// applied afterwards by taking the missing column(s) from the neighbouring lane, zero outside
+// the row.  All kh*kw loads of a thread are issued before the first use.  The sums keep the
+// (ky, kx) ascending order of the reference.
+template <int KH, int KW, int PW, int LPR>
+__global__ __launch_bounds__(256) void col2im_same_kernel(const float *__restrict__ cols, float *__restrict__ gx,
+                                                          ConvGeom g, unsigned rows_total)
+{
+    constexpr int RPW = 64 / LPR;  // rows per wave
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane & (LPR - 1);
+    const int W4 = g.W >> 2;
+    const bool in_row = q < W4;
+    const unsigned P = (unsigned)(g.OH * g.OW);
+    for (unsigned r = (blockIdx.x * 4u + wave) * RPW + lane / LPR; r - lane / LPR < rows_total;
+         r += gridDim.x * 4u * RPW) {
+        const bool active = in_row && r < rows_total;
+        const unsigned plane = r / (unsigned)g.H;
+        const int iy = (int)(r - plane * (unsigned)g.H);
+        const float *cp = cols + (long long)plane * (KH * KW) * P + q * 4;
+        float4 v[KH][KW];
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky) {
+            const int oy = iy + g.ph - ky * g.dh;
+            const bool ok = active && (unsigned)oy < (unsigned)g.OH;
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx)
+                v[ky][kx] = ok ? ld_stream(reinterpret_cast<const float4 *>(cp + (unsigned)(ky * KW + kx) * P + (unsigned)oy * g.OW))
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx) {
+                const int d = PW - kx;  // source column = destination column + d
+                const float4 c = v[ky][kx];
+                if (d == 0) {
+                    a0 += c.x; a1 += c.y; a2 += c.z; a3 += c.w;
+                } else if (d > 0) {
+                    // columns 4q+d .. 4q+d+3: own elements d..3, then the next lane's 0..d-1
+                    const bool has = q + 1 < W4;
+                    const float nx = __shfl_down(c.x, 1, LPR), ny = __shfl_down(c.y, 1, LPR), nz = __shfl_down(c.z, 1, LPR);
+                    const float e0 = has ? nx : 0.f, e1 = has ? ny : 0.f, e2 = has ? nz : 0.f;
+                    if (d == 1) { a0 += c.y; a1 += c.z; a2 += c.w; a3 += e0; }
+                    else if (d == 2) { a0 += c.z; a1 += c.w; a2 += e0; a3 += e1; }
+                    else { a0 += c.w; a1 += e0; a2 += e1; a3 += e2; }
+                } else {
+                    // columns 4q+d .. : the previous lane's last -d elements, then own 0..3+d
+                    const bool has = q > 0;
+                    const float py = __shfl_up(c.y, 1, LPR), pz = __shfl_up(c.z, 1, LPR), pw_ = __shfl_up(c.w, 1, LPR);
+                    const float e1 = has ? py : 0.f, e2 = has ? pz : 0.f, e3 = has ? pw_ : 0.f;
+                    if (d == -1) { a0 += e3; a1 += c.x; a2 += c.y; a3 += c.z; }
+                    else if (d == -2) { a0 += e2; a1 += e3; a2 += c.x; a3 += c.y; }
+                    else { a0 += e1; a1 += e2; a2 += e3; a3 += c.x; }
+                }
+            }
+        if (active) st_stream(reinterpret_cast<float4 *>(gx + (long long)r * g.W + q * 4), make_float4(a0, a1, a2, a3));
+    }
+}
+
+template <int KH, int KW, int PW>
+static void launch_col2im_same(hipStream_t st, const float *cols, float *gx, const ConvGeom &g, long long rows)
+{
+    const int W4 = g.W >> 2;
+    const int lpr = W4 <= 4 ? 4 : W4 <= 8 ? 8 : W4 <= 16 ? 16 : W4 <= 32 ? 32 : 64;
+    const long long rows_per_block = 4 * (64 / lpr);
+    long long blocks = (rows + rows_per_block - 1) / rows_per_block;
+    if (blocks > 1048576) blocks = 1048576;
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (lpr) {
+        case 4: hipLaunchKernelGGL((col2im_same_kernel<KH, KW, PW, 4>), grid, block, 0, st, cols, gx, g, (unsigned)rows); break;
+        case 8: hipLaunchKernelGGL((col2im_same_kernel<KH, KW, PW, 8>), grid, block, 0, st, cols, gx, g, (unsigned)rows); break;
+        case 16: hipLaunchKernelGGL((col2im_same_kernel<KH, KW, PW, 16>), grid, block, 0, st, cols, gx, g, (unsigned)rows); break;
+        case 32: hipLaunchKernelGGL((col2im_same_kernel<KH, KW, PW, 32>), grid, block, 0, st, cols, gx, g, (unsigned)rows); break;
+        default: hipLaunchKernelGGL((col2im_same_kernel<KH, KW, PW, 64>), grid, block, 0, st, cols, gx, g, (unsigned)rows); break;
+    }
+}
+
 // Stride 2 on both axes: one thread per 2x2 block of destination pixels.  Every tap (ky, kx)
 // feeds exactly one pixel of the block (the one whose offset has the right parity), so a thread
 // reads each of the kh*kw planes once, at consecutive positions for consecutive threads, and no
@@ -258,6 +340,83 @@ static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int k
 
 using namespace ag;
 
+// im2col for the "same"-size stride-1 convolutions (W == OW, W % 4 == 0, W <= 256, dilation 1
+// along x): the mirror image of col2im_same_kernel.  LPR lanes share one output row, each owning
+// four consecutive columns.  A lane loads its own four columns of the kh input rows with aligned
+// 128-bit loads (zero outside the image), builds the kw horizontally shifted versions with one
+// lane exchange each, and streams the kh*kw results to their planes with aligned 128-bit
+// non-temporal stores.  No LDS, no divisions besides one per thread.
+template <int KH, int KW, int PW, int LPR>
+__global__ __launch_bounds__(256) void im2col_same_kernel(const float *__restrict__ x, float *__restrict__ cols,
+                                                          ConvGeom g, unsigned rows_total)
+{
+    constexpr int RPW = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane & (LPR - 1);
+    const int W4 = g.W >> 2;
+    const bool in_row = q < W4;
+    const unsigned P = (unsigned)(g.OH * g.OW);
+    for (unsigned r = (blockIdx.x * 4u + wave) * RPW + lane / LPR; r - lane / LPR < rows_total;
+         r += gridDim.x * 4u * RPW) {
+        const bool active = in_row && r < rows_total;
+        const unsigned plane = r / (unsigned)g.OH;
+        const int oy = (int)(r - plane * (unsigned)g.OH);
+        const float *xp = x + (long long)plane * g.H * g.W + q * 4;
+        float4 v[KH];
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky) {
+            const int iy = oy - g.ph + ky * g.dh;
+            const bool ok = active && (unsigned)iy < (unsigned)g.H;
+            v[ky] = ok ? *reinterpret_cast<const float4 *>(xp + (unsigned)iy * g.W) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float *cp = cols + (long long)plane * (KH * KW) * P + (unsigned)oy * g.OW + q * 4;
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx) {
+                const int d = kx - PW;  // source column = output column + d
+                const float4 c = v[ky];
+                float4 o;
+                if (d == 0) {
+                    o = c;
+                } else if (d > 0) {
+                    const bool has = q + 1 < W4;
+                    const float nx = __shfl_down(c.x, 1, LPR), ny = __shfl_down(c.y, 1, LPR), nz = __shfl_down(c.z, 1, LPR);
+                    const float e0 = has ? nx : 0.f, e1 = has ? ny : 0.f, e2 = has ? nz : 0.f;
+                    if (d == 1) o = make_float4(c.y, c.z, c.w, e0);
+                    else if (d == 2) o = make_float4(c.z, c.w, e0, e1);
+                    else o = make_float4(c.w, e0, e1, e2);
+                } else {
+                    const bool has = q > 0;
+                    const float py = __shfl_up(c.y, 1, LPR), pz = __shfl_up(c.z, 1, LPR), pw_ = __shfl_up(c.w, 1, LPR);
+                    const float e1 = has ? py : 0.f, e2 = has ? pz : 0.f, e3 = has ? pw_ : 0.f;
+                    if (d == -1) o = make_float4(e3, c.x, c.y, c.z);
+                    else if (d == -2) o = make_float4(e2, e3, c.x, c.y);
+                    else o = make_float4(e1, e2, e3, c.x);
+                }
+                if (active) st_stream(reinterpret_cast<float4 *>(cp + (unsigned)(ky * KW + kx) * P), o);
+            }
+    }
+}
+
+template <int KH, int KW, int PW>
+static void launch_im2col_same(hipStream_t st, const float *x, float *cols, const ConvGeom &g, long long rows)
+{
+    const int W4 = g.W >> 2;
+    const int lpr = W4 <= 4 ? 4 : W4 <= 8 ? 8 : W4 <= 16 ? 16 : W4 <= 32 ? 32 : 64;
+    const long long rows_per_block = 4 * (64 / lpr);
+    long long blocks = (rows + rows_per_block - 1) / rows_per_block;
+    if (blocks > 1048576) blocks = 1048576;
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (lpr) {
+        case 4: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 4>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
+        case 8: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 8>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
+        case 16: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 16>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
+        case 32: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 32>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
+        default: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 64>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
+    }
+}
+
 extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *cols, int B, int C,
                                      int H, int W, int kh, int kw, int ph, int pw, int sh, int sw,
                                      int dh, int dw)
@@ -272,6 +431,18 @@ extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *
     if (planes == 0 || OH <= 0 || OW <= 0) return AG_OK;
     AG_REQUIRE(x && cols, AG_ERR_INVALID_DIMS, "im2col: null pointer");
     ConvGeom g{C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW};
+
+    const bool same = sh == 1 && sw == 1 && dw == 1 && OW == W && ph == pw && W % 4 == 0 && W <= 256 &&
+                      aligned16(x) && aligned16(cols) && planes * OH < 0x7fffffffLL &&
+                      (long long)kh * kw * OH * OW < 0x7fffffffLL && (long long)H * W < 0x7fffffffLL;
+    if (same && kh == 3 && kw == 3 && pw == 1) {
+        launch_im2col_same<3, 3, 1>(as_stream(stream), x, cols, g, planes * OH);
+        return check_launch("im2col");
+    }
+    if (same && kh == 5 && kw == 5 && pw == 2) {
+        launch_im2col_same<5, 5, 2>(as_stream(stream), x, cols, g, planes * OH);
+        return check_launch("im2col");
+    }
 
     const int WL = (OW - 1) * sw + (kw - 1) * dw + 1;  // staged row length
     const int rows_min = (kh - 1) * dh + 1;            // input rows for one output row
@@ -321,7 +492,13 @@ extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, floa
     AG_REQUIRE(gx && (cols || OH == 0 || OW == 0), AG_ERR_INVALID_DIMS, "col2im: null pointer");
     AG_REQUIRE((long long)H * W <= 0x7fffffffLL, AG_ERR_INVALID_DIMS, "col2im: plane too large");
     ConvGeom g{C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, OH, OW};
-    if (sh == 1 && sw == 1 && W % 4 == 0 && aligned16(gx)) {
+    const bool same = sh == 1 && sw == 1 && dw == 1 && OW == W && W % 4 == 0 && W <= 256 && aligned16(gx) &&
+                      aligned16(cols) && planes * H < 0x7fffffffLL && (long long)kh * kw * OH * OW < 0x7fffffffLL;
+    if (same && kh == 3 && kw == 3 && pw == 1) {
+        launch_col2im_same<3, 3, 1>(as_stream(stream), cols, gx, g, planes * H);
+    } else if (same && kh == 5 && kw == 5 && pw == 2) {
+        launch_col2im_same<5, 5, 2>(as_stream(stream), cols, gx, g, planes * H);
+    } else if (sh == 1 && sw == 1 && W % 4 == 0 && aligned16(gx)) {
         const long long groups = planes * H * (W / 4);
         long long blocks = (groups + 255) / 256;
         if (blocks > 262144) blocks = 262144;

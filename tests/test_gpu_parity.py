@@ -75,6 +75,12 @@ GEOMS = [  # B, C, H, W, kh, kw, pad, stride, dil
     (1, 1, 4, 4, 1, 1, 0, 1, 1),
     (1, 2, 70, 300, 3, 3, 1, 1, 1),   # several row bands per plane
     (1, 1, 3, 9000, 3, 3, 1, 1, 1),   # row too wide to stage: direct path
+    (2, 3, 12, 16, 5, 5, 2, 1, 1),    # 5x5 "same": shifts of two columns, four lanes per row
+    (1, 2, 6, 64, 3, 3, 1, 1, 1),     # a row fills its sixteen lanes exactly
+    (1, 1, 5, 128, 3, 3, 1, 1, 1),    # thirty-two lanes per row
+    (1, 1, 3, 256, 3, 3, 1, 1, 1),    # one row per wave
+    (3, 1, 5, 8, 3, 3, 1, 1, 1),      # rows do not fill the last wave
+    (1, 2, 9, 12, 3, 3, 1, 1, 2),     # dilation keeps the general stride-1 kernel
 ]
 
 
