@@ -38,11 +38,11 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 # true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 KIB = 1024.0
 TRAFFIC_BYTES = {
-    "gemm_fwd": (920481.0 * 2.0 + 401408.0) * KIB,
-    "gemm_filter_grad": (1157507.4 * 2.0 + 73728.0) * KIB,
-    "gemm_input_grad": (291922.1 * 2.0 + 1806336.0) * KIB,
-    "im2col": (124964.5 * 2.0 + 1806336.2) * KIB,
-    "col2im": (920882.1 * 2.0 + 200704.0) * KIB,
+    "gemm_fwd": (918691.3 * 2.0 + 401408.0) * KIB,
+    "gemm_filter_grad": ((1116497.5 + 36881.9) * 2.0 + 73728.0 + 288.0) * KIB,  # GEMM + fold of the split partials
+    "gemm_input_grad": (212984.1 * 2.0 + 1806336.0) * KIB,
+    "im2col": (112668.1 * 2.0 + 1806380.7) * KIB,
+    "col2im": (919260.8 * 2.0 + 200704.0) * KIB,
 }
 
 

@@ -358,20 +358,35 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
     else run(std::false_type{});
 }
 
-// C[m][n] = alpha * sum_s partial[s][m][n] + beta * C[m][n], s ascending.
+// C[m][n] = alpha * sum_s partial[s][m][n] + beta * C[m][n].  A block folds 32 consecutive
+// elements: thread (g, e) adds the partials s = g, g + 8, g + 16, ... of element e (eight
+// independent chains keep enough loads in flight), then the eight group sums are added in
+// ascending g.  The order is fixed, so the result is deterministic.
 __global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__restrict__ partial, int splits,
                                                           long long split_stride, float *__restrict__ C,
                                                           int M, int N, long long ldc, float alpha,
                                                           float beta)
 {
+    __shared__ float part[8][32];
     const long long total = (long long)M * N;
-    for (long long e = blockIdx.x * 256LL + threadIdx.x; e < total; e += gridDim.x * 256LL) {
+    const int e_in = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    for (long long e0 = blockIdx.x * 32LL; e0 < total; e0 += gridDim.x * 32LL) {
+        const long long e = e0 + e_in;
         float acc = 0.f;
-        for (int s = 0; s < splits; ++s) acc += partial[s * split_stride + e];
-        const int m = (int)(e / N), n = (int)(e - (long long)m * N);
-        float *dst = C + m * ldc + n;
-        const float r = alpha * acc;
-        *dst = beta == 0.f ? r : r + beta * *dst;
+        if (e < total)
+            for (int s = grp; s < splits; s += 8) acc += partial[s * split_stride + e];
+        part[grp][e_in] = acc;
+        __syncthreads();
+        if (grp == 0 && e < total) {
+            float sum = part[0][e_in];
+#pragma unroll
+            for (int g = 1; g < 8; ++g) sum += part[g][e_in];
+            const int m = (int)(e / N), n = (int)(e - (long long)m * N);
+            float *dst = C + m * ldc + n;
+            const float r = alpha * sum;
+            *dst = beta == 0.f ? r : r + beta * *dst;
+        }
+        __syncthreads();
     }
 }
 
@@ -626,7 +641,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (ag_status_t s = check_launch(who)) return s;
     if (p.splits > 1) {
         const long long total = (long long)c.M * c.N;
-        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 256) > 4096 ? 4096 : cdiv(total, 256))),
+        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
                            dim3(256), 0, st, static_cast<const float *>(ws), p.splits, p.sCsplit, real_c, c.M,
                            c.N, c.ldc, c.alpha, c.beta);
         return check_launch(who);

@@ -336,10 +336,6 @@ static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int k
     return AG_OK;
 }
 
-}  // namespace ag
-
-using namespace ag;
-
 // im2col for the "same"-size stride-1 convolutions (W == OW, W % 4 == 0, W <= 256, dilation 1
 // along x): the mirror image of col2im_same_kernel.  LPR lanes share one output row, each owning
 // four consecutive columns.  A lane loads its own four columns of the kh input rows with aligned
@@ -416,6 +412,10 @@ static void launch_im2col_same(hipStream_t st, const float *x, float *cols, cons
         default: hipLaunchKernelGGL((im2col_same_kernel<KH, KW, PW, 64>), grid, block, 0, st, x, cols, g, (unsigned)rows); break;
     }
 }
+
+}  // namespace ag
+
+using namespace ag;
 
 extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *cols, int B, int C,
                                      int H, int W, int kh, int kw, int ph, int pw, int sh, int sw,

@@ -254,6 +254,143 @@ static ag_status_t pool_geom(const char *who, int B, int C, int H, int W, int si
     return AG_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Stride-2 backward without LDS (window 2 or 3, W % 4 == 0, W <= 256).  LPR lanes (a power of
+// two >= W/4) share one plane; lane q owns input columns 4q .. 4q+3 and reads the two outputs 2q
+// and 2q+1 whose windows start there.  A lane walks a chunk of output rows top to bottom and
+// writes every input row once with an aligned 128-bit streaming store.
+// ---------------------------------------------------------------------------------------------
+// A chunk of output rows [oy0, oy1) owns the input rows
+// [2*oy0, 2*oy1) (the last chunk also the rows below the last window, which receive nothing).
+// Every pixel adds the gradients of the windows that selected it in ascending (oy, ox) order,
+// the order of the reference's scatter loop, so the sums are bit-identical.  For the 3-wide
+// window the contributions of window row oy to input row 2*oy+2 are carried to the next
+// iteration, and a chunk first recomputes what the window row above it contributes to its top row.
+template <bool EXACT, int SIZE, int LPR>
+__global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__restrict__ gy,
+                                                             const float *__restrict__ argmax,
+                                                             const int32_t *__restrict__ idx_local,
+                                                             float *__restrict__ gx, PoolGeom g, int rows_per_chunk,
+                                                             int chunks, unsigned groups_total)
+{
+    constexpr int GPW = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane & (LPR - 1);
+    const bool in_row = q < (g.W >> 2);
+    const int W = g.W;
+    for (unsigned grp = (blockIdx.x * 4u + wave) * GPW + lane / LPR; grp - lane / LPR < groups_total;
+         grp += gridDim.x * 4u * GPW) {
+        const bool active = in_row && grp < groups_total;
+        const unsigned plane = grp / (unsigned)chunks;
+        const int chunk = (int)(grp - plane * (unsigned)chunks);
+        const int oy0 = chunk * rows_per_chunk;
+        const int oy1 = grp < groups_total ? min(oy0 + rows_per_chunk, g.OH) : oy0;
+        const bool last_chunk = chunk == chunks - 1;
+        const long long base = (long long)plane * g.H * W;
+        const long long obase = (long long)plane * g.OH * g.OW;
+        float *gxp = gx + base + q * 4;
+        const bool va = active && 2 * q < g.OW, vb = active && 2 * q + 1 < g.OW;
+        // gradient and selected plane-local position of outputs (oy, 2q) and (oy, 2q+1)
+        struct Out {
+            float ga, gb;
+            long long ia, ib;
+        };
+        auto load_out = [&](int oy) {
+            Out o;
+            const long long at = obase + (long long)oy * g.OW + 2 * q;
+            o.ga = va ? gy[at] : 0.f;
+            o.gb = vb ? gy[at + 1] : 0.f;
+            if (EXACT) {
+                o.ia = va ? (long long)idx_local[at] : -1;
+                o.ib = vb ? (long long)idx_local[at + 1] : -1;
+            } else {
+                // whole-tensor offsets as stored by the forward pass; made plane-local here
+                o.ia = va ? (long long)argmax[at] - base : -1;
+                o.ib = vb ? (long long)argmax[at + 1] - base : -1;
+            }
+            return o;
+        };
+        // Adds what window row `o` (with the neighbour's second window `pg`, `pi`) gives to the
+        // four pixels of input row iy, pixel by pixel in ascending ox.
+        auto add_row = [&](float (&acc)[4], const Out &o, float pg, long long pi, int iy) {
+            const long long r = (long long)iy * W + 4 * q;
+            if (SIZE == 3) {
+                acc[0] = pi == r ? acc[0] + pg : acc[0];
+                acc[0] = o.ia == r ? acc[0] + o.ga : acc[0];
+                acc[1] = o.ia == r + 1 ? acc[1] + o.ga : acc[1];
+                acc[2] = o.ia == r + 2 ? acc[2] + o.ga : acc[2];
+                acc[2] = o.ib == r + 2 ? acc[2] + o.gb : acc[2];
+                acc[3] = o.ib == r + 3 ? acc[3] + o.gb : acc[3];
+            } else {
+                acc[0] = o.ia == r ? acc[0] + o.ga : acc[0];
+                acc[1] = o.ia == r + 1 ? acc[1] + o.ga : acc[1];
+                acc[2] = o.ib == r + 2 ? acc[2] + o.gb : acc[2];
+                acc[3] = o.ib == r + 3 ? acc[3] + o.gb : acc[3];
+            }
+        };
+        auto neighbour = [&](const Out &o, float &pg, long long &pi) {
+            pg = __shfl_up(o.gb, 1, LPR);
+            const int lo = __shfl_up((int)(o.ib & 0xffffffffll), 1, LPR), hi = __shfl_up((int)(o.ib >> 32), 1, LPR);
+            pi = q > 0 ? (((long long)hi << 32) | (unsigned)lo) : -1;
+            if (q == 0) pg = 0.f;
+        };
+        auto store_row = [&](int iy, const float (&acc)[4]) {
+            if (active) st_stream(reinterpret_cast<float4 *>(gxp + iy * W), make_float4(acc[0], acc[1], acc[2], acc[3]));
+        };
+        float carry[4] = {0.f, 0.f, 0.f, 0.f};
+        Out cur;
+        cur.ga = cur.gb = 0.f;
+        cur.ia = cur.ib = -1;
+        if (SIZE == 3 && oy0 > 0 && oy0 < oy1) {
+            const Out above = load_out(oy0 - 1);
+            float pg;
+            long long pi;
+            neighbour(above, pg, pi);
+            add_row(carry, above, pg, pi, 2 * oy0);
+        }
+        if (oy0 < oy1) cur = load_out(oy0);
+        for (int oy = oy0; oy < oy1; ++oy) {
+            Out nxt;
+            nxt.ga = nxt.gb = 0.f;
+            nxt.ia = nxt.ib = -1;
+            if (oy + 1 < oy1) nxt = load_out(oy + 1);
+            float pg = 0.f;
+            long long pi = -1;
+            if (SIZE == 3) neighbour(cur, pg, pi);
+            float a0[4] = {carry[0], carry[1], carry[2], carry[3]}, a1[4] = {0.f, 0.f, 0.f, 0.f};
+            add_row(a0, cur, pg, pi, 2 * oy);
+            add_row(a1, cur, pg, pi, 2 * oy + 1);
+            store_row(2 * oy, a0);
+            store_row(2 * oy + 1, a1);
+            if (SIZE == 3) {
+                carry[0] = carry[1] = carry[2] = carry[3] = 0.f;
+                add_row(carry, cur, pg, pi, 2 * oy + 2);
+            }
+            cur = nxt;
+        }
+        if (last_chunk && grp < groups_total) {
+            // rows below the last window row: the carried row (3-wide window), then zeros
+            int iy = 2 * g.OH;
+            if (SIZE == 3 && iy < g.H) {
+                store_row(iy, carry);
+                ++iy;
+            }
+            const float z[4] = {0.f, 0.f, 0.f, 0.f};
+            for (; iy < g.H; ++iy) store_row(iy, z);
+        }
+    }
+}
+
+static int lanes_per_row(int W)
+{
+    const int W4 = W >> 2;
+    return W4 <= 4 ? 4 : W4 <= 8 ? 8 : W4 <= 16 ? 16 : W4 <= 32 ? 32 : 64;
+}
+
+// Output rows per chunk: short chunks give more independent streams, long ones re-read fewer
+// halo rows; nine rows of a 27-row plane measured well.
+static int pool_chunk_rows(int OH) { return OH <= 12 ? OH : (OH + (OH + 8) / 9 - 1) / ((OH + 8) / 9); }
+
 constexpr long long kExactFloatIndexLimit = 1LL << 24;
 
 }  // namespace ag
@@ -307,6 +444,33 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
     AG_REQUIRE(idx_local || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
                "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the int32 plane-local indices",
                (long long)B * C * H * W);
+    if (stride == 2 && (size == 2 || size == 3) && W % 4 == 0 && W <= 256 && aligned16(gx) && g.OH > 0 && g.OW > 0 &&
+        (long long)B * C * g.OH < 0x7fffffffLL && (long long)H * W < 0x7fffffffLL) {
+        const int rpc = pool_chunk_rows(g.OH), chunks = (g.OH + rpc - 1) / rpc;
+        const long long groups = (long long)B * C * chunks;
+        const int lpr = lanes_per_row(W);
+        long long blocks = (groups + 4 * (64 / lpr) - 1) / (4 * (64 / lpr));
+        if (blocks > 1048576) blocks = 1048576;
+#define AG_POOL_BWD_S2(EX, SZ, LP)                                                                            \
+    hipLaunchKernelGGL((maxpool_bwd_s2_kernel<EX, SZ, LP>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), \
+                       gy, argmax, idx_local, gx, g, rpc, chunks, (unsigned)groups)
+#define AG_POOL_BWD_S2_LPR(EX, SZ)                      \
+    switch (lpr) {                                      \
+        case 4: AG_POOL_BWD_S2(EX, SZ, 4); break;       \
+        case 8: AG_POOL_BWD_S2(EX, SZ, 8); break;       \
+        case 16: AG_POOL_BWD_S2(EX, SZ, 16); break;     \
+        case 32: AG_POOL_BWD_S2(EX, SZ, 32); break;     \
+        default: AG_POOL_BWD_S2(EX, SZ, 64); break;     \
+    }
+        if (idx_local) {
+            if (size == 3) { AG_POOL_BWD_S2_LPR(true, 3) } else { AG_POOL_BWD_S2_LPR(true, 2) }
+        } else {
+            if (size == 3) { AG_POOL_BWD_S2_LPR(false, 3) } else { AG_POOL_BWD_S2_LPR(false, 2) }
+        }
+#undef AG_POOL_BWD_S2_LPR
+#undef AG_POOL_BWD_S2
+        return check_launch("max_pool2d_grad");
+    }
     // LDS-staged path: W % 4 == 0 (128-bit stores) and the windows of a band fit the budget
     const long long orow_bytes = (long long)g.OW * 8;  // gy + index per output
     if (W % 4 == 0 && aligned16(gx) && g.OH > 0 && g.OW > 0 &&

@@ -426,7 +426,10 @@ def test_max_pool_reference_vector(K, golden):
 
 
 POOL_CASES = [(2, 3, 6, 6, 2, 2), (2, 3, 7, 9, 3, 2), (1, 2, 8, 8, 3, 1), (3, 32, 28, 28, 2, 2),
-              (2, 16, 56, 56, 3, 2), (1, 1, 5, 7, 2, 3), (1, 3, 33, 65, 3, 2)]
+              (2, 16, 56, 56, 3, 2), (1, 1, 5, 7, 2, 3), (1, 3, 33, 65, 3, 2),
+              # stride-2 register kernels: one lane group per plane, 4 .. 64 lanes per row, chunked rows
+              (2, 3, 8, 4, 2, 2), (1, 2, 64, 64, 3, 2), (1, 2, 30, 128, 3, 2), (1, 1, 9, 256, 2, 2),
+              (5, 3, 40, 12, 3, 2), (1, 1, 4, 4, 3, 2), (7, 1, 5, 8, 3, 2), (3, 2, 27, 20, 2, 2)]
 
 
 @pytest.mark.parametrize("case", POOL_CASES)
@@ -454,6 +457,24 @@ def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
     for idx in (None, il):
         ggy = host(K.max_pool2d_grad_grad(dev(ggx), am, idx, size, 0, stride))
         assert np.array_equal(ggy, orc.maxpool2d_gradgrad(ggx, oam, oy.shape))
+
+
+@pytest.mark.parametrize("case", [(2, 4, 56, 56, 3, 2), (2, 4, 28, 28, 2, 2), (1, 3, 21, 16, 3, 2)])
+def test_max_pool_many_ties(K, orc, rng, case):
+    """Small integer inputs: almost every window has several equal maxima; the first in row-major
+    window order must be selected, and the backward must route each gradient to exactly that pixel."""
+    B, C, H, W, size, stride = case
+    x = rng.integers(0, 3, (B, C, H, W)).astype(np.float32)
+    say("max_pool ties", case)
+    y, am, il = K.max_pool2d(dev(x), size, 0, stride)
+    oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, stride)
+    assert np.array_equal(host(y), oy) and np.array_equal(host(il), oil)
+    assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32))
+    gy = rng.standard_normal(oy.shape).astype(np.float32)
+    ogx, _ = orc.maxpool2d_bwd(gy, oam, x.shape)
+    for idx in (None, il):
+        gx = host(K.max_pool2d_grad(dev(gy), am, idx, x.shape, size, 0, stride))
+        assert np.array_equal(gx.view(np.uint32), ogx.view(np.uint32))
 
 
 def test_max_pool_nan_window_and_pad_error(K, orc):
