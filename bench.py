@@ -298,7 +298,73 @@ def micro(torch, Kn, capi, dev):
     ms = time_events(torch, lambda: Kn.batch_matmul(A, Bm), 10)
     tf = 2.0 * 64 * 512 ** 3 / ms / 1e9
     res["batch_matmul_64x512"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    res.update(graph_steps())
     return res
+
+
+def graph_steps():
+    """Configurations 1 and 2 end to end through the host operator layer (graph build, evaluation,
+    gradients, Adam), host arrays fed every step as the reference's examples do.  These steps are
+    tens of MFLOP: launch- and copy-latency bound, reported as wall-clock time only."""
+    import time
+
+    import numpy as np
+
+    import rust_autograd_amd.graph as G
+
+    rng = np.random.default_rng(5)
+
+    def glorot(shape):
+        sc = np.sqrt(6.0 / (int(np.prod(shape[1:])) + shape[0] * int(np.prod(shape[2:]))))
+        return rng.uniform(-sc, sc, shape).astype(np.float32)
+
+    out = {}
+    # config 1: conv(1->32, 3x3, pad 1) -> ReLU -> max_pool 2x2 -> sum; grads w.r.t. x and w
+    env = G.VariableEnvironment()
+    wid = env.set("w", glorot((32, 1, 3, 3)))
+    xv = rng.random((64, 1, 28, 28), dtype=np.float32)
+
+    def c1_step():
+        c = env.context()
+        x, w = c.placeholder("x", [-1, 1, 28, 28]), c.variable(wid)
+        loss = c.reduce_sum(c.max_pool2d(c.relu(c.conv2d(x, w, 1, 1)), 2, 0, 2), [0, 1, 2, 3])
+        c.eval(c.grad([loss], [x, w]), {"x": xv})
+
+    # config 2: the small CNN of examples/cnn_mnist.rs with Adam, batch 128
+    env2 = G.VariableEnvironment()
+    params = {"w1": glorot((32, 1, 3, 3)), "w2": glorot((64, 32, 3, 3)),
+              "w3": rng.uniform(-0.04, 0.04, (3136, 10)).astype(np.float32),
+              "b1": np.zeros((1, 32, 28, 28), np.float32), "b2": np.zeros((1, 64, 14, 14), np.float32),
+              "b3": np.zeros((1, 10), np.float32)}
+    ids = {k: env2.set(k, a) for k, a in params.items()}
+    names = list(params)
+    adam = G.Adam(env2, [ids[k] for k in names], alpha=1e-3)
+    x2 = rng.random((128, 1, 28, 28), dtype=np.float32)
+    y2 = rng.integers(0, 10, (128, 1)).astype(np.float32)
+
+    def c2_step():
+        c = env2.context()
+        v = {k: c.variable(ids[k]) for k in names}
+        x, t = c.placeholder("x", [-1, 1, 28, 28]), c.placeholder("y", [-1, 1])
+        z = c.max_pool2d(c.relu(c.conv2d(x, v["w1"], 1, 1) + v["b1"]), 2, 0, 2)
+        z = c.max_pool2d(c.relu(c.conv2d(z, v["w2"], 1, 1) + v["b2"]), 2, 0, 2)
+        logits = c.matmul(c.reshape(z, [-1, 3136]), v["w3"]) + v["b3"]
+        loss = c.reduce_mean(c.sparse_softmax_cross_entropy(logits, t), [0], False)
+        grads = c.grad([loss], [v[k] for k in names])
+        adam.update([v[k] for k in names], grads, c, {"x": x2, "y": y2})
+
+    for name, step, images in (("config1_conv_block_step", c1_step, 64), ("config2_cnn_adam_step", c2_step, 128)):
+        for _ in range(3):
+            step()
+        ts = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            step()  # evaluation synchronises before it returns
+            ts.append((time.perf_counter() - t0) * 1e3)
+        ts.sort()
+        out[name] = {"ms": round(ts[len(ts) // 2], 3), "images/s": round(images / ts[len(ts) // 2] * 1e3, 1),
+                     "note": "graph build + host feeds + evaluation through libag_host.so, wall clock"}
+    return out
 
 
 if __name__ == "__main__":
