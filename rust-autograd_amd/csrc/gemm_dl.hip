@@ -154,14 +154,46 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     struct Item {
         int m0, n0, bz, sp, kb0, nt;
     };
-    auto decode = [&](unsigned w) {
-        const unsigned lb = xcd_remap(w, total);
-        const unsigned z = lb / tiles, t_in = lb % tiles;
+    // Item w has the logical position xcd_remap(w) = (z * tiles_n + tn) * tiles_m + tm.  The block
+    // walks items blockIdx.x, blockIdx.x + gridDim.x, ...; with the grid a multiple of the XCD
+    // count (the host sees to it) the logical position advances by gridDim.x / 8 every time, so
+    // the (tm, tn, z) digits are stepped with a few scalar adds instead of being divided out
+    // again for every item.
+    struct Cursor {
+        int tm, tn, z;
+    };
+    Cursor step, first;
+    {
+        const unsigned stride = gridDim.x / kXcds;
+        step.tm = (int)(stride % (unsigned)p.tiles_m);
+        step.tn = (int)(stride / (unsigned)p.tiles_m % (unsigned)p.tiles_n);
+        step.z = (int)(stride / tiles);
+        unsigned g = xcd_remap(blockIdx.x, total);
+        first.tm = (int)(g % (unsigned)p.tiles_m);
+        g /= (unsigned)p.tiles_m;
+        first.tn = (int)(g % (unsigned)p.tiles_n);
+        first.z = (int)(g / (unsigned)p.tiles_n);
+    }
+    auto cursor_next = [&](Cursor &c) {
+        c.tm += step.tm;
+        const int carry_m = c.tm >= p.tiles_m;
+        c.tm -= carry_m ? p.tiles_m : 0;
+        c.tn += step.tn + carry_m;
+        const int carry_n = c.tn >= p.tiles_n;
+        c.tn -= carry_n ? p.tiles_n : 0;
+        c.z += step.z + carry_n;
+    };
+    auto item_of = [&](const Cursor &c) {
         Item it;
-        it.m0 = (int)(t_in % p.tiles_m) * BM;
-        it.n0 = (int)(t_in / p.tiles_m) * BN;
-        it.bz = (int)(z / p.splits);
-        it.sp = (int)(z % p.splits);
+        it.m0 = c.tm * BM;
+        it.n0 = c.tn * BN;
+        if (p.splits == 1) {
+            it.bz = c.z;
+            it.sp = 0;
+        } else {
+            it.bz = c.z / p.splits;
+            it.sp = c.z % p.splits;
+        }
         it.kb0 = it.sp * p.kb_per_split;
         it.nt = (min(p.kbatch, it.kb0 + p.kb_per_split) - it.kb0) * kt_per;
         return it;
@@ -175,8 +207,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     LoadB ldr_b;
     const float *pa = nullptr, *pb = nullptr;  // origin of the next k tile to fetch
     int fkt = 0, f_left = 0;
+    Cursor fcur = first;
     auto f_begin = [&]() {
-        const Item it = decode(fw);
+        const Item it = item_of(fcur);
         ldr_a.init(lda, it.m0, p.M, wave, lane);
         ldr_b.init(ldb, it.n0, p.N, wave, lane);
         pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
@@ -188,7 +221,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         if (--f_left == 0) {
             fw += gridDim.x;
             f_valid = fw < total;
-            if (f_valid) f_begin();
+            if (f_valid) {
+                cursor_next(fcur);
+                f_begin();
+            }
         } else if (++fkt == kt_per) {
             fkt = 0;
             pa += wrap_a;
@@ -287,8 +323,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 for (int j = 0; j < NI; ++j) {
                     float *dst = Cb + (long long)(row_base + i * 32) * ldc + col_base + j * 32;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        dst[(long long)(8 * (v / 4) + (v % 4)) * ldc] = alpha * acc[i][j][v];
+                    for (int v = 0; v < 16; ++v)  // written once, read by a later kernel: streaming stores
+                        st_stream(dst + (long long)(8 * (v / 4) + (v % 4)) * ldc, alpha * acc[i][j][v]);
                 }
             return true;
         } else {
@@ -365,7 +401,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     else wait_loads_then_barrier<0>();
 
     unsigned cw = blockIdx.x;
-    Item ci = decode(cw);
+    Cursor ccur = first;
+    Item ci = item_of(ccur);
     const float *cur = lds;  // ring slot being multiplied
     const float *const ring_end = lds + STAGES * TILE;
     read_frags(cur, 0, af[0], bf[0]);
@@ -405,7 +442,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         if (last_item) break;
         after_epilogue = counted;
         cw += gridDim.x;
-        ci = decode(cw);
+        cursor_next(ccur);
+        ci = item_of(ccur);
     }
 }
 
@@ -417,7 +455,8 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
     if (ka == KA_ && kb == KB_) {                                                                     \
         auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_>;                                 \
         long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \
-        if (g > p.total_blocks) g = p.total_blocks;                                                   \
+        if (g >= p.total_blocks) g = p.total_blocks;        /* one item per block */                 \
+        else g = g >= kXcds ? g - g % kXcds : kXcds;         /* the kernel steps items by grid / 8 */ \
         hipLaunchKernelGGL(kern, dim3((unsigned)g), dim3(NT), 0, st, p);                              \
         return;                                                                                       \
     }
