@@ -617,11 +617,20 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.alpha = c.alpha; p.beta = c.beta;
     p.sCsplit = (long long)c.M * c.N;
 
-    int cfg = choose_cfg(c.M, c.N, c.K, (long long)c.batch * p.splits, c.kbatch > 1, direct_ok(c));
+    // Independent batches that share A and are n-contiguous in B and C can be laid side by side
+    // along n (direct-to-LDS kernel): N = batch * n is then tiled without padding every batch.
+    const bool foldable = direct_ok(c) && c.batch > 1 && p.splits == 1 && c.kbatch == 1 && c.sA == 0 &&
+                          !c.transB && c.N % 4 == 0 && (long long)c.N * c.batch < 0x7fffffffLL &&
+                          c.sB < (1LL << 30) && c.sB % 4 == 0;
+    int cfg = choose_cfg(c.M, foldable ? c.N * c.batch : c.N, c.K, foldable ? 1 : (long long)c.batch * p.splits,
+                         c.kbatch > 1, direct_ok(c));
     if (cfg >= kFirstDirectCfg && !direct_ok(c)) cfg = 0;  // a forced configuration that cannot run
+    const bool fold = foldable && cfg >= kFirstDirectCfg && c.N >= kCfgs[cfg].bn;
+    p.n_img = fold ? c.N : 0;
+    if (fold) p.N = c.N * c.batch;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
-    p.tiles_n = (int)cdiv(c.N, kCfgs[cfg].bn);
-    const long long blocks = (long long)p.tiles_m * p.tiles_n * c.batch * p.splits;
+    p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
+    const long long blocks = (long long)p.tiles_m * p.tiles_n * (fold ? 1 : c.batch) * p.splits;
     AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "%s: too many tiles (%lld)", who, blocks);
     p.total_blocks = (unsigned)blocks;
 

@@ -82,6 +82,28 @@ struct DirectTile {
             }
         }
     }
+    // Folded batch (m/n-contiguous operand only): the tile starts at column r0 of one batch and
+    // may run on into the next one, `next` elements further (0 when there is no next batch: those
+    // columns are clamped like any column beyond the operand).
+    __device__ inline void init_folded(int ld, int r0, int n_img, unsigned next, int wave, int lane)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int pos = (i * NW + wave) * 64 + lane;
+            const int k = pos / CPR, cn = (pos % CPR) ^ (((k >> 2) & 1) * 8);
+            int n = r0 + cn * 4;
+            unsigned extra = 0;
+            if (n >= n_img) {
+                if (next != 0) {
+                    n -= n_img;
+                    extra = next;
+                } else {
+                    n = n_img - 4;
+                }
+            }
+            off[i] = ((unsigned)(k * ld + n) + extra) * 4u;
+        }
+    }
     __device__ static inline long long k_step(int ld) { return KC ? BK : (long long)BK * ld; }
 
     // Load number `i` (a constant after unrolling) of this wave.
@@ -153,6 +175,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 
     struct Item {
         int m0, n0, bz, sp, kb0, nt;
+        int r0;  // folded batch: n0 = bz * n_img + r0
     };
     // Item w has the logical position xcd_remap(w) = (z * tiles_n + tn) * tiles_m + tm.  The block
     // walks items blockIdx.x, blockIdx.x + gridDim.x, ...; with the grid a multiple of the XCD
@@ -187,7 +210,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         Item it;
         it.m0 = c.tm * BM;
         it.n0 = c.tn * BN;
-        if (p.splits == 1) {
+        it.r0 = 0;
+        if (p.n_img != 0) {
+            it.bz = it.n0 / p.n_img;
+            it.r0 = it.n0 - it.bz * p.n_img;
+            it.sp = 0;
+        } else if (p.splits == 1) {
             it.bz = c.z;
             it.sp = 0;
         } else {
@@ -211,7 +239,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
         ldr_a.init(lda, it.m0, p.M, wave, lane);
-        ldr_b.init(ldb, it.n0, p.N, wave, lane);
+        if (!KB && p.n_img != 0) {
+            const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
+            ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
+        } else {
+            ldr_b.init(ldb, it.n0, p.N, wave, lane);
+        }
         pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
         pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
         fkt = 0;
@@ -315,13 +348,19 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         }
         const bool full = it.m0 + BM <= p.M && it.n0 + BN <= p.N;
         const int row_base = it.m0 + wm * WM + 4 * half;
-        const int col_base = it.n0 + wn * WN + l31;
+        // column inside batch it.bz; a folded tile may run on into the next batch, whose columns
+        // sit sC - n_img elements further
+        const int col_base = (p.n_img != 0 ? it.r0 : it.n0) + wn * WN + l31;
+        const int col_end = p.n_img != 0 ? p.n_img : p.N;
+        const long long next_img = p.sC - p.n_img;
         if (full && beta == 0.f) {
+            // interior tile, overwrite: straight stores
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j) {
-                    float *dst = Cb + (long long)(row_base + i * 32) * ldc + col_base + j * 32;
+                    const int col = col_base + j * 32;
+                    float *dst = Cb + (long long)(row_base + i * 32) * ldc + col + (col >= col_end ? next_img : 0);
 #pragma unroll
                     for (int v = 0; v < 16; ++v)  // written once, read by a later kernel: streaming stores
                         st_stream(dst + (long long)(8 * (v / 4) + (v % 4)) * ldc, alpha * acc[i][j][v]);
@@ -333,11 +372,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 #pragma unroll
                 for (int j = 0; j < NI; ++j) {
                     const int col = col_base + j * 32;
+                    // beyond the operand: past N, or (folded) past the last batch
+                    const bool col_ok = p.n_img != 0 ? it.n0 + wn * WN + l31 + j * 32 < p.N : col < p.N;
+                    const long long shift = col >= col_end ? next_img : 0;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
-                        if (row < p.M && col < p.N) {
-                            float *dst = Cb + (long long)row * ldc + col;
+                        if (row < p.M && col_ok) {
+                            float *dst = Cb + (long long)row * ldc + col + shift;
                             const float r = alpha * acc[i][j][v];
                             *dst = beta == 0.f ? r : r + beta * *dst;
                         }

@@ -24,6 +24,10 @@ struct GemmParams {
     float alpha, beta;
     int tiles_m, tiles_n;
     unsigned total_blocks;
+    // Folded batch (direct-to-LDS kernel only): A shared by all batches and B, C n-contiguous, so
+    // the batches are laid side by side along n -- column g of the folded problem is column
+    // g % n_img of batch g / n_img -- and N = batch * n_img is tiled without padding every batch.
+    int n_img;  // 0 = not folded
 };
 
 constexpr int kXcds = 8;

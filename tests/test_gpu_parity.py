@@ -222,6 +222,33 @@ def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb):
         assert_close(host(c), truth, f"direct gemm {m}x{n}x{k}x{batch}")
 
 
+@pytest.mark.parametrize("tb", [0, 1])
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("cfg", DIRECT_CFGS + [-1])
+def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
+    """A shared by all batches (stride 0, the conv filter matrix): with B and C n-contiguous the
+    batches are tiled side by side along n, so tiles straddle two batches and the last tile runs
+    past the last batch; with B transposed the batches stay separate.  alpha / beta included."""
+    L = K.capi.lib()
+    for (m, n, k, batch, beta) in ((128, 300, 64, 7, 0.0), (200, 260, 32, 3, 0.0), (192, 512, 96, 4, 0.0),
+                                   (64, 296, 64, 5, -0.5)):
+        a = rng.random((k, m) if ta else (m, k), dtype=np.float32)
+        b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
+        c0 = rng.random((batch, m, n), dtype=np.float32)
+        say("gemm folded cfg", cfg, ta, tb, m, n, k, batch, beta)
+        c = dev(c0)
+        L.ag_gemm_force_config(cfg)
+        try:
+            K.gemm(ta, tb, m, n, k, 2.0, dev(a), a.shape[1], 0, dev(b), b.shape[2], b.shape[1] * b.shape[2], beta, c, n,
+                   m * n, batch)
+        finally:
+            L.ag_gemm_force_config(-1)
+        A = a.T if ta else a
+        Bm = b.transpose(0, 2, 1) if tb else b
+        truth = 2.0 * (A.astype(np.float64)[None] @ Bm.astype(np.float64)) + beta * c0
+        assert_close(host(c), truth, f"folded gemm {m}x{n}x{k}x{batch}")
+
+
 @pytest.mark.parametrize("cfg", DIRECT_CFGS)
 def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg):
     """The filter-gradient form (sum over images, split into a workspace and folded) and the
