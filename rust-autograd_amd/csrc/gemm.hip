@@ -413,6 +413,9 @@ static int num_cus()
     return cus;
 }
 
+// Blocks of the direct-to-LDS kernel's persistent grid: one per CU, a multiple of the XCD count.
+static long long direct_grid(int cus) { return cus >= kXcds ? cus - cus % kXcds : kXcds; }
+
 template <typename Kern>
 static int resident_blocks(Kern kern, int threads, int fallback)
 {
@@ -456,7 +459,7 @@ static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
                                 {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
                                 {128, 128}, {192, 128}, {128, 64},
-                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}};
+                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
@@ -628,11 +631,48 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     const bool fold = foldable && cfg >= kFirstDirectCfg && c.N >= kCfgs[cfg].bn;
     p.n_img = fold ? c.N : 0;
     if (fold) p.N = c.N * c.batch;
+    p.n_off = 0;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * (fold ? 1 : c.batch) * p.splits;
     AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "%s: too many tiles (%lld)", who, blocks);
     p.total_blocks = (unsigned)blocks;
+
+    // A persistent grid of G blocks takes ceil(items / G) rounds; when the last round would be
+    // mostly idle (12.25 rounds at the headline forward shape) the folded problem is cut in two
+    // launches: whole rounds of the chosen tile, then the remaining columns with a narrower tile
+    // (128 x 64 or 128 x 128) that fills the chip once more for a fraction of a round.
+    int tail_cfg = -1;
+    GemmParams tail = p;
+    if (fold && g_force_cfg < 0 && kCfgs[cfg].bm == 128 && p.tiles_m == 1) {
+        const long long G = direct_grid(num_cus());
+        const long long rounds = blocks / G, rem = blocks % G;
+        if (rounds >= 1 && rem > 0) {
+            const int bn = kCfgs[cfg].bn;
+            const long long main_cols = rounds * G * bn;
+            double best = (double)rounds + 1.0 - 0.05;
+            static const int narrow[] = {18, 13};  // 128 x 64, 128 x 128
+            static const double eff[] = {0.85, 0.92};
+            for (int t = 0; t < 2; ++t) {
+                const int bnt = kCfgs[narrow[t]].bn;
+                if (bnt >= bn) continue;
+                const long long items = cdiv(p.N - main_cols, bnt);
+                const double cost = (double)rounds + (double)cdiv(items, G) * bnt / bn / eff[t];
+                if (cost < best) {
+                    best = cost;
+                    tail_cfg = narrow[t];
+                }
+            }
+            if (tail_cfg >= 0) {
+                tail.n_off = (int)main_cols;
+                tail.tiles_n = (int)cdiv(p.N - main_cols, kCfgs[tail_cfg].bn);
+                tail.total_blocks = (unsigned)tail.tiles_n;
+                p.N = (int)main_cols;
+                p.tiles_n = (int)(rounds * G);
+                p.total_blocks = (unsigned)p.tiles_n;
+            }
+        }
+    }
 
     float *real_c = c.C;
     if (p.splits > 1) {
@@ -648,6 +688,10 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (cfg >= kFirstDirectCfg) launch_direct(st, cfg, !c.transA, c.transB != 0, p, num_cus(), g_grid_scale);
     else launch(st, cfg, la, lb, p);
     if (ag_status_t s = check_launch(who)) return s;
+    if (tail_cfg >= 0) {
+        launch_direct(st, tail_cfg, !c.transA, c.transB != 0, tail, num_cus(), g_grid_scale);
+        if (ag_status_t s = check_launch(who)) return s;
+    }
     if (p.splits > 1) {
         const long long total = (long long)c.M * c.N;
         hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),

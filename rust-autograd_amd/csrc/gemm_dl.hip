@@ -209,7 +209,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     auto item_of = [&](const Cursor &c) {
         Item it;
         it.m0 = c.tm * BM;
-        it.n0 = c.tn * BN;
+        it.n0 = p.n_off + c.tn * BN;
         it.r0 = 0;
         if (p.n_img != 0) {
             it.bz = it.n0 / p.n_img;
@@ -517,7 +517,8 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
         case 14: launch_dl<128, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 15: launch_dl<256, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        default: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        default: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
     }
 }
 

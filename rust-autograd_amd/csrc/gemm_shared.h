@@ -28,6 +28,7 @@ struct GemmParams {
     // the batches are laid side by side along n -- column g of the folded problem is column
     // g % n_img of batch g / n_img -- and N = batch * n_img is tiled without padding every batch.
     int n_img;  // 0 = not folded
+    int n_off;  // folded: first column of this launch (a launch may cover a column range only)
 };
 
 constexpr int kXcds = 8;

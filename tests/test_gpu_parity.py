@@ -196,7 +196,7 @@ def test_gemm_every_tile_configuration(K, rng, cfg):
     assert_close(got_t, truth, "gemm TT")
 
 
-DIRECT_CFGS = list(range(13, 18))  # operand tiles loaded from global memory straight into LDS
+DIRECT_CFGS = list(range(13, 19))  # operand tiles loaded from global memory straight into LDS
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
@@ -230,8 +230,12 @@ def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
     batches are tiled side by side along n, so tiles straddle two batches and the last tile runs
     past the last batch; with B transposed the batches stay separate.  alpha / beta included."""
     L = K.capi.lib()
-    for (m, n, k, batch, beta) in ((128, 300, 64, 7, 0.0), (200, 260, 32, 3, 0.0), (192, 512, 96, 4, 0.0),
-                                   (64, 296, 64, 5, -0.5)):
+    shapes = [(128, 300, 64, 7, 0.0), (200, 260, 32, 3, 0.0), (192, 512, 96, 4, 0.0), (64, 296, 64, 5, -0.5)]
+    if cfg == -1:
+        # more tiles than the persistent grid has blocks: whole rounds, then a narrow-tile launch
+        # for the remaining columns, which starts in the middle of a batch
+        shapes.append((128, 3136, 32, 24, 0.0))
+    for (m, n, k, batch, beta) in shapes:
         a = rng.random((k, m) if ta else (m, k), dtype=np.float32)
         b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
         c0 = rng.random((batch, m, n), dtype=np.float32)
