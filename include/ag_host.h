@@ -38,6 +38,9 @@ int agh_env_set(agh_env *env, const char *ns, const char *name, const float *dat
 int agh_env_find(agh_env *env, const char *ns, const char *name);
 int agh_env_shape(agh_env *env, int var_id, int64_t *shape_out, int max_rank); /* returns the rank */
 int agh_env_read(agh_env *env, int var_id, float *out, size_t n);
+/* Overwrites the variable's array in place (same element count), as writing through
+ * env.get_array_by_id(id).borrow_mut() does (src/variable.rs:695-703). */
+int agh_env_write(agh_env *env, int var_id, const float *data, size_t n);
 
 /* ---- graph construction (one context = one `env.run(|ctx| ...)` closure) --------------------- */
 agh_ctx *agh_ctx_new(agh_env *env);
@@ -63,6 +66,8 @@ int agh_sparse_softmax_cross_entropy(agh_ctx *ctx, int logits, int labels);
 int agh_stop_gradient(agh_ctx *ctx, int x);
 /* tensor_ops::grad(ys, xs): writes nx tensor ids to out. */
 int agh_grad(agh_ctx *ctx, const int *ys, int ny, const int *xs, int nx, int *out);
+/* tensor_ops::grad_with_default(ys, xs, ys_grads): ys_grads[i] is the known gradient of ys[i]. */
+int agh_grad_with_default(agh_ctx *ctx, const int *ys, const int *ys_grads, int ny, const int *xs, int nx, int *out);
 /* optimizers::grad_helper(losses, namespace): returns the number of (variable, gradient) pairs. */
 int agh_grad_helper(agh_ctx *ctx, const int *losses, int n, const char *ns, int *vars_out, int *grads_out, int max_out);
 

@@ -67,6 +67,7 @@ class NdArray {
     NdArray reshaped(const Shape &shape) const;  // same storage, new extents (len must match)
     NdArray deep_copy() const;
     std::vector<float> to_host() const;  // synchronises the stream
+    void copy_from_host(const float *data);  // overwrites the elements in place; synchronises
 
   private:
     Shape shape_;
@@ -296,6 +297,8 @@ Tensor scalar(float v, Graph *g);
 Tensor zeros_like(Tensor x);      // zeros(shape(x)): what grad() returns for a non-differentiable x
 Tensor stop_gradient(Tensor x);
 std::vector<Tensor> grad(const std::vector<Tensor> &ys, const std::vector<Tensor> &xs);   // :94
+std::vector<Tensor> grad_with_default(const std::vector<Tensor> &ys, const std::vector<Tensor> &xs,
+                                      const std::vector<Tensor> &ys_grads);                  // :130
 }  // namespace tensor_ops
 
 // ---------------------------------------------------------------------------------------------

@@ -79,6 +79,16 @@ int agh_env_read(agh_env *env, int var_id, float *out, size_t n)
     });
 }
 
+int agh_env_write(agh_env *env, int var_id, const float *data, size_t n)
+{
+    return guard([&] {
+        NdArray &a = env->env.array(var_id);
+        if (a.len() != n) throw Panic("agh_env_write: element count differs");
+        a.copy_from_host(data);
+        return 0;
+    });
+}
+
 agh_ctx *agh_ctx_new(agh_env *env) { return new agh_ctx(&env->env); }
 void agh_ctx_free(agh_ctx *ctx) { delete ctx; }
 
@@ -158,6 +168,21 @@ int agh_grad(agh_ctx *c, const int *ys, int ny, const int *xs, int nx, int *out)
         for (int i = 0; i < ny; ++i) y.push_back(T(c, ys[i]));
         for (int i = 0; i < nx; ++i) x.push_back(T(c, xs[i]));
         const std::vector<Tensor> g = tensor_ops::grad(y, x);
+        for (int i = 0; i < nx; ++i) out[i] = g[(size_t)i].id;
+        return 0;
+    });
+}
+
+int agh_grad_with_default(agh_ctx *c, const int *ys, const int *ys_grads, int ny, const int *xs, int nx, int *out)
+{
+    return guard([&] {
+        std::vector<Tensor> y, gy, x;
+        for (int i = 0; i < ny; ++i) {
+            y.push_back(T(c, ys[i]));
+            gy.push_back(T(c, ys_grads[i]));
+        }
+        for (int i = 0; i < nx; ++i) x.push_back(T(c, xs[i]));
+        const std::vector<Tensor> g = tensor_ops::grad_with_default(y, x, gy);
         for (int i = 0; i < nx; ++i) out[i] = g[(size_t)i].id;
         return 0;
     });

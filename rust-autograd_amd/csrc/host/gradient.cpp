@@ -72,13 +72,16 @@ struct HeapNode {
     bool operator<(const HeapNode &o) const { return topo_rank < o.topo_rank; }  // max-heap by rank
 };
 
-GradientMap compute_gradients(Graph &g, const std::vector<Tensor> &ys, const std::vector<Tensor> &xs)
+// `gys`: already known gradients of `ys` (gradient.rs:36-50); null = a scalar one for every y.
+GradientMap compute_gradients(Graph &g, const std::vector<Tensor> &ys, const std::vector<Tensor> &xs,
+                              const std::vector<Tensor> *gys = nullptr)
 {
     GradientMap map = init_gradient_map(g, ys, xs);
-    const Tensor start_gy = tensor_ops::scalar(1.f, &g);
+    if (gys && gys->size() != ys.size()) throw Panic("grad_with_default: ys and ys_grads differ in length");
     std::priority_queue<HeapNode> heap;
-    for (const Tensor &y : ys) {
-        map.at(y.id).gradients.push_back(start_gy);
+    for (size_t i = 0; i < ys.size(); ++i) {
+        const Tensor &y = ys[i];
+        map.at(y.id).gradients.push_back(gys ? (*gys)[i] : tensor_ops::scalar(1.f, &g));
         heap.push(HeapNode{y.id, g.node(y.id).topo_rank});
     }
     while (!heap.empty()) {
@@ -123,6 +126,24 @@ std::vector<Tensor> grad(const std::vector<Tensor> &ys, const std::vector<Tensor
             ret.push_back(it->second.gradient());
         else
             ret.push_back(zeros_like(x));  // not differentiable (mod.rs:108-111)
+    }
+    return ret;
+}
+
+std::vector<Tensor> grad_with_default(const std::vector<Tensor> &ys, const std::vector<Tensor> &xs,
+                                      const std::vector<Tensor> &ys_grads)
+{
+    // mod.rs:130-153: no sum_all wrapping, the given gradients start the back-propagation
+    if (ys.empty()) throw Panic("grad_with_default: no ys");
+    Graph &g = *ys[0].graph;
+    GradientMap map = compute_gradients(g, ys, xs, &ys_grads);
+    std::vector<Tensor> ret;
+    for (const Tensor &x : xs) {
+        auto it = map.find(x.id);
+        if (it != map.end() && it->second.on_backprop_path && !it->second.gradients.empty())
+            ret.push_back(it->second.gradient());
+        else
+            ret.push_back(zeros_like(x));
     }
     return ret;
 }

@@ -798,7 +798,8 @@ struct ReshapeLike : Op {  // gradient of Reshape: back to the extents of input 
     }
     void grad(GradientContext &ctx) const override
     {
-        ctx.append_input_grad(std::nullopt);
+        // a reshape again (array_ops.rs:226-238); the input that only lends its extents gets none
+        ctx.append_input_grad(build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReshapeLike>()));
         ctx.append_input_grad(std::nullopt);
     }
 };

@@ -121,6 +121,15 @@ NdArray NdArray::from_host(const Shape &shape, const float *data)
     return a;
 }
 
+void NdArray::copy_from_host(const float *data)
+{
+    if (len())
+        check(hipMemcpyAsync(ptr(), data, len() * sizeof(float), hipMemcpyHostToDevice,
+                             static_cast<hipStream_t>(current_stream())),
+              "hipMemcpy H2D");
+    synchronize();
+}
+
 NdArray NdArray::reshaped(const Shape &shape) const
 {
     if (product(shape) != len()) throw Panic("NdArray::reshaped: element count differs");

@@ -28,6 +28,7 @@ PROTOTYPES = {
     "agh_env_find": (_i, [_p, _s, _s]),
     "agh_env_shape": (_i, [_p, _i, _lp, _i]),
     "agh_env_read": (_i, [_p, _i, _fp, _z]),
+    "agh_env_write": (_i, [_p, _i, _fp, _z]),
     "agh_ctx_new": (_p, [_p]),
     "agh_ctx_free": (None, [_p]),
     "agh_variable": (_i, [_p, _i]),
@@ -50,6 +51,7 @@ PROTOTYPES = {
     "agh_sparse_softmax_cross_entropy": (_i, [_p, _i, _i]),
     "agh_stop_gradient": (_i, [_p, _i]),
     "agh_grad": (_i, [_p, _ip, _i, _ip, _i, _ip]),
+    "agh_grad_with_default": (_i, [_p, _ip, _ip, _i, _ip, _i, _ip]),
     "agh_grad_helper": (_i, [_p, _ip, _i, _s, _ip, _ip, _i]),
     "agh_num_nodes": (_i, [_p]),
     "agh_op_name": (_s, [_p, _i]),
@@ -133,6 +135,11 @@ class VariableEnvironment:
         out = np.empty([buf[i] for i in range(rank)], dtype=np.float32)
         _check(lib().agh_env_read(self._h, var_id, out.ctypes.data_as(_fp), out.size))
         return out
+
+    def write(self, var_id, array):
+        """Overwrites a variable in place (what `get_array_by_id(id).borrow_mut()` is used for)."""
+        a = _f32(array)
+        _check(lib().agh_env_write(self._h, var_id, a.ctypes.data_as(_fp), a.size))
 
     def context(self):
         return Context(self)
@@ -272,6 +279,14 @@ class Context:
         xi, nx = _ints(t.id for t in xs)
         out = (C.c_int * max(nx, 1))()
         _check(lib().agh_grad(self._h, yi, ny, xi, nx, out))
+        return [self._t(out[i]) for i in range(nx)]
+
+    def grad_with_default(self, ys, xs, ys_grads):
+        yi, ny = _ints(t.id for t in ys)
+        gi, _ = _ints(t.id for t in ys_grads)
+        xi, nx = _ints(t.id for t in xs)
+        out = (C.c_int * max(nx, 1))()
+        _check(lib().agh_grad_with_default(self._h, yi, gi, ny, xi, nx, out))
         return [self._t(out[i]) for i in range(nx)]
 
     def grad_helper(self, losses, namespace=""):

@@ -428,3 +428,138 @@ def test_variables_are_shared_between_contexts_and_updated_in_place(G, orc, rng)
         assert_close(env.array(wid), p, f"Adam step {step}")
     # with a constant-sign gradient Adam moves every element by about alpha per step
     assert np.abs(env.array(wid) - (wv - 1.0)).max() < 0.05
+
+
+# ------------------------------------------------------------------------------- the reference's own gradient tests
+def check_theoretical_grads(G, env, c, objective, gradients, var_ids, eps=1e-2, tol=2e-2):
+    """src/test_helper.rs:9-140: the analytic gradients of sum_all(objective) w.r.t. shared variables
+    against central differences obtained by rewriting the variable in place and re-evaluating the
+    same graph.  The reference runs this in f64 with eps 1e-3 / tol 1e-2; in f32 the step is ten
+    times larger so that rounding of the objective (about 1e-6 relative) stays below the tolerance."""
+    obj = c.sum_all(objective)
+    th = c.eval(gradients)
+    for vid, g_th in zip(var_ids, th):
+        assert not isinstance(g_th, G.OpError), g_th
+        base = env.array(vid)
+        flat = base.reshape(-1)
+        assert g_th.size == flat.size
+        for i in range(flat.size):
+            vals = []
+            for sgn in (+1.0, -1.0):
+                pert = flat.copy()
+                pert[i] += sgn * eps
+                env.write(vid, pert.reshape(base.shape))
+                vals.append(float(c.eval([obj])[0]))
+            env.write(vid, base)
+            g_num = (vals[0] - vals[1]) / (2 * eps)
+            assert abs(g_num - float(g_th.reshape(-1)[i])) <= tol * max(1.0, abs(g_num)), (
+                f"gradient check: numerical={g_num}, theoretical={g_th.reshape(-1)[i]} at element {i}")
+
+
+def ref_env(G, rng, shapes):
+    env = G.VariableEnvironment()
+    ids = [env.set(f"v{i}", rng.standard_normal(s).astype(np.float32)) for i, s in enumerate(shapes)]
+    return env, ids
+
+
+def test_ref_conv2d_transpose(G, rng):                      # tests/test_tensor_ops_grad.rs:1358
+    env, (xi, wi) = ref_env(G, rng, [(3, 2, 2, 2), (2, 3, 2, 2)])
+    c = env.context()
+    x, w = c.variable(xi), c.variable(wi)
+    y = c.conv2d_transpose(x, w, 0, 1)
+    check_theoretical_grads(G, env, c, y, c.grad([y], [w]), [wi])
+
+
+def test_ref_conv2d_transpose_filter_grad(G, rng):          # :1374 (second order; the answer is zero)
+    env, (xi, wi) = ref_env(G, rng, [(2, 2, 2, 2), (2, 3, 2, 2)])
+    c = env.context()
+    x, w = c.variable(xi), c.variable(wi)
+    y = c.conv2d_transpose(x, w, 0, 1)
+    g = c.grad([y], [w])[0]
+    check_theoretical_grads(G, env, c, g, c.grad([g], [w]), [wi])
+
+
+def test_ref_conv2d_filter_grad(G, rng):                    # :1399 (second order; the answer is zero)
+    env, (xi, wi) = ref_env(G, rng, [(2, 3, 5, 5), (2, 3, 2, 2)])
+    c = env.context()
+    x, w = c.variable(xi), c.variable(wi)
+    y = c.conv2d(x, w, 0, 1)
+    g = c.grad([y], [w])[0]
+    check_theoretical_grads(G, env, c, g, c.grad([g], [w]), [wi])
+
+
+def test_ref_conv2d_grad(G, rng):                           # :1423 grad_with_default, then w.r.t. gy
+    env, (xi, wi) = ref_env(G, rng, [(2, 3, 5, 5), (2, 3, 2, 2)])
+    # The reference feeds ones of shape [2,2,2,2] although y is [2,2,4,4]; its input gradient then
+    # has the extent rebuilt from gy (3x3).  Here the gradient takes x's extent, so gy has y's shape.
+    gyi = env.set("gy", np.ones((2, 2, 4, 4), np.float32))
+    c = env.context()
+    x, w, gy = c.variable(xi), c.variable(wi), c.variable(gyi)
+    y = c.conv2d(x, w, 0, 1)
+    g = c.grad_with_default([y], [x], [gy])[0]
+    check_theoretical_grads(G, env, c, g, [c.grad([g], [gy])[0]], [gyi])
+
+
+def test_ref_conv2d_xw_grad(G, rng):                        # :1449 d(filter grad)/dx
+    env, (xi, wi) = ref_env(G, rng, [(2, 3, 5, 5), (2, 3, 2, 2)])
+    c = env.context()
+    x, w = c.variable(xi), c.variable(wi)
+    y = c.conv2d(x, w, 0, 1)
+    g = c.grad([y], [w])[0]
+    check_theoretical_grads(G, env, c, g, c.grad([g], [x]), [xi])
+
+
+def test_ref_conv2d(G, rng):                                # :1473 pad 1, stride 2
+    env, (xi, wi) = ref_env(G, rng, [(2, 3, 5, 5), (2, 3, 3, 3)])
+    c = env.context()
+    x, w = c.variable(xi), c.variable(wi)
+    y = c.conv2d(x, w, 1, 2)
+    check_theoretical_grads(G, env, c, y, c.grad([y], [x, w]), [xi, wi])
+
+
+def test_ref_max_pool2d(G):                                 # :1496
+    env = G.VariableEnvironment()
+    xi = env.set("x", np.linspace(0.0, 1.0, 9, dtype=np.float32))
+    c = env.context()
+    x = c.variable(xi)
+    y = c.max_pool2d(c.reshape(x, [1, 1, 3, 3]), 2, 0, 1)
+    check_theoretical_grads(G, env, c, y, c.grad([y], [x]), [xi])
+
+
+def test_ref_max_pool2d_grad(G):                            # :1508 runs MaxPool2DGradGrad
+    env = G.VariableEnvironment()
+    xi = env.set("x", np.linspace(0.0, 1.0, 36, dtype=np.float32))
+    gyi = env.set("gy", np.linspace(0.0, 1.0, 16, dtype=np.float32).reshape(2, 2, 2, 2))
+    c = env.context()
+    x, gy = c.variable(xi), c.variable(gyi)
+    y = c.max_pool2d(c.reshape(x, [2, 2, 3, 3]), 2, 0, 1)
+    g = c.grad_with_default([y], [x], [gy])[0]
+    check_theoretical_grads(G, env, c, g, [c.grad([g], [gy])[0]], [gyi])
+
+
+def test_ref_matmul_and_batch_matmul(G, rng):               # :457, :479
+    env, (ai, bi) = ref_env(G, rng, [(4, 2), (2, 3)])
+    c = env.context()
+    a, b = c.variable(ai), c.variable(bi)
+    z = c.matmul(a, b)
+    check_theoretical_grads(G, env, c, z, c.grad([z], [a, b]), [ai, bi])
+    env, (ai, bi) = ref_env(G, rng, [(2, 4, 2), (2, 2, 3)])
+    c = env.context()
+    a, b = c.variable(ai), c.variable(bi)
+    z = c.batch_matmul(a, b)
+    check_theoretical_grads(G, env, c, z, c.grad([z], [a, b]), [ai, bi])
+
+
+def test_ref_reduce_and_wx_plus_b(G, rng):                  # :523, :627-:690
+    env, (xi,) = ref_env(G, rng, [(3, 2, 3)])
+    for keep in (False, True):
+        for op in ("reduce_mean", "reduce_sum"):
+            c = env.context()
+            x = c.variable(xi)
+            z = getattr(c, op)(x, [1], keep)
+            check_theoretical_grads(G, env, c, z, c.grad([z], [x]), [xi])
+    env, (xi, wi, bi) = ref_env(G, rng, [(2, 3), (3, 4), (1, 4)])
+    c = env.context()
+    x, w, b = c.variable(xi), c.variable(wi), c.variable(bi)
+    z = c.matmul(x, w) + b
+    check_theoretical_grads(G, env, c, z, c.grad([z], [b]), [bi])
