@@ -185,6 +185,8 @@ def main():
     ws = torch.empty(max(16, L.ag_conv2d_filter_grad_f32_workspace(Bn, CK, P, K)), dtype=torch.uint8, device=dev)
     st, ptr, chk = Kn._stream, Kn._ptr, capi.check
     T = Timer(torch)
+    geom = (Bn, K, OH, OH, C, KH, KH, PAD, H, W)
+    assert 0 < L.ag_conv_input_grad_scratch_floats(*geom) <= gcols.numel()
 
     def step():
         T.run("im2col", lambda: chk(L.ag_im2col_f32(st(), ptr(x), ptr(cols), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
@@ -194,10 +196,10 @@ def main():
         T.run("gemm_filter_grad", lambda: chk(L.ag_gemm_batchsum_f32(st(), 0, 1, K, CK, P, 1.0, ptr(gy), P, K * P,
                                                                      ptr(cols), P, CK * P, 0.0, ptr(gw), CK, Bn,
                                                                      ptr(ws), ws.numel())))
-        T.run("gemm_input_grad", lambda: chk(L.ag_gemm_f32(st(), 1, 0, CK, P, K, 1.0, ptr(w), CK, 0, ptr(gy), P,
-                                                           K * P, 0.0, ptr(gcols), P, CK * P, Bn)))
-        T.run("col2im", lambda: chk(L.ag_col2im_f32(st(), ptr(gcols), ptr(gx), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
-                                                    STRIDE, DIL, DIL, OH, OH)))
+        # Conv2DTranspose (the input gradient): the two stages ag_conv2d_transpose_f32 runs for a
+        # stride-1 convolution, launched separately so that each gets its own events
+        T.run("input_grad_prepare", lambda: chk(L.ag_conv_input_grad_prepare_f32(st(), ptr(gy), ptr(w), ptr(gcols), *geom)))
+        T.run("gemm_input_grad", lambda: chk(L.ag_conv_input_grad_gemm_f32(st(), ptr(gcols), ptr(gx), *geom)))
 
     if args.pmc_calibration:
         src = torch.ones(1 << 28, device=dev)
@@ -224,19 +226,21 @@ def main():
     for name in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"):
         tf = gemm_flop / (per[name] * 1e-3) / 1e12
         kernels[name] = {"ms": round(per[name], 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
-    for name in ("im2col", "col2im"):
-        gbs = col_bytes / (per[name] * 1e-3) / 1e9
+    prep_bytes = 4.0 * (gy.numel() + L.ag_conv_input_grad_scratch_floats(*geom))  # read gy, write its bordered copy
+    for name, nbytes in (("im2col", col_bytes), ("input_grad_prepare", prep_bytes)):
+        gbs = nbytes / (per[name] * 1e-3) / 1e9
         kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
     if Bn == B:
         for name in kernels:
-            kernels[name]["traffic_bytes"] = round(TRAFFIC_BYTES[name])
+            if name in TRAFFIC_BYTES:
+                kernels[name]["traffic_bytes"] = round(TRAFFIC_BYTES[name])
     gemm_ms = sum(per[n] for n in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"))
     gemm_tf = 3 * gemm_flop / (gemm_ms * 1e-3) / 1e12
     dominant = max(("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"), key=lambda n: per[n])
     dom_tf = gemm_flop / (per[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(dom_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4),
-                "traffic": round(TRAFFIC_BYTES[dominant]) if Bn == B else None,
+                "traffic": round(TRAFFIC_BYTES[dominant]) if Bn == B and dominant in TRAFFIC_BYTES else None,
                 "gemm_phase_TFLOP/s": round(gemm_tf, 2),
                 "gemm_phase_frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)}
 
@@ -249,7 +253,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"C4 conv2d fwd+bwd: x [{Bn},{C},{H},{W}] N(0,1), w [{K},{C},{KH},{KH}] glorot-uniform, "
-                               f"stride {STRIDE} pad {PAD}; im2col + 3 fp32-MFMA GEMMs + col2im per step"},
+                               f"stride {STRIDE} pad {PAD}; im2col, forward GEMM, filter-gradient GEMM, column-free input-gradient GEMM per step"},
         "roofline": roofline, "kernels": kernels,
     }
     if not args.no_cpu:
@@ -273,6 +277,25 @@ def micro(torch, Kn, capi, dev):
     ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), 10)
     res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
     del x, y, am, il, gy
+
+    # the column-materialising input gradient (what the reference does per image): W^T . gy, then col2im
+    Bn, Cc, Kf, Hh = 256, 64, 128, 56
+    Pp, CKk = Hh * Hh, Cc * 9
+    L = capi.lib()
+    st, ptr, chk = Kn._stream, Kn._ptr, capi.check
+    wt = torch.randn(Kf, CKk, device=dev, generator=g) * 0.1
+    gyy = torch.randn(Bn, Kf, Pp, device=dev, generator=g)
+    gc = torch.empty(Bn, CKk, Pp, device=dev)
+    gxx = torch.empty(Bn, Cc, Hh, Hh, device=dev)
+    ms = time_events(torch, lambda: chk(L.ag_gemm_f32(st(), 1, 0, CKk, Pp, Kf, 1.0, ptr(wt), CKk, 0, ptr(gyy), Pp, Kf * Pp,
+                                                      0.0, ptr(gc), Pp, CKk * Pp, Bn)), 10)
+    tf = 2.0 * Kf * Pp * CKk * Bn / ms / 1e9
+    res["gemm_input_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    ms = time_events(torch, lambda: chk(L.ag_col2im_f32(st(), ptr(gc), ptr(gxx), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1, Hh, Hh)), 10)
+    cb = 4.0 * (gc.numel() + gxx.numel())
+    res["col2im"] = {"ms": round(ms, 4), "GB/s": round(cb / ms / 1e6, 1), "frac_hbm": round(cb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "traffic_bytes": round(TRAFFIC_BYTES["col2im"])}
+    del wt, gyy, gc, gxx
 
     # reduce_sum (to scalar) and Adam on 2^26 elements
     n = 1 << 26

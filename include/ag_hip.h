@@ -134,6 +134,21 @@ ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const f
                                     float *gcols, int B, int ych, int yh, int yw, int xch, int kh,
                                     int kw, int pad, int stride, int dilation, int xh, int xw);
 
+/* The two stages of the stride-1, dilation-1 input gradient that ag_conv2d_transpose_f32 runs
+ * when the geometry allows it (no counterpart in the reference, which always materialises the
+ * columns): `prepare` writes a zero-bordered copy of gy and the filter in tap-major order into
+ * `scratch`; `gemm` accumulates gx over the kh*kw taps in one contraction that reads them.
+ * ag_conv_input_grad_scratch_floats returns the scratch size in floats, or 0 when the geometry
+ * is not supported (then use ag_conv2d_transpose_f32). */
+size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int yw, int xch, int kh, int kw,
+                                         int pad, int xh, int xw);
+ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w,
+                                           float *scratch, int B, int ych, int yh, int yw, int xch,
+                                           int kh, int kw, int pad, int xh, int xw);
+ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch, float *gx, int B,
+                                        int ych, int yh, int yw, int xch, int kh, int kw, int pad,
+                                        int xh, int xw);
+
 /* Replaces Conv2DTransposeFilterGrad::compute -> conv2d_transpose_filter_grad_impl
  * (conv2d_transpose.rs:433-451, 303-431).  x [B,ych,yh,yw] (input of the transposed conv),
  * gy [B,xch,H,W] (gradient of its output) -> gw [ych,xch,kh,kw].  `gycols` is caller scratch of
@@ -245,6 +260,9 @@ void ag_gemm_force_config(int cfg);
 void ag_gemm_force_splits(int splits);
 /* Experiment hook: blocks per CU of the persistent GEMM grid (0 = as many as stay resident). */
 void ag_gemm_force_grid(int blocks_per_cu);
+/* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): stride-1 calls may use the
+ * implicit input-gradient GEMM, which never writes the columns. */
+void ag_conv_fused_input_grad(int on);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -92,6 +92,10 @@ PROTOTYPES = {
     "ag_gemm_force_config": (None, [c_i]),
     "ag_gemm_force_splits": (None, [c_i]),
     "ag_gemm_force_grid": (None, [c_i]),
+    "ag_conv_fused_input_grad": (None, [c_i]),
+    "ag_conv_input_grad_scratch_floats": (C.c_size_t, [c_i] * 10),
+    "ag_conv_input_grad_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 10),
+    "ag_conv_input_grad_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 10),
 }
 
 _lib = None

@@ -3,6 +3,7 @@
 // batched: one im2col launch and one strided-batched GEMM launch per operator instead of one
 // task per image, and one split-accumulation GEMM instead of an image-sequential beta=1 loop.
 #include "ag_internal.h"
+#include "gemm_shared.h"
 
 using namespace ag;
 
@@ -56,6 +57,81 @@ extern "C" ag_status_t ag_conv2d_filter_grad_f32(ag_stream_t stream, const float
                                 (long long)CK * P, 0.f, gw, CK, B, ws, ws_bytes);
 }
 
+namespace ag {
+
+static bool g_fused_input_grad = true;  // experiment hook, see ag_conv_fused_input_grad
+
+// gyp[plane][r][s] = gy[plane][r - top][s - left] inside the image, 0 in the border; four
+// consecutive elements of the flattened padded plane per thread (its extent is a multiple of 4).
+__global__ __launch_bounds__(256) void pad_border_kernel(const float *__restrict__ gy, float *__restrict__ gyp,
+                                                         long long quads, int OH, int OW, int Hp, int Wp, int top,
+                                                         int left)
+{
+    const int plane_quads = Hp * Wp / 4;
+    for (long long qd = blockIdx.x * 256LL + threadIdx.x; qd < quads; qd += gridDim.x * 256LL) {
+        const long long plane = qd / plane_quads;
+        const int e0 = (int)(qd - plane * plane_quads) * 4;
+        const float *src = gy + plane * (long long)OH * OW;
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int r = (e0 + t) / Wp, s = (e0 + t) - r * Wp;
+            const int oy = r - top, ox = s - left;
+            v[t] = ((unsigned)oy < (unsigned)OH && (unsigned)ox < (unsigned)OW) ? src[oy * OW + ox] : 0.f;
+        }
+        st_stream(reinterpret_cast<float4 *>(gyp) + qd, make_float4(v[0], v[1], v[2], v[3]));
+    }
+}
+
+// wr[c][tap][k] = w[k][c][tap]  (tap = ky*kw + kx): the filter as the k-contiguous left operand of
+// the implicit input-gradient GEMM.
+__global__ __launch_bounds__(256) void filter_taps_kernel(const float *__restrict__ w, float *__restrict__ wr, int Kf,
+                                                          int C, int taps)
+{
+    const int total = Kf * C * taps;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int k = e % Kf, tap = e / Kf % taps, c = e / (Kf * taps);
+        wr[e] = w[((long long)k * C + c) * taps + tap];
+    }
+}
+
+// Geometry of the implicit (column-free) stride-1 input gradient.
+struct FusedGeom {
+    int Hp, Wp;
+    long long gyp_floats, wr_floats;  // scratch layout: zero-bordered gy, then the tap-major filter
+};
+
+// False when the geometry does not allow the implicit path.
+static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad, int xh, int xw, FusedGeom *g)
+{
+    if (pad > kh - 1 || pad > kw - 1 || ych % 32 != 0 || B < 1 || xch < 1) return false;
+    if (yh != xh + 2 * pad - kh + 1 || yw != xw + 2 * pad - kw + 1 || yh < 1 || yw < 1) return false;
+    g->Hp = xh + kh - 1;
+    g->Wp = xw + kw - 1;
+    // padded planes and the per-image column range must be multiples of four elements
+    while (((long long)xh * g->Wp) % 4 != 0 || ((long long)g->Hp * g->Wp) % 4 != 0)
+        if (++g->Wp > xw + kw + 6) return false;
+    const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
+    g->gyp_floats = (long long)B * ych * plane + 1024;  // slack: the last taps read a little past a plane
+    g->wr_floats = (long long)xch * kh * kw * ych;
+    return n_img >= 256 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
+}
+
+static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const FusedGeom &g,
+                                 int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad)
+{
+    const long long quads = (long long)B * ych * g.Hp * g.Wp / 4;
+    long long blocks = (quads + 255) / 256;
+    if (blocks > 1048576) blocks = 1048576;
+    hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, gy, scratch, quads, yh, yw, g.Hp,
+                       g.Wp, kh - 1 - pad, kw - 1 - pad);
+    hipLaunchKernelGGL(filter_taps_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w,
+                       scratch + g.gyp_floats, ych, xch, kh * kw);
+    return check_launch("conv2d_transpose");
+}
+
+}  // namespace ag
+
 extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const float *w,
                                                float *gx, float *gcols, int B, int ych, int yh, int yw,
                                                int xch, int kh, int kw, int pad, int stride, int dilation,
@@ -73,6 +149,17 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
                AG_ERR_INCOMPATIBLE_SHAPE,
                "conv2d_transpose: output %dx%d too small for input %dx%d (k=%dx%d stride=%d pad=%d dilation=%d)", xh,
                xw, yh, yw, kh, kw, stride, pad, dilation);
+    // Stride 1, dilation 1: the gradient is accumulated over filter taps inside one GEMM that
+    // reads a zero-bordered copy of gy; the columns (conv2d_transpose.rs:148-151) are never
+    // written.  The sum runs over (tap, filter) instead of filters then taps, within tolerance.
+    FusedGeom fg;
+    if (stride == 1 && dilation == 1 && g_fused_input_grad &&
+        fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
+        aligned16(gcols) && aligned16(gx)) {
+        if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad)) return s;
+        return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
+                                    fg.Wp);
+    }
     // gcols_b[M x P] = w^T[M x ych] * gy_b[ych x P]               conv2d_transpose.rs:114-116,167-182
     if (ag_status_t s = ag_gemm_f32(stream, 1, 0, (int)M, (int)P, ych, 1.f, w, (int)M, 0, gy, (int)P,
                                     (long long)ych * P, 0.f, gcols, (int)P, M * P, B))
@@ -106,4 +193,38 @@ extern "C" ag_status_t ag_conv2d_transpose_filter_grad_f32(ag_stream_t stream, c
     // gw[ych x N] = sum_b x_b[ych x P] * gycols_b[N x P]^T        conv2d_transpose.rs:354-381
     return ag_gemm_batchsum_f32(stream, 0, 1, ych, (int)N, (int)P, 1.f, x, (int)P, (long long)ych * P, gycols,
                                 (int)P, N * P, 0.f, gw, (int)N, B, ws, ws_bytes);
+}
+
+// Experiment hook (not part of the operator surface): 0 makes ag_conv2d_transpose_f32 always take
+// the GEMM + col2im path, 1 (default) lets stride-1 calls use the implicit input-gradient GEMM.
+extern "C" void ag_conv_fused_input_grad(int on) { ag::g_fused_input_grad = on != 0; }
+
+// The two stages of the column-free stride-1 input gradient, for callers that time or schedule
+// them separately.  `scratch` holds ag_conv_input_grad_scratch_floats() floats (0 = this
+// geometry takes the GEMM + col2im path and the staged entry points refuse it).
+extern "C" size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad,
+                                                    int xh, int xw)
+{
+    FusedGeom g;
+    return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) ? (size_t)(g.gyp_floats + g.wr_floats) : 0;
+}
+
+extern "C" ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w, float *scratch,
+                                                      int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad,
+                                                      int xh, int xw)
+{
+    FusedGeom g;
+    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch), AG_ERR_INVALID_DIMS,
+               "conv_input_grad_prepare: geometry not supported by the column-free path");
+    return fused_prepare(as_stream(stream), gy, w, scratch, g, B, ych, yh, yw, xch, kh, kw, pad);
+}
+
+extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch, float *gx, int B, int ych,
+                                                   int yh, int yw, int xch, int kh, int kw, int pad, int xh, int xw)
+{
+    FusedGeom g;
+    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch) && aligned16(gx),
+               AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: geometry not supported by the column-free path");
+    return gemm_conv_input_grad(as_stream(stream), scratch + g.gyp_floats, scratch, gx, B, xch, ych, xh, xw, kh, kw, g.Hp,
+                                g.Wp);
 }

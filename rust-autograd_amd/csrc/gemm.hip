@@ -459,7 +459,7 @@ static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
                                 {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
                                 {128, 128}, {192, 128}, {128, 64},
-                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}};
+                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}, {64, 256}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
@@ -632,6 +632,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.n_img = fold ? c.N : 0;
     if (fold) p.N = c.N * c.batch;
     p.n_off = 0;
+    p.conv_wp = p.conv_w = p.conv_kw = 0;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * (fold ? 1 : c.batch) * p.splits;
@@ -700,6 +701,34 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         return check_launch(who);
     }
     return AG_OK;
+}
+
+// Implicit input gradient of a stride-1 convolution on the direct-to-LDS kernel (see the conv_*
+// fields of GemmParams): gx[b][c] = sum over taps and filters of wr[c][tap][k] * gyp[b][k] shifted.
+// wr [C][kh*kw*Kf] (k fastest), gyp [B][Kf][Hp][Wp] zero-bordered, gx [B][C][H][W].
+ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp)
+{
+    GemmParams p;
+    p.A = wr; p.B = gyp; p.C = gx;
+    p.M = C; p.K = Kf;
+    p.n_img = H * Wp;
+    p.N = B * p.n_img;
+    p.lda = (long long)kh * kw * Kf; p.ldb = (long long)Hp * Wp; p.ldc = (long long)H * W;
+    p.sA = 0; p.sB = (long long)Kf * Hp * Wp; p.sC = (long long)C * H * W;
+    p.sAk = Kf; p.sBk = 0;
+    p.kbatch = kh * kw; p.kb_per_split = p.kbatch; p.splits = 1; p.sCsplit = 0;
+    p.alpha = 1.f; p.beta = 0.f;
+    p.n_off = 0;
+    p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
+    const int cfg = C <= 64 ? kDirectCfg64 : 14;  // 64 x 256 or 128 x 256
+    p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
+    p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
+    const long long blocks = (long long)p.tiles_m * p.tiles_n;
+    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "conv2d_transpose: too many tiles (%lld)", blocks);
+    p.total_blocks = (unsigned)blocks;
+    launch_direct(st, cfg, true, false, p, num_cus(), g_grid_scale);
+    return check_launch("conv2d_transpose");
 }
 
 static int g_force_splits = 0;  // experiment hook, see ag_gemm_force_splits

@@ -234,7 +234,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     LoadA ldr_a;
     LoadB ldr_b;
     const float *pa = nullptr, *pb = nullptr;  // origin of the next k tile to fetch
-    int fkt = 0, f_left = 0;
+    int fkt = 0, f_left = 0, f_kx = 0;
+    const int conv_first_shift = p.conv_wp != 0 ? (p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1) : 0;
     Cursor fcur = first;
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
@@ -247,6 +248,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         }
         pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
         pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
+        if (p.conv_wp != 0) {  // first tap (0, 0): the largest shift
+            pb += conv_first_shift;
+            f_kx = 0;
+        }
         fkt = 0;
         f_left = it.nt;
     };
@@ -257,6 +262,23 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             if (f_valid) {
                 cursor_next(fcur);
                 f_begin();
+            }
+        } else if (p.conv_wp != 0) {
+            // Implicit input gradient: for one group of 32 filters all taps are visited in turn
+            // (they read nearly the same rows of B, which stay in the cache), then the next group.
+            if (++fkt == p.kbatch) {  // fkt counts taps here
+                fkt = 0;
+                f_kx = 0;
+                pa += BK - (long long)(p.kbatch - 1) * p.sAk;
+                pb += step_b + conv_first_shift;  // the last tap has shift 0
+            } else {
+                pa += p.sAk;
+                if (++f_kx == p.conv_kw) {  // next tap: one column to the left, or up a row
+                    f_kx = 0;
+                    pb += p.conv_kw - 1 - p.conv_wp;
+                } else {
+                    pb -= 1;
+                }
             }
         } else if (++fkt == kt_per) {
             fkt = 0;
@@ -345,6 +367,36 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             ldc = p.ldc;
             alpha = p.alpha;
             beta = p.beta;
+        }
+        if (p.conv_wp != 0) {
+            // implicit input gradient: column -> pixel of the (possibly next) image; the columns
+            // of the zero border are dropped
+            const int row_base = it.m0 + wm * WM + 4 * half;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                int col = it.r0 + wn * WN + l31 + j * 32;
+                const bool in_range = it.n0 + wn * WN + l31 + j * 32 < p.N;
+                long long img = 0;
+                if (col >= p.n_img) {
+                    col -= p.n_img;
+                    img = p.sC;
+                }
+                const int iy = col / p.conv_wp, ix = col - iy * p.conv_wp;
+                const bool ok = in_range && ix < p.conv_w;
+                float *dst0 = Cb + img + iy * p.conv_w + ix;
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
+                        if (ok && row < p.M) {
+                            float *dst = dst0 + (long long)row * ldc;
+                            const float r = alpha * acc[i][j][v];
+                            *dst = beta == 0.f ? r : r + beta * *dst;
+                        }
+                    }
+            }
+            return false;
         }
         const bool full = it.m0 + BM <= p.M && it.n0 + BN <= p.N;
         const int row_base = it.m0 + wm * WM + 4 * half;
@@ -518,7 +570,8 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
         case 15: launch_dl<256, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        default: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 18: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        default: launch_dl<64, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
     }
 }
 

@@ -29,6 +29,12 @@ struct GemmParams {
     // g % n_img of batch g / n_img -- and N = batch * n_img is tiled without padding every batch.
     int n_img;  // 0 = not folded
     int n_off;  // folded: first column of this launch (a launch may cover a column range only)
+    // Implicit input gradient of a stride-1 convolution (direct-to-LDS kernel, folded batch):
+    // B is the zero-bordered upstream gradient [batch][K][Hp][conv_wp]; the accumulated "batches"
+    // are the kh*kw filter taps, tap (ky, kx) reading B shifted by (kh-1-ky)*conv_wp + (kw-1-kx)
+    // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
+    // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
+    int conv_wp, conv_w, conv_kw;
 };
 
 constexpr int kXcds = 8;
@@ -46,5 +52,9 @@ __device__ inline unsigned xcd_remap(unsigned id, unsigned total)
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
 constexpr int kFirstDirectCfg = 13;
 void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
+ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
+// Direct-to-LDS configuration with a 64-row tile (64 x 256), used by the implicit input gradient.
+constexpr int kDirectCfg64 = 19;
 
 }  // namespace ag

@@ -385,10 +385,42 @@ def test_conv2d_forward_and_gradients(K, orc, rng, case):
     assert np.array_equal(host(gx), orc.col2im(host(gcols), C, H, W, k, k, p, p, s, s, d, d, OH, OW))
     # the reference's reconstructed size (may be a crop)
     say("conv2d input grad, reference size", case)
-    gx_ref = host(K.conv2d_transpose(dev(gy), dev(w), p, s, d))
+    gx_ref = host(K.conv2d_transpose(dev(gy), dev(w), p, s, d, return_cols=True)[0])  # same path as gx above
     rh, rw = gx_ref.shape[2:]
     assert rh == orc.conv_transpose_out_size(OH, k, p, s, d) and rh <= H
     assert np.array_equal(gx_ref, host(gx)[:, :, :rh, :rw])
+
+
+FUSED_CASES = [  # B, C (input channels of the conv), K (filters), H, W, k, pad
+    (2, 64, 128, 56, 56, 3, 1),   # north star, 2 of 256 images
+    (5, 32, 32, 20, 24, 3, 1),    # tiles straddle several images
+    (2, 16, 64, 18, 18, 5, 2),    # 5x5
+    (2, 8, 32, 20, 20, 3, 0),     # no padding: the gradient is wider than gy on every side
+    (3, 8, 32, 17, 17, 3, 1),     # odd width: the padded row gets an extra column
+    (2, 96, 32, 16, 20, 3, 1),    # more than 64 input channels: 128-row tiles
+    (1, 7, 64, 30, 30, 3, 2),     # pad equal to k - 1
+]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_conv2d_input_grad_fused_matches_columns_path(K, orc, rng, case):
+    """Stride-1 input gradient: the implicit GEMM over filter taps (no columns) against the f64
+    oracle and against the library's own GEMM + col2im path."""
+    B, C, Kc, H, W, k, p = case
+    L = K.capi.lib()
+    OH, OW = H + 2 * p - k + 1, W + 2 * p - k + 1
+    gy = rng.standard_normal((B, Kc, OH, OW)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    say("fused input grad", case)
+    gx_fused = host(K.conv2d_transpose(dev(gy), dev(w), p, 1, 1, out_hw=(H, W)))
+    say("columns input grad", case)
+    gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, 1, out_hw=(H, W), return_cols=True)
+    o64 = orc.conv2d_transpose(gy.astype(np.float64), w.astype(np.float64), p, 1, 1, out_hw=(H, W))
+    oabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1, out_hw=(H, W))
+    assert gx_fused.shape == o64.shape
+    assert_close_conditioned(gx_fused, o64, oabs, "fused input grad")
+    assert_close_conditioned(host(gx_cols), o64, oabs, "columns input grad")
+    assert_close_conditioned(gx_fused, host(gx_cols).astype(np.float64), oabs, "fused vs columns")
 
 
 def test_conv2d_all_ones_closed_form(K):
