@@ -273,8 +273,15 @@ def micro(torch, Kn, capi, dev):
     y, am, il = Kn.max_pool2d(x, 3, 0, 2)
     gy = torch.randn_like(y)
     by = 4.0 * (x.numel() + 2 * y.numel())
-    ms = time_events(torch, lambda: Kn.max_pool2d(x, 3, 0, 2), 10)
-    res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    Lp = capi.lib()
+    sp, pp, cp = Kn._stream, Kn._ptr, capi.check
+    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), pp(il), 256, 128, 56, 56, 3, 0, 2)), 10)
+    res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                          "note": "also writes the exact int32 index (95.6 MB, not counted) that the backward needs above 2^24 elements"}
+    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), None, 256, 128, 56, 56, 3, 0, 2)), 10)
+    res["maxpool_fwd_reference_outputs"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+                                            "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                            "note": "y and the f32-encoded argmax only, the reference's two outputs"}
     ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), 10)
     res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
     del x, y, am, il, gy
