@@ -329,8 +329,47 @@ def micro(torch, Kn, capi, dev):
     ms = time_events(torch, lambda: Kn.batch_matmul(A, Bm), 10)
     tf = 2.0 * 64 * 512 ** 3 / ms / 1e9
     res["batch_matmul_64x512"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+    res.update(other_conv_configs(torch, Kn, dev, g))
     res.update(graph_steps())
     return res
+
+
+def other_conv_configs(torch, Kn, dev, g):
+    """Operator-level conv2d forward + both gradients at the remaining convolution configurations
+    (stride-2 variant of the headline; dilated and transposed convolutions of configuration 5)."""
+    out = {}
+
+    def conv_case(name, Bn, Cc, Kf, Hh, k, pad, stride, dil):
+        x = torch.randn(Bn, Cc, Hh, Hh, device=dev, generator=g)
+        w = torch.randn(Kf, Cc, k, k, device=dev, generator=g) * 0.05
+        y, cols = Kn.conv2d(x, w, pad, stride, dil)
+        gy = torch.randn_like(y)
+
+        def step():
+            yy, cc = Kn.conv2d(x, w, pad, stride, dil)
+            Kn.conv2d_filter_grad(cc, gy, tuple(w.shape))
+            Kn.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(Hh, Hh))
+
+        ms = time_events(torch, step, 8)
+        flop = 3 * 2.0 * Bn * Kf * y.shape[2] * y.shape[3] * Cc * k * k
+        out[name] = {"ms": round(ms, 4), "images/s": round(Bn / ms * 1e3, 1), "TFLOP/s": round(flop / ms / 1e9, 2)}
+
+    conv_case("conv2d_fwd_bwd_stride2_B256_64to128_56x56", 256, 64, 128, 56, 3, 1, 2, 1)
+    conv_case("conv2d_fwd_bwd_dilated_B32_256to256_14x14", 32, 256, 256, 14, 3, 2, 1, 2)
+    # transposed convolution 128 -> 64, 4x4, stride 2, pad 1: [32,128,14,14] -> [32,64,28,28], forward and both gradients
+    x = torch.randn(32, 128, 14, 14, device=dev, generator=g)
+    w = (torch.rand(128, 64, 4, 4, device=dev, generator=g) - 0.5) * 0.2
+    yt = Kn.conv2d_transpose(x, w, 1, 2)
+    go = torch.randn_like(yt)
+
+    def tstep():
+        Kn.conv2d_transpose(x, w, 1, 2)
+        Kn.conv2d(go, w, 1, 2)                                  # gradient w.r.t. the input of the transposed conv
+        Kn.conv2d_transpose_filter_grad(x, go, tuple(w.shape), 1, 2)
+
+    ms = time_events(torch, tstep, 8)
+    out["conv2d_transpose_fwd_bwd_B32_128to64_14to28"] = {"ms": round(ms, 4), "images/s": round(32 / ms * 1e3, 1)}
+    return out
 
 
 def graph_steps():
