@@ -423,6 +423,32 @@ def test_conv2d_input_grad_fused_matches_columns_path(K, orc, rng, case):
     assert_close_conditioned(gx_fused, host(gx_cols).astype(np.float64), oabs, "fused vs columns")
 
 
+def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
+    """ag_conv_input_grad_{scratch_floats,prepare,gemm}: the two stages a caller may launch itself."""
+    L = K.capi.lib()
+    B, C, Kc, H, W, k, p = 3, 24, 64, 20, 28, 3, 1
+    geom = (B, Kc, H, W, C, k, k, p, H, W)
+    n = L.ag_conv_input_grad_scratch_floats(*geom)
+    assert n > B * Kc * (H + 2) * (W + 2)
+    gy = rng.standard_normal((B, Kc, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    scratch = torch.empty(n, device="cuda")
+    gx = torch.empty(B, C, H, W, device="cuda")
+    gyd, wd = dev(gy), dev(w)  # kept alive: a temporary would be freed and reused before the launch
+    say("staged input grad")
+    K.check(L.ag_conv_input_grad_prepare_f32(K._stream(), K._ptr(gyd), K._ptr(wd), K._ptr(scratch), *geom))
+    K.check(L.ag_conv_input_grad_gemm_f32(K._stream(), K._ptr(scratch), K._ptr(gx), *geom))
+    o64 = orc.conv2d_transpose(gy.astype(np.float64), w.astype(np.float64), p, 1, 1, out_hw=(H, W))
+    oabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1, out_hw=(H, W))
+    assert_close_conditioned(host(gx), o64, oabs, "staged input grad")
+    # geometries the column-free path does not take report 0 and are refused
+    assert L.ag_conv_input_grad_scratch_floats(B, 48, H, W, C, k, k, p, H, W) == 0          # filters not a multiple of 32
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 8, 8) == 0           # fewer than 256 columns per image
+    with pytest.raises(K.capi.InvalidDims, match="not supported"):
+        K.check(L.ag_conv_input_grad_prepare_f32(K._stream(), K._ptr(gyd), K._ptr(wd), K._ptr(scratch), B, 48, H, W,
+                                                 C, k, k, p, H, W))
+
+
 def test_conv2d_all_ones_closed_form(K):
     """Ones input and ones filter: y = C * (number of in-bounds taps); exact integers in f32."""
     B, C, Kc, H = 2, 64, 128, 56
