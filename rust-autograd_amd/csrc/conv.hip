@@ -114,7 +114,8 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + 1024;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
-    return n_img >= 256 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
+    // a tile (64 x 128 for up to 64 channels, else 128 x 256) may straddle two images, not three
+    return n_img >= (xch <= 64 ? 128 : 256) && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
 }
 
 static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const FusedGeom &g,

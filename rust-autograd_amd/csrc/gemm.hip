@@ -459,7 +459,7 @@ static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
                                 {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
                                 {128, 128}, {192, 128}, {128, 64},
-                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}, {64, 256}};
+                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}, {64, 128}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
@@ -721,7 +721,7 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     p.alpha = 1.f; p.beta = 0.f;
     p.n_off = 0;
     p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
-    const int cfg = C <= 64 ? kDirectCfg64 : 14;  // 64 x 256 or 128 x 256
+    const int cfg = C <= 64 ? kDirectCfg64 : 14;  // 64 x 128 or 128 x 256
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n;

@@ -571,7 +571,7 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
         case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 18: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        default: launch_dl<64, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        default: launch_dl<64, 128, 32, 32, 64, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
     }
 }
 

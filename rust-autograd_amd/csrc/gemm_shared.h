@@ -54,7 +54,7 @@ constexpr int kFirstDirectCfg = 13;
 void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
                                  int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
-// Direct-to-LDS configuration with a 64-row tile (64 x 256), used by the implicit input gradient.
+// Direct-to-LDS configuration with a 64-row tile (64 x 128, two blocks per CU), used by the implicit input gradient.
 constexpr int kDirectCfg64 = 19;
 
 }  // namespace ag

@@ -399,6 +399,7 @@ FUSED_CASES = [  # B, C (input channels of the conv), K (filters), H, W, k, pad
     (3, 8, 32, 17, 17, 3, 1),     # odd width: the padded row gets an extra column
     (2, 96, 32, 16, 20, 3, 1),    # more than 64 input channels: 128-row tiles
     (1, 7, 64, 30, 30, 3, 2),     # pad equal to k - 1
+    (4, 32, 64, 14, 14, 3, 1),    # config 2's second convolution: 224 padded columns per image
 ]
 
 
@@ -443,7 +444,7 @@ def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
     assert_close_conditioned(host(gx), o64, oabs, "staged input grad")
     # geometries the column-free path does not take report 0 and are refused
     assert L.ag_conv_input_grad_scratch_floats(B, 48, H, W, C, k, k, p, H, W) == 0          # filters not a multiple of 32
-    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 8, 8) == 0           # fewer than 256 columns per image
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 8, 8) == 0           # fewer than 128 columns per image
     with pytest.raises(K.capi.InvalidDims, match="not supported"):
         K.check(L.ag_conv_input_grad_prepare_f32(K._stream(), K._ptr(gyd), K._ptr(wd), K._ptr(scratch), B, 48, H, W,
                                                  C, k, k, p, H, W))
