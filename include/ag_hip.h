@@ -228,6 +228,11 @@ ag_status_t ag_relu_grad_f32(ag_stream_t stream, const float *x, const float *gy
 /* AddOp with a row-vector right operand: y[r][c] = x[r][c] + bias[c] (binary_ops.rs:147-166, 304-346). */
 ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const float *bias, float *y,
                             size_t rows, size_t cols);
+/* AddOp with a right operand that has the left operand's rank and extent 1 on the axes it is
+ * broadcast along, e.g. a [1,C,1,1] bias on NCHW (binary_ops.rs:147-166, 304-346; the conv biases of
+ * examples/cnn_mnist.rs).  bshape[i] must be shape[i] or 1; rank <= 8. */
+ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
+                                 const int *shape, const int *bshape, int rank);
 /* MaybeReduceSum for that operand: out[c] = sum_r gy[r][c], r ascending (binary_ops.rs:39-105). */
 ag_status_t ag_bias_grad_f32(ag_stream_t stream, const float *gy, float *out, size_t rows,
                              size_t cols);

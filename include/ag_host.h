@@ -41,6 +41,18 @@ int agh_env_read(agh_env *env, int var_id, float *out, size_t n);
 /* Overwrites the variable's array in place (same element count), as writing through
  * env.get_array_by_id(id).borrow_mut() does (src/variable.rs:695-703). */
 int agh_env_write(agh_env *env, int var_id, const float *data, size_t n);
+int agh_env_len(agh_env *env); /* number of variable arrays (named or not) */
+/* Persistence in the reference's own on-disk format: serde_json of {"array_list":[{"v":1,"dim":[..],
+ * "data":[..]},..],"name_to_id":{"ns\u0001name":id,..}} (src/variable.rs:470-480).
+ * agh_env_save = VariableEnvironment::save (:549-554); agh_env_load = ::load (:487-490), NULL on error;
+ * agh_env_initialize = ::initialize (:493-503), replacing the arrays and names of `env`.
+ * A file that cannot be opened or parsed gives -1 / NULL and a message in agh_last_error(). */
+int agh_env_save(agh_env *env, const char *path);
+agh_env *agh_env_load(const char *path);
+int agh_env_initialize(agh_env *env, const char *path);
+/* Reads a saved environment and writes it again, in host memory only (no device is touched):
+ * checks a file and brings it to the exact text agh_env_save produces. */
+int agh_env_file_rewrite(const char *src_path, const char *dst_path);
 
 /* ---- graph construction (one context = one `env.run(|ctx| ...)` closure) --------------------- */
 agh_ctx *agh_ctx_new(agh_env *env);

@@ -26,7 +26,7 @@ echo "built $out"
 # kernel library next to it.
 host_out="$here/../libag_host.so"
 /opt/rocm/bin/hipcc -O2 -std=c++17 -fPIC -fvisibility=hidden -Wall -I"$here/../../include" -I"$here/host" -I/opt/rocm/include \
-    -x c++ "$here/host/runtime.cpp" "$here/host/ops.cpp" "$here/host/gradient.cpp" "$here/host/capi_host.cpp" \
+    -x c++ "$here/host/runtime.cpp" "$here/host/ops.cpp" "$here/host/gradient.cpp" "$here/host/persist.cpp" "$here/host/capi_host.cpp" \
     -D__HIP_PLATFORM_AMD__ -shared -o "$host_out" -L"$here/.." -lag_hip -L/opt/rocm/lib -lamdhip64 \
     -Wl,-rpath,'$ORIGIN' -Wl,-rpath,/opt/rocm/lib
 echo "built $host_out"

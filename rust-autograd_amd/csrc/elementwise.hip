@@ -40,6 +40,32 @@ __global__ __launch_bounds__(256) void add_bias_kernel(const float *__restrict__
     AG_EW_LOOP(i, n) y[i] = x[i] + bias[i % cols];
 }
 
+// Right operand broadcast along any of its axes of extent 1.  `dims` are the left operand's extents
+// after adjacent axes with the same broadcast state have been merged (outermost first), `bstride`
+// the right operand's element stride for each merged axis (0 where it is broadcast).
+struct BroadcastGeom {
+    unsigned dims[6];
+    unsigned bstride[6];
+    int rank;
+};
+
+__global__ __launch_bounds__(256) void add_broadcast_kernel(const float *__restrict__ x,
+                                                            const float *__restrict__ b,
+                                                            float *__restrict__ y, size_t n, BroadcastGeom g)
+{
+    AG_EW_LOOP(i, n)
+    {
+        size_t rest = i, bi = 0;
+        for (int d = g.rank - 1; d > 0; --d) {
+            const size_t q = rest / g.dims[d];
+            bi += (rest - q * g.dims[d]) * g.bstride[d];
+            rest = q;
+        }
+        bi += rest * g.bstride[0];
+        y[i] = x[i] + b[bi];
+    }
+}
+
 // out[c] = sum over rows, ascending (ndarray sum_axis(0) order used by MaybeReduceSum).
 __global__ __launch_bounds__(256) void bias_grad_kernel(const float *__restrict__ gy,
                                                         float *__restrict__ out, size_t rows, size_t cols)
@@ -163,6 +189,47 @@ extern "C" ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const
 {
     AG_REQUIRE(rows * cols == 0 || (x && bias && y), AG_ERR_INVALID_DIMS, "add: null pointer");
     AG_EW_ENTRY("add", add_bias_kernel, rows * cols, x, bias, y, rows * cols, cols);
+}
+
+extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
+                                            const int *shape, const int *bshape, int rank)
+{
+    AG_REQUIRE(rank >= 1 && rank <= 8 && shape && bshape, AG_ERR_INVALID_DIMS, "add: rank %d not in 1..8", rank);
+    size_t n = 1;
+    for (int i = 0; i < rank; ++i) {
+        AG_REQUIRE(shape[i] >= 0 && (bshape[i] == shape[i] || bshape[i] == 1), AG_ERR_INCOMPATIBLE_SHAPE,
+                   "add: axis %d of the right operand has extent %d, the left %d", i, bshape[i], shape[i]);
+        n *= (size_t)shape[i];
+    }
+    if (n == 0) return AG_OK;
+    AG_REQUIRE(x && b && y, AG_ERR_INVALID_DIMS, "add: null pointer");
+    // merge neighbours with the same broadcast state; axes of extent 1 join either kind
+    BroadcastGeom g{};
+    bool prev_bc = false;
+    size_t bstride = 1;
+    unsigned rev_dims[8], rev_bstride[8];
+    int groups = 0;
+    for (int i = rank - 1; i >= 0; --i) {
+        if (shape[i] == 1) continue;
+        const bool bc = bshape[i] == 1;
+        if (groups > 0 && bc == prev_bc) {
+            AG_REQUIRE((size_t)rev_dims[groups - 1] * (size_t)shape[i] <= 0xffffffffu, AG_ERR_INVALID_DIMS, "add: extent too large");
+            rev_dims[groups - 1] *= (unsigned)shape[i];
+        } else {
+            rev_dims[groups] = (unsigned)shape[i];
+            rev_bstride[groups] = bc ? 0u : (unsigned)bstride;
+            ++groups;
+        }
+        if (!bc) bstride *= (size_t)shape[i];
+        prev_bc = bc;
+    }
+    AG_REQUIRE(groups <= 6 && bstride <= 0xffffffffu, AG_ERR_INVALID_DIMS, "add: broadcast pattern with %d groups of axes not supported", groups);
+    if (groups == 0) {
+        rev_dims[0] = 1, rev_bstride[0] = 0, groups = 1;
+    }
+    g.rank = groups;
+    for (int i = 0; i < groups; ++i) g.dims[i] = rev_dims[groups - 1 - i], g.bstride[i] = rev_bstride[groups - 1 - i];
+    AG_EW_ENTRY("add", add_broadcast_kernel, n, x, b, y, n, g);
 }
 
 extern "C" ag_status_t ag_bias_grad_f32(ag_stream_t stream, const float *gy, float *out, size_t rows,

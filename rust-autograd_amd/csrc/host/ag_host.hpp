@@ -41,6 +41,12 @@ struct Panic : std::runtime_error {
     using std::runtime_error::runtime_error;
 };
 
+// A file that cannot be read, written or parsed while saving or loading variables; the reference
+// returns these as `Err(Box<dyn Error>)` (src/variable.rs:487, 549, 556).
+struct PersistError : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
 // ---------------------------------------------------------------------------------------------
 // device arrays
 // ---------------------------------------------------------------------------------------------
@@ -202,6 +208,20 @@ class TensorBuilder {  // src/tensor.rs:609-803
 // ---------------------------------------------------------------------------------------------
 // variables                                                              src/variable.rs
 // ---------------------------------------------------------------------------------------------
+// Host-memory image of a saved environment: what the reference serialises (src/variable.rs:470-480).
+struct SavedArray {
+    Shape dim;
+    std::vector<float> data;  // row-major
+};
+struct SavedEnvironment {
+    std::vector<SavedArray> array_list;
+    std::map<std::string, int> name_to_id;  // "namespace\x01name" -> index into array_list
+};
+std::string to_json(const SavedEnvironment &env);     // the text serde_json writes for it
+SavedEnvironment from_json(const std::string &text);  // throws PersistError
+SavedEnvironment read_saved_environment(const std::string &path);
+void write_saved_environment(const SavedEnvironment &env, const std::string &path);
+
 class VariableEnvironment {
   public:
     // `namespace_id` "" is the default namespace.  Names are unique inside a namespace.
@@ -214,6 +234,12 @@ class VariableEnvironment {
 
     // Runs `f` with a fresh graph bound to this environment (src/variable.rs:670-683).
     void run(const std::function<void(Context &)> &f);
+
+    // Persistence in the reference's JSON format (src/variable.rs:483-500, 549-554).  `initialize`
+    // replaces this environment's arrays and names with the saved ones.  Throw PersistError.
+    void save(const std::string &path) const;
+    static VariableEnvironment load(const std::string &path);
+    void initialize(const std::string &path);
 
   private:
     std::vector<NdArray> arrays_;

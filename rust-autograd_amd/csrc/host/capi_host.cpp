@@ -89,6 +89,45 @@ int agh_env_write(agh_env *env, int var_id, const float *data, size_t n)
     });
 }
 
+int agh_env_len(agh_env *env) { return (int)env->env.size(); }
+
+int agh_env_save(agh_env *env, const char *path)
+{
+    return guard([&] {
+        env->env.save(path);
+        return 0;
+    });
+}
+
+agh_env *agh_env_load(const char *path)
+{
+    agh_env *env = new agh_env();
+    if (guard([&] {
+            env->env.initialize(path);
+            return 0;
+        }) != 0) {
+        delete env;
+        return nullptr;
+    }
+    return env;
+}
+
+int agh_env_initialize(agh_env *env, const char *path)
+{
+    return guard([&] {
+        env->env.initialize(path);
+        return 0;
+    });
+}
+
+int agh_env_file_rewrite(const char *src_path, const char *dst_path)
+{
+    return guard([&] {
+        write_saved_environment(read_saved_environment(src_path), dst_path);
+        return 0;
+    });
+}
+
 agh_ctx *agh_ctx_new(agh_env *env) { return new agh_ctx(&env->env); }
 void agh_ctx_free(agh_ctx *ctx) { delete ctx; }
 

@@ -674,6 +674,24 @@ static bool broadcasts_over_rows(const Shape &a, const Shape &b)
     return b.size() + 1 == a.size() && std::equal(a.begin() + 1, a.end(), b.begin());
 }
 
+// True when `b` has `a`'s rank and every axis of `b` is either `a`'s or 1 (ndarray broadcasting of
+// operands of equal rank); a one-element `b` of any rank counts as all ones (binary_ops.rs:54-60).
+static bool broadcasts_along_axes(const Shape &a, const Shape &b, std::vector<int> *bshape)
+{
+    size_t blen = 1;
+    for (const int64_t d : b) blen *= (size_t)d;
+    if (a.empty() || a.size() > 8) return false;
+    bshape->assign(a.size(), 1);
+    if (blen == 1) return true;
+    if (b.size() != a.size()) return false;
+    for (size_t i = 0; i < a.size(); ++i) {
+        if (b[i] != a[i] && b[i] != 1) return false;
+        if (a[i] > 0x7fffffff) return false;
+        (*bshape)[i] = (int)b[i];
+    }
+    return true;
+}
+
 struct MaybeReduceSum : Op {
     const char *name() const override { return "MaybeReduceSum"; }
     OpError compute(ComputeContext &ctx) const override
@@ -687,6 +705,25 @@ struct MaybeReduceSum : Op {
             NdArray out = NdArray::empty(x.shape());
             const size_t rows = (size_t)gy.shape()[0];
             const OpError e = from_status(ag_bias_grad_f32(ctx.stream(), gy.ptr(), out.ptr(), rows, gy.len() / rows));
+            if (!e.ok()) return e;
+            ctx.append_output(out);
+            return OpError::none();
+        }
+        std::vector<int> xshape;
+        if (broadcasts_along_axes(gy.shape(), x.shape(), &xshape)) {
+            // sum over every axis the operand was broadcast along (binary_ops.rs:69-87)
+            std::vector<int> shape(gy.shape().begin(), gy.shape().end()), axes;
+            for (int i = 0; i < (int)shape.size(); ++i)
+                if (xshape[(size_t)i] == 1 && shape[(size_t)i] > 1) axes.push_back(i);
+            if (axes.empty()) {  // same elements, other extents of 1 (binary_ops.rs:62-66)
+                ctx.append_output_view(gy.reshaped(x.shape()));
+                return OpError::none();
+            }
+            NdArray out = NdArray::empty(x.shape());
+            const size_t nb = ag_reduce_sum_f32_workspace(shape.data(), (int)shape.size(), axes.data(), (int)axes.size());
+            NdArray ws = workspace(nb);
+            const OpError e = from_status(ag_reduce_sum_f32(ctx.stream(), gy.ptr(), out.ptr(), shape.data(), (int)shape.size(),
+                                                            axes.data(), (int)axes.size(), 0, ws.ptr(), ws.len() * 4));
             if (!e.ok()) return e;
             ctx.append_output(out);
             return OpError::none();
@@ -714,6 +751,9 @@ struct AddOp : Op {  // binary_ops.rs:147-166, 304-346
         } else if (broadcasts_over_rows(a.shape(), b.shape())) {
             const size_t rows = (size_t)a.shape()[0];
             e = from_status(ag_add_bias_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), rows, a.len() / rows));
+        } else if (std::vector<int> bshape; broadcasts_along_axes(a.shape(), b.shape(), &bshape)) {
+            const std::vector<int> shape(a.shape().begin(), a.shape().end());
+            e = from_status(ag_add_broadcast_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), shape.data(), bshape.data(), (int)shape.size()));
         } else {
             return OpError::make(ErrorKind::IncompatibleShape,
                                  "AddOp: unsupported broadcast " + shape_str(a.shape()) + " + " + shape_str(b.shape()));

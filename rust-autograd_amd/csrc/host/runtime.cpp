@@ -407,11 +407,11 @@ static std::string full_name(const std::string &ns, const std::string &name) { r
 
 VariableID VariableEnvironment::set(const std::string &namespace_id, const std::string &name, NdArray array)
 {
-    const std::string key = full_name(namespace_id, name);
-    if (name_to_id_.count(key)) throw Panic("Bad variable name: " + name + " is already registered");
+    // register_variable (src/variable.rs:347-358): a name that is already taken is bound to the new
+    // array; the old array stays in the list under its id
     const VariableID id = (VariableID)arrays_.size();
     arrays_.push_back(std::move(array));
-    name_to_id_[key] = id;
+    name_to_id_[full_name(namespace_id, name)] = id;
     return id;
 }
 

@@ -29,6 +29,11 @@ PROTOTYPES = {
     "agh_env_shape": (_i, [_p, _i, _lp, _i]),
     "agh_env_read": (_i, [_p, _i, _fp, _z]),
     "agh_env_write": (_i, [_p, _i, _fp, _z]),
+    "agh_env_len": (_i, [_p]),
+    "agh_env_save": (_i, [_p, _s]),
+    "agh_env_load": (_p, [_s]),
+    "agh_env_initialize": (_i, [_p, _s]),
+    "agh_env_file_rewrite": (_i, [_s, _s]),
     "agh_ctx_new": (_p, [_p]),
     "agh_ctx_free": (None, [_p]),
     "agh_variable": (_i, [_p, _i]),
@@ -111,9 +116,41 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+class PersistError(Exception):
+    """A saved environment that cannot be read, written or parsed (`Err(Box<dyn Error>)` of
+    `VariableEnvironment::save/load/initialize`, src/variable.rs:487-503, 549-563)."""
+
+
+def _check_file(rc):
+    if rc is None or (isinstance(rc, int) and rc < 0):
+        raise PersistError(lib().agh_last_error().decode())
+    return rc
+
+
+def rewrite_saved_environment(src_path, dst_path):
+    """Parses a saved environment and writes it again, in host memory only."""
+    _check_file(lib().agh_env_file_rewrite(os.fsencode(src_path), os.fsencode(dst_path)))
+
+
 class VariableEnvironment:
-    def __init__(self):
-        self._h = _check(lib().agh_env_new())
+    def __init__(self, _handle=None):
+        self._h = _handle if _handle is not None else _check(lib().agh_env_new())
+
+    @classmethod
+    def load(cls, path):
+        """`VariableEnvironment::<f32>::load(path)` (src/variable.rs:487-490)."""
+        return cls(_check_file(lib().agh_env_load(os.fsencode(path))))
+
+    def save(self, path):
+        """`env.save(path)` (src/variable.rs:549-554): the reference's JSON format."""
+        _check_file(lib().agh_env_save(self._h, os.fsencode(path)))
+
+    def initialize(self, path):
+        """`env.initialize(path)` (src/variable.rs:493-503): replaces arrays and names."""
+        _check_file(lib().agh_env_initialize(self._h, os.fsencode(path)))
+
+    def __len__(self):
+        return _check(lib().agh_env_len(self._h))
 
     def __del__(self):
         if getattr(self, "_h", None) and _LIB is not None:

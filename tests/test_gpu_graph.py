@@ -563,3 +563,112 @@ def test_ref_reduce_and_wx_plus_b(G, rng):                  # :523, :627-:690
     x, w, b = c.variable(xi), c.variable(wi), c.variable(bi)
     z = c.matmul(x, w) + b
     check_theoretical_grads(G, env, c, z, c.grad([z], [b]), [bi])
+
+
+# ------------------------------------------------------------------------------- saved environments
+def test_ref_save_and_load(G, rng, tmp_path):                # src/variable.rs:811-841
+    path = str(tmp_path / "model.json")
+    env = G.VariableEnvironment()
+    a = rng.standard_normal((2, 3)).astype(np.float32)
+    b = rng.standard_normal((2, 3)).astype(np.float32)
+    ida, idb = env.set("a", a), env.set("b", b)
+    env.save(path)
+    loaded = G.VariableEnvironment.load(path)
+    assert len(loaded) == len(env) == 2
+    for vid, want in ((ida, a), (idb, b)):
+        # the reference asserts 1e-6; shortest-round-trip digits give the same bits back
+        assert loaded.array(vid).tobytes() == want.tobytes()
+    assert loaded.find("a") == ida and loaded.find("b") == idb and loaded.find("c") is None
+
+
+def test_ref_save_and_init(G, rng, tmp_path):                # src/variable.rs:843-866
+    path = str(tmp_path / "model.json")
+    env = G.VariableEnvironment()
+    a = env.set("a", rng.standard_normal((2, 3)).astype(np.float32))
+    b = env.set("b", rng.standard_normal((2, 3)).astype(np.float32))
+    before = [env.array(a), env.array(b)]
+    for _ in range(10):
+        c = env.context()
+        c.variable(a), c.variable(b)
+        env.save(path)            # saving from inside a run, over the previous file
+    env.initialize(path)
+    assert [env.array(a).tobytes(), env.array(b).tobytes()] == [x.tobytes() for x in before]
+
+
+def test_training_resumes_identically_from_a_saved_environment(G, rng, tmp_path):
+    # parameters in the default namespace, Adam's m/v/t in the optimizer's namespace, every shape
+    # rank (0-d t, 4-d filter); a run that is saved, reloaded and continued must match one that
+    # was never interrupted, bit for bit
+    path = str(tmp_path / "train.json")
+    x = rng.standard_normal((4, 2, 8, 8)).astype(np.float32)
+
+    def make():
+        r = np.random.default_rng(3)
+        env = G.VariableEnvironment()
+        wid = env.set("w", (0.3 * r.standard_normal((3, 2, 3, 3))).astype(np.float32))
+        bid = env.set("b", np.zeros((1, 3, 1, 1), np.float32), namespace="bias")
+        return env, wid, bid
+
+    def step(env, adam, wid, bid):
+        c = env.context()
+        w, b = c.variable(wid), c.variable(bid)
+        y = c.relu(c.add(c.conv2d(c.placeholder("x", [-1, 2, 8, 8]), w, 1, 1), b))
+        loss = c.sum_all(c.mul(y, y))
+        gw, gb = c.grad([loss], [w, b])
+        adam.update([w, b], [gw, gb], c, feeds={"x": x})
+
+    env1, wid, bid = make()
+    adam1 = G.Adam(env1, [wid, bid], alpha=0.05)
+    for _ in range(4):
+        step(env1, adam1, wid, bid)
+
+    env2, _, _ = make()
+    adam2 = G.Adam(env2, [wid, bid], alpha=0.05)
+    for _ in range(2):
+        step(env2, adam2, wid, bid)
+    env2.save(path)
+    text = open(path).read()
+    assert text.startswith('{"array_list":[{"v":1,"dim":[3,2,3,3],"data":[') and '"bias\\u0001b":1' in text
+    env3 = G.VariableEnvironment.load(path)
+    assert len(env3) == len(env2) and env3.find("b", namespace="bias") == bid
+    for vid in range(len(env2)):
+        assert env3.array(vid).tobytes() == env2.array(vid).tobytes(), f"loaded variable {vid}"
+    # Adam::new always registers fresh m, v, t (src/optimizers/adam.rs:84-101), so a run is continued
+    # with the optimizer it already has, after `initialize` put the saved arrays back in place
+    for _ in range(3):
+        step(env2, adam2, wid, bid)     # wander off ...
+    env2.initialize(path)               # ... and come back to the saved state
+    for _ in range(2):
+        step(env2, adam2, wid, bid)
+    for vid in range(len(env1)):
+        assert env2.array(vid).tobytes() == env1.array(vid).tobytes(), f"variable {vid}"
+
+
+def test_a_name_registered_twice_is_bound_to_the_newer_array(G):   # src/variable.rs:347-358
+    env = G.VariableEnvironment()
+    first = env.set("w", np.zeros((2,), np.float32))
+    second = env.set("w", np.ones((3,), np.float32))
+    assert (first, second) == (0, 1) and env.find("w") == second and len(env) == 2
+    assert env.array(first).shape == (2,) and env.array(second).shape == (3,)
+
+
+@pytest.mark.parametrize("shape,bshape", [((4, 3, 6, 6), (1, 3, 1, 1)), ((5, 7), (5, 1)), ((3, 4, 5), (1, 1, 1)),
+                                          ((3, 4, 5), (1, 4, 1))])
+def test_add_broadcast_and_the_reduced_gradient(G, rng, shape, bshape):
+    # AddOp with ndarray broadcasting of a unit-extent operand and MaybeReduceSum
+    # (binary_ops.rs:39-105, 147-166): d sum(w * (x + b)) / db = w summed over the broadcast axes
+    x = rng.standard_normal(shape).astype(np.float32)
+    b = rng.standard_normal(bshape).astype(np.float32)
+    w = rng.standard_normal(shape).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    xt, bt, wt = (c.variable(env.set(n, a)) for n, a in (("x", x), ("b", b), ("w", w)))
+    y = c.add(xt, bt)
+    gx, gb = c.grad([c.mul(y, wt)], [xt, bt])
+    yv, gxv, gbv = c.eval([y, gx, gb])
+    assert np.array_equal(yv, x + b)
+    assert np.array_equal(gxv, w)
+    axes = tuple(i for i, (s, t) in enumerate(zip(shape, bshape)) if t == 1 and s > 1)
+    want = w.astype(np.float64).sum(axis=axes, keepdims=True)
+    assert gbv.shape == tuple(bshape)
+    assert_close(gbv, want, "bias gradient", scale=np.abs(w).astype(np.float64).sum(axis=axes, keepdims=True))

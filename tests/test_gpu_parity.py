@@ -708,6 +708,26 @@ def test_relu_bias_addn_mul_fill(K, orc, rng):
     assert np.all(host(K.fill((3, 5), 1.5)) == 1.5)
 
 
+@pytest.mark.parametrize("shape,bshape", [
+    ((4, 3, 8, 8), (1, 3, 1, 1)),       # the conv bias of examples/cnn_mnist.rs
+    ((5, 7, 9), (5, 1, 9)), ((5, 7, 9), (1, 7, 1)), ((6, 10), (1, 10)), ((6, 10), (6, 1)),
+    ((2, 3, 4, 5, 6), (2, 1, 4, 1, 6)), ((3, 1, 4), (1, 1, 4)), ((7,), (1,)), ((2, 3), (2, 3)),
+])
+def test_add_with_an_operand_broadcast_along_its_unit_axes(K, rng, shape, bshape):
+    # one rounding per element: numpy's own broadcast add is the exact answer
+    x = rng.standard_normal(shape).astype(np.float32)
+    b = rng.standard_normal(bshape).astype(np.float32)
+    say(f"add_broadcast {shape} + {bshape}")
+    assert np.array_equal(host(K.add_broadcast(dev(x), dev(b))), x + b)
+
+
+def test_add_broadcast_rejects_other_extents(K, rng):
+    from rust_autograd_amd import capi
+    x, b = dev(np.zeros((4, 3), np.float32)), dev(np.zeros((2, 3), np.float32))
+    with pytest.raises(capi.IncompatibleShape):
+        K.add_broadcast(x, b)
+
+
 def test_sparse_softmax_cross_entropy(K, orc, rng):
     logits = (rng.standard_normal((128, 10)) * 3).astype(np.float32)
     labels = rng.integers(0, 10, size=(128, 1)).astype(np.float32)
