@@ -310,6 +310,15 @@ def micro(torch, Kn, capi, dev):
     a = torch.randn(n, device=dev, generator=g)
     ms = time_events(torch, lambda: Kn.sum_all(a), 10)
     res["sum_all_2^26"] = {"ms": round(ms, 4), "GB/s": round(4.0 * n / ms / 1e6, 1), "frac_hbm": round(4.0 * n / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    # axis reductions over the pool input's shape: the per-channel (conv bias) gradient, one axis, the rows
+    a4 = torch.randn(Bn, Kf, Hh, Hh, device=dev, generator=g)
+    for name, axes in (("reduce_sum_[256,128,56,56]_axes_0_2_3", [0, 2, 3]), ("reduce_sum_[256,128,56,56]_axis_0", [0]),
+                       ("reduce_mean_[256,128,56,56]_axes_2_3", [2, 3])):
+        fn = Kn.reduce_mean if "mean" in name else Kn.reduce_sum
+        ms = time_events(torch, lambda: fn(a4, axes), 10)
+        res[name] = {"ms": round(ms, 4), "GB/s": round(4.0 * a4.numel() / ms / 1e6, 1),
+                     "frac_hbm": round(4.0 * a4.numel() / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del a4
     p, m, v = torch.randn(n, device=dev, generator=g), torch.zeros(n, device=dev), torch.zeros(n, device=dev)
     t = torch.ones(1, device=dev)
     ms = time_events(torch, lambda: Kn.adam_update(p, a, m, v, t), 10)

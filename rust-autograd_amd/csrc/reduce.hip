@@ -8,6 +8,13 @@
 // (inner > 1), or a short folded axis, each thread owns one output and adds along the axis
 // sequentially, which is the reference's own order (bit-identical sums); a long innermost axis
 // uses one wave per row instead (tolerance-level agreement).
+//
+// Inputs of 2^20 elements and more take the streaming folds instead: neighbouring axes with the
+// same state are merged, the last folded group goes first (it reads the whole input, every later
+// step a small intermediate), and every step keeps many independent 128-bit streaming loads in
+// flight per thread over contiguous memory -- a group of lanes per row for a trailing group, a
+// thread per output column (split along the folded axis until the chip is full) otherwise.  Sums
+// agree with the sequential order to rounding.
 #include "ag_internal.h"
 
 namespace ag {
@@ -47,19 +54,28 @@ __global__ __launch_bounds__(kSumThreads) void sum_stage1_kernel(const float *__
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     size_t done = 0;
     if (vec) {
+        // Each block streams one contiguous run of the input, eight 128-bit loads in flight per
+        // thread: measured 7.0 TB/s on MI355X against 5.4 TB/s for loads a whole grid apart.
         const size_t n4 = n / 4;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
-        size_t i = tid;
-        // four independent 128-bit loads in flight per thread
-        for (; i + 3 * nthreads < n4; i += 4 * nthreads) {
-            const float4 v0 = ld_stream(x4 + i), v1 = ld_stream(x4 + i + nthreads), v2 = ld_stream(x4 + i + 2 * nthreads),
-                         v3 = ld_stream(x4 + i + 3 * nthreads);
-            a0 += (v0.x + v1.x) + (v2.x + v3.x);
-            a1 += (v0.y + v1.y) + (v2.y + v3.y);
-            a2 += (v0.z + v1.z) + (v2.z + v3.z);
-            a3 += (v0.w + v1.w) + (v2.w + v3.w);
+        const size_t per_block = (n4 + gridDim.x - 1) / gridDim.x;
+        const size_t b0 = blockIdx.x * per_block;
+        const size_t b1 = b0 + per_block < n4 ? b0 + per_block : n4;
+        size_t i = b0 + threadIdx.x;
+        constexpr int U = 8;
+        for (; i + (U - 1) * kSumThreads < b1; i += U * kSumThreads) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = ld_stream(x4 + i + u * kSumThreads);
+#pragma unroll
+            for (int u = 0; u < U; u += 2) {
+                a0 += v[u].x + v[u + 1].x;
+                a1 += v[u].y + v[u + 1].y;
+                a2 += v[u].z + v[u + 1].z;
+                a3 += v[u].w + v[u + 1].w;
+            }
         }
-        for (; i < n4; i += nthreads) {
+        for (; i < b1; i += kSumThreads) {
             const float4 v = x4[i];
             a0 += v.x;
             a1 += v.y;
@@ -142,6 +158,148 @@ __global__ __launch_bounds__(256) void fold_last_axis_kernel(const float *__rest
         for (size_t i = lane; i < len; i += 64) acc += p[i];
         acc = wave_sum(acc);
         if (lane == 0) out[r] = apply_scale ? acc * scale : acc;
+    }
+}
+
+// ---- streaming folds (large inputs) ------------------------------------------------------------
+
+// x [rows][len] -> out [rows]: G lanes per row, rows of one wave adjacent in memory.
+template <int G, bool VEC>
+__global__ __launch_bounds__(256) void fold_rows_kernel(const float *__restrict__ x, float *__restrict__ out,
+                                                        size_t rows, size_t len, float scale, int apply_scale)
+{
+    const unsigned lane = threadIdx.x % G;
+    const size_t row = (blockIdx.x * 256ull + threadIdx.x) / G;
+    const bool live = row < rows;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (live) {
+        const float *p = x + row * len;
+        if (VEC) {
+            const float4 *p4 = reinterpret_cast<const float4 *>(p);
+            const size_t len4 = len / 4;
+            size_t j = lane;
+            for (; j + 3 * G < len4; j += 4 * G) {
+                const float4 v0 = ld_stream(p4 + j), v1 = ld_stream(p4 + j + G), v2 = ld_stream(p4 + j + 2 * G),
+                             v3 = ld_stream(p4 + j + 3 * G);
+                a0 += (v0.x + v1.x) + (v2.x + v3.x);
+                a1 += (v0.y + v1.y) + (v2.y + v3.y);
+                a2 += (v0.z + v1.z) + (v2.z + v3.z);
+                a3 += (v0.w + v1.w) + (v2.w + v3.w);
+            }
+            for (; j < len4; j += G) {
+                const float4 v = ld_stream(p4 + j);
+                a0 += v.x;
+                a1 += v.y;
+                a2 += v.z;
+                a3 += v.w;
+            }
+        } else {
+            size_t j = lane;
+            for (; j + 3 * G < len; j += 4 * G) {
+                a0 += ld_stream(p + j);
+                a1 += ld_stream(p + j + G);
+                a2 += ld_stream(p + j + 2 * G);
+                a3 += ld_stream(p + j + 3 * G);
+            }
+            for (; j < len; j += G) a0 += ld_stream(p + j);
+        }
+    }
+    float s = (a0 + a1) + (a2 + a3);
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) s += __shfl_down(s, off, G);
+    if (live && lane == 0) out[row] = apply_scale ? s * scale : s;
+}
+
+// Few long rows: x [rows][len] -> part [rows][splits]; block (row, split) streams elements
+// [split*chunk, min(len, (split+1)*chunk)) of its row (chunk a multiple of 4).
+template <bool VEC>
+__global__ __launch_bounds__(256) void fold_rows_split_kernel(const float *__restrict__ x, float *__restrict__ part,
+                                                              size_t len, unsigned splits, size_t chunk)
+{
+    __shared__ float lds[4];
+    const size_t row = blockIdx.x / splits;
+    const unsigned sp = blockIdx.x % splits;
+    const size_t e0 = (size_t)sp * chunk, e1 = e0 + chunk < len ? e0 + chunk : len;
+    const float *p = x + row * len;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (VEC) {
+        const float4 *p4 = reinterpret_cast<const float4 *>(p);
+        const size_t q1 = e1 / 4;
+        size_t i = e0 / 4 + threadIdx.x;
+        constexpr int U = 8;
+        for (; i + (U - 1) * 256 < q1; i += U * 256) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = ld_stream(p4 + i + u * 256);
+#pragma unroll
+            for (int u = 0; u < U; u += 2) {
+                a0 += v[u].x + v[u + 1].x;
+                a1 += v[u].y + v[u + 1].y;
+                a2 += v[u].z + v[u + 1].z;
+                a3 += v[u].w + v[u + 1].w;
+            }
+        }
+        for (; i < q1; i += 256) {
+            const float4 v = ld_stream(p4 + i);
+            a0 += v.x;
+            a1 += v.y;
+            a2 += v.z;
+            a3 += v.w;
+        }
+    } else {
+        size_t i = e0 + threadIdx.x;
+        for (; i + 3 * 256 < e1; i += 4 * 256) {
+            a0 += ld_stream(p + i);
+            a1 += ld_stream(p + i + 256);
+            a2 += ld_stream(p + i + 512);
+            a3 += ld_stream(p + i + 768);
+        }
+        for (; i < e1; i += 256) a0 += ld_stream(p + i);
+    }
+    const float s = block_sum((a0 + a1) + (a2 + a3), lds);
+    if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+
+template <typename T>
+__device__ inline T vec_zero();
+template <>
+__device__ inline float vec_zero<float>() { return 0.f; }
+template <>
+__device__ inline float4 vec_zero<float4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ inline float vadd(float a, float b) { return a + b; }
+__device__ inline float4 vadd(const float4 &a, const float4 &b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+__device__ inline float vscale(float a, float s) { return a * s; }
+__device__ inline float4 vscale(const float4 &a, float s) { return make_float4(a.x * s, a.y * s, a.z * s, a.w * s); }
+
+// x [outer][len][inner] -> out [outer][splits][inner], T = float4 when inner is a multiple of 4:
+// one thread per output column (of T), rows [split*chunk, min(len, (split+1)*chunk)) added with
+// eight loads in flight.  grid = (column blocks, splits, min(outer, 65535)).
+template <typename T>
+__global__ __launch_bounds__(256) void fold_cols_kernel(const float *__restrict__ x, float *__restrict__ out,
+                                                        size_t outer, size_t len, size_t inner_t, size_t chunk,
+                                                        float scale, int apply_scale)
+{
+    const size_t col = blockIdx.x * 256ull + threadIdx.x;
+    if (col >= inner_t) return;
+    const unsigned sp = blockIdx.y, splits = gridDim.y;
+    const size_t r0 = (size_t)sp * chunk, r1 = r0 + chunk < len ? r0 + chunk : len;
+    for (size_t o = blockIdx.z; o < outer; o += gridDim.z) {
+        const T *p = reinterpret_cast<const T *>(x) + (o * len + r0) * inner_t + col;
+        T acc0 = vec_zero<T>(), acc1 = vec_zero<T>();
+        size_t r = r0;
+        constexpr int U = 8;
+        for (; r + U <= r1; r += U) {
+            T v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = ld_stream(p + u * inner_t);
+            acc0 = vadd(acc0, vadd(vadd(v[0], v[1]), vadd(v[2], v[3])));
+            acc1 = vadd(acc1, vadd(vadd(v[4], v[5]), vadd(v[6], v[7])));
+            p += U * inner_t;
+        }
+        for (; r < r1; ++r, p += inner_t) acc0 = vadd(acc0, ld_stream(p));
+        T sum = vadd(acc0, acc1);
+        if (apply_scale) sum = vscale(sum, scale);
+        reinterpret_cast<T *>(out)[(o * splits + sp) * inner_t + col] = sum;
     }
 }
 
@@ -277,6 +435,185 @@ static void reduce_ws_layout(const int *shape, int rank, const int *sorted_axes,
     }
 }
 
+// ---- plan of the streaming folds -----------------------------------------------------------------
+constexpr size_t kStreamMinElements = (size_t)1 << 20;
+constexpr size_t kStreamBlocks = 2048;  // blocks a fold is split into, at least, when its shape allows
+
+struct StreamStep {
+    int kind;  // 0: lanes per row; 1: blocks per row, then 0 over the partials; 2: thread per column
+    size_t outer, len, inner;
+    unsigned splits;
+    size_t chunk;
+};
+struct StreamPlan {
+    int n_steps;
+    StreamStep step[kMaxRank];
+    bool scalar;      // every element is folded: the whole-array sum
+    size_t pingpong;  // floats of each of the two intermediate buffers
+    size_t partial;   // floats for the partial sums of split folds
+};
+
+static size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+
+static void plan_step(StreamStep *st)
+{
+    st->splits = 1;
+    st->chunk = st->len;
+    if (st->inner == 1) {
+        st->kind = 0;
+        if (st->len >= 16384 && st->outer < kStreamBlocks) {
+            size_t sp = ceil_div(kStreamBlocks, st->outer);
+            if (sp > st->len / 4096) sp = st->len / 4096;
+            if (sp >= 2) {
+                st->kind = 1;
+                st->chunk = (ceil_div(st->len, sp) + 3) & ~(size_t)3;
+                st->splits = (unsigned)ceil_div(st->len, st->chunk);
+            }
+        }
+    } else {
+        st->kind = 2;
+        const size_t inner_t = st->inner % 4 == 0 ? st->inner / 4 : st->inner;
+        const size_t blocks = ceil_div(inner_t, 256) * (st->outer < 65535 ? st->outer : 65535);
+        size_t sp = ceil_div(kStreamBlocks, blocks);
+        if (sp > st->len / 16) sp = st->len / 16;
+        if (sp > 65535) sp = 65535;
+        if (sp >= 2) {
+            st->chunk = ceil_div(st->len, sp);
+            st->splits = (unsigned)ceil_div(st->len, st->chunk);
+        }
+    }
+}
+
+// False when the input is small or nothing is folded: the sequential folds handle those.
+static bool plan_stream(const int *shape, int rank, const int *sorted_axes, int n_axes, StreamPlan *pl)
+{
+    size_t total = 1;
+    for (int i = 0; i < rank; ++i) total *= (size_t)shape[i];
+    if (n_axes == 0 || total < kStreamMinElements) return false;
+    size_t ext[kMaxRank];
+    bool red[kMaxRank];
+    int ng = 0;
+    bool any = false;
+    for (int i = 0; i < rank; ++i) {
+        if (shape[i] == 1) continue;
+        bool r = false;
+        for (int j = 0; j < n_axes; ++j) r |= sorted_axes[j] == i;
+        any |= r;
+        if (ng > 0 && red[ng - 1] == r) {
+            ext[ng - 1] *= (size_t)shape[i];
+        } else {
+            ext[ng] = (size_t)shape[i];
+            red[ng] = r;
+            ++ng;
+        }
+    }
+    if (!any) return false;
+    pl->n_steps = 0;
+    pl->pingpong = pl->partial = 0;
+    pl->scalar = ng == 1;
+    if (pl->scalar) {
+        pl->partial = kSumBlocks;
+        return true;
+    }
+    for (;;) {
+        int j = -1, left = 0;
+        for (int g = 0; g < ng; ++g)
+            if (red[g]) {
+                j = g;
+                ++left;
+            }
+        if (j < 0) break;
+        StreamStep st{};
+        st.outer = st.inner = 1;
+        for (int g = 0; g < j; ++g) st.outer *= ext[g];
+        for (int g = j + 1; g < ng; ++g) st.inner *= ext[g];
+        st.len = ext[j];
+        plan_step(&st);
+        const size_t result = st.outer * st.inner;
+        if (left > 1 && ((result + 3) & ~(size_t)3) > pl->pingpong) pl->pingpong = (result + 3) & ~(size_t)3;
+        if (st.splits > 1 && result * st.splits > pl->partial) pl->partial = result * st.splits;
+        pl->step[pl->n_steps++] = st;
+        // drop the folded group; the kept groups on either side become one
+        int w = 0;
+        for (int g = 0; g < ng; ++g) {
+            if (g == j) continue;
+            if (w > 0 && red[w - 1] == red[g]) {
+                ext[w - 1] *= ext[g];
+            } else {
+                ext[w] = ext[g];
+                red[w] = red[g];
+                ++w;
+            }
+        }
+        ng = w;
+    }
+    return true;
+}
+
+static void launch_fold_rows(hipStream_t st, const float *src, float *dst, size_t rows, size_t len, float scale, int sc)
+{
+    const bool vec = len % 4 == 0 && aligned16(src);
+    const size_t lanes = vec ? len / 4 : len;
+    const int G = lanes >= 32 ? 64 : lanes >= 8 ? 16 : 4;
+    const dim3 grid((unsigned)ceil_div(rows * (size_t)G, 256)), block(256);
+#define AG_FOLD_ROWS(GG)                                                                                               \
+    do {                                                                                                               \
+        if (vec) hipLaunchKernelGGL((fold_rows_kernel<GG, true>), grid, block, 0, st, src, dst, rows, len, scale, sc);  \
+        else hipLaunchKernelGGL((fold_rows_kernel<GG, false>), grid, block, 0, st, src, dst, rows, len, scale, sc);     \
+    } while (0)
+    if (G == 64) AG_FOLD_ROWS(64);
+    else if (G == 16) AG_FOLD_ROWS(16);
+    else AG_FOLD_ROWS(4);
+#undef AG_FOLD_ROWS
+}
+
+static void launch_fold_cols(hipStream_t st, const float *src, float *dst, size_t outer, size_t len, size_t inner,
+                             unsigned splits, size_t chunk, float scale, int sc)
+{
+    const bool vec = inner % 4 == 0 && aligned16(src) && aligned16(dst);
+    const size_t inner_t = vec ? inner / 4 : inner;
+    const dim3 grid((unsigned)ceil_div(inner_t, 256), splits, (unsigned)(outer < 65535 ? outer : 65535)), block(256);
+    if (vec) hipLaunchKernelGGL((fold_cols_kernel<float4>), grid, block, 0, st, src, dst, outer, len, inner_t, chunk, scale, sc);
+    else hipLaunchKernelGGL((fold_cols_kernel<float>), grid, block, 0, st, src, dst, outer, len, inner_t, chunk, scale, sc);
+}
+
+static void run_stream(hipStream_t st, const StreamPlan &pl, const float *x, size_t total, float *out, float *ws,
+                       float scale, int do_scale)
+{
+    float *buf[2] = {ws, ws + pl.pingpong};
+    float *part = ws + 2 * pl.pingpong;
+    if (pl.scalar) {
+        size_t blocks = ceil_div(total, kSumThreads * 16);
+        if (blocks > (size_t)kSumBlocks) blocks = kSumBlocks;
+        hipLaunchKernelGGL(sum_stage1_kernel, dim3((unsigned)blocks), dim3(kSumThreads), 0, st, x, total, part);
+        hipLaunchKernelGGL(sum_stage2_kernel, dim3(1), dim3(kSumThreads), 0, st, part, (int)blocks,
+                           do_scale ? scale : 1.0f, out);
+        return;
+    }
+    const float *cur = x;
+    for (int i = 0; i < pl.n_steps; ++i) {
+        const StreamStep &s = pl.step[i];
+        const bool last = i == pl.n_steps - 1;
+        float *dst = last ? out : buf[i & 1];
+        const int sc = last ? do_scale : 0;
+        if (s.kind == 0) {
+            launch_fold_rows(st, cur, dst, s.outer, s.len, scale, sc);
+        } else if (s.kind == 1) {
+            const bool vec = s.len % 4 == 0 && aligned16(cur);
+            const dim3 grid((unsigned)(s.outer * s.splits)), block(256);
+            if (vec) hipLaunchKernelGGL((fold_rows_split_kernel<true>), grid, block, 0, st, cur, part, s.len, s.splits, s.chunk);
+            else hipLaunchKernelGGL((fold_rows_split_kernel<false>), grid, block, 0, st, cur, part, s.len, s.splits, s.chunk);
+            launch_fold_rows(st, part, dst, s.outer, s.splits, scale, sc);
+        } else if (s.splits > 1) {
+            launch_fold_cols(st, cur, part, s.outer, s.len, s.inner, s.splits, s.chunk, 1.f, 0);
+            launch_fold_cols(st, part, dst, s.outer, s.splits, s.inner, 1, s.splits, scale, sc);
+        } else {
+            launch_fold_cols(st, cur, dst, s.outer, s.len, s.inner, 1, s.len, scale, sc);
+        }
+        cur = dst;
+    }
+}
+
 extern "C" size_t ag_reduce_sum_f32_workspace(const int *shape, int rank, const int *axes, int n_axes)
 {
     int ax[kMaxRank];
@@ -293,7 +630,10 @@ extern "C" size_t ag_reduce_sum_f32_workspace(const int *shape, int rank, const 
         }
     size_t pp, sf;
     reduce_ws_layout(shape, rank, ax, n_axes, &pp, &sf);
-    return sizeof(float) * (2 * pp + sf) + 32;
+    size_t floats = 2 * pp + sf;
+    StreamPlan pl;
+    if (plan_stream(shape, rank, ax, n_axes, &pl) && 2 * pl.pingpong + pl.partial > floats) floats = 2 * pl.pingpong + pl.partial;
+    return sizeof(float) * floats + 32;
 }
 
 extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, float *out,
@@ -326,6 +666,22 @@ extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, flo
         hipLaunchKernelGGL(scale_copy_kernel, dim3(grid_for(total, 256)), dim3(256), 0, st, x, out, total,
                            1.f, 0);
         return check_launch("reduce_sum");
+    }
+    StreamPlan pl;
+    if (plan_stream(shape, rank, ax, n_axes, &pl)) {
+        const size_t need = sizeof(float) * (2 * pl.pingpong + pl.partial);
+        AG_REQUIRE(need == 0 || (ws && ws_bytes >= need), AG_ERR_INVALID_DIMS,
+                   "reduce_sum: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+        bool fits = true;  // launch limits of the streaming kernels
+        for (int i = 0; i < pl.n_steps; ++i) {
+            const StreamStep &s = pl.step[i];
+            const size_t blocks = s.kind == 0 ? ceil_div(s.outer, 4) : s.kind == 1 ? s.outer * s.splits : ceil_div(s.inner, 256);
+            fits &= blocks < (size_t)kMaxGridX;
+        }
+        if (fits) {
+            run_stream(st, pl, x, total, out, static_cast<float *>(ws), scale, do_scale);
+            return check_launch(mean ? "reduce_mean" : "reduce_sum");
+        }
     }
     size_t pp, sf;
     reduce_ws_layout(shape, rank, ax, n_axes, &pp, &sf);

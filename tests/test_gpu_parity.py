@@ -653,6 +653,53 @@ def test_reduce_large_rows_and_columns(K, rng):
     assert_close(host(K.reduce_sum(dev(x), [0])), x.astype(np.float64).sum(0), "column sums")
 
 
+STREAM_CASES = [
+    ((1 << 20,), [0]), ((3 << 19,), [0]), ((1048583,), [0]),                 # everything folded
+    ((2048, 1024), [1]), ((2048, 1024), [0]), ((2048, 1031), [1]), ((2050, 1031), [0]),
+    ((40000, 56), [1]), ((30000, 37), [1]), ((300000, 6), [1]), ((200000, 8), [1]),   # short trailing rows
+    ((3, 400000), [1]), ((7, 300001), [1]),                                  # few long rows: split over blocks
+    ((4096, 512), [0]), ((20000, 64), [0]), ((100000, 12), [0]), ((600000, 2), [0]),  # leading fold, wide to narrow
+    ((32, 64, 28, 28), [0, 2, 3]), ((32, 64, 28, 28), [1]), ((32, 64, 28, 28), [2, 3]), ((32, 64, 28, 28), [0]),
+    ((32, 64, 28, 28), [3]), ((32, 64, 28, 28), [0, 1]), ((32, 64, 28, 28), [1, 3]), ((32, 64, 28, 28), [0, 1, 2, 3]),
+    ((16, 1, 33, 1, 2049), [0, 4]), ((5, 70000, 3), [1]), ((70000, 5, 3), [0, 2]),
+]
+
+
+@pytest.mark.parametrize("shape,axes", STREAM_CASES)
+def test_reduce_large_inputs(K, rng, shape, axes):
+    # 2^20 elements and more: neighbouring axes merged, streaming folds; agreement with the f64 sum to
+    # f32 rounding of a pairwise-like order (far inside 1e-4 of the sum of magnitudes)
+    x = rng.standard_normal(shape).astype(np.float32)
+    say("reduce large", shape, axes)
+    ax = tuple(axes)
+    for mean, keep in ((False, False), (True, True)):
+        got = host(K.reduce_sum(dev(x), axes, keep, mean))
+        truth = x.astype(np.float64).sum(axis=ax, keepdims=keep)
+        cond = np.abs(x).astype(np.float64).sum(axis=ax, keepdims=keep)
+        if mean:
+            n = float(np.prod([shape[a] for a in ax]))
+            truth, cond = truth / n, cond / n
+        assert got.shape == truth.shape
+        assert_close_conditioned(got, truth, cond, f"reduce {shape} {axes} mean={mean}")
+    # small integers add exactly in f32 in any order: every element is counted once, in the right output
+    xi = rng.integers(-8, 9, size=shape).astype(np.float32)
+    exact = xi.astype(np.int64).sum(axis=ax).astype(np.float32)
+    assert np.array_equal(host(K.reduce_sum(dev(xi), axes)), exact)
+    n = np.float32(np.prod([shape[a] for a in ax], dtype=np.float64))
+    assert np.array_equal(host(K.reduce_mean(dev(xi), axes)), exact * (np.float32(1) / n))
+
+
+def test_reduce_large_input_from_an_unaligned_view(K, rng):
+    # a 4-byte-aligned start address: the 128-bit paths must not be taken
+    base = dev(rng.standard_normal(3 + 2048 * 1024).astype(np.float32))
+    x = base[3:].view(2048, 1024)
+    say("reduce large unaligned")
+    xh = host(x).astype(np.float64)
+    for axes in ([0], [1], [0, 1]):
+        got = host(K.reduce_sum(x, axes))
+        assert_close_conditioned(got, xh.sum(axis=tuple(axes)), np.abs(xh).sum(axis=tuple(axes)), f"unaligned {axes}")
+
+
 def test_broadcast_grad(K, orc, rng):
     gy = rng.standard_normal((3, 1, 5, 1)).astype(np.float32)
     say("broadcast_grad")
