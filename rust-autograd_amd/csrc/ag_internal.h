@@ -47,6 +47,9 @@ __device__ inline void st_stream(float *p, float v) { __builtin_nontemporal_stor
 __device__ inline void st_stream(int *p, int v) { __builtin_nontemporal_store(v, p); }
 #endif
 
+// Validates reduction axes (range, rank <= 8) and writes them to `sorted` in ascending order.
+ag_status_t check_axes(const char *who, const int *shape, int rank, const int *axes, int n_axes, int *sorted);
+
 }  // namespace ag
 
 #define AG_REQUIRE(cond, code, ...)                      \

@@ -18,53 +18,172 @@ static unsigned ew_grid(size_t n, int per_thread)
 #define AG_EW_LOOP(i, n) \
     for (size_t i = blockIdx.x * 256ull + threadIdx.x; i < (n); i += gridDim.x * 256ull)
 
-// activation_ops.rs:155-159  x.max(0)  (f32::max: NaN input yields 0)
-__global__ __launch_bounds__(256) void relu_kernel(const float *__restrict__ x, float *__restrict__ y,
-                                                   size_t n)
+// Every streaming elementwise operator is a functor with `one(i)` (element i) and `vec(q)` (elements
+// 4q..4q+3 through 128-bit streaming loads and stores).  With 16-byte aligned operands each thread
+// of a one-shot grid handles one group of four, and one thread finishes a partial last group
+// (copy-like kernels measured 6.2-6.7 TB/s this way on MI355X against 4.6-5.7 TB/s for scalar
+// grid-strided loops); otherwise one element per thread, grid-strided.
+template <typename F>
+__global__ __launch_bounds__(256) void ew_vec_kernel(size_t n4, size_t n, F f)
 {
-    AG_EW_LOOP(i, n) { const float v = x[i]; y[i] = v > 0.f ? v : 0.f; }
+    const size_t i = blockIdx.x * 256ull + threadIdx.x;
+    if (i < n4) {
+        f.vec(i);
+    } else if (i == n4) {
+        for (size_t e = n4 * 4; e < n; ++e) f.one(e);
+    }
 }
+
+template <typename F>
+__global__ __launch_bounds__(256) void ew_scalar_kernel(size_t n, F f)
+{
+    AG_EW_LOOP(i, n) f.one(i);
+}
+
+__device__ inline const float4 *as4(const float *p) { return reinterpret_cast<const float4 *>(p); }
+__device__ inline float4 *as4(float *p) { return reinterpret_cast<float4 *>(p); }
+
+// activation_ops.rs:155-159  x.max(0)  (f32::max: NaN input yields 0)
+struct ReluF {
+    const float *x;
+    float *y;
+    static __device__ float f(float v) { return v > 0.f ? v : 0.f; }
+    __device__ void one(size_t i) const { y[i] = f(x[i]); }
+    __device__ void vec(size_t q) const
+    {
+        const float4 v = ld_stream(as4(x) + q);
+        st_stream(as4(y) + q, make_float4(f(v.x), f(v.y), f(v.z), f(v.w)));
+    }
+};
 
 // activation_ops.rs:161-166  greater(x, 0) * gy
-__global__ __launch_bounds__(256) void relu_grad_kernel(const float *__restrict__ x,
-                                                        const float *__restrict__ gy,
-                                                        float *__restrict__ gx, size_t n)
-{
-    AG_EW_LOOP(i, n) gx[i] = (x[i] > 0.f ? 1.f : 0.f) * gy[i];
-}
+struct ReluGradF {
+    const float *x, *gy;
+    float *gx;
+    static __device__ float f(float v, float g) { return (v > 0.f ? 1.f : 0.f) * g; }
+    __device__ void one(size_t i) const { gx[i] = f(x[i], gy[i]); }
+    __device__ void vec(size_t q) const
+    {
+        const float4 v = ld_stream(as4(x) + q), g = ld_stream(as4(gy) + q);
+        st_stream(as4(gx) + q, make_float4(f(v.x, g.x), f(v.y, g.y), f(v.z, g.z), f(v.w, g.w)));
+    }
+};
 
-__global__ __launch_bounds__(256) void add_bias_kernel(const float *__restrict__ x,
-                                                       const float *__restrict__ bias,
-                                                       float *__restrict__ y, size_t n, size_t cols)
-{
-    AG_EW_LOOP(i, n) y[i] = x[i] + bias[i % cols];
-}
+struct PtrPack {
+    const float *p[8];
+};
 
-// Right operand broadcast along any of its axes of extent 1.  `dims` are the left operand's extents
-// after adjacent axes with the same broadcast state have been merged (outermost first), `bstride`
-// the right operand's element stride for each merged axis (0 where it is broadcast).
+// array_ops.rs:503-535  ((x0 + x1) + x2) + ...
+struct AddNF {
+    PtrPack xs;
+    int count;
+    float *out;
+    __device__ void one(size_t i) const
+    {
+        float acc = xs.p[0][i];
+        for (int j = 1; j < count; ++j) acc += xs.p[j][i];
+        out[i] = acc;
+    }
+    __device__ void vec(size_t q) const
+    {
+        float4 acc = ld_stream(as4(xs.p[0]) + q);
+        for (int j = 1; j < count; ++j) {
+            const float4 v = ld_stream(as4(xs.p[j]) + q);
+            acc.x += v.x;
+            acc.y += v.y;
+            acc.z += v.z;
+            acc.w += v.w;
+        }
+        st_stream(as4(out) + q, acc);
+    }
+};
+
+struct MulF {
+    const float *a, *b;
+    float *out;
+    __device__ void one(size_t i) const { out[i] = a[i] * b[i]; }
+    __device__ void vec(size_t q) const
+    {
+        const float4 u = ld_stream(as4(a) + q), v = ld_stream(as4(b) + q);
+        st_stream(as4(out) + q, make_float4(u.x * v.x, u.y * v.y, u.z * v.z, u.w * v.w));
+    }
+};
+
+template <bool DIVIDE>
+struct ScaleF {
+    const float *a;
+    float s;
+    float *out;
+    __device__ float f(float v) const { return DIVIDE ? v / s : v * s; }
+    __device__ void one(size_t i) const { out[i] = f(a[i]); }
+    __device__ void vec(size_t q) const
+    {
+        const float4 v = ld_stream(as4(a) + q);
+        st_stream(as4(out) + q, make_float4(f(v.x), f(v.y), f(v.z), f(v.w)));
+    }
+};
+
+struct FillF {
+    float *out;
+    float v;
+    __device__ void one(size_t i) const { out[i] = v; }
+    __device__ void vec(size_t q) const { st_stream(as4(out) + q, make_float4(v, v, v, v)); }
+};
+
+// Broadcast of an operand `b` along its axes of extent 1.  `dims` are the result's extents after
+// neighbouring axes with the same broadcast state have been merged (outermost first), `bstride` the
+// stride of `b` for each merged axis in elements (0 where it is broadcast).
 struct BroadcastGeom {
-    unsigned dims[6];
-    unsigned bstride[6];
+    unsigned dims[8];
+    unsigned bstride[8];
     int rank;
 };
 
-__global__ __launch_bounds__(256) void add_broadcast_kernel(const float *__restrict__ x,
-                                                            const float *__restrict__ b,
-                                                            float *__restrict__ y, size_t n, BroadcastGeom g)
-{
-    AG_EW_LOOP(i, n)
+// ADD: y = x + b (AddOp, binary_ops.rs:147-166, 304-346); otherwise y = b (ReduceGradCommon,
+// reduction_ops.rs:459-512).  I = unsigned when the result has fewer than 2^32 elements.  `vec`
+// needs an innermost merged extent that is a multiple of 4.
+template <bool ADD, typename I>
+struct BroadcastF {
+    const float *x, *b;
+    float *y;
+    BroadcastGeom g;
+    __device__ void one(size_t i) const
     {
-        size_t rest = i, bi = 0;
+        I rest = (I)i, bi = 0;
         for (int d = g.rank - 1; d > 0; --d) {
-            const size_t q = rest / g.dims[d];
+            const I q = rest / g.dims[d];
             bi += (rest - q * g.dims[d]) * g.bstride[d];
             rest = q;
         }
         bi += rest * g.bstride[0];
-        y[i] = x[i] + b[bi];
+        y[i] = ADD ? x[i] + b[bi] : b[bi];
     }
-}
+    __device__ void vec(size_t q4) const
+    {
+        const int last = g.rank - 1;
+        const I inner4 = g.dims[last] >> 2;
+        I rest = (I)q4 / inner4;
+        I bi = ((I)q4 - rest * inner4) * 4 * g.bstride[last];
+        for (int d = last - 1; d > 0; --d) {
+            const I q = rest / g.dims[d];
+            bi += (rest - q * g.dims[d]) * g.bstride[d];
+            rest = q;
+        }
+        if (last > 0) bi += rest * g.bstride[0];
+        float4 bv;
+        if (g.bstride[last] == 0) {
+            const float s = b[bi];
+            bv = make_float4(s, s, s, s);
+        } else {
+            bv = *reinterpret_cast<const float4 *>(b + bi);
+        }
+        if (ADD) {
+            const float4 v = ld_stream(as4(x) + q4);
+            bv = make_float4(v.x + bv.x, v.y + bv.y, v.z + bv.z, v.w + bv.w);
+        }
+        st_stream(as4(y) + q4, bv);
+    }
+};
 
 // out[c] = sum over rows, ascending (ndarray sum_axis(0) order used by MaybeReduceSum).
 __global__ __launch_bounds__(256) void bias_grad_kernel(const float *__restrict__ gy,
@@ -72,47 +191,20 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const float *__restrict_
 {
     AG_EW_LOOP(c, cols)
     {
+        // eight loads in flight, added in row order
         float acc = 0.f;
-        for (size_t r = 0; r < rows; ++r) acc += gy[r * cols + c];
+        const float *p = gy + c;
+        size_t r = 0;
+        for (; r + 8 <= rows; r += 8, p += 8 * cols) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = p[u * cols];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; r < rows; ++r, p += cols) acc += *p;
         out[c] = acc;
     }
-}
-
-struct PtrPack {
-    const float *p[8];
-};
-
-__global__ __launch_bounds__(256) void add_n_kernel(PtrPack xs, int count, float *__restrict__ out, size_t n)
-{
-    AG_EW_LOOP(i, n)
-    {
-        float acc = xs.p[0][i];
-        for (int j = 1; j < count; ++j) acc += xs.p[j][i];
-        out[i] = acc;
-    }
-}
-
-__global__ __launch_bounds__(256) void mul_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                  float *__restrict__ out, size_t n)
-{
-    AG_EW_LOOP(i, n) out[i] = a[i] * b[i];
-}
-
-__global__ __launch_bounds__(256) void scale_kernel(const float *__restrict__ a, float s,
-                                                    float *__restrict__ out, size_t n)
-{
-    AG_EW_LOOP(i, n) out[i] = a[i] * s;
-}
-
-__global__ __launch_bounds__(256) void div_scalar_kernel(const float *__restrict__ a, float s,
-                                                         float *__restrict__ out, size_t n)
-{
-    AG_EW_LOOP(i, n) out[i] = a[i] / s;
-}
-
-__global__ __launch_bounds__(256) void fill_kernel(float *__restrict__ out, float v, size_t n)
-{
-    AG_EW_LOOP(i, n) out[i] = v;
 }
 
 // One thread per row (class counts are small): log_softmax = x - (ln(sum exp(x - max)) + max),
@@ -142,6 +234,49 @@ __global__ __launch_bounds__(256) void sparse_xent_kernel(const float *__restric
     }
 }
 
+// The same arithmetic with the 256 rows of a block staged through LDS (row pitch odd, so the
+// per-row scans are free of bank conflicts): global loads and stores are then contiguous across
+// the wave instead of one row apart.  For up to 63 classes.
+__global__ __launch_bounds__(256) void sparse_xent_lds_kernel(const float *__restrict__ logits,
+                                                              const float *__restrict__ labels,
+                                                              float *__restrict__ loss,
+                                                              float *__restrict__ lsm, size_t rows,
+                                                              unsigned classes, unsigned pitch)
+{
+    extern __shared__ float tile[];
+    const size_t r0 = blockIdx.x * 256ull;
+    const unsigned nrows = rows - r0 < 256 ? (unsigned)(rows - r0) : 256u;
+    const unsigned count = nrows * classes;
+    const float *src = logits + r0 * classes;
+    float *dst = lsm + r0 * classes;
+    for (unsigned e = threadIdx.x; e < count; e += 256) {
+        const unsigned r = e / classes;
+        tile[r * pitch + (e - r * classes)] = src[e];
+    }
+    __syncthreads();
+    if (threadIdx.x < nrows) {
+        float *row = tile + threadIdx.x * pitch;
+        float mx = -FLT_MAX;
+        for (unsigned c = 0; c < classes; ++c) mx = fmaxf(mx, row[c]);
+        float s = 0.f;
+        for (unsigned c = 0; c < classes; ++c) s += expf(row[c] - mx);
+        const float lse = logf(s) + mx;
+        const size_t label = (size_t)labels[r0 + threadIdx.x];
+        float picked = 0.f;
+        for (unsigned c = 0; c < classes; ++c) {
+            const float v = row[c] - lse;
+            row[c] = v;
+            if (c == label) picked = v;
+        }
+        loss[r0 + threadIdx.x] = -picked;
+    }
+    __syncthreads();
+    for (unsigned e = threadIdx.x; e < count; e += 256) {
+        const unsigned r = e / classes;
+        dst[e] = tile[r * pitch + (e - r * classes)];
+    }
+}
+
 // xent_ops.rs:139-153  (exp(log_softmax) - onehot(label)) * gy[row]
 __global__ __launch_bounds__(256) void sparse_xent_grad_kernel(const float *__restrict__ lsm,
                                                                const float *__restrict__ labels,
@@ -163,48 +298,30 @@ __global__ __launch_bounds__(256) void sparse_xent_grad_kernel(const float *__re
 
 using namespace ag;
 
-#define AG_EW_ENTRY(name, kernel, nexpr, ...)                                                     \
-    do {                                                                                          \
-        const size_t n__ = (nexpr);                                                               \
-        if (n__ == 0) return AG_OK;                                                               \
-        hipLaunchKernelGGL(kernel, dim3(ew_grid(n__, 4)), dim3(256), 0, as_stream(stream), __VA_ARGS__); \
-        return check_launch(name);                                                                \
-    } while (0)
-
-extern "C" ag_status_t ag_relu_f32(ag_stream_t stream, const float *x, float *y, size_t n)
+template <typename F>
+static ag_status_t ew_launch(const char *name, ag_stream_t stream, size_t n, bool vec, const F &f)
 {
-    AG_REQUIRE(n == 0 || (x && y), AG_ERR_INVALID_DIMS, "relu: null pointer");
-    AG_EW_ENTRY("relu", relu_kernel, n, x, y, n);
+    if (n == 0) return AG_OK;
+    const size_t n4 = n / 4, blocks = (n4 + 256) / 256;  // n4 + 1 threads: the last finishes a partial group
+    if (vec && blocks <= (size_t)kMaxGridX)
+        hipLaunchKernelGGL((ew_vec_kernel<F>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), n4, n, f);
+    else
+        hipLaunchKernelGGL((ew_scalar_kernel<F>), dim3(ew_grid(n, 4)), dim3(256), 0, as_stream(stream), n, f);
+    return check_launch(name);
 }
 
-extern "C" ag_status_t ag_relu_grad_f32(ag_stream_t stream, const float *x, const float *gy, float *gx,
-                                        size_t n)
+// Merges neighbouring axes with the same broadcast state (axes of extent 1 join either kind).
+static ag_status_t make_broadcast_geom(const char *who, const int *shape, const int *bshape, int rank,
+                                       BroadcastGeom *g, size_t *n_out)
 {
-    AG_REQUIRE(n == 0 || (x && gy && gx), AG_ERR_INVALID_DIMS, "relu_grad: null pointer");
-    AG_EW_ENTRY("relu_grad", relu_grad_kernel, n, x, gy, gx, n);
-}
-
-extern "C" ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const float *bias, float *y,
-                                       size_t rows, size_t cols)
-{
-    AG_REQUIRE(rows * cols == 0 || (x && bias && y), AG_ERR_INVALID_DIMS, "add: null pointer");
-    AG_EW_ENTRY("add", add_bias_kernel, rows * cols, x, bias, y, rows * cols, cols);
-}
-
-extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
-                                            const int *shape, const int *bshape, int rank)
-{
-    AG_REQUIRE(rank >= 1 && rank <= 8 && shape && bshape, AG_ERR_INVALID_DIMS, "add: rank %d not in 1..8", rank);
+    AG_REQUIRE(rank >= 0 && rank <= 8 && (rank == 0 || (shape && bshape)), AG_ERR_INVALID_DIMS, "%s: rank %d not in 0..8", who, rank);
     size_t n = 1;
     for (int i = 0; i < rank; ++i) {
         AG_REQUIRE(shape[i] >= 0 && (bshape[i] == shape[i] || bshape[i] == 1), AG_ERR_INCOMPATIBLE_SHAPE,
-                   "add: axis %d of the right operand has extent %d, the left %d", i, bshape[i], shape[i]);
+                   "%s: axis %d of the broadcast operand has extent %d, the result %d", who, i, bshape[i], shape[i]);
         n *= (size_t)shape[i];
     }
-    if (n == 0) return AG_OK;
-    AG_REQUIRE(x && b && y, AG_ERR_INVALID_DIMS, "add: null pointer");
-    // merge neighbours with the same broadcast state; axes of extent 1 join either kind
-    BroadcastGeom g{};
+    *n_out = n;
     bool prev_bc = false;
     size_t bstride = 1;
     unsigned rev_dims[8], rev_bstride[8];
@@ -213,7 +330,7 @@ extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, 
         if (shape[i] == 1) continue;
         const bool bc = bshape[i] == 1;
         if (groups > 0 && bc == prev_bc) {
-            AG_REQUIRE((size_t)rev_dims[groups - 1] * (size_t)shape[i] <= 0xffffffffu, AG_ERR_INVALID_DIMS, "add: extent too large");
+            AG_REQUIRE((size_t)rev_dims[groups - 1] * (size_t)shape[i] <= 0xffffffffu, AG_ERR_INVALID_DIMS, "%s: extent too large", who);
             rev_dims[groups - 1] *= (unsigned)shape[i];
         } else {
             rev_dims[groups] = (unsigned)shape[i];
@@ -223,13 +340,76 @@ extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, 
         if (!bc) bstride *= (size_t)shape[i];
         prev_bc = bc;
     }
-    AG_REQUIRE(groups <= 6 && bstride <= 0xffffffffu, AG_ERR_INVALID_DIMS, "add: broadcast pattern with %d groups of axes not supported", groups);
+    AG_REQUIRE(bstride <= 0xffffffffu, AG_ERR_INVALID_DIMS, "%s: operand too large", who);
     if (groups == 0) {
         rev_dims[0] = 1, rev_bstride[0] = 0, groups = 1;
     }
-    g.rank = groups;
-    for (int i = 0; i < groups; ++i) g.dims[i] = rev_dims[groups - 1 - i], g.bstride[i] = rev_bstride[groups - 1 - i];
-    AG_EW_ENTRY("add", add_broadcast_kernel, n, x, b, y, n, g);
+    g->rank = groups;
+    for (int i = 0; i < groups; ++i) g->dims[i] = rev_dims[groups - 1 - i], g->bstride[i] = rev_bstride[groups - 1 - i];
+    return AG_OK;
+}
+
+template <bool ADD>
+static ag_status_t launch_broadcast(const char *name, ag_stream_t stream, const float *x, const float *b, float *y,
+                                    const BroadcastGeom &g, size_t n)
+{
+    const int last = g.rank - 1;
+    const bool vec = g.dims[last] % 4 == 0 && aligned16(y) && (!ADD || aligned16(x)) && (g.bstride[last] == 0 || aligned16(b));
+    if (n <= 0xffffffffu) return ew_launch(name, stream, n, vec, BroadcastF<ADD, unsigned>{x, b, y, g});
+    return ew_launch(name, stream, n, vec, BroadcastF<ADD, size_t>{x, b, y, g});
+}
+
+extern "C" ag_status_t ag_relu_f32(ag_stream_t stream, const float *x, float *y, size_t n)
+{
+    AG_REQUIRE(n == 0 || (x && y), AG_ERR_INVALID_DIMS, "relu: null pointer");
+    return ew_launch("relu", stream, n, aligned16(x) && aligned16(y), ReluF{x, y});
+}
+
+extern "C" ag_status_t ag_relu_grad_f32(ag_stream_t stream, const float *x, const float *gy, float *gx,
+                                        size_t n)
+{
+    AG_REQUIRE(n == 0 || (x && gy && gx), AG_ERR_INVALID_DIMS, "relu_grad: null pointer");
+    return ew_launch("relu_grad", stream, n, aligned16(x) && aligned16(gy) && aligned16(gx), ReluGradF{x, gy, gx});
+}
+
+extern "C" ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const float *bias, float *y,
+                                       size_t rows, size_t cols)
+{
+    AG_REQUIRE(rows * cols == 0 || (x && bias && y), AG_ERR_INVALID_DIMS, "add: null pointer");
+    AG_REQUIRE(rows <= 0x7fffffffu && cols <= 0x7fffffffu, AG_ERR_INVALID_DIMS, "add: extent too large");
+    const int shape[2] = {(int)rows, (int)cols}, bshape[2] = {1, (int)cols};
+    BroadcastGeom g{};
+    size_t n;
+    if (ag_status_t s = make_broadcast_geom("add", shape, bshape, 2, &g, &n)) return s;
+    if (n == 0) return AG_OK;
+    return launch_broadcast<true>("add", stream, x, bias, y, g, n);
+}
+
+extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
+                                            const int *shape, const int *bshape, int rank)
+{
+    AG_REQUIRE(rank >= 1, AG_ERR_INVALID_DIMS, "add: rank %d not in 1..8", rank);
+    BroadcastGeom g{};
+    size_t n;
+    if (ag_status_t s = make_broadcast_geom("add", shape, bshape, rank, &g, &n)) return s;
+    if (n == 0) return AG_OK;
+    AG_REQUIRE(x && b && y, AG_ERR_INVALID_DIMS, "add: null pointer");
+    return launch_broadcast<true>("add", stream, x, b, y, g, n);
+}
+
+extern "C" ag_status_t ag_broadcast_grad_f32(ag_stream_t stream, const float *gy, float *gx,
+                                             const int *shape, int rank, const int *axes, int n_axes)
+{
+    int sorted[8], bshape[8];
+    if (ag_status_t s = check_axes("reduce_grad", shape, rank, axes, n_axes, sorted)) return s;
+    for (int d = 0; d < rank; ++d) bshape[d] = shape[d];
+    for (int j = 0; j < n_axes; ++j) bshape[sorted[j]] = 1;
+    BroadcastGeom g{};
+    size_t n;
+    if (ag_status_t s = make_broadcast_geom("reduce_grad", shape, bshape, rank, &g, &n)) return s;
+    if (n == 0) return AG_OK;
+    AG_REQUIRE(gy && gx, AG_ERR_INVALID_DIMS, "reduce_grad: null pointer");
+    return launch_broadcast<false>("reduce_grad", stream, nullptr, gy, gx, g, n);
 }
 
 extern "C" ag_status_t ag_bias_grad_f32(ag_stream_t stream, const float *gy, float *out, size_t rows,
@@ -247,37 +427,49 @@ extern "C" ag_status_t ag_add_n_f32(ag_stream_t stream, const float *const *xs, 
 {
     AG_REQUIRE(count >= 1 && count <= 8, AG_ERR_INVALID_DIMS, "add_n: between 1 and 8 inputs supported, got %d", count);
     AG_REQUIRE(xs && (n == 0 || out), AG_ERR_INVALID_DIMS, "add_n: null pointer");
-    PtrPack pk{};
+    AddNF f{};
+    bool vec = aligned16(out);
     for (int i = 0; i < count; ++i) {
         AG_REQUIRE(xs[i] || n == 0, AG_ERR_INVALID_DIMS, "add_n: input %d is null", i);
-        pk.p[i] = xs[i];
+        f.xs.p[i] = xs[i];
+        vec = vec && aligned16(xs[i]);
     }
-    AG_EW_ENTRY("add_n", add_n_kernel, n, pk, count, out, n);
+    f.count = count;
+    f.out = out;
+    return ew_launch("add_n", stream, n, vec, f);
 }
 
 extern "C" ag_status_t ag_mul_f32(ag_stream_t stream, const float *a, const float *b, float *out, size_t n)
 {
     AG_REQUIRE(n == 0 || (a && b && out), AG_ERR_INVALID_DIMS, "mul: null pointer");
-    AG_EW_ENTRY("mul", mul_kernel, n, a, b, out, n);
+    return ew_launch("mul", stream, n, aligned16(a) && aligned16(b) && aligned16(out), MulF{a, b, out});
 }
 
 extern "C" ag_status_t ag_scale_f32(ag_stream_t stream, const float *a, float s, float *out, size_t n)
 {
     AG_REQUIRE(n == 0 || (a && out), AG_ERR_INVALID_DIMS, "scale: null pointer");
-    AG_EW_ENTRY("scale", scale_kernel, n, a, s, out, n);
+    return ew_launch("scale", stream, n, aligned16(a) && aligned16(out), ScaleF<false>{a, s, out});
 }
 
 extern "C" ag_status_t ag_div_scalar_f32(ag_stream_t stream, const float *a, float s, float *out, size_t n)
 {
     AG_REQUIRE(n == 0 || (a && out), AG_ERR_INVALID_DIMS, "div: null pointer");
-    AG_EW_ENTRY("div", div_scalar_kernel, n, a, s, out, n);
+    return ew_launch("div", stream, n, aligned16(a) && aligned16(out), ScaleF<true>{a, s, out});
 }
 
 extern "C" ag_status_t ag_fill_f32(ag_stream_t stream, float *out, float value, size_t n)
 {
     AG_REQUIRE(n == 0 || out, AG_ERR_INVALID_DIMS, "fill: null pointer");
-    AG_EW_ENTRY("fill", fill_kernel, n, out, value, n);
+    return ew_launch("fill", stream, n, aligned16(out), FillF{out, value});
 }
+
+#define AG_EW_ENTRY(name, kernel, nexpr, ...)                                                     \
+    do {                                                                                          \
+        const size_t n__ = (nexpr);                                                               \
+        if (n__ == 0) return AG_OK;                                                               \
+        hipLaunchKernelGGL(kernel, dim3(ew_grid(n__, 4)), dim3(256), 0, as_stream(stream), __VA_ARGS__); \
+        return check_launch(name);                                                                \
+    } while (0)
 
 extern "C" ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const float *logits,
                                                   const float *labels, float *loss, float *log_softmax,
@@ -288,6 +480,12 @@ extern "C" ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const floa
     AG_REQUIRE(rows == 0 || (logits && labels && loss && log_softmax), AG_ERR_INVALID_DIMS,
                "SparseSoftmaxCrossEntropy: null pointer");
     if (rows == 0) return AG_OK;
+    if (classes <= 63 && (rows + 255) / 256 <= (size_t)kMaxGridX) {
+        const unsigned pitch = (unsigned)classes | 1u;
+        hipLaunchKernelGGL(sparse_xent_lds_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 256 * pitch * sizeof(float),
+                           as_stream(stream), logits, labels, loss, log_softmax, rows, (unsigned)classes, pitch);
+        return check_launch("SparseSoftmaxCrossEntropy");
+    }
     hipLaunchKernelGGL(sparse_xent_kernel, dim3(ew_grid(rows, 1)), dim3(256), 0, as_stream(stream), logits,
                        labels, loss, log_softmax, rows, classes);
     return check_launch("SparseSoftmaxCrossEntropy");

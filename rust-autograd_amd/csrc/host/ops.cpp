@@ -704,7 +704,15 @@ struct MaybeReduceSum : Op {
         if (broadcasts_over_rows(gy.shape(), x.shape())) {
             NdArray out = NdArray::empty(x.shape());
             const size_t rows = (size_t)gy.shape()[0];
-            const OpError e = from_status(ag_bias_grad_f32(ctx.stream(), gy.ptr(), out.ptr(), rows, gy.len() / rows));
+            OpError e;
+            if (gy.len() >= ((size_t)1 << 20) && rows <= 0x7fffffff && gy.len() / rows <= 0x7fffffff) {
+                // large gradients: the streaming fold over axis 0 instead of one sequential chain per column
+                const int shape[2] = {(int)rows, (int)(gy.len() / rows)}, axis = 0;
+                NdArray ws = workspace(ag_reduce_sum_f32_workspace(shape, 2, &axis, 1));
+                e = from_status(ag_reduce_sum_f32(ctx.stream(), gy.ptr(), out.ptr(), shape, 2, &axis, 1, 0, ws.ptr(), ws.len() * 4));
+            } else {
+                e = from_status(ag_bias_grad_f32(ctx.stream(), gy.ptr(), out.ptr(), rows, gy.len() / rows));
+            }
             if (!e.ok()) return e;
             ctx.append_output(out);
             return OpError::none();

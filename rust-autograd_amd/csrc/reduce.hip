@@ -311,28 +311,6 @@ __global__ __launch_bounds__(256) void scale_copy_kernel(const float *__restrict
         out[i] = apply_scale ? x[i] * scale : x[i];
 }
 
-struct BroadcastShape {
-    int rank;
-    int dim[kMaxRank];       // extents of gx
-    long long gstride[kMaxRank];  // stride of that axis inside gy (0 for reduced axes)
-};
-
-__global__ __launch_bounds__(256) void broadcast_kernel(const float *__restrict__ gy,
-                                                        float *__restrict__ gx, BroadcastShape s,
-                                                        size_t total)
-{
-    for (size_t flat = blockIdx.x * 256ull + threadIdx.x; flat < total; flat += gridDim.x * 256ull) {
-        size_t rem = flat;
-        long long src = 0;
-        for (int d = s.rank - 1; d >= 0; --d) {
-            const size_t c = rem % (size_t)s.dim[d];
-            rem /= (size_t)s.dim[d];
-            src += (long long)c * s.gstride[d];
-        }
-        gx[flat] = gy[src];
-    }
-}
-
 // Split a long fold with few outputs so that the whole chip takes part.  Returns the number of
 // splits (1 = no split) and the rows per split.
 static size_t fold_splits(size_t outer, size_t len, size_t inner, size_t *chunk)
@@ -354,7 +332,7 @@ static unsigned grid_for(size_t work_items, int per_block)
     return (unsigned)b;
 }
 
-static ag_status_t check_axes(const char *who, const int *shape, int rank, const int *axes, int n_axes,
+ag_status_t check_axes(const char *who, const int *shape, int rank, const int *axes, int n_axes,
                               int *sorted)
 {
     AG_REQUIRE(rank >= 0 && rank <= kMaxRank, AG_ERR_INVALID_DIMS, "%s: rank %d not in [0,%d]", who, rank, kMaxRank);
@@ -717,28 +695,4 @@ extern "C" ag_status_t ag_reduce_sum_f32(ag_stream_t stream, const float *x, flo
         cur = dst;
     }
     return check_launch(mean ? "reduce_mean" : "reduce_sum");
-}
-
-extern "C" ag_status_t ag_broadcast_grad_f32(ag_stream_t stream, const float *gy, float *gx,
-                                             const int *shape, int rank, const int *axes, int n_axes)
-{
-    int ax[kMaxRank];
-    if (ag_status_t s = check_axes("reduce_grad", shape, rank, axes, n_axes, ax)) return s;
-    BroadcastShape bs;
-    bs.rank = rank;
-    size_t total = 1;
-    long long stride = 1;
-    for (int d = rank - 1; d >= 0; --d) {
-        bool red = false;
-        for (int j = 0; j < n_axes; ++j) red |= ax[j] == d;
-        bs.dim[d] = shape[d];
-        bs.gstride[d] = red ? 0 : stride;
-        if (!red) stride *= shape[d];
-        total *= (size_t)shape[d];
-    }
-    if (total == 0) return AG_OK;
-    AG_REQUIRE(gy && gx, AG_ERR_INVALID_DIMS, "reduce_grad: null pointer");
-    hipLaunchKernelGGL(broadcast_kernel, dim3(grid_for(total, 256)), dim3(256), 0, as_stream(stream), gy,
-                       gx, bs, total);
-    return check_launch("reduce_grad");
 }

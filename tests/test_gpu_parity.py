@@ -775,6 +775,46 @@ def test_add_broadcast_rejects_other_extents(K, rng):
         K.add_broadcast(x, b)
 
 
+@pytest.mark.parametrize("n,offset", [(1, 0), (3, 0), (4, 0), (1027, 0), (4096, 0), (100003, 0), (4099, 1), (8192, 3)])
+def test_elementwise_vector_and_scalar_paths_agree_with_numpy(K, orc, rng, n, offset):
+    # 128-bit path (aligned operands, with and without a partial last group) and the scalar path
+    # (operands that start 4 or 12 bytes past an aligned address): one rounding per element, so
+    # numpy's f32 arithmetic is the exact answer
+    say(f"elementwise n={n} offset={offset}")
+    mk = lambda: rng.standard_normal(n + offset).astype(np.float32)
+    xa, ya, za = mk(), mk(), mk()
+    x, y, z = (dev(a)[offset:] for a in (xa, ya, za))
+    xa, ya, za = xa[offset:], ya[offset:], za[offset:]
+    assert np.array_equal(host(K.relu(x)), np.maximum(xa, 0))
+    assert np.array_equal(host(K.relu_grad(x, y)), (xa > 0).astype(np.float32) * ya)
+    assert np.array_equal(host(K.add_n([x, y, z])), (xa + ya) + za)
+    assert np.array_equal(host(K.mul(x, y)), xa * ya)
+    assert np.array_equal(host(K.scale(x, 0.3)), xa * np.float32(0.3))
+    assert np.all(host(K.fill((n,), -2.5)) == -2.5)
+
+
+@pytest.mark.parametrize("shape,axes", [((64, 32, 14, 14), [0, 1, 2, 3]), ((8, 16, 12, 12), [0, 2, 3]), ((8, 16, 12, 12), [1]),
+                                        ((5, 7, 9), [2]), ((5, 7, 9), [0]), ((6, 8), [1]), ((3, 4, 5, 6, 7), [1, 3]),
+                                        ((128, 1), [0]), ((4, 4), [])])
+def test_broadcast_grad_patterns(K, rng, shape, axes):
+    gshape = [1 if i in axes else s for i, s in enumerate(shape)]
+    gy = rng.standard_normal(gshape).astype(np.float32)
+    say(f"broadcast_grad {shape} {axes}")
+    assert np.array_equal(host(K.broadcast_grad(dev(gy), shape, axes)), np.broadcast_to(gy, shape))
+
+
+def test_sparse_softmax_cross_entropy_many_rows_and_class_counts(K, orc, rng):
+    # several blocks, a partial last block, odd and even class counts, more classes than the staged kernel takes
+    for rows, classes in ((1000, 10), (257, 7), (513, 32), (300, 63), (200, 64), (130, 100)):
+        logits = (rng.standard_normal((rows, classes)) * 3).astype(np.float32)
+        labels = rng.integers(0, classes, size=(rows, 1)).astype(np.float32)
+        say(f"xent {rows}x{classes}")
+        loss, lsm = K.sparse_softmax_cross_entropy(dev(logits), dev(labels))
+        oloss, olsm = orc.sparse_softmax_xent(logits, labels)
+        assert_close(host(loss), oloss, f"xent loss {rows}x{classes}")
+        assert_close(host(lsm), olsm, f"log softmax {rows}x{classes}")
+
+
 def test_sparse_softmax_cross_entropy(K, orc, rng):
     logits = (rng.standard_normal((128, 10)) * 3).astype(np.float32)
     labels = rng.integers(0, 10, size=(128, 1)).astype(np.float32)
