@@ -38,11 +38,11 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 # true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 KIB = 1024.0
 TRAFFIC_BYTES = {
-    "gemm_fwd": ((898692.1 + 19691.6) * 2.0 + 393226.0 + 8192.2) * KIB,          # whole rounds + narrow-tile tail
-    "gemm_filter_grad": ((1116520.0 + 36883.6) * 2.0 + 73730.5 + 288.0) * KIB,   # GEMM + fold of the split partials
-    "gemm_input_grad": (234831.1 * 2.0 + 225667.5) * KIB,                        # implicit GEMM over the filter taps
+    "gemm_fwd": ((898691.8 + 19691.6) * 2.0 + 393230.8 + 8192.0) * KIB,          # whole rounds + narrow-tile tail
+    "gemm_filter_grad": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
+    "gemm_input_grad": (232938.5 * 2.0 + 215922.3) * KIB,                        # implicit GEMM over the filter taps
     "input_grad_prepare": ((207225.9 + 1165.0) * 2.0 + 430592.0 + 288.0) * KIB,  # zero-bordered gy + tap-major filter
-    "im2col": (112660.4 * 2.0 + 1806379.2) * KIB,
+    "im2col": (112667.1 * 2.0 + 1806374.2) * KIB,
     "col2im": (919260.8 * 2.0 + 200704.0) * KIB,
 }
 
