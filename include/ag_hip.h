@@ -105,6 +105,16 @@ ag_status_t ag_gemm_batchsum_f32(ag_stream_t stream, int transA, int transB, int
                                  const float *B, int ldb, long long strideB, float beta, float *C,
                                  int ldc, int batch, void *ws, size_t ws_bytes);
 
+/* Replaces MatMul::compute (dot_ops.rs:564-606, mat_mul_impl_blas :142-234): C[M x N] = op(A) . op(B),
+ * row-major, alpha 1, beta 0.  Same result as ag_gemm_f32 with batch 1; a product with few output
+ * tiles and a long contraction (K >= 512, e.g. the [128,3136].[3136,10] dense layer of
+ * examples/cnn_mnist.rs) is cut into slices of K that are computed by different blocks and summed in
+ * slice order, which needs the workspace. */
+size_t ag_matmul_f32_workspace(int M, int N, int K);
+ag_status_t ag_matmul_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K,
+                          const float *A, int lda, const float *B, int ldb, float *C, int ldc,
+                          void *ws, size_t ws_bytes);
+
 /* ---- convolution operators ------------------------------------------------------------------ */
 
 /* Replaces Conv2D::compute -> conv2d_impl -> fast_im2col_gemm_fused_kernel

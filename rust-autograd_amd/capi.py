@@ -61,6 +61,8 @@ PROTOTYPES = {
     "ag_gemm_f32": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_f, c_p, c_i, c_ll, c_p, c_i, c_ll, c_f, c_p,
                           c_i, c_ll, c_i]),
     "ag_gemm_batchsum_f32_workspace": (c_sz, [c_i] * 4),
+    "ag_matmul_f32_workspace": (c_sz, [c_i] * 3),
+    "ag_matmul_f32": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_p, c_i, c_p, c_i, c_p, c_i, c_p, c_sz]),
     "ag_gemm_batchsum_f32": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_f, c_p, c_i, c_ll, c_p, c_i, c_ll,
                                    c_f, c_p, c_i, c_i, c_p, c_sz]),
     "ag_conv2d_fwd_f32": (c_i, [c_p] * 5 + [c_i] * 10),

@@ -748,6 +748,20 @@ static int choose_splits(int M, int N, int K, int kbatch)
     return (int)cdiv(kbatch, per);
 }
 
+// A single product with few output tiles and a long contraction is cut into `s` slices of the
+// contraction that are summed like the images of an accumulated-batch GEMM, so that more than a
+// handful of blocks work on it.  Returns s (1 = no split); K / s is a multiple of 4.
+static int matmul_slices(int M, int N, int K)
+{
+    const long long tiles = cdiv(M, 64) * cdiv(N, 64);
+    if (tiles >= 64 || K < 512) return 1;
+    long long want = cdiv(256, tiles);
+    if (want > K / 64) want = K / 64;
+    for (long long s = want; s >= 2; --s)
+        if (K % s == 0 && (K / s) % 4 == 0) return (int)s;
+    return 1;
+}
+
 }  // namespace ag
 
 using namespace ag;
@@ -787,4 +801,24 @@ extern "C" ag_status_t ag_gemm_batchsum_f32(ag_stream_t stream, int transA, int 
     GemmCall c{transA, transB, M, N, K, alpha, beta, A, lda, 0, strideA, B, ldb, 0, strideB, C, ldc, 0, 1, batch};
     const int splits = (M > 0 && N > 0 && batch > 0) ? choose_splits(M, N, K, batch) : 1;
     return run_gemm(as_stream(stream), "gemm_batchsum", c, ws, ws_bytes, splits);
+}
+
+extern "C" size_t ag_matmul_f32_workspace(int M, int N, int K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 16;
+    const int s = matmul_slices(M, N, K);
+    return s > 1 ? ag_gemm_batchsum_f32_workspace(M, N, K / s, s) : 16;
+}
+
+extern "C" ag_status_t ag_matmul_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K, const float *A,
+                                     int lda, const float *B, int ldb, float *C, int ldc, void *ws, size_t ws_bytes)
+{
+    const int s = (M > 0 && N > 0 && K > 0) ? matmul_slices(M, N, K) : 1;
+    if (s <= 1) return ag_gemm_f32(stream, transA, transB, M, N, K, 1.f, A, lda, 0, B, ldb, 0, 0.f, C, ldc, 0, 1);
+    const int Kc = K / s;
+    // slice i of the contraction: columns of op(A), rows of op(B)
+    const long long strideA = transA ? (long long)Kc * lda : Kc;
+    const long long strideB = transB ? Kc : (long long)Kc * ldb;
+    return ag_gemm_batchsum_f32(stream, transA, transB, M, N, Kc, 1.f, A, lda, strideA, B, ldb, strideB, 0.f, C, ldc, s, ws,
+                                ws_bytes);
 }

@@ -436,10 +436,11 @@ struct MatMul : Op {
                                      std::to_string(k2) + " \xc3\x97 " + std::to_string(n) +
                                      " are not compatible for matrix multiplication");
         NdArray c = NdArray::empty({m, n});
-        const OpError e = from_status(ag_gemm_f32(ctx.stream(), transpose_a, transpose_b, (int)m, (int)n, (int)k, 1.f, a.ptr(),
-                                                  (int)std::max<int64_t>(a.shape()[1], 1), 0, b.ptr(),
-                                                  (int)std::max<int64_t>(b.shape()[1], 1), 0, 0.f, c.ptr(),
-                                                  (int)std::max<int64_t>(n, 1), 0, 1));
+        NdArray ws = workspace(ag_matmul_f32_workspace((int)m, (int)n, (int)k));
+        const OpError e = from_status(ag_matmul_f32(ctx.stream(), transpose_a, transpose_b, (int)m, (int)n, (int)k, a.ptr(),
+                                                    (int)std::max<int64_t>(a.shape()[1], 1), b.ptr(),
+                                                    (int)std::max<int64_t>(b.shape()[1], 1), c.ptr(),
+                                                    (int)std::max<int64_t>(n, 1), ws.ptr(), ws.len() * 4));
         if (!e.ok()) return e;
         ctx.append_output(c);
         return OpError::none();

@@ -88,8 +88,11 @@ def matmul(a, b, transpose_a=False, transpose_b=False):
         raise capi.IncompatibleShape(
             f"ndarray: inputs {m} × {k} and {k2} × {n} are not compatible for matrix multiplication")
     c = _empty((m, n), a)
-    return gemm(transpose_a, transpose_b, m, n, k, 1.0, a, max(a.shape[1], 1), 0, b, max(b.shape[1], 1), 0, 0.0,
-                c, max(n, 1), 0, 1)
+    L = capi.lib()
+    ws = _ws(L.ag_matmul_f32_workspace(m, n, k), a)
+    check(L.ag_matmul_f32(_stream(), int(transpose_a), int(transpose_b), m, n, k, _ptr(a), max(a.shape[1], 1), _ptr(b),
+                          max(b.shape[1], 1), _ptr(c), max(n, 1), _ptr(ws), ws.numel()))
+    return c
 
 
 def batch_matmul(a, b, transpose_a=False, transpose_b=False):

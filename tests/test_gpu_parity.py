@@ -321,6 +321,27 @@ def test_gemm_batchsum_matches_sequential_accumulation(K, orc, rng, batch):
     assert np.array_equal(host(c), host(c2))
 
 
+@pytest.mark.parametrize("m,n,k", [(128, 10, 3136), (10, 128, 3136), (64, 64, 4096), (7, 5, 1000), (130, 70, 2048),
+                                   (128, 10, 3137), (128, 10, 1022), (200, 300, 512)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_long_contraction_few_tiles(K, rng, m, n, k, ta, tb):
+    """MatMul with few output tiles and a long K: the contraction is cut into slices summed in order
+    (K without a suitable divisor, or with many tiles, stays one product)."""
+    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+    say(f"matmul sliced {m}x{n}x{k} ta={ta} tb={tb}")
+    A = (a.T if ta else a).astype(np.float64)
+    Bm = (b.T if tb else b).astype(np.float64)
+    got = host(K.matmul(dev(a), dev(b), ta, tb))
+    assert_close_conditioned(got, A @ Bm, np.abs(A) @ np.abs(Bm), "sliced matmul")
+    assert np.array_equal(got, host(K.matmul(dev(a), dev(b), ta, tb)))   # deterministic
+    # small integers: every product is counted exactly once whatever the slicing
+    ai = rng.integers(-3, 4, size=a.shape).astype(np.float32)
+    bi = rng.integers(-3, 4, size=b.shape).astype(np.float32)
+    exact = (ai.T if ta else ai).astype(np.int64) @ (bi.T if tb else bi).astype(np.int64)
+    assert np.array_equal(host(K.matmul(dev(ai), dev(bi), ta, tb)), exact.astype(np.float32))
+
+
 def test_gemm_degenerate_k_and_beta(K, rng):
     c0 = rng.random((5, 6), dtype=np.float32)
     c = dev(c0)
