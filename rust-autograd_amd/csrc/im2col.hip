@@ -324,6 +324,42 @@ __global__ __launch_bounds__(256) void col2im_stride2_kernel(const float *__rest
     }
 }
 
+// The same for the usual geometries (dilation 1, W and H even) with the window and the padding known
+// at compile time: no run-time loops or parity tests, 32-bit offsets inside a plane, one streaming
+// load per tap (consecutive lanes read consecutive positions) and two 64-bit streaming stores (the
+// lanes of a wave write 512 contiguous bytes per row).  Same visiting order.
+template <int KH, int KW, int PH, int PW>
+__global__ __launch_bounds__(256) void col2im_stride2_vec_kernel(const float *__restrict__ cols,
+                                                                 float *__restrict__ gx, ConvGeom g,
+                                                                 unsigned nblk)
+{
+    const unsigned gi = blockIdx.x * 256u + threadIdx.x;
+    if (gi >= nblk) return;
+    const unsigned BW = (unsigned)g.W >> 1, BH = (unsigned)g.H >> 1;
+    const unsigned rowi = gi / BW, bx = gi - rowi * BW;  // (plane, by)
+    const unsigned plane = rowi / BH, by = rowi - plane * BH;
+    const unsigned P = (unsigned)(g.OH * g.OW);
+    const float *cp = cols + (long long)plane * (KH * KW) * P;
+    float acc[2][2] = {};
+#pragma unroll
+    for (int ky = 0; ky < KH; ++ky) {
+        const int ry = (ky - PH) & 1;
+        const int ty = 2 * (int)by + ry + PH - ky;
+        const int oy = ty >> 1;
+        const bool vy = ty >= 0 && oy < g.OH;
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx) {
+            const int rx = (kx - PW) & 1;
+            const int tx = 2 * (int)bx + rx + PW - kx;
+            const int ox = tx >> 1;
+            if (vy && tx >= 0 && ox < g.OW) acc[ry][rx] += ld_stream(cp + (unsigned)(ky * KW + kx) * P + oy * g.OW + ox);
+        }
+    }
+    float *dst = gx + (long long)plane * g.H * g.W + (2 * by) * (unsigned)g.W + 2 * bx;
+    *reinterpret_cast<float2 *>(dst) = make_float2(acc[0][0], acc[0][1]);
+    *reinterpret_cast<float2 *>(dst + g.W) = make_float2(acc[1][0], acc[1][1]);
+}
+
 static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int kh, int kw, int ph,
                               int pw, int sh, int sw, int dh, int dw)
 {
@@ -508,6 +544,15 @@ extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, floa
         else
             hipLaunchKernelGGL((col2im_unit_vec4_kernel<0, 0>), dim3((unsigned)blocks), dim3(256), 0,
                                as_stream(stream), cols, gx, g, groups);
+    } else if (sh == 2 && sw == 2 && dh == 1 && dw == 1 && W % 2 == 0 && H % 2 == 0 && (reinterpret_cast<uintptr_t>(gx) & 7u) == 0 &&
+               ((kh == 3 && kw == 3) || (kh == 4 && kw == 4)) && ph == 1 && pw == 1 &&
+               planes * (H / 2) * (W / 2) < 0xffffffffLL && (long long)kh * kw * OH * OW < 0x7fffffffLL) {
+        const unsigned nblk = (unsigned)(planes * (H / 2) * (W / 2));
+        const dim3 grid((nblk + 255) / 256), block(256);
+        if (kh == 3)
+            hipLaunchKernelGGL((col2im_stride2_vec_kernel<3, 3, 1, 1>), grid, block, 0, as_stream(stream), cols, gx, g, nblk);
+        else
+            hipLaunchKernelGGL((col2im_stride2_vec_kernel<4, 4, 1, 1>), grid, block, 0, as_stream(stream), cols, gx, g, nblk);
     } else if (sh == 2 && sw == 2) {
         const long long nblk = planes * ((H + 1) / 2) * ((W + 1) / 2);
         long long blocks = (nblk + 255) / 256;
