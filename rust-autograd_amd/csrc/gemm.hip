@@ -494,12 +494,13 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
 {
     if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg;
     if (direct) {
-        static const int dl[] = {14, 15, 16, 17, 13};  // 128x256, 256x128, 192x128, 128x192, 128x128
-        static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.92};
+        // 128x256, 256x128, 192x128, 128x192, 128x128, and 64x128 (two blocks per CU) for outputs of up to 64 rows
+        static const int dl[] = {14, 15, 16, 17, 13, kDirectCfg64};
+        static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.92, 0.8};
         int best = -1;
         double best_cost = 1e300;
         long long best_blocks = 0;
-        for (int c = 0; c < 5; ++c) {
+        for (int c = 0; c < 6; ++c) {
             const TileCfg &t = kCfgs[dl[c]];
             const long long tm = cdiv(M, t.bm), tn = cdiv(N, t.bn);
             const double cost = (double)tm * t.bm * tn * t.bn / eff[c];
@@ -509,7 +510,7 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
                 best_blocks = tm * tn * zcount;
             }
         }
-        if (best_blocks >= 256) return best;
+        if (best_blocks >= (best == kDirectCfg64 ? 128 : 256)) return best;
     }
     static const int short_k[] = {11, 10, 12, 8};  // 192x128, 128x128, 128x64, 64x64 (BK 16)
     static const int long_k[] = {0, 1, 2, 3};      // 128x128, 128x64, 64x128, 64x64 (BK 32)

@@ -200,7 +200,7 @@ def test_gemm_every_tile_configuration(K, rng, cfg):
     assert_close(got_t, truth, "gemm TT")
 
 
-DIRECT_CFGS = list(range(13, 19))  # operand tiles loaded from global memory straight into LDS
+DIRECT_CFGS = list(range(13, 20))  # operand tiles loaded from global memory straight into LDS
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
@@ -239,6 +239,8 @@ def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
         # more tiles than the persistent grid has blocks: whole rounds, then a narrow-tile launch
         # for the remaining columns, which starts in the middle of a batch
         shapes.append((128, 3136, 32, 24, 0.0))
+        # an output of 64 rows (the second convolution of the small CNN): the 64 x 128 tile, chosen automatically
+        shapes.append((64, 196, 288, 128, 0.0))
     for (m, n, k, batch, beta) in shapes:
         a = rng.random((k, m) if ta else (m, k), dtype=np.float32)
         b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
