@@ -4,9 +4,14 @@
 A "step" is one conv2d forward + backward over one synthetic batch at the headline shape
 (B=256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, f32):
 
-    forward      im2col(x) -> cols ;  y   = W . cols            (Conv2D)
-    filter grad  gW = sum_b gy_b . cols_b^T                      (Conv2DFilterGrad)
-    input grad   gcols = W^T . gy ;  gx = col2im(gcols)          (Conv2DTranspose)
+    forward      x' = zero-bordered x ;  y  = sum over taps  W[tap] . shift(x', tap)      (Conv2D)
+    filter grad  gy' = zero-bordered gy ; gW[tap] = sum_b gy'_b . shift(x'_b, tap)^T       (Conv2DFilterGrad)
+    input grad   gx = sum over taps  W[tap]^T . shift(gy', tap)                             (Conv2DTranspose)
+
+Each contraction is one implicit GEMM over the filter taps: the im2col columns the reference
+materialises (conv2d.rs:25-112, conv2d_transpose.rs:148-151) are never written.  The
+column-materialising kernels (im2col, the GEMMs over columns, col2im) serve the other geometries
+and are timed in the per-kernel section.
 
 Inputs are resident in HBM before the timed region.  Every kernel launch inside the timed steps
 is bracketed by events on the launch stream, so the per-kernel figures and the roofline object
@@ -38,10 +43,10 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 # true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 KIB = 1024.0
 TRAFFIC_BYTES = {
-    "gemm_fwd": ((898691.8 + 19691.6) * 2.0 + 393230.8 + 8192.0) * KIB,          # whole rounds + narrow-tile tail
-    "gemm_filter_grad": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
-    "gemm_input_grad": (232938.5 * 2.0 + 215922.3) * KIB,                        # implicit GEMM over the filter taps
-    "input_grad_prepare": ((207225.9 + 1165.0) * 2.0 + 430592.0 + 288.0) * KIB,  # zero-bordered gy + tap-major filter
+    # the step (column-free): to be refreshed from profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt
+    # per-kernel section (column-materialising operators)
+    "gemm_fwd_columns": ((898691.8 + 19691.6) * 2.0 + 393230.8 + 8192.0) * KIB,          # whole rounds + narrow-tile tail
+    "gemm_filter_grad_columns": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
     "im2col": (112667.1 * 2.0 + 1806374.2) * KIB,
     "col2im": (919260.8 * 2.0 + 200704.0) * KIB,
 }
@@ -177,30 +182,31 @@ def main():
     s = (6.0 / K) ** 0.5
     w = (torch.rand(K, C, KH, KH, device=dev, generator=g) * 2 - 1) * s
     gy = torch.randn(Bn, K, OH, OH, device=dev, generator=g)
-    cols = torch.empty(Bn, CK, P, device=dev)
     y = torch.empty(Bn, K, OH, OH, device=dev)
-    gcols = torch.empty(Bn, CK, P, device=dev)
     gx = torch.empty(Bn, C, H, W, device=dev)
     gw = torch.empty(K, C, KH, KH, device=dev)
     L = capi.lib()
-    ws = torch.empty(max(16, L.ag_conv2d_filter_grad_f32_workspace(Bn, CK, P, K)), dtype=torch.uint8, device=dev)
     st, ptr, chk = Kn._stream, Kn._ptr, capi.check
     T = Timer(torch)
-    geom = (Bn, K, OH, OH, C, KH, KH, PAD, H, W)
-    assert 0 < L.ag_conv_input_grad_scratch_floats(*geom) <= gcols.numel()
+    fgeom = (Bn, C, H, W, K, KH, KH, PAD)                # forward / filter gradient
+    igeom = (Bn, K, OH, OH, C, KH, KH, PAD, H, W)        # input gradient
+    n_xpad, n_gypad = L.ag_conv2d_nocols_scratch_floats(*fgeom), L.ag_conv_input_grad_scratch_floats(*igeom)
+    assert n_xpad > 0 and n_gypad > 0, "the headline geometry takes the column-free path"
+    xpad = torch.empty(n_xpad, device=dev)
+    gypad = torch.empty(n_gypad, device=dev)
+    ws = torch.empty(max(16, L.ag_conv2d_filter_grad_nocols_f32_workspace(*fgeom)), dtype=torch.uint8, device=dev)
 
     def step():
-        T.run("im2col", lambda: chk(L.ag_im2col_f32(st(), ptr(x), ptr(cols), Bn, C, H, W, KH, KH, PAD, PAD, STRIDE,
-                                                    STRIDE, DIL, DIL)))
-        T.run("gemm_fwd", lambda: chk(L.ag_gemm_f32(st(), 0, 0, K, P, CK, 1.0, ptr(w), CK, 0, ptr(cols), P, CK * P,
-                                                    0.0, ptr(y), P, K * P, Bn)))
-        T.run("gemm_filter_grad", lambda: chk(L.ag_gemm_batchsum_f32(st(), 0, 1, K, CK, P, 1.0, ptr(gy), P, K * P,
-                                                                     ptr(cols), P, CK * P, 0.0, ptr(gw), CK, Bn,
-                                                                     ptr(ws), ws.numel())))
-        # Conv2DTranspose (the input gradient): the two stages ag_conv2d_transpose_f32 runs for a
-        # stride-1 convolution, launched separately so that each gets its own events
-        T.run("input_grad_prepare", lambda: chk(L.ag_conv_input_grad_prepare_f32(st(), ptr(gy), ptr(w), ptr(gcols), *geom)))
-        T.run("gemm_input_grad", lambda: chk(L.ag_conv_input_grad_gemm_f32(st(), ptr(gcols), ptr(gx), *geom)))
+        # Conv2D forward: zero-bordered copy of x (kept for the filter gradient), then one implicit GEMM over the taps
+        T.run("fwd_prepare", lambda: chk(L.ag_conv2d_nocols_prepare_f32(st(), ptr(x), ptr(w), ptr(xpad), *fgeom)))
+        T.run("gemm_fwd", lambda: chk(L.ag_conv2d_nocols_gemm_f32(st(), ptr(xpad), ptr(y), *fgeom)))
+        # zero-bordered copy of gy, shared by both gradients
+        T.run("input_grad_prepare", lambda: chk(L.ag_conv_input_grad_prepare_f32(st(), ptr(gy), ptr(w), ptr(gypad), *igeom)))
+        # Conv2DFilterGrad: GEMM over the flattened padded planes, summed over images
+        T.run("gemm_filter_grad", lambda: chk(L.ag_conv2d_filter_grad_nocols_f32(st(), ptr(xpad), ptr(gypad), ptr(gw), *fgeom,
+                                                                                 ptr(ws), ws.numel())))
+        # Conv2DTranspose (the input gradient): implicit GEMM over the taps
+        T.run("gemm_input_grad", lambda: chk(L.ag_conv_input_grad_gemm_f32(st(), ptr(gypad), ptr(gx), *igeom)))
 
     if args.pmc_calibration:
         src = torch.ones(1 << 28, device=dev)
@@ -222,13 +228,12 @@ def main():
     per = T.totals()
 
     gemm_flop = 2.0 * K * P * CK * Bn            # identical for the three contractions
-    col_bytes = 4.0 * (Bn * C * H * W + Bn * CK * P)
     kernels = {}
     for name in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"):
         tf = gemm_flop / (per[name] * 1e-3) / 1e12
         kernels[name] = {"ms": round(per[name], 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
-    prep_bytes = 4.0 * (gy.numel() + L.ag_conv_input_grad_scratch_floats(*geom))  # read gy, write its bordered copy
-    for name, nbytes in (("im2col", col_bytes), ("input_grad_prepare", prep_bytes)):
+    # bordered copies: read the tensor once, write its padded planes once
+    for name, nbytes in (("fwd_prepare", 4.0 * (x.numel() + n_xpad)), ("input_grad_prepare", 4.0 * (gy.numel() + n_gypad))):
         gbs = nbytes / (per[name] * 1e-3) / 1e9
         kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
     if Bn == B:
@@ -254,7 +259,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"C4 conv2d fwd+bwd: x [{Bn},{C},{H},{W}] N(0,1), w [{K},{C},{KH},{KH}] glorot-uniform, "
-                               f"stride {STRIDE} pad {PAD}; im2col, forward GEMM, filter-gradient GEMM, column-free input-gradient GEMM per step"},
+                               f"stride {STRIDE} pad {PAD}; forward, filter gradient and input gradient per step, each an implicit (column-free) GEMM over zero-bordered copies of x / gy"},
         "roofline": roofline, "kernels": kernels,
     }
     if not args.no_cpu:
@@ -286,7 +291,8 @@ def micro(torch, Kn, capi, dev):
     res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
     del x, y, am, il, gy
 
-    # the column-materialising input gradient (what the reference does per image): W^T . gy, then col2im
+    # the column-materialising operators (what the reference does per image): im2col + W . cols, gy . cols^T summed
+    # over images, W^T . gy + col2im
     Bn, Cc, Kf, Hh = 256, 64, 128, 56
     Pp, CKk = Hh * Hh, Cc * 9
     L = capi.lib()
@@ -295,12 +301,30 @@ def micro(torch, Kn, capi, dev):
     gyy = torch.randn(Bn, Kf, Pp, device=dev, generator=g)
     gc = torch.empty(Bn, CKk, Pp, device=dev)
     gxx = torch.empty(Bn, Cc, Hh, Hh, device=dev)
+    xx = torch.randn(Bn, Cc, Hh, Hh, device=dev, generator=g)
+    yy = torch.empty(Bn, Kf, Pp, device=dev)
+    gww = torch.empty(Kf, CKk, device=dev)
+    wsf = torch.empty(max(16, L.ag_conv2d_filter_grad_f32_workspace(Bn, CKk, Pp, Kf)), dtype=torch.uint8, device=dev)
+    cb = 4.0 * (gc.numel() + gxx.numel())
+    gf = 2.0 * Kf * Pp * CKk * Bn
+    ms = time_events(torch, lambda: chk(L.ag_im2col_f32(st(), ptr(xx), ptr(gc), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1)), 10)
+    res["im2col"] = {"ms": round(ms, 4), "GB/s": round(cb / ms / 1e6, 1), "frac_hbm": round(cb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "traffic_bytes": round(TRAFFIC_BYTES["im2col"])}
+    ms = time_events(torch, lambda: chk(L.ag_gemm_f32(st(), 0, 0, Kf, Pp, CKk, 1.0, ptr(wt), CKk, 0, ptr(gc), Pp, CKk * Pp, 0.0,
+                                                      ptr(yy), Pp, Kf * Pp, Bn)), 10)
+    res["gemm_fwd_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(gf / ms / 1e9, 2), "frac_mfma": round(gf / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+                               "traffic_bytes": round(TRAFFIC_BYTES["gemm_fwd_columns"])}
+    ms = time_events(torch, lambda: chk(L.ag_gemm_batchsum_f32(st(), 0, 1, Kf, CKk, Pp, 1.0, ptr(gyy), Pp, Kf * Pp, ptr(gc), Pp,
+                                                               CKk * Pp, 0.0, ptr(gww), CKk, Bn, ptr(wsf), wsf.numel())), 10)
+    res["gemm_filter_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(gf / ms / 1e9, 2),
+                                       "frac_mfma": round(gf / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+                                       "traffic_bytes": round(TRAFFIC_BYTES["gemm_filter_grad_columns"])}
+    del xx, yy, gww, wsf
     ms = time_events(torch, lambda: chk(L.ag_gemm_f32(st(), 1, 0, CKk, Pp, Kf, 1.0, ptr(wt), CKk, 0, ptr(gyy), Pp, Kf * Pp,
                                                       0.0, ptr(gc), Pp, CKk * Pp, Bn)), 10)
     tf = 2.0 * Kf * Pp * CKk * Bn / ms / 1e9
     res["gemm_input_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
     ms = time_events(torch, lambda: chk(L.ag_col2im_f32(st(), ptr(gc), ptr(gxx), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1, Hh, Hh)), 10)
-    cb = 4.0 * (gc.numel() + gxx.numel())
     res["col2im"] = {"ms": round(ms, 4), "GB/s": round(cb / ms / 1e6, 1), "frac_hbm": round(cb / ms / 1e6 / HBM_PEAK_GBS, 4),
                      "traffic_bytes": round(TRAFFIC_BYTES["col2im"])}
     del wt, gyy, gc, gxx

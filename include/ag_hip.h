@@ -159,6 +159,34 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch
                                         int ych, int yh, int yw, int xch, int kh, int kw, int pad,
                                         int xh, int xw);
 
+/* Column-free stride-1, dilation-1 convolution: forward and filter gradient without the im2col
+ * columns.  No counterpart in the reference, which always materialises them (Conv2D::compute ->
+ * fast_im2col_gemm_fused_kernel, conv2d.rs:25-112; conv2d_filter_grad_impl, conv2d.rs:631-734); the
+ * results are those of ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32 within the floating-point
+ * tolerance (other summation order).  The forward writes a zero-bordered copy of x into `xpad`
+ * (ag_conv2d_nocols_scratch_floats() floats; 0 = geometry not supported: square window, C a multiple
+ * of 32, planes of at least 128 or 256 padded elements) and runs one implicit GEMM over the filter
+ * taps.  The filter gradient contracts that copy with the zero-bordered upstream gradient that
+ * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images in
+ * splits that need the workspace; "same" convolutions only (2*pad == kh-1 == kw-1, K a multiple of
+ * 32), so that both copies share one padded plane shape.  A NaN or infinity in x can reach the
+ * gradient of the neighbouring channel as well (the contraction runs a few elements past a plane,
+ * against border zeros of the gradient). */
+size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad);
+ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y,
+                                     float *xpad, int B, int C, int H, int W, int K, int kh, int kw,
+                                     int pad);
+/* The two stages of ag_conv2d_fwd_nocols_f32 (bordered copy of x and tap-major filter; the GEMM). */
+ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, const float *w, float *xpad,
+                                         int B, int C, int H, int W, int K, int kh, int kw, int pad);
+ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C,
+                                      int H, int W, int K, int kh, int kw, int pad);
+size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw,
+                                                  int pad);
+ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, const float *xpad, const float *gypad,
+                                             float *gw, int B, int C, int H, int W, int K, int kh,
+                                             int kw, int pad, void *ws, size_t ws_bytes);
+
 /* Replaces Conv2DTransposeFilterGrad::compute -> conv2d_transpose_filter_grad_impl
  * (conv2d_transpose.rs:433-451, 303-431).  x [B,ych,yh,yw] (input of the transposed conv),
  * gy [B,xch,H,W] (gradient of its output) -> gw [ych,xch,kh,kw].  `gycols` is caller scratch of

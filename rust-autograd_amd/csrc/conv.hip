@@ -83,6 +83,16 @@ __global__ __launch_bounds__(256) void pad_border_kernel(const float *__restrict
     }
 }
 
+// Zeroes the slack before and after the padded planes: the implicit filter gradient multiplies what
+// it reads there by border zeros of the gradient, which must not meet a NaN bit pattern.
+__global__ void zero_slack_kernel(float *lead, int n_lead, float *tail, int n_tail)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n_lead + n_tail; i += gridDim.x * blockDim.x) {
+        if (i < n_lead) lead[i] = 0.f;
+        else tail[i - n_lead] = 0.f;
+    }
+}
+
 // wr[c][tap][k] = w[k][c][tap]  (tap = ky*kw + kx): the filter as the k-contiguous left operand of
 // the implicit input-gradient GEMM.
 __global__ __launch_bounds__(256) void filter_taps_kernel(const float *__restrict__ w, float *__restrict__ wr, int Kf,
@@ -92,6 +102,19 @@ __global__ __launch_bounds__(256) void filter_taps_kernel(const float *__restric
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int k = e % Kf, tap = e / Kf % taps, c = e / (Kf * taps);
         wr[e] = w[((long long)k * C + c) * taps + tap];
+    }
+}
+
+// wf[k][tap'][c] = w[k][c][taps - 1 - tap']: the filter as the left operand of the implicit forward
+// GEMM.  The GEMM visits its taps from the largest shift to none (the order the input gradient
+// needs), so a correlation lists them reversed.
+__global__ __launch_bounds__(256) void filter_taps_fwd_kernel(const float *__restrict__ w, float *__restrict__ wf, int Kf,
+                                                              int C, int taps)
+{
+    const int total = Kf * C * taps;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int c = e % C, tap = e / C % taps, k = e / (C * taps);
+        wf[e] = w[((long long)k * C + c) * taps + (taps - 1 - tap)];
     }
 }
 
@@ -126,12 +149,121 @@ static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w
     if (blocks > 1048576) blocks = 1048576;
     hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, gy, scratch, quads, yh, yw, g.Hp,
                        g.Wp, kh - 1 - pad, kw - 1 - pad);
+    // the implicit filter gradient may read a few elements past the last plane and expects zeros
+    hipLaunchKernelGGL(zero_slack_kernel, dim3(4), dim3(256), 0, st, scratch, 0, scratch + quads * 4,
+                       (int)(g.gyp_floats - quads * 4));
     hipLaunchKernelGGL(filter_taps_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w,
                        scratch + g.gyp_floats, ych, xch, kh * kw);
     return check_launch("conv2d_transpose");
 }
 
+// The column-free forward is the same implicit GEMM with the roles exchanged: the input x takes the
+// place of the upstream gradient (bordered by `pad`), the C input channels are contracted and the K
+// filters are the output rows.  Leading slack: the implicit filter gradient reads up to one padded
+// row and column before the first plane.
+constexpr long long kFwdLeadFloats = 1024;
+
+static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, FusedGeom *g)
+{
+    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
+    if (OH < 1 || OW < 1 || pad > kh - 1 || pad > kw - 1) return false;
+    // seen as an input gradient: "gy" = x [C, H, W], "gx" = y [K, OH, OW], border kh-1-pad' = pad
+    return kh == kw && fused_geom(B, C, H, W, K, kh, kw, kh - 1 - pad, OH, OW, g);
+}
+
+// Positions of the flattened padded plane that the implicit filter gradient contracts over: all
+// rows that hold gradient values, rounded up to the GEMM's k tile.  0 = the rounding would reach
+// past zeros.
+static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
+{
+    // past the end of a plane the next plane's top border (pad rows and pad elements of zeros) or the
+    // zeroed slack follows
+    const long long kq = (((long long)(OH + pad) * g.Wp + 31) / 32) * 32;
+    return kq <= (long long)g.Hp * g.Wp + (long long)pad * g.Wp + pad ? (int)kq : 0;
+}
+
 }  // namespace ag
+
+// ---- column-free stride-1 convolution: forward and filter gradient ------------------------------
+// No counterpart of these three in the reference, which always materialises the columns
+// (conv2d.rs:25-112, 631-734); they compute the same y and gw from a zero-bordered copy of x.
+// `xpad`: ag_conv2d_nocols_scratch_floats() floats, written by the forward and read by the filter
+// gradient.  0 floats = geometry not supported (use ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32).
+extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad)
+{
+    FusedGeom g;
+    if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g)) return 0;
+    return (size_t)(kFwdLeadFloats + g.gyp_floats + g.wr_floats);
+}
+
+// The two stages of the forward, for callers that time or schedule them separately.
+extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, const float *w, float *xpad, int B,
+                                                    int C, int H, int W, int K, int kh, int kw, int pad)
+{
+    FusedGeom g;
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad), AG_ERR_INVALID_DIMS,
+               "conv2d (column-free): geometry not supported");
+    AG_REQUIRE(x && w && xpad, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    hipStream_t st = as_stream(stream);
+    float *xp = xpad + kFwdLeadFloats, *wf = xp + g.gyp_floats;
+    const long long quads = (long long)B * C * g.Hp * g.Wp / 4;
+    long long blocks = (quads + 255) / 256;
+    if (blocks > 1048576) blocks = 1048576;
+    hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, x, xp, quads, H, W, g.Hp, g.Wp, pad, pad);
+    hipLaunchKernelGGL(zero_slack_kernel, dim3(8), dim3(256), 0, st, xpad, (int)kFwdLeadFloats, xp + quads * 4,
+                       (int)(g.gyp_floats - quads * 4));
+    hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
+                       kh * kw);
+    return check_launch("conv2d");
+}
+
+extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C, int H, int W,
+                                                 int K, int kh, int kw, int pad)
+{
+    FusedGeom g;
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
+               "conv2d (column-free): geometry not supported");
+    AG_REQUIRE(xpad && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    const float *xp = xpad + kFwdLeadFloats;
+    return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1,
+                                kh, kw, g.Hp, g.Wp);
+}
+
+extern "C" ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y, float *xpad,
+                                                int B, int C, int H, int W, int K, int kh, int kw, int pad)
+{
+    if (ag_status_t s = ag_conv2d_nocols_prepare_f32(stream, x, w, xpad, B, C, H, W, K, kh, kw, pad)) return s;
+    return ag_conv2d_nocols_gemm_f32(stream, xpad, y, B, C, H, W, K, kh, kw, pad);
+}
+
+// gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the first
+// B*K*Hp*Wp floats of its scratch); the geometry must be a "same" convolution (2*pad == k-1) so
+// that x and gy share one padded plane shape.
+extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw, int pad)
+{
+    FusedGeom g;
+    if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g)) return 0;
+    const int kq = filter_grad_positions(g, H + 2 * pad - kh + 1, pad);
+    return kq ? gemm_conv_filter_grad_workspace(B, K, C, kh * kw, kq) : 0;
+}
+
+extern "C" ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, const float *xpad, const float *gypad, float *gw,
+                                                        int B, int C, int H, int W, int K, int kh, int kw, int pad, void *ws,
+                                                        size_t ws_bytes)
+{
+    FusedGeom g, gg;
+    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
+    AG_REQUIRE(2 * pad == kh - 1 && 2 * pad == kw - 1 && K % 4 == 0 && C >= 1 &&
+                   fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg) &&
+                   g.Hp == gg.Hp && g.Wp == gg.Wp && aligned16(xpad) && aligned16(gypad),
+               AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): geometry not supported");
+    const int kq = filter_grad_positions(g, OH, pad);
+    AG_REQUIRE(kq > 0 && (long long)C * g.Hp * g.Wp < (1LL << 30), AG_ERR_INVALID_DIMS,
+               "conv2d_filter_grad (column-free): plane too small or too many channels");
+    AG_REQUIRE(gw, AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): null output");
+    return gemm_conv_filter_grad(as_stream(stream), gypad, xpad + kFwdLeadFloats, gw, ws, ws_bytes, B, K, C, kh, kw, pad, g.Hp,
+                                 g.Wp, kq);
+}
 
 extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const float *w,
                                                float *gx, float *gcols, int B, int ych, int yh, int yw,

@@ -634,6 +634,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (fold) p.N = c.N * c.batch;
     p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
+    p.rows_taps = p.rows_kw = p.rows_wp = 0;
+    p.rows_plane = 0;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * (fold ? 1 : c.batch) * p.splits;
@@ -722,6 +724,8 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     p.alpha = 1.f; p.beta = 0.f;
     p.n_off = 0;
     p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
+    p.rows_taps = p.rows_kw = p.rows_wp = 0;
+    p.rows_plane = 0;
     const int cfg = C <= 64 ? kDirectCfg64 : 14;  // 64 x 128 or 128 x 256
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
@@ -730,6 +734,69 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     p.total_blocks = (unsigned)blocks;
     launch_direct(st, cfg, true, false, p, num_cus(), g_grid_scale);
     return check_launch("conv2d_transpose");
+}
+
+constexpr int kConvFilterGradCfg = 17;  // 128 x 192 tiles, both operands k-contiguous
+
+static int conv_filter_grad_splits(int B, int Kf, int C, int taps, int kq)
+{
+    (void)kq;
+    // as many splits as give the chip a few rounds of tiles; every split sums whole images
+    const long long tiles = cdiv(Kf, kCfgs[kConvFilterGradCfg].bm) * cdiv((long long)C * taps, kCfgs[kConvFilterGradCfg].bn);
+    long long want = cdiv(4096, tiles);
+    if (want > B) want = B;
+    const long long per = cdiv(B, want);
+    return (int)cdiv(B, per);
+}
+
+size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq)
+{
+    const int splits = conv_filter_grad_splits(B, Kf, C, taps, kq);
+    return splits > 1 ? sizeof(float) * (size_t)splits * Kf * C * taps : 16;
+}
+
+ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
+                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq)
+{
+    const int taps = kh * kw;
+    const long long plane = (long long)Hp * Wp;
+    GemmParams p;
+    p.A = gyp;
+    p.B = xp - ((long long)pad * Wp + pad);  // tap (0, 0) reads `pad` rows and columns before the position
+    p.M = Kf; p.N = C * taps; p.K = kq;
+    p.lda = plane; p.ldb = plane; p.ldc = p.N;
+    p.sA = p.sB = p.sC = 0;
+    p.sAk = (long long)Kf * plane; p.sBk = (long long)C * plane;
+    p.kbatch = B;
+    p.splits = conv_filter_grad_splits(B, Kf, C, taps, kq);
+    p.kb_per_split = (int)cdiv(B, p.splits);
+    p.splits = (int)cdiv(B, p.kb_per_split);
+    p.sCsplit = (long long)p.M * p.N;
+    p.alpha = 1.f; p.beta = 0.f;
+    p.n_img = 0; p.n_off = 0;
+    p.conv_wp = p.conv_w = p.conv_kw = 0;
+    p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)plane;
+    p.C = gw;
+    if (p.splits > 1) {
+        const size_t need = sizeof(float) * (size_t)p.splits * p.M * p.N;
+        AG_REQUIRE(ws && ws_bytes >= need, AG_ERR_INVALID_DIMS, "conv2d_filter_grad: workspace of %zu bytes needed, %zu given",
+                   need, ws_bytes);
+        p.C = static_cast<float *>(ws);
+    }
+    const int cfg = kConvFilterGradCfg;
+    p.tiles_m = (int)cdiv(p.M, kCfgs[cfg].bm);
+    p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
+    p.total_blocks = (unsigned)((long long)p.tiles_m * p.tiles_n * p.splits);
+    launch_direct(st, cfg, true, true, p, num_cus(), g_grid_scale);
+    if (ag_status_t s = check_launch("conv2d_filter_grad")) return s;
+    if (p.splits > 1) {
+        const long long total = (long long)p.M * p.N;
+        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
+                           dim3(256), 0, st, static_cast<const float *>(ws), p.splits, p.sCsplit, gw, p.M, p.N,
+                           (long long)p.N, 1.f, 0.f);
+        return check_launch("conv2d_filter_grad");
+    }
+    return AG_OK;
 }
 
 static int g_force_splits = 0;  // experiment hook, see ag_gemm_force_splits

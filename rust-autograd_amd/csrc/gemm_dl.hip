@@ -82,6 +82,20 @@ struct DirectTile {
             }
         }
     }
+    // k-contiguous rows that are (channel, tap) pairs of a zero-bordered input (implicit filter
+    // gradient): row n starts (n / taps) * plane + ky * wp + kx elements after the origin.
+    __device__ inline void init_conv_rows(int row0, int rows, int taps, int kw, int wp, unsigned plane, int wave, int lane)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int pos = (i * NW + wave) * 64 + lane;
+            const int r = pos / CPR, c = (pos % CPR) ^ kc_swizzle<BK>(r);
+            const int row = min(row0 + r, rows - 1);
+            const int ch = row / taps, tap = row - ch * taps;
+            const int ky = tap / kw, kx = tap - ky * kw;
+            off[i] = ((unsigned)ch * plane + (unsigned)(ky * wp + kx + c * 4)) * 4u;
+        }
+    }
     // Folded batch (m/n-contiguous operand only): the tile starts at column r0 of one batch and
     // may run on into the next one, `next` elements further (0 when there is no next batch: those
     // columns are clamped like any column beyond the operand).
@@ -243,6 +257,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         if (!KB && p.n_img != 0) {
             const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
             ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
+        } else if (KB && p.rows_taps != 0) {
+            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, wave, lane);
         } else {
             ldr_b.init(ldb, it.n0, p.N, wave, lane);
         }

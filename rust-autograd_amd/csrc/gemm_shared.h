@@ -35,6 +35,12 @@ struct GemmParams {
     // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
     // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
     int conv_wp, conv_w, conv_kw;
+    // Implicit filter gradient of a stride-1 convolution (direct-to-LDS kernel, k-contiguous B): row n
+    // of B is (channel n / rows_taps, tap n % rows_taps) of a zero-bordered input [..][C][Hp][rows_wp]
+    // and starts (channel * rows_plane + ky * rows_wp + kx) elements after B; the contraction runs
+    // over the flattened padded plane.  0 = rows of B are ldb apart.
+    int rows_taps, rows_kw, rows_wp;
+    unsigned rows_plane;
 };
 
 constexpr int kXcds = 8;
@@ -52,6 +58,13 @@ __device__ inline unsigned xcd_remap(unsigned id, unsigned total)
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
 constexpr int kFirstDirectCfg = 13;
 void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
+// Implicit filter gradient: gw[k][c][tap] = sum over images and padded-plane positions q of
+// gyp[b][k][q] * xp[b][c][q + (ky - pad) * Wp + (kx - pad)].  gyp, xp: zero-bordered [B][.][Hp][Wp]
+// with the same border `pad` on every side; `kq` (a multiple of 32, at most Hp * Wp) positions
+// cover every non-zero element of gyp.  `ws`: partial sums of the split over images.
+size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq);
+ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
+                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq);
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
                                  int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
 // Direct-to-LDS configuration with a 64-row tile (64 x 128, two blocks per CU), used by the implicit input gradient.

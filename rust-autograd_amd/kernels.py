@@ -196,6 +196,55 @@ def conv2d_transpose(gy, w, pad, stride, dilation=1, out_hw=None, return_cols=Fa
     return (gx, gcols) if return_cols else gx
 
 
+def conv2d_nocols(x, w, pad):
+    """Column-free stride-1 forward: (y, xpad) or None when the geometry is not supported.  `xpad`
+    (the zero-bordered input) is what conv2d_filter_grad_nocols reads instead of the columns."""
+    x, w = _f32(x, "conv2d"), _f32(w, "conv2d")
+    B, Cc, H, W = x.shape
+    Kf, C2, kh, kw = w.shape
+    if Cc != C2:
+        raise capi.IncompatibleShape(f"conv2d: Number of input channels ({Cc}) must match second filter dim ({C2})")
+    L = capi.lib()
+    n = L.ag_conv2d_nocols_scratch_floats(B, Cc, H, W, Kf, kh, kw, pad)
+    if n == 0:
+        return None
+    xpad = torch.empty(n, dtype=torch.float32, device=x.device)
+    y = _empty((B, Kf, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1), x)
+    check(L.ag_conv2d_fwd_nocols_f32(_stream(), _ptr(x), _ptr(w), _ptr(y), _ptr(xpad), B, Cc, H, W, Kf, kh, kw, pad))
+    return y, xpad
+
+
+def conv_input_grad_staged(gy, w, pad, x_hw):
+    """The two stages of the column-free stride-1 input gradient: (gx, scratch); the scratch starts
+    with the zero-bordered gy that conv2d_filter_grad_nocols takes.  None when not supported."""
+    gy, w = _f32(gy, "conv2d_transpose"), _f32(w, "conv2d_transpose")
+    B, ych, yh, yw = gy.shape
+    _, xch, kh, kw = w.shape
+    xh, xw = x_hw
+    L = capi.lib()
+    n = L.ag_conv_input_grad_scratch_floats(B, ych, yh, yw, xch, kh, kw, pad, xh, xw)
+    if n == 0:
+        return None
+    scratch = torch.empty(n, dtype=torch.float32, device=gy.device)
+    gx = _empty((B, xch, xh, xw), gy)
+    check(L.ag_conv_input_grad_prepare_f32(_stream(), _ptr(gy), _ptr(w), _ptr(scratch), B, ych, yh, yw, xch, kh, kw, pad, xh, xw))
+    check(L.ag_conv_input_grad_gemm_f32(_stream(), _ptr(scratch), _ptr(gx), B, ych, yh, yw, xch, kh, kw, pad, xh, xw))
+    return gx, scratch
+
+
+def conv2d_filter_grad_nocols(xpad, gypad, x_shape, w_shape, pad):
+    """Column-free filter gradient of a "same" stride-1 convolution from the zero-bordered copies of
+    x (conv2d_nocols) and gy (conv_input_grad_staged)."""
+    B, Cc, H, W = x_shape
+    Kf, _, kh, kw = w_shape
+    L = capi.lib()
+    gw = _empty(w_shape, xpad)
+    ws = _ws(L.ag_conv2d_filter_grad_nocols_f32_workspace(B, Cc, H, W, Kf, kh, kw, pad), xpad)
+    check(L.ag_conv2d_filter_grad_nocols_f32(_stream(), _ptr(xpad), _ptr(gypad), _ptr(gw), B, Cc, H, W, Kf, kh, kw, pad,
+                                             _ptr(ws), ws.numel()))
+    return gw
+
+
 def conv2d_transpose_filter_grad(x, gy, w_shape, pad, stride, dilation=1):
     """Conv2DTransposeFilterGrad::compute (conv2d_transpose.rs:433-451)."""
     x, gy = _f32(x, "conv2d_transpose_filter_grad"), _f32(gy, "conv2d_transpose_filter_grad")

@@ -418,6 +418,86 @@ def test_conv2d_forward_and_gradients(K, orc, rng, case):
     assert np.array_equal(gx_ref, host(gx)[:, :, :rh, :rw])
 
 
+NOCOLS_CASES = [  # B, C (a multiple of 32), K (filters), H, W, k, pad
+    (2, 64, 128, 56, 56, 3, 1),   # north star, 2 of 256 images
+    (5, 32, 32, 20, 24, 3, 1),    # 64-row output tiles straddle several images
+    (3, 32, 64, 18, 18, 5, 2),    # 5x5 "same"
+    (2, 64, 160, 17, 17, 3, 1),   # odd width; more than 128 filters: two row tiles
+    (4, 32, 64, 14, 14, 3, 1),    # config 2's second convolution
+    (2, 32, 32, 20, 20, 3, 0),    # no padding: forward only (the filter gradient needs a "same" convolution)
+    (2, 32, 64, 24, 24, 3, 2),    # pad equal to k - 1: forward only
+]
+
+
+@pytest.mark.parametrize("case", NOCOLS_CASES)
+def test_conv2d_column_free_forward_and_filter_grad(K, orc, rng, case):
+    """Stride-1 convolution without the im2col columns: the forward as one implicit GEMM over the
+    filter taps of a zero-bordered x, and (for "same" convolutions) the filter gradient as a GEMM
+    over the flattened padded planes of x and gy.  Against the f64 oracle and the columns path."""
+    B, C, Kc, H, W, k, p = case
+    OH, OW = H + 2 * p - k + 1, W + 2 * p - k + 1
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, OH, OW)).astype(np.float32)
+    say("column-free forward", case)
+    res = K.conv2d_nocols(dev(x), dev(w), p)
+    assert res is not None, "geometry expected to be supported"
+    y, xpad = res
+    y64, _ = orc.conv2d_fwd(x.astype(np.float64), w.astype(np.float64), p, 1, 1)
+    yabs, _ = orc.conv2d_fwd(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1)
+    assert tuple(y.shape) == y64.shape
+    assert_close_conditioned(host(y), y64, yabs, "column-free forward")
+    y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
+    assert_close_conditioned(host(y_cols), y64, yabs, "columns forward")
+    if 2 * p != k - 1:
+        return
+    say("column-free filter gradient", case)
+    staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+    assert staged is not None
+    gx, gypad = staged
+    gw = host(K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p))
+    _, cols64 = orc.conv2d_fwd(x.astype(np.float64), w.astype(np.float64), p, 1, 1)
+    _, colsabs = orc.conv2d_fwd(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1)
+    gw64 = orc.conv2d_filter_grad(cols64, gy.astype(np.float64), w.shape)
+    gwabs = orc.conv2d_filter_grad(colsabs, np.abs(gy).astype(np.float64), w.shape)
+    assert gw.shape == gw64.shape
+    assert_close_conditioned(gw, gw64, gwabs, "column-free filter gradient")
+    assert_close_conditioned(host(K.conv2d_filter_grad(cols, dev(gy), w.shape)), gw64, gwabs, "columns filter gradient")
+    # deterministic, and the input gradient that shares the bordered gy is the usual one
+    assert np.array_equal(gw, host(K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p)))
+    gx64 = orc.conv2d_transpose(gy.astype(np.float64), w.astype(np.float64), p, 1, 1, out_hw=(H, W))
+    gxabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1, out_hw=(H, W))
+    assert_close_conditioned(host(gx), gx64, gxabs, "staged input gradient")
+
+
+def test_conv2d_column_free_exact_on_small_integers(K, rng):
+    # integer-valued data: every product and partial sum is exact in f32, so the column-free results
+    # must equal the columns path bit for bit (a shifted tap, a dropped row or a border that is not
+    # zero cannot hide in a tolerance)
+    B, C, Kc, H, W, k, p = 3, 32, 64, 22, 26, 3, 1
+    x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
+    say("column-free exact")
+    y, xpad = K.conv2d_nocols(dev(x), dev(w), p)
+    y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
+    assert np.array_equal(host(y), host(y_cols))
+    gx, gypad = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+    gw = K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p)
+    assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape)))
+
+
+def test_conv2d_column_free_refuses_other_geometries(K, rng):
+    L = K.capi.lib()
+    assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1) == 0      # C not a multiple of 32
+    assert L.ag_conv2d_nocols_scratch_floats(2, 32, 4, 4, 32, 3, 3, 1) == 0       # plane too small
+    assert K.conv2d_nocols(dev(np.zeros((2, 3, 28, 28), np.float32)), dev(np.zeros((32, 3, 3, 3), np.float32)), 1) is None
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 32, 3, 3, 0) >= 0
+    x = dev(np.zeros(4096, np.float32))
+    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 32, 3, 3, 0, None, 0)
+    assert rc == 4 and b"geometry not supported" in L.ag_last_error()
+
+
 FUSED_CASES = [  # B, C (input channels of the conv), K (filters), H, W, k, pad
     (2, 64, 128, 56, 56, 3, 1),   # north star, 2 of 256 images
     (5, 32, 32, 20, 24, 3, 1),    # tiles straddle several images
