@@ -43,7 +43,12 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 # true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 KIB = 1024.0
 TRAFFIC_BYTES = {
-    # the step (column-free): to be refreshed from profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt
+    # the step (column-free)
+    "gemm_fwd": (170285.8 * 2.0 + 608000.4) * KIB,                                       # implicit GEMM over bordered x
+    "gemm_filter_grad": ((339673.1 + 36883.5) * 2.0 + 73730.8 + 288.0) * KIB,            # implicit GEMM + fold of the split partials
+    "gemm_input_grad": (233062.8 * 2.0 + 215040.8) * KIB,                                # implicit GEMM over bordered gy
+    "fwd_prepare": ((155428.3 * 2.0 + 322944.0) * 2 / 3 + 445.5 * 2.0 + 288.0) * KIB,    # pad_border averages x (64 ch) and gy (128 ch)
+    "input_grad_prepare": ((155428.3 * 2.0 + 322944.0) * 4 / 3 + 1165.0 * 2.0 + 288.0) * KIB,
     # per-kernel section (column-materialising operators)
     "gemm_fwd_columns": ((898691.8 + 19691.6) * 2.0 + 393230.8 + 8192.0) * KIB,          # whole rounds + narrow-tile tail
     "gemm_filter_grad_columns": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
