@@ -388,6 +388,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             // implicit input gradient: column -> pixel of the (possibly next) image; the columns
             // of the zero border are dropped
             const int row_base = it.m0 + wm * WM + 4 * half;
+            float *dst0[NI];
+            bool ok[NI];
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 int col = it.r0 + wn * WN + l31 + j * 32;
@@ -398,20 +400,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                     img = p.sC;
                 }
                 const int iy = col / p.conv_wp, ix = col - iy * p.conv_wp;
-                const bool ok = in_range && ix < p.conv_w;
-                float *dst0 = Cb + img + iy * p.conv_w + ix;
+                ok[j] = in_range && ix < p.conv_w;
+                dst0[j] = Cb + img + iy * p.conv_w + ix;
+            }
+            // rows outermost: the segments of one output row leave back to back, so the cache lines
+            // they share are completed before they can be evicted
 #pragma unroll
-                for (int i = 0; i < MI; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
-                        if (ok && row < p.M) {
-                            float *dst = dst0 + (long long)row * ldc;
+                for (int v = 0; v < 16; ++v) {
+                    const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        if (ok[j] && row < p.M) {
+                            float *dst = dst0[j] + (long long)row * ldc;
                             const float r = alpha * acc[i][j][v];
                             *dst = beta == 0.f ? r : r + beta * *dst;
                         }
-                    }
-            }
+                }
             return false;
         }
         const bool full = it.m0 + BM <= p.M && it.n0 + BN <= p.N;
