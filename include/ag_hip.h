@@ -181,6 +181,12 @@ ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, con
                                          int B, int C, int H, int W, int K, int kh, int kw, int pad);
 ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C,
                                       int H, int W, int K, int kh, int kw, int pad);
+/* The forward GEMM over an existing bordered copy with another filter: what Conv2DWithCols
+ * (conv2d.rs:589-629) becomes when its "columns" input is such a copy.  wf: K*C*kh*kw floats. */
+ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, const float *xpad, const float *w,
+                                             float *wf, float *y, int B, int C, int H, int W, int K,
+                                             int kh, int kw, int pad);
+/* 0 = geometry not supported by the column-free filter gradient. */
 size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw,
                                                   int pad);
 ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, const float *xpad, const float *gypad,

@@ -103,6 +103,7 @@ PROTOTYPES = {
     "ag_conv2d_fwd_nocols_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
     "ag_conv2d_nocols_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8),
     "ag_conv2d_nocols_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 8),
+    "ag_conv2d_nocols_with_filter_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32_workspace": (c_sz, [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8 + [c_p, c_sz]),
 }

@@ -236,14 +236,35 @@ extern "C" ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float 
     return ag_conv2d_nocols_gemm_f32(stream, xpad, y, B, C, H, W, K, kh, kw, pad);
 }
 
+// The forward GEMM over an existing bordered copy with another filter (Conv2DWithCols, conv2d.rs:
+// 589-629, when the "columns" it is given are a bordered input): `wf` receives K*C*kh*kw floats.
+extern "C" ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, const float *xpad, const float *w, float *wf,
+                                                        float *y, int B, int C, int H, int W, int K, int kh, int kw, int pad)
+{
+    FusedGeom g;
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y) && aligned16(wf),
+               AG_ERR_INVALID_DIMS, "conv2d (column-free): geometry not supported");
+    AG_REQUIRE(xpad && w && wf && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    hipStream_t st = as_stream(stream);
+    hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
+                       kh * kw);
+    if (ag_status_t s = check_launch("conv2d")) return s;
+    return gemm_conv_input_grad(st, wf, xpad + kFwdLeadFloats, y, B, K, C, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1, kh, kw,
+                                g.Hp, g.Wp);
+}
+
 // gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the first
 // B*K*Hp*Wp floats of its scratch); the geometry must be a "same" convolution (2*pad == k-1) so
 // that x and gy share one padded plane shape.
 extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw, int pad)
 {
-    FusedGeom g;
-    if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g)) return 0;
-    const int kq = filter_grad_positions(g, H + 2 * pad - kh + 1, pad);
+    FusedGeom g, gg;
+    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
+    if (2 * pad != kh - 1 || 2 * pad != kw - 1 || K % 4 != 0 || !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) ||
+        !fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg) || g.Hp != gg.Hp || g.Wp != gg.Wp ||
+        (long long)C * g.Hp * g.Wp >= (1LL << 30))
+        return 0;
+    const int kq = filter_grad_positions(g, OH, pad);
     return kq ? gemm_conv_filter_grad_workspace(B, K, C, kh * kw, kq) : 0;
 }
 

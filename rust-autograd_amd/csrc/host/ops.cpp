@@ -154,10 +154,29 @@ struct Conv2DFilterGrad : Op, ConvHyper {  // conv2d.rs:736-776
     const char *name() const override { return "Conv2DFilterGrad"; }
     OpError compute(ComputeContext &ctx) const override
     {
-        const NdArray cols = ctx.input(0), gy = ctx.input(1), w = ctx.input(2);  // must be columns
+        const NdArray cols = ctx.input(0), gy = ctx.input(1), w = ctx.input(2);
         const int B = (int)gy.shape()[0], K = (int)gy.shape()[1], P = (int)(gy.shape()[2] * gy.shape()[3]);
         const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
         NdArray gw = NdArray::empty(w.shape());
+        if (cols.ndim() == 1) {  // the zero-bordered input of a column-free Conv2D (stride 1, dilation 1)
+            const int C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
+            const int OH = (int)gy.shape()[2], OW = (int)gy.shape()[3];
+            const int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
+            const size_t n_gyp = ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, H, W);
+            const size_t nb = ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad);
+            if (n_gyp == 0 || nb == 0 || cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad))
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: the bordered input does not match gy and the filter");
+            NdArray gyp = NdArray::empty({(int64_t)n_gyp});
+            OpError e = from_status(
+                ag_conv_input_grad_prepare_f32(ctx.stream(), gy.ptr(), w.ptr(), gyp.ptr(), B, K, OH, OW, C, kh, kw, pad, H, W));
+            if (!e.ok()) return e;
+            NdArray ws = workspace(nb);
+            e = from_status(ag_conv2d_filter_grad_nocols_f32(ctx.stream(), cols.ptr(), gyp.ptr(), gw.ptr(), B, C, H, W, K, kh, kw,
+                                                             pad, ws.ptr(), ws.len() * 4));
+            if (!e.ok()) return e;
+            ctx.append_output(gw);
+            return OpError::none();
+        }
         const size_t nb = ag_conv2d_filter_grad_f32_workspace(B, CK, P, K);
         NdArray ws = workspace(nb);
         const OpError e = from_status(
@@ -175,6 +194,24 @@ struct Conv2DWithCols : Op, ConvHyper {  // conv2d.rs:589-629
     OpError compute(ComputeContext &ctx) const override
     {
         const NdArray cols = ctx.input(0), w = ctx.input(1);
+        if (cols.ndim() == 1) {
+            // the zero-bordered input of a column-free Conv2D; the third input (only its extents are
+            // read) has the shape of the result
+            if (ctx.num_inputs() < 3) return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: columns expected");
+            const NdArray like = ctx.input(2);
+            const int B = (int)like.shape()[0], OH = (int)like.shape()[2], OW = (int)like.shape()[3];
+            const int K = (int)w.shape()[0], C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
+            const int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
+            if (cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad))
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: the bordered input does not match the filter");
+            NdArray y = NdArray::empty({B, K, OH, OW});
+            NdArray wf = NdArray::empty(w.shape());
+            const OpError e = from_status(ag_conv2d_nocols_with_filter_f32(ctx.stream(), cols.ptr(), w.ptr(), wf.ptr(), y.ptr(), B, C,
+                                                                           H, W, K, kh, kw, pad));
+            if (!e.ok()) return e;
+            ctx.append_output(y);
+            return OpError::none();
+        }
         // cols carries [B, C*kh*kw, OH, OW] here (the reference labels it [B,C,kw,kh,OH,OW], conv2d.rs:484)
         const int B = (int)cols.shape()[0], K = (int)w.shape()[0];
         const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
@@ -209,6 +246,20 @@ struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
         if (OH <= 0 || OW <= 0)
             return OpError::make(ErrorKind::IncompatibleShape, "conv2d: filter extent exceeds the padded input");
         NdArray y = NdArray::empty({B, K, OH, OW});
+        // Column-free path when all three contractions of this convolution support it: the second
+        // output, which only Conv2DFilterGrad and Conv2DWithCols read, is then the zero-bordered
+        // input (rank 1) instead of the columns.
+        const size_t n_xpad = (stride == 1 && dilation == 1) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad) : 0;
+        if (n_xpad > 0 && ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad) > 0 &&
+            ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, H, W) > 0) {
+            NdArray xpad = NdArray::empty({(int64_t)n_xpad});
+            const OpError e = from_status(
+                ag_conv2d_fwd_nocols_f32(ctx.stream(), x.ptr(), w.ptr(), y.ptr(), xpad.ptr(), B, C, H, W, K, kh, kw, pad));
+            if (!e.ok()) return e;
+            ctx.append_output(y);
+            ctx.append_output(xpad);
+            return OpError::none();
+        }
         NdArray cols = NdArray::empty({B, (int64_t)C * kh * kw, OH, OW});
         const OpError e = from_status(ag_conv2d_fwd_f32(ctx.stream(), x.ptr(), w.ptr(), y.ptr(), cols.ptr(), B, C, H, W, K, kh,
                                                         kw, pad, stride, dilation));
@@ -263,6 +314,7 @@ void Conv2DFilterGrad::grad(GradientContext &ctx) const
     const Tensor ggy = g->builder()
                            .append_input(cols, false)
                            .append_input(ggw, false)
+                           .append_input(tensor_ops::stop_gradient(gy), false)  // extents of the result
                            .append_backprop_input(x0)
                            .append_backprop_input(ggw)
                            .build(std::make_unique<Conv2DWithCols>(ConvHyper{pad, stride, dilation}));

@@ -691,3 +691,53 @@ def test_add_broadcast_and_the_reduced_gradient(G, rng, shape, bshape):
     want = w.astype(np.float64).sum(axis=axes, keepdims=True)
     assert gbv.shape == tuple(bshape)
     assert_close(gbv, want, "bias gradient", scale=np.abs(w).astype(np.float64).sum(axis=axes, keepdims=True))
+
+
+# ------------------------------------------------------------------------------- column-free convolution in the graph
+@pytest.mark.parametrize("B,Cin,Cout,H,k,pad", [(4, 32, 64, 12, 3, 1), (2, 64, 128, 20, 3, 1), (3, 32, 32, 16, 5, 2)])
+def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, pad):
+    # channel counts that are multiples of 32, "same" stride-1 convolution: Conv2D keeps a zero-bordered
+    # input instead of the columns and all three operators run column-free; values against the oracle
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = glorot(rng, (Cout, Cin, k, k))
+    env = G.VariableEnvironment()
+    c = env.context()
+    x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+    y = c.conv2d(x, w, pad, 1)
+    gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+    second = c.nth_tensor(y, 1)
+    say(f"column-free conv through the graph B={B} C={Cin} K={Cout} H={H} k={k}")
+    yv, gxv, gwv, kept = c.eval([y, gx, gw, second], {"x": xv, "w": wv})
+    assert kept.ndim == 1, "Conv2D is expected to keep the bordered input, not the columns, at this shape"
+    oy, ocols = orc.conv2d_fwd(xv, wv, pad, 1, 1)
+    assert_close(yv, oy, "y", scale=1.0)
+    gyv = (2 * yv).astype(np.float32)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, 1, 1, out_hw=(H, H)), "gx", scale=np.abs(gxv).max(), rtol=2e-4)
+
+
+def test_conv2d_column_free_second_order(G, orc, rng):
+    # the gradient of the filter gradient: w.r.t. x (Conv2DTranspose of the incoming gradient) and
+    # w.r.t. gy (Conv2DWithCols, here over the bordered input)
+    B, Cin, Cout, H = 2, 32, 32, 12
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = glorot(rng, (Cout, Cin, 3, 3))
+    rv = rng.standard_normal(wv.shape).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x, w, r = (c.placeholder(n, list(a.shape)) for n, a in (("x", xv), ("w", wv), ("r", rv)))
+    y = c.conv2d(x, w, 1, 1)
+    gys = c.mul(y, y)
+    (gw,) = c.grad([c.sum_all(gys)], [w])          # gw = filter_grad(x, gy = 2y)
+    (ggx,) = c.grad([c.sum_all(c.mul(gw, r))], [x])
+    say("column-free second order")
+    gwv, ggxv = c.eval([gw, ggx], {"x": xv, "w": wv, "r": rv})
+    # f(x) = <filter_grad(x, 2 conv(x, w)), r>; with gy = 2 conv(x, w):
+    # df/dx = conv_transpose(gy, r) + conv_transpose(2 conv(x, r), w)
+    oy, ocols = orc.conv2d_fwd(xv, wv, 1, 1, 1)
+    gyv = (2 * oy).astype(np.float32)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    oyr, _ = orc.conv2d_fwd(xv, rv, 1, 1, 1)
+    want = orc.conv2d_transpose(gyv, rv, 1, 1, 1, out_hw=(H, H)).astype(np.float64) + \
+        orc.conv2d_transpose((2 * oyr).astype(np.float32), wv, 1, 1, 1, out_hw=(H, H)).astype(np.float64)
+    assert_close(ggxv, want, "ggx", scale=np.abs(want).max(), rtol=3e-4)
