@@ -129,11 +129,18 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
 {
     if (pad > kh - 1 || pad > kw - 1 || ych % 32 != 0 || B < 1 || xch < 1) return false;
     if (yh != xh + 2 * pad - kh + 1 || yw != xw + 2 * pad - kw + 1 || yh < 1 || yw < 1) return false;
-    g->Hp = xh + kh - 1;
-    g->Wp = xw + kw - 1;
-    // padded planes and the per-image column range must be multiples of four elements
-    while (((long long)xh * g->Wp) % 4 != 0 || ((long long)g->Hp * g->Wp) % 4 != 0)
-        if (++g->Wp > xw + kw + 6) return false;
+    // A padded row holds the left border (kw-1-pad zeros) and the data; it needs no right border of
+    // its own: a read that runs past the end of a row by up to kw-1-pad elements lands in the left
+    // border of the next row, which is just as zero.  The row pitch and the plane (rows added at the
+    // bottom) grow until the per-image column range and the plane are multiples of four elements.
+    g->Wp = yw + (kw - 1 - pad);
+    for (;; ++g->Wp) {
+        if (g->Wp > xw + kw + 6) return false;
+        if (((long long)xh * g->Wp) % 4 != 0) continue;
+        g->Hp = xh + kh - 1;
+        while (((long long)g->Hp * g->Wp) % 4 != 0) ++g->Hp;
+        break;
+    }
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + 1024;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
