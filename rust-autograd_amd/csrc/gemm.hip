@@ -732,8 +732,45 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     const long long blocks = (long long)p.tiles_m * p.tiles_n;
     AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "conv2d_transpose: too many tiles (%lld)", blocks);
     p.total_blocks = (unsigned)blocks;
+    // whole rounds of the persistent grid with the wide tile, then the remaining columns with a
+    // narrower one (as for the folded GEMM over columns)
+    int tail_cfg = -1;
+    GemmParams tail = p;
+    if (cfg == 14 && p.tiles_m == 1 && g_grid_scale <= 0) {
+        const long long G = direct_grid(num_cus());
+        const long long rounds = blocks / G, rem = blocks % G;
+        if (rounds >= 1 && rem > 0) {
+            const int bn = kCfgs[cfg].bn;
+            const long long main_cols = rounds * G * bn;
+            double best = (double)rounds + 1.0 - 0.05;
+            static const int narrow[] = {18, 13};  // 128 x 64, 128 x 128
+            static const double eff[] = {0.85, 0.92};
+            for (int t = 0; t < 2; ++t) {
+                const int bnt = kCfgs[narrow[t]].bn;
+                const long long items = cdiv(p.N - main_cols, bnt);
+                const double cost = (double)rounds + (double)cdiv(items, G) * bnt / bn / eff[t];
+                if (cost < best && p.n_img >= bnt) {
+                    best = cost;
+                    tail_cfg = narrow[t];
+                }
+            }
+            if (tail_cfg >= 0) {
+                tail.n_off = (int)main_cols;
+                tail.tiles_n = (int)cdiv(p.N - main_cols, kCfgs[tail_cfg].bn);
+                tail.total_blocks = (unsigned)tail.tiles_n;
+                p.N = (int)main_cols;
+                p.tiles_n = (int)(rounds * G);
+                p.total_blocks = (unsigned)p.tiles_n;
+            }
+        }
+    }
     launch_direct(st, cfg, true, false, p, num_cus(), g_grid_scale);
-    return check_launch("conv2d_transpose");
+    if (ag_status_t s = check_launch("conv2d_transpose")) return s;
+    if (tail_cfg >= 0) {
+        launch_direct(st, tail_cfg, true, false, tail, num_cus(), g_grid_scale);
+        return check_launch("conv2d_transpose");
+    }
+    return AG_OK;
 }
 
 constexpr int kConvFilterGradCfg = 17;  // 128 x 192 tiles, both operands k-contiguous

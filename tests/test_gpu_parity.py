@@ -470,11 +470,15 @@ def test_conv2d_column_free_forward_and_filter_grad(K, orc, rng, case):
     assert_close_conditioned(host(gx), gx64, gxabs, "staged input gradient")
 
 
-def test_conv2d_column_free_exact_on_small_integers(K, rng):
+@pytest.mark.parametrize("B,C,Kc,H,W,k,p", [
+    (3, 32, 64, 22, 26, 3, 1),
+    (22, 64, 128, 56, 56, 3, 1),   # more tiles than the persistent grid has blocks: whole rounds, then a narrow-tile launch
+    (2, 32, 32, 16, 16, 5, 2),
+])
+def test_conv2d_column_free_exact_on_small_integers(K, rng, B, C, Kc, H, W, k, p):
     # integer-valued data: every product and partial sum is exact in f32, so the column-free results
     # must equal the columns path bit for bit (a shifted tap, a dropped row or a border that is not
     # zero cannot hide in a tolerance)
-    B, C, Kc, H, W, k, p = 3, 32, 64, 22, 26, 3, 1
     x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
     w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
     gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
