@@ -67,17 +67,22 @@ __global__ __launch_bounds__(256) void pad_border_kernel(const float *__restrict
                                                          long long quads, int OH, int OW, int Hp, int Wp, int top,
                                                          int left)
 {
-    const int plane_quads = Hp * Wp / 4;
+    const unsigned plane_quads = (unsigned)(Hp * Wp) / 4u;
     for (long long qd = blockIdx.x * 256LL + threadIdx.x; qd < quads; qd += gridDim.x * 256LL) {
-        const long long plane = qd / plane_quads;
-        const int e0 = (int)(qd - plane * plane_quads) * 4;
+        // one division for the plane, one for the row; (row, column) then step along the four elements
+        const long long plane = quads <= 0xffffffffLL ? (long long)((unsigned)qd / plane_quads) : qd / plane_quads;
+        const unsigned e0 = (unsigned)(qd - plane * plane_quads) * 4u;
+        int r = (int)(e0 / (unsigned)Wp), sx = (int)(e0 - (unsigned)r * (unsigned)Wp);
         const float *src = gy + plane * (long long)OH * OW;
         float v[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int r = (e0 + t) / Wp, s = (e0 + t) - r * Wp;
-            const int oy = r - top, ox = s - left;
+            const int oy = r - top, ox = sx - left;
             v[t] = ((unsigned)oy < (unsigned)OH && (unsigned)ox < (unsigned)OW) ? src[oy * OW + ox] : 0.f;
+            if (++sx == Wp) {
+                sx = 0;
+                ++r;
+            }
         }
         st_stream(reinterpret_cast<float4 *>(gyp) + qd, make_float4(v[0], v[1], v[2], v[3]));
     }
