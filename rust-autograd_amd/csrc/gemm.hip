@@ -497,20 +497,27 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
         // 128x256, 256x128, 192x128, 128x192, 128x128, and 64x128 (two blocks per CU) for outputs of up to 64 rows
         static const int dl[] = {14, 15, 16, 17, 13, kDirectCfg64};
         static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.92, 0.8};
+        // The cheapest tile among those that give the chip at least half a round of blocks: padded
+        // area over efficiency, counted in whole rounds of the persistent grid while there are few
+        // of them (264 blocks on 256 CUs take two rounds, 200 take one).
         int best = -1;
         double best_cost = 1e300;
-        long long best_blocks = 0;
         for (int c = 0; c < 6; ++c) {
             const TileCfg &t = kCfgs[dl[c]];
             const long long tm = cdiv(M, t.bm), tn = cdiv(N, t.bn);
-            const double cost = (double)tm * t.bm * tn * t.bn / eff[c];
+            const long long blocks = tm * tn * zcount;
+            const long long grid = direct_grid(num_cus()) * (dl[c] == kDirectCfg64 ? 2 : 1);
+            if (blocks < direct_grid(num_cus()) / 2) continue;
+            const long long counted = blocks < 8 * grid ? cdiv(blocks, grid) * grid : blocks;
+            // equal round counts: the tile with less padding wins
+            const double padding = (double)tm * t.bm * tn * t.bn / ((double)M * N) - 1.0;
+            const double cost = (double)counted * t.bm * t.bn / zcount / eff[c] * (1.0 + 0.5 * padding);
             if (cost < best_cost * 0.995) {
                 best_cost = cost;
                 best = dl[c];
-                best_blocks = tm * tn * zcount;
             }
         }
-        if (best_blocks >= (best == kDirectCfg64 ? 128 : 256)) return best;
+        if (best >= 0) return best;
     }
     static const int short_k[] = {11, 10, 12, 8};  // 192x128, 128x128, 128x64, 64x64 (BK 16)
     static const int long_k[] = {0, 1, 2, 3};      // 128x128, 128x64, 64x128, 64x64 (BK 32)
@@ -588,8 +595,11 @@ __global__ __launch_bounds__(256) void scale_c_kernel(float *C, int M, int N, lo
     }
 }
 
+// `partials_only` >= 0 (split accumulations only): the partial sums are written from split slot
+// `partials_only` of the workspace onwards and left for the caller to fold; `*used_splits` receives
+// their number.
 static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, void *ws, size_t ws_bytes,
-                            int splits)
+                            int splits, int partials_only = -1, int *used_splits = nullptr)
 {
     if (ag_status_t s = validate(who, c)) return s;
     if (c.M == 0 || c.N == 0 || c.batch == 0) return AG_OK;
@@ -601,6 +611,42 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         return check_launch(who);
     }
     AG_REQUIRE(c.A && c.B, AG_ERR_INVALID_DIMS, "%s: null operand", who);
+    // A long contraction that misses the direct-to-LDS kernel only because K is not a multiple of
+    // its k tile: the whole tiles go there, the remaining K % 32 are accumulated on top by the
+    // register-staged kernel (2-3 % of the work).
+    if (c.K % 32 != 0 && c.K >= 256 && (c.kbatch > 1 || c.K >= 1024) && g_force_cfg < 0 && !direct_ok(c)) {
+        GemmCall body = c;
+        body.K = c.K - c.K % 32;
+        if (direct_ok(body)) {
+            GemmCall rest = c;
+            rest.K = c.K % 32;
+            rest.beta = 1.f;
+            rest.A = c.A + (c.transA ? (long long)body.K * c.lda : (long long)body.K);
+            rest.B = c.B + (c.transB ? (long long)body.K : (long long)body.K * c.ldb);
+            const size_t slot = sizeof(float) * (size_t)c.M * c.N;
+            if (splits > 1 && partials_only < 0 && c.batch == 1 && ws && ws_bytes >= 2 * (size_t)splits * slot) {
+                // both passes leave their partial sums side by side; one fold adds them all
+                int s_body = 0, s_rest = 0;
+                if (ag_status_t s = run_gemm(st, who, body, ws, ws_bytes, splits, 0, &s_body)) return s;
+                if (s_body <= 1) {  // the body did not split after all and has written C
+                    rest.beta = 1.f;
+                    return run_gemm(st, who, rest, ws, ws_bytes, splits);
+                }
+                rest.beta = c.beta;
+                // the tail is a few per cent of the work: an eighth of the splits keeps its partial sums small
+                if (ag_status_t s = run_gemm(st, who, rest, ws, ws_bytes, splits >= 16 ? splits / 8 : 2, s_body, &s_rest)) return s;
+                // rest split: fold everything onto beta * C; rest not split: it has written
+                // alpha * rest + beta * C, the body's partial sums are added on top
+                const long long total = (long long)c.M * c.N;
+                hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
+                                   dim3(256), 0, st, static_cast<const float *>(ws), s_rest > 1 ? s_body + s_rest : s_body, total,
+                                   c.C, c.M, c.N, c.ldc, c.alpha, s_rest > 1 ? c.beta : 1.f);
+                return check_launch(who);
+            }
+            if (ag_status_t s = run_gemm(st, who, body, ws, ws_bytes, splits)) return s;
+            return run_gemm(st, who, rest, ws, ws_bytes, splits);
+        }
+    }
     // tile offsets inside one operand slice are 32-bit
     const long long a_span = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
     const long long b_span = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
@@ -679,12 +725,14 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     }
 
     float *real_c = c.C;
+    if (used_splits) *used_splits = p.splits;
+    const int first_slot = partials_only > 0 ? partials_only : 0;
     if (p.splits > 1) {
-        const size_t need = sizeof(float) * (size_t)p.splits * c.M * c.N;
+        const size_t need = sizeof(float) * (size_t)(first_slot + p.splits) * c.M * c.N;
         AG_REQUIRE(c.batch == 1, AG_ERR_INVALID_DIMS, "%s: split accumulation with independent batches", who);
         AG_REQUIRE(ws && ws_bytes >= need, AG_ERR_INVALID_DIMS, "%s: workspace of %zu bytes needed, %zu given",
                    who, need, ws_bytes);
-        p.C = static_cast<float *>(ws);
+        p.C = static_cast<float *>(ws) + (size_t)first_slot * c.M * c.N;
     }
     // A is k-contiguous when not transposed; B is k-contiguous when transposed.
     const int la = loader_kind(!c.transA, c.A, c.lda, c.K, c.sA, c.sAk);
@@ -696,7 +744,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         launch_direct(st, tail_cfg, !c.transA, c.transB != 0, tail, num_cus(), g_grid_scale);
         if (ag_status_t s = check_launch(who)) return s;
     }
-    if (p.splits > 1) {
+    if (p.splits > 1 && partials_only < 0) {
         const long long total = (long long)c.M * c.N;
         hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
                            dim3(256), 0, st, static_cast<const float *>(ws), p.splits, p.sCsplit, real_c, c.M,
@@ -895,7 +943,9 @@ extern "C" size_t ag_gemm_batchsum_f32_workspace(int M, int N, int K, int batch)
 {
     if (M <= 0 || N <= 0 || batch <= 0) return 16;
     const int splits = choose_splits(M, N, K, batch);
-    return splits > 1 ? sizeof(float) * (size_t)splits * M * N : 16;
+    // a contraction with a K tail runs as two passes that keep their partial sums side by side
+    const size_t passes = (K % 32 != 0 && K >= 256) ? 2 : 1;
+    return splits > 1 ? sizeof(float) * passes * (size_t)splits * M * N : 16;
 }
 
 extern "C" ag_status_t ag_gemm_batchsum_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K,

@@ -348,6 +348,43 @@ def test_matmul_long_contraction_few_tiles(K, rng, m, n, k, ta, tb):
     assert np.array_equal(host(K.matmul(dev(ai), dev(bi), ta, tb)), exact.astype(np.float32))
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_long_k_with_a_tail(K, rng, ta, tb):
+    """K = 32 q + r: whole k tiles on the direct-to-LDS kernel, the remaining r accumulated on top."""
+    for (m, n, k, batch, beta) in ((256, 384, 1040, 3, 0.0), (128, 512, 2060, 2, 0.5)):
+        a = rng.standard_normal((batch, k, m) if ta else (batch, m, k)).astype(np.float32)
+        b = rng.standard_normal((batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+        c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
+        c = dev(c0)
+        say("gemm K tail", ta, tb, m, n, k, batch, beta)
+        K.gemm(ta, tb, m, n, k, 1.5, dev(a), a.shape[2], a.shape[1] * a.shape[2], dev(b), b.shape[2],
+               b.shape[1] * b.shape[2], beta, c, n, m * n, batch)
+        A = (a.transpose(0, 2, 1) if ta else a).astype(np.float64)
+        Bm = (b.transpose(0, 2, 1) if tb else b).astype(np.float64)
+        truth = 1.5 * (A @ Bm) + beta * c0
+        assert_close_conditioned(host(c), truth, 1.5 * (np.abs(A) @ np.abs(Bm)) + abs(beta) * np.abs(c0), "gemm with a K tail")
+
+
+@pytest.mark.parametrize("beta", [0.0, 2.0])
+def test_gemm_batchsum_long_k_with_a_tail(K, rng, beta):
+    """The stride-2 filter gradient's contraction (784 positions per image = 24 k tiles + 16)."""
+    m, n, k, batch = 128, 576, 784, 40
+    a = rng.standard_normal((batch, m, k)).astype(np.float32)
+    b = rng.standard_normal((batch, n, k)).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    c = dev(c0)
+    say("gemm_batchsum K tail", beta)
+    K.gemm_batchsum(0, 1, m, n, k, 1.0, dev(a), k, m * k, dev(b), k, n * k, beta, c, n, batch)
+    truth = np.einsum("bmk,bnk->mn", a.astype(np.float64), b.astype(np.float64)) + beta * c0
+    absdot = np.einsum("bmk,bnk->mn", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64)) + abs(beta) * np.abs(c0)
+    assert_close_conditioned(host(c), truth, absdot, "batchsum with a K tail")
+    ai = rng.integers(-2, 3, a.shape).astype(np.float32)
+    bi = rng.integers(-2, 3, b.shape).astype(np.float32)
+    ci = dev(np.zeros((m, n), np.float32))
+    K.gemm_batchsum(0, 1, m, n, k, 1.0, dev(ai), k, m * k, dev(bi), k, n * k, 0.0, ci, n, batch)
+    assert np.array_equal(host(ci), np.einsum("bmk,bnk->mn", ai.astype(np.int64), bi.astype(np.int64)).astype(np.float32))
+
+
 def test_gemm_degenerate_k_and_beta(K, rng):
     c0 = rng.random((5, 6), dtype=np.float32)
     c = dev(c0)
