@@ -249,7 +249,9 @@ struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
         // Column-free path when all three contractions of this convolution support it: the second
         // output, which only Conv2DFilterGrad and Conv2DWithCols read, is then the zero-bordered
         // input (rank 1) instead of the columns.
-        const size_t n_xpad = (stride == 1 && dilation == 1) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad) : 0;
+        // (small problems are launch-bound and the column path has fewer launches: from 64 MB of columns on)
+        const bool large = (long long)B * C * kh * kw * OH * OW >= (16LL << 20);
+        const size_t n_xpad = (large && stride == 1 && dilation == 1) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad) : 0;
         if (n_xpad > 0 && ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad) > 0 &&
             ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, H, W) > 0) {
             NdArray xpad = NdArray::empty({(int64_t)n_xpad});

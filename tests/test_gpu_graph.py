@@ -694,7 +694,7 @@ def test_add_broadcast_and_the_reduced_gradient(G, rng, shape, bshape):
 
 
 # ------------------------------------------------------------------------------- column-free convolution in the graph
-@pytest.mark.parametrize("B,Cin,Cout,H,k,pad", [(4, 32, 64, 12, 3, 1), (2, 64, 128, 20, 3, 1), (3, 32, 32, 16, 5, 2)])
+@pytest.mark.parametrize("B,Cin,Cout,H,k,pad", [(64, 32, 64, 32, 3, 1), (24, 64, 128, 36, 3, 1), (32, 32, 32, 28, 5, 2)])
 def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, pad):
     # channel counts that are multiples of 32, "same" stride-1 convolution: Conv2D keeps a zero-bordered
     # input instead of the columns and all three operators run column-free; values against the oracle
@@ -719,7 +719,7 @@ def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, p
 def test_conv2d_column_free_second_order(G, orc, rng):
     # the gradient of the filter gradient: w.r.t. x (Conv2DTranspose of the incoming gradient) and
     # w.r.t. gy (Conv2DWithCols, here over the bordered input)
-    B, Cin, Cout, H = 2, 32, 32, 12
+    B, Cin, Cout, H = 64, 32, 32, 32   # 18.9 M column elements: above the size from which Conv2D goes column-free
     xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
     wv = glorot(rng, (Cout, Cin, 3, 3))
     rv = rng.standard_normal(wv.shape).astype(np.float32)
@@ -731,7 +731,8 @@ def test_conv2d_column_free_second_order(G, orc, rng):
     (gw,) = c.grad([c.sum_all(gys)], [w])          # gw = filter_grad(x, gy = 2y)
     (ggx,) = c.grad([c.sum_all(c.mul(gw, r))], [x])
     say("column-free second order")
-    gwv, ggxv = c.eval([gw, ggx], {"x": xv, "w": wv, "r": rv})
+    gwv, ggxv, kept = c.eval([gw, ggx, c.nth_tensor(y, 1)], {"x": xv, "w": wv, "r": rv})
+    assert kept.ndim == 1, "Conv2D is expected to keep the bordered input at this shape"
     # f(x) = <filter_grad(x, 2 conv(x, w)), r>; with gy = 2 conv(x, w):
     # df/dx = conv_transpose(gy, r) + conv_transpose(2 conv(x, r), w)
     oy, ocols = orc.conv2d_fwd(xv, wv, 1, 1, 1)
