@@ -528,6 +528,42 @@ def test_conv2d_column_free_exact_on_small_integers(K, rng, B, C, Kc, H, W, k, p
     assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape)))
 
 
+def test_conv2d_column_free_random_geometries_exact(K):
+    # a fixed sample of geometries (odd extents, every padding from 0 to k-1, channel counts on both sides of
+    # the 64-row tile, images smaller and larger than a tile): integer-valued data, so forward, filter
+    # gradient and input gradient must equal the columns path bit for bit wherever the library accepts
+    # the geometry
+    r = np.random.default_rng(20240611)
+    L = K.capi.lib()
+    ran_fwd = ran_bwd = 0
+    for _ in range(40):
+        k = int(r.choice([3, 3, 5]))
+        p = int(r.integers(0, k))
+        B = int(r.integers(1, 6))
+        C = int(r.choice([32, 64, 96]))
+        Kc = int(r.choice([32, 64, 96, 160]))
+        H, W = int(r.integers(max(k, 9), 41)), int(r.integers(max(k, 9), 41))
+        OH, OW = H + 2 * p - k + 1, W + 2 * p - k + 1
+        x = r.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+        gy = r.integers(-2, 3, (B, Kc, OH, OW)).astype(np.float32)
+        say("column-free random geometry", (B, C, Kc, H, W, k, p))
+        y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
+        res = K.conv2d_nocols(dev(x), dev(w), p)
+        if res is not None:
+            ran_fwd += 1
+            assert np.array_equal(host(res[0]), host(y_cols)), (B, C, Kc, H, W, k, p)
+        gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, 1, out_hw=(H, W), return_cols=True)
+        staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+        if staged is not None:
+            assert np.array_equal(host(staged[0]), host(gx_cols)), (B, C, Kc, H, W, k, p)
+        if res is not None and staged is not None and L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p) > 0:
+            ran_bwd += 1
+            gw = K.conv2d_filter_grad_nocols(res[1], staged[1], x.shape, w.shape, p)
+            assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape))), (B, C, Kc, H, W, k, p)
+    assert ran_fwd >= 20 and ran_bwd >= 5, (ran_fwd, ran_bwd)
+
+
 def test_conv2d_column_free_refuses_other_geometries(K, rng):
     L = K.capi.lib()
     assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1) == 0      # C not a multiple of 32
