@@ -54,6 +54,8 @@ TRAFFIC_BYTES = {
     "gemm_filter_grad_columns": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
     "im2col": (112667.1 * 2.0 + 1806374.2) * KIB,
     "col2im": (919260.8 * 2.0 + 200704.0) * KIB,
+    "maxpool_fwd": (198682.5 * 2.0 + 301828.7) * KIB,   # x in; y, f32 index and int32 index out
+    "maxpool_bwd": (113241.7 * 2.0 + 418113.7) * KIB,   # gy and int32 index in (rows shared by two chunks read twice); gx out
 }
 
 
@@ -66,6 +68,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
     ap.add_argument("--cpu-images", type=int, default=32, help="images in the CPU baseline sample")
+    ap.add_argument("--pool-only", action="store_true",
+                    help="run only the two pooling kernels of the per-kernel section, three times each (for counter passes)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch one plain copy kernel (ag_scale_f32 by 1.0) over 2^28 floats, "
                          "so that a rocprofv3 --pmc run of this command holds a kernel of known traffic "
@@ -181,6 +185,17 @@ def main():
     OH = Kn.conv_out_size(H, KH, PAD, STRIDE, DIL)
     P, CK = OH * OH, C * KH * KH
 
+    if args.pool_only:
+        xp_ = torch.randn(256, 128, 56, 56, device=dev)
+        yp_, am_, il_ = Kn.max_pool2d(xp_, 3, 0, 2)
+        for _ in range(2):
+            Kn.max_pool2d(xp_, 3, 0, 2)
+        for _ in range(3):
+            Kn.max_pool2d_grad(yp_, am_, il_, tuple(xp_.shape), 3, 0, 2)
+        torch.cuda.synchronize()
+        print(json.dumps({"pool_only": True, "launches": 3}))
+        return
+
     g = torch.Generator(device=dev)
     g.manual_seed(1234)
     x = torch.randn(Bn, C, H, W, device=dev, generator=g)
@@ -287,13 +302,17 @@ def micro(torch, Kn, capi, dev):
     sp, pp, cp = Kn._stream, Kn._ptr, capi.check
     ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), pp(il), 256, 128, 56, 56, 3, 0, 2)), 10)
     res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "note": "also writes the exact int32 index (95.6 MB, not counted) that the backward needs above 2^24 elements"}
+                          "traffic_bytes": round(TRAFFIC_BYTES["maxpool_fwd"]),
+                          "frac_hbm_of_traffic": round(TRAFFIC_BYTES["maxpool_fwd"] / ms / 1e6 / HBM_PEAK_GBS, 4),
+                          "note": "also writes the exact int32 index (95.6 MB, not counted in GB/s) that the backward needs above 2^24 elements"}
     ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), None, 256, 128, 56, 56, 3, 0, 2)), 10)
     res["maxpool_fwd_reference_outputs"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
                                             "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
                                             "note": "y and the f32-encoded argmax only, the reference's two outputs"}
     ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), 10)
-    res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                          "traffic_bytes": round(TRAFFIC_BYTES["maxpool_bwd"]),
+                          "frac_hbm_of_traffic": round(TRAFFIC_BYTES["maxpool_bwd"] / ms / 1e6 / HBM_PEAK_GBS, 4)}
     del x, y, am, il, gy
 
     # the column-materialising operators (what the reference does per image): im2col + W . cols, gy . cols^T summed
