@@ -564,6 +564,31 @@ def test_conv2d_column_free_random_geometries_exact(K):
     assert ran_fwd >= 20 and ran_bwd >= 5, (ran_fwd, ran_bwd)
 
 
+def test_conv2d_column_free_headline_size_matches_columns_path(K):
+    # the benchmark's own shape (B=256, 64 -> 128 channels, 56x56, 3x3): the three column-free results
+    # against the library's column path, which the smaller cases pin to the oracle
+    B, C, Kc, H, k, p = 256, 64, 128, 56, 3, 1
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    x = torch.randn(B, C, H, H, device="cuda", generator=g)
+    w = (torch.rand(Kc, C, k, k, device="cuda", generator=g) * 2 - 1) * (6.0 / Kc) ** 0.5
+    gy = torch.randn(B, Kc, H, H, device="cuda", generator=g)
+    say("column-free at the headline size")
+    y, xpad = K.conv2d_nocols(x, w, p)
+    y_cols, cols = K.conv2d(x, w, p, 1, 1)
+    scale_y = float(y_cols.abs().max())
+    assert float((y - y_cols).abs().max()) <= 1e-5 + 1e-4 * scale_y
+    del y, y_cols
+    gx, gypad = K.conv_input_grad_staged(gy, w, p, (H, H))
+    gw = K.conv2d_filter_grad_nocols(xpad, gypad, tuple(x.shape), tuple(w.shape), p)
+    gw_cols = K.conv2d_filter_grad(cols, gy, tuple(w.shape))
+    # a filter-gradient element sums 802 816 products of N(0,1) values: compare on the scale of such a sum
+    assert float((gw - gw_cols).abs().max()) <= 1e-4 * float(gw_cols.abs().max())
+    del cols, xpad
+    gx_cols, _ = K.conv2d_transpose(gy, w, p, 1, 1, out_hw=(H, H), return_cols=True)
+    assert float((gx - gx_cols).abs().max()) <= 1e-5 + 1e-4 * float(gx_cols.abs().max())
+
+
 def test_conv2d_column_free_refuses_other_geometries(K, rng):
     L = K.capi.lib()
     assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1) == 0      # C not a multiple of 32
