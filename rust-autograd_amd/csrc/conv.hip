@@ -190,8 +190,8 @@ static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
 {
     // past the end of a plane the next plane's top border (pad rows and pad elements of zeros) or the
     // zeroed slack follows
-    const long long kq = (((long long)(OH + pad) * g.Wp + 31) / 32) * 32;
-    return kq <= (long long)g.Hp * g.Wp + (long long)pad * g.Wp + pad ? (int)kq : 0;
+    const long long kq = (((long long)OH * g.Wp + 31) / 32) * 32;
+    return kq <= (long long)(g.Hp - pad) * g.Wp ? (int)kq : 0;
 }
 
 }  // namespace ag

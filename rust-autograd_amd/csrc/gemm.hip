@@ -846,8 +846,8 @@ ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float 
     const int taps = kh * kw;
     const long long plane = (long long)Hp * Wp;
     GemmParams p;
-    p.A = gyp;
-    p.B = xp - ((long long)pad * Wp + pad);  // tap (0, 0) reads `pad` rows and columns before the position
+    p.A = gyp + ((long long)pad * Wp + pad);  // positions are counted from the first gradient value
+    p.B = xp;
     p.M = Kf; p.N = C * taps; p.K = kq;
     p.lda = plane; p.ldb = plane; p.ldc = p.N;
     p.sA = p.sB = p.sC = 0;

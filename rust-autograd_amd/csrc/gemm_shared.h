@@ -58,10 +58,11 @@ __device__ inline unsigned xcd_remap(unsigned id, unsigned total)
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
 constexpr int kFirstDirectCfg = 13;
 void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
-// Implicit filter gradient: gw[k][c][tap] = sum over images and padded-plane positions q of
-// gyp[b][k][q] * xp[b][c][q + (ky - pad) * Wp + (kx - pad)].  gyp, xp: zero-bordered [B][.][Hp][Wp]
-// with the same border `pad` on every side; `kq` (a multiple of 32, at most Hp * Wp) positions
-// cover every non-zero element of gyp.  `ws`: partial sums of the split over images.
+// Implicit filter gradient: gw[k][c][tap] = sum over images and positions q, counted from the first
+// gradient value of a plane, of gyp[b][k][q + pad * Wp + pad] * xp[b][c][q + ky * Wp + kx].  gyp, xp:
+// zero-bordered [B][.][Hp][Wp] with the same border `pad`; `kq` (a multiple of 32) positions cover
+// every non-zero element of gyp and end inside the zero rows below it.  `ws`: partial sums of the
+// split over images.
 size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq);
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
                                   int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq);
