@@ -44,9 +44,9 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 KIB = 1024.0
 TRAFFIC_BYTES = {
     # the step (column-free)
-    "gemm_fwd": ((157893.0 + 5455.7) * 2.0 + 392905.2 + 15116.0) * KIB,                  # implicit GEMM over bordered x + narrow-tile tail
-    "gemm_filter_grad": ((333275.1 + 36883.5) * 2.0 + 73731.8 + 288.0) * KIB,            # implicit GEMM + fold of the split partials
-    "gemm_input_grad": (232747.0 * 2.0 + 201514.1) * KIB,                                # implicit GEMM over bordered gy
+    "gemm_fwd": ((158390.0 + 5455.7) * 2.0 + 392641.7 + 15116.0) * KIB,                  # implicit GEMM over bordered x + narrow-tile tail
+    "gemm_filter_grad": ((327022.7 + 36883.4) * 2.0 + 73730.3 + 288.0) * KIB,            # implicit GEMM + fold of the split partials
+    "gemm_input_grad": (232756.5 * 2.0 + 201655.9) * KIB,                                # implicit GEMM over bordered gy
     "fwd_prepare": ((155175.4 * 2.0 + 328320.0) * 2 / 3 + 445.5 * 2.0 + 288.0) * KIB,    # pad_border averages x (64 ch) and gy (128 ch)
     "input_grad_prepare": ((155175.4 * 2.0 + 328320.0) * 4 / 3 + 1165.0 * 2.0 + 288.0) * KIB,
     # per-kernel section (column-materialising operators)
