@@ -490,7 +490,9 @@ static long long cdiv(long long a, long long b) { return (a + b - 1) / b; }
 // tiles per output tile, and the accumulated-batch GEMMs, take the BK = 16 family with a
 // three-tile LDS ring, long contractions take BK = 32.  Problems too small to give every CU a
 // block fall back to 64 x 64 tiles of the register-staged kernel.
-static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bool direct)
+// `tail_split`: the launch will be cut into whole rounds plus a narrow-tile tail (folded batch with
+// one row of tiles), so a partly filled last round costs nothing here.
+static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bool direct, bool tail_split = false)
 {
     if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg;
     if (direct) {
@@ -508,7 +510,8 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
             const long long blocks = tm * tn * zcount;
             const long long grid = direct_grid(num_cus()) * (dl[c] == kDirectCfg64 ? 2 : 1);
             if (blocks < direct_grid(num_cus()) / 2) continue;
-            const long long counted = blocks < 8 * grid ? cdiv(blocks, grid) * grid : blocks;
+            const bool whole_rounds = blocks < 8 * grid && !(tail_split && t.bm == 128 && tm == 1);
+            const long long counted = whole_rounds ? cdiv(blocks, grid) * grid : blocks;
             // equal round counts: the tile with less padding wins
             const double padding = (double)tm * t.bm * tn * t.bn / ((double)M * N) - 1.0;
             const double cost = (double)counted * t.bm * t.bn / zcount / eff[c] * (1.0 + 0.5 * padding);
@@ -617,7 +620,10 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (c.K % 32 != 0 && c.K >= 256 && (c.kbatch > 1 || c.K >= 1024) && g_force_cfg < 0 && !direct_ok(c)) {
         GemmCall body = c;
         body.K = c.K - c.K % 32;
-        if (direct_ok(body)) {
+        // only when the body really lands on the direct-to-LDS kernel (enough tiles for it)
+        const int eff_splits = splits < 1 ? 1 : (int)cdiv(c.kbatch, cdiv(c.kbatch, splits));
+        if (direct_ok(body) &&
+            choose_cfg(body.M, body.N, body.K, (long long)body.batch * eff_splits, body.kbatch > 1, true) >= kFirstDirectCfg) {
             GemmCall rest = c;
             rest.K = c.K % 32;
             rest.beta = 1.f;
@@ -673,7 +679,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
                           !c.transB && c.N % 4 == 0 && (long long)c.N * c.batch < 0x7fffffffLL &&
                           c.sB < (1LL << 30) && c.sB % 4 == 0;
     int cfg = choose_cfg(c.M, foldable ? c.N * c.batch : c.N, c.K, foldable ? 1 : (long long)c.batch * p.splits,
-                         c.kbatch > 1, direct_ok(c));
+                         c.kbatch > 1, direct_ok(c), foldable && g_force_cfg < 0);
     if (cfg >= kFirstDirectCfg && !direct_ok(c)) cfg = 0;  // a forced configuration that cannot run
     const bool fold = foldable && cfg >= kFirstDirectCfg && c.N >= kCfgs[cfg].bn;
     p.n_img = fold ? c.N : 0;
