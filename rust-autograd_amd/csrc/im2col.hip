@@ -360,6 +360,39 @@ __global__ __launch_bounds__(256) void col2im_stride2_vec_kernel(const float *__
     *reinterpret_cast<float2 *>(dst + g.W) = make_float2(acc[1][0], acc[1][1]);
 }
 
+// Stride 2, 3x3 window, pad 1, dilation 1 on an even image (W == 2 * OW, OW % 4 == 0): a thread
+// owns four consecutive outputs of one row.  Per window row it loads the nine input elements they
+// touch (two aligned 128-bit loads and the element to their left), picks the three column phases
+// out of registers and streams one aligned 128-bit store per tap.  No LDS, no run-time loops.
+__global__ __launch_bounds__(256) void im2col_s2_k3_kernel(const float *__restrict__ x, float *__restrict__ cols,
+                                                           ConvGeom g, unsigned ngroups)
+{
+    const unsigned gi = blockIdx.x * 256u + threadIdx.x;
+    if (gi >= ngroups) return;
+    const unsigned OW4 = (unsigned)g.OW >> 2;
+    const unsigned rowi = gi / OW4, q = gi - rowi * OW4;  // (plane, oy), group of four outputs
+    const unsigned plane = rowi / (unsigned)g.OH, oy = rowi - plane * (unsigned)g.OH;
+    const unsigned P = (unsigned)(g.OH * g.OW);
+    const float *xp = x + (long long)plane * g.H * g.W;
+    float *dst = cols + (long long)plane * 9 * P + oy * (unsigned)g.OW + 4 * q;
+    const int ix0 = 8 * (int)q;  // first even column; the window of output ox starts at 2*ox - 1
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int iy = 2 * (int)oy + ky - 1;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+        float left = 0.f;
+        if ((unsigned)iy < (unsigned)g.H) {
+            const float *row = xp + iy * g.W + ix0;
+            a = *reinterpret_cast<const float4 *>(row);
+            b = *reinterpret_cast<const float4 *>(row + 4);
+            if (ix0 > 0) left = row[-1];
+        }
+        st_stream(reinterpret_cast<float4 *>(dst + (unsigned)(ky * 3 + 0) * P), make_float4(left, a.y, a.w, b.y));
+        st_stream(reinterpret_cast<float4 *>(dst + (unsigned)(ky * 3 + 1) * P), make_float4(a.x, a.z, b.x, b.z));
+        st_stream(reinterpret_cast<float4 *>(dst + (unsigned)(ky * 3 + 2) * P), make_float4(a.y, a.w, b.y, b.w));
+    }
+}
+
 static ag_status_t check_geom(const char *who, int B, int C, int H, int W, int kh, int kw, int ph,
                               int pw, int sh, int sw, int dh, int dw)
 {
@@ -477,6 +510,14 @@ extern "C" ag_status_t ag_im2col_f32(ag_stream_t stream, const float *x, float *
     }
     if (same && kh == 5 && kw == 5 && pw == 2) {
         launch_im2col_same<5, 5, 2>(as_stream(stream), x, cols, g, planes * OH);
+        return check_launch("im2col");
+    }
+
+    if (sh == 2 && sw == 2 && dh == 1 && dw == 1 && kh == 3 && kw == 3 && ph == 1 && pw == 1 && W == 2 * OW && OW % 4 == 0 &&
+        aligned16(x) && aligned16(cols) && planes * OH * (OW / 4) < 0xffffffffLL && 9LL * OH * OW < 0x7fffffffLL &&
+        (long long)H * W < 0x7fffffffLL) {
+        const unsigned ngroups = (unsigned)(planes * OH * (OW / 4));
+        hipLaunchKernelGGL(im2col_s2_k3_kernel, dim3((ngroups + 255) / 256), dim3(256), 0, as_stream(stream), x, cols, g, ngroups);
         return check_launch("im2col");
     }
 

@@ -81,7 +81,9 @@ GEOMS = [  # B, C, H, W, kh, kw, pad, stride, dil
     (1, 1, 3, 256, 3, 3, 1, 1, 1),    # one row per wave
     (3, 1, 5, 8, 3, 3, 1, 1, 1),      # rows do not fill the last wave
     (1, 2, 9, 12, 3, 3, 1, 1, 2),     # dilation keeps the general stride-1 kernel
-    (1, 3, 8, 12, 3, 3, 1, 2, 1),     # stride 2, two 2x2 blocks per thread
+    (1, 3, 8, 12, 3, 3, 1, 2, 1),     # stride 2
+    (2, 2, 9, 16, 3, 3, 1, 2, 1),     # stride 2, odd height, eight outputs per row: four outputs per thread
+    (1, 2, 6, 32, 3, 3, 1, 2, 1),     # the same, several groups per row
     (2, 2, 6, 8, 4, 4, 1, 2, 1),      # the same with the 4x4 window of the transposed convolution
     (1, 2, 7, 8, 3, 3, 1, 2, 1),      # odd height: general stride-2 kernel
     (1, 2, 8, 10, 3, 3, 1, 2, 1),     # width not a multiple of 4: general stride-2 kernel
