@@ -43,9 +43,122 @@ extern "C" ag_status_t ag_conv2d_with_cols_f32(ag_stream_t stream, const float *
                        (long long)K * P, B);
 }
 
+namespace ag {
+
+// Filter gradient of a thin first layer (few filters, C*kh*kw of a few dozen at most, e.g. the
+// 1 -> 32 channel 3x3 convolution of the small CNN): the output is a few hundred numbers summed
+// over every position of every image, which leaves a tiled GEMM with one or two tiles per image.
+// Here a block takes chunks of 128 positions, stages the K x 128 and CK x 128 operand slices in LDS
+// (odd pitch: conflict-free) and every thread accumulates up to eight of the K*CK outputs over all
+// the chunks of the block; one partial result per block, folded in block order by a second kernel.
+constexpr int kThinChunk = 128, kThinPitch = kThinChunk + 1, kThinMaxK = 64, kThinMaxCK = 32, kThinMaxBlocks = 512;
+
+__global__ __launch_bounds__(256) void thin_filter_grad_kernel(const float *__restrict__ cols, const float *__restrict__ gy,
+                                                               float *__restrict__ partial, int B, int CK, int P, int K,
+                                                               int chunks, long long items)
+{
+    __shared__ float s_gy[kThinMaxK * kThinPitch];
+    __shared__ float s_co[kThinMaxCK * kThinPitch];
+    const int outputs = K * CK;
+    float acc[8] = {};
+    for (long long item = blockIdx.x; item < items; item += gridDim.x) {
+        const long long b = item / chunks;
+        const int p0 = (int)(item - b * chunks) * kThinChunk, np = min(kThinChunk, P - p0);
+        const float *gyb = gy + (b * K) * (long long)P + p0, *cob = cols + (b * CK) * (long long)P + p0;
+        // thread -> position c of the chunk and every second row; all loads are issued before the
+        // first LDS write, so their latencies overlap
+        const int c = threadIdx.x & (kThinChunk - 1), rg = threadIdx.x >> 7;
+        const bool in = c < np;
+        float vg[kThinMaxK / 2], vc[kThinMaxCK / 2];
+#pragma unroll
+        for (int j = 0; j < kThinMaxK / 2; ++j) {
+            const int r = rg + 2 * j;
+            vg[j] = (in && r < K) ? gyb[(long long)r * P + c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < kThinMaxCK / 2; ++j) {
+            const int r = rg + 2 * j;
+            vc[j] = (in && r < CK) ? cob[(long long)r * P + c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < kThinMaxK / 2; ++j)
+            if (rg + 2 * j < K) s_gy[(rg + 2 * j) * kThinPitch + c] = vg[j];
+#pragma unroll
+        for (int j = 0; j < kThinMaxCK / 2; ++j)
+            if (rg + 2 * j < CK) s_co[(rg + 2 * j) * kThinPitch + c] = vc[j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int o = threadIdx.x + j * 256;
+            if (o < outputs) {
+                const float *a = s_gy + (o / CK) * kThinPitch, *c = s_co + (o % CK) * kThinPitch;
+                // eight independent chains: the LDS reads of one do not wait for the adds of another
+                float part[8] = {};
+#pragma unroll 2
+                for (int q = 0; q < kThinChunk; q += 8)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) part[u] += a[q + u] * c[q + u];
+                acc[j] += ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int o = threadIdx.x + j * 256;
+        if (o < outputs) partial[(long long)blockIdx.x * outputs + o] = acc[j];
+    }
+}
+
+// 32 outputs per block; eight groups of threads each add every eighth partial result (eight loads
+// in flight), then the group sums are added in group order: a fixed order, so deterministic.
+__global__ __launch_bounds__(256) void thin_filter_grad_fold_kernel(const float *__restrict__ partial, float *__restrict__ gw,
+                                                                    int outputs, int blocks)
+{
+    __shared__ float part[8][32];
+    const int oi = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int o = blockIdx.x * 32 + oi;
+    float sum = 0.f;
+    if (o < outputs) {
+        int b = grp;
+        for (; b + 56 < blocks; b += 64) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(long long)(b + 8 * u) * outputs + o];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += v[u];
+        }
+        for (; b < blocks; b += 8) sum += partial[(long long)b * outputs + o];
+    }
+    part[grp][oi] = sum;
+    __syncthreads();
+    if (grp == 0 && o < outputs) {
+        float total = part[0][oi];
+#pragma unroll
+        for (int g2 = 1; g2 < 8; ++g2) total += part[g2][oi];
+        gw[o] = total;
+    }
+}
+
+static bool thin_filter_grad(int B, int CK, int P, int K)
+{
+    return K >= 1 && K <= kThinMaxK && CK >= 1 && CK <= kThinMaxCK && K * CK <= 2048 && P >= 64 && B >= 1;
+}
+
+static long long thin_blocks(int B, int P)
+{
+    const long long items = (long long)B * ((P + kThinChunk - 1) / kThinChunk);
+    return items < kThinMaxBlocks ? items : kThinMaxBlocks;
+}
+
+}  // namespace ag
+
 extern "C" size_t ag_conv2d_filter_grad_f32_workspace(int B, int CK, int P, int K)
 {
-    return ag_gemm_batchsum_f32_workspace(K, CK, P, B);
+    // (also the workspace of ag_conv2d_transpose_filter_grad_f32, which always runs the GEMM)
+    const size_t gemm = ag_gemm_batchsum_f32_workspace(K, CK, P, B);
+    const size_t thin = ag::thin_filter_grad(B, CK, P, K) ? sizeof(float) * (size_t)ag::thin_blocks(B, P) * K * CK : 0;
+    return thin > gemm ? thin : gemm;
 }
 
 extern "C" ag_status_t ag_conv2d_filter_grad_f32(ag_stream_t stream, const float *cols, const float *gy,
@@ -53,6 +166,19 @@ extern "C" ag_status_t ag_conv2d_filter_grad_f32(ag_stream_t stream, const float
                                                  size_t ws_bytes)
 {
     // gw[K x CK] = sum_b gy_b[K x P] * cols_b[CK x P]^T        conv2d.rs:662-687
+    if (ag::thin_filter_grad(B, CK, P, K)) {
+        const long long blocks = ag::thin_blocks(B, P);
+        const size_t need = sizeof(float) * (size_t)blocks * K * CK;
+        AG_REQUIRE(cols && gy && gw, AG_ERR_INVALID_DIMS, "conv2d_filter_grad: null pointer");
+        AG_REQUIRE(ws && ws_bytes >= need, AG_ERR_INVALID_DIMS, "conv2d_filter_grad: workspace of %zu bytes needed, %zu given",
+                   need, ws_bytes);
+        const int chunks = (P + ag::kThinChunk - 1) / ag::kThinChunk;
+        hipLaunchKernelGGL(ag::thin_filter_grad_kernel, dim3((unsigned)blocks), dim3(256), 0, ag::as_stream(stream), cols, gy,
+                           static_cast<float *>(ws), B, CK, P, K, chunks, (long long)B * chunks);
+        hipLaunchKernelGGL(ag::thin_filter_grad_fold_kernel, dim3((unsigned)((K * CK + 31) / 32)), dim3(256), 0,
+                           ag::as_stream(stream), static_cast<const float *>(ws), gw, K * CK, (int)blocks);
+        return ag::check_launch("conv2d_filter_grad");
+    }
     return ag_gemm_batchsum_f32(stream, 0, 1, K, CK, P, 1.f, gy, P, (long long)K * P, cols, P,
                                 (long long)CK * P, 0.f, gw, CK, B, ws, ws_bytes);
 }

@@ -387,6 +387,28 @@ def test_gemm_batchsum_long_k_with_a_tail(K, rng, beta):
     assert np.array_equal(host(ci), np.einsum("bmk,bnk->mn", ai.astype(np.int64), bi.astype(np.int64)).astype(np.float32))
 
 
+@pytest.mark.parametrize("B,C,Kc,H,W,k", [(64, 1, 32, 28, 28, 3), (5, 3, 64, 17, 19, 3), (130, 1, 8, 12, 12, 5), (2, 2, 16, 40, 40, 3),
+                                          (1100, 1, 4, 8, 8, 3)])
+def test_conv2d_filter_grad_of_a_thin_first_layer(K, orc, rng, B, C, Kc, H, W, k):
+    """Few filters and C*kh*kw of a few dozen at most: the chunked-positions kernel instead of a GEMM with one
+    tile per image (partial chunks, more work items than blocks, every output counted once)."""
+    p = k // 2
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, H, W)).astype(np.float32)
+    say("thin filter grad", B, C, Kc, H, W, k)
+    cols = K.im2col(dev(x), k, k, p, p, 1, 1, 1, 1)
+    gw = host(K.conv2d_filter_grad(cols, dev(gy), (Kc, C, k, k)))
+    ocols = orc.im2col(x.astype(np.float64), k, k, p, p, 1, 1, 1, 1)
+    truth = orc.conv2d_filter_grad(ocols, gy.astype(np.float64), (Kc, C, k, k))
+    absdot = orc.conv2d_filter_grad(np.abs(ocols), np.abs(gy).astype(np.float64), (Kc, C, k, k))
+    assert_close_conditioned(gw, truth, absdot, "thin filter gradient")
+    xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+    gi = rng.integers(-2, 3, gy.shape).astype(np.float32)
+    gwi = host(K.conv2d_filter_grad(K.im2col(dev(xi), k, k, p, p, 1, 1, 1, 1), dev(gi), (Kc, C, k, k)))
+    exact = orc.conv2d_filter_grad(orc.im2col(xi.astype(np.float64), k, k, p, p, 1, 1, 1, 1), gi.astype(np.float64), (Kc, C, k, k))
+    assert np.array_equal(gwi, exact.astype(np.float32))
+
+
 def test_gemm_degenerate_k_and_beta(K, rng):
     c0 = rng.random((5, 6), dtype=np.float32)
     c = dev(c0)
