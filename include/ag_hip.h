@@ -18,8 +18,11 @@
  *   - status 1..5 are the five variants of the reference's `OpError`
  *     (src/op.rs:66-73) in declaration order; 100 + n is hipError_t n;
  *   - nothing throws or aborts across this boundary;
- *   - functions are re-entrant; the only mutable global is the thread-local
- *     error string.
+ *   - functions are re-entrant: the mutable state of the library is the
+ *     thread-local error string and caches of device properties that are filled
+ *     once under a lock.  The library also exports a few ag_test_* symbols for its own
+ *     test-suite (rust-autograd_amd/csrc/ag_test_hooks.h); they set thread-local
+ *     overrides and are not part of this boundary.
  */
 #ifndef AG_HIP_H
 #define AG_HIP_H
@@ -301,17 +304,6 @@ ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const float *logits, 
 ag_status_t ag_sparse_softmax_xent_grad_f32(ag_stream_t stream, const float *log_softmax,
                                             const float *labels, const float *gy, float *gx,
                                             size_t rows, size_t classes);
-
-/* Experiment hook, not part of the operator surface: force GEMM tile configuration `cfg`
- * (-1 restores the automatic choice) for later calls in this process. */
-void ag_gemm_force_config(int cfg);
-/* Experiment hook: force the split count of accumulated-batch GEMMs (0 = automatic). */
-void ag_gemm_force_splits(int splits);
-/* Experiment hook: blocks per CU of the persistent GEMM grid (0 = as many as stay resident). */
-void ag_gemm_force_grid(int blocks_per_cu);
-/* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): stride-1 calls may use the
- * implicit input-gradient GEMM, which never writes the columns. */
-void ag_conv_fused_input_grad(int on);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

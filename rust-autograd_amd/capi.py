@@ -92,10 +92,6 @@ PROTOTYPES = {
     "ag_fill_f32": (c_i, [c_p, c_p, c_f, c_sz]),
     "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
-    "ag_gemm_force_config": (None, [c_i]),
-    "ag_gemm_force_splits": (None, [c_i]),
-    "ag_gemm_force_grid": (None, [c_i]),
-    "ag_conv_fused_input_grad": (None, [c_i]),
     "ag_conv_input_grad_scratch_floats": (C.c_size_t, [c_i] * 10),
     "ag_conv_input_grad_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 10),
     "ag_conv_input_grad_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 10),
@@ -106,6 +102,14 @@ PROTOTYPES = {
     "ag_conv2d_nocols_with_filter_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32_workspace": (c_sz, [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8 + [c_p, c_sz]),
+}
+
+# Test hooks (csrc/ag_test_hooks.h): thread-local overrides used by the test-suite, not part of the boundary.
+TEST_HOOKS = {
+    "ag_test_gemm_force_config": (None, [c_i]),
+    "ag_test_gemm_force_splits": (None, [c_i]),
+    "ag_test_gemm_force_grid": (None, [c_i]),
+    "ag_test_conv_fused_input_grad": (None, [c_i]),
 }
 
 _lib = None
@@ -120,7 +124,7 @@ def lib():
                 f"{LIB_PATH} is missing: build it with rust-autograd_amd/csrc/build.sh "
                 "(there is no CPU fallback)")
         handle = C.CDLL(LIB_PATH)
-        for name, (res, args) in PROTOTYPES.items():
+        for name, (res, args) in list(PROTOTYPES.items()) + list(TEST_HOOKS.items()):
             fn = getattr(handle, name)  # AttributeError names the missing symbol
             fn.restype = res
             fn.argtypes = args

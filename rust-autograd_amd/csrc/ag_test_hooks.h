@@ -1,0 +1,29 @@
+/* Test hooks of libag_hip.so: exported for the library's own test-suite and tuning runs, NOT part of
+ * the operator boundary (include/ag_hip.h).  Every hook sets an override that is local to the
+ * calling thread, so other threads' calls are never affected. */
+#ifndef AG_TEST_HOOKS_H
+#define AG_TEST_HOOKS_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+/* Force GEMM tile configuration `cfg` for later calls of this thread (-1 = automatic choice). */
+void ag_test_gemm_force_config(int cfg);
+/* Force the split count of accumulated-batch GEMMs (0 = automatic). */
+void ag_test_gemm_force_splits(int splits);
+/* Blocks per CU of the persistent GEMM grid (0 = as many as stay resident). */
+void ag_test_gemm_force_grid(int blocks_per_cu);
+/* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): it may take the implicit GEMM. */
+void ag_test_conv_fused_input_grad(int on);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif /* AG_TEST_HOOKS_H */

@@ -3,6 +3,7 @@
 // batched: one im2col launch and one strided-batched GEMM launch per operator instead of one
 // task per image, and one split-accumulation GEMM instead of an image-sequential beta=1 loop.
 #include "ag_internal.h"
+#include "ag_test_hooks.h"
 #include "gemm_shared.h"
 
 using namespace ag;
@@ -185,7 +186,7 @@ extern "C" ag_status_t ag_conv2d_filter_grad_f32(ag_stream_t stream, const float
 
 namespace ag {
 
-static bool g_fused_input_grad = true;  // experiment hook, see ag_conv_fused_input_grad
+static thread_local bool g_fused_input_grad = true;  // test hook (ag_test_hooks.h), per calling thread
 
 // gyp[plane][r][s] = gy[plane][r - top][s - left] inside the image, 0 in the border; four
 // consecutive elements of the flattened padded plane per thread (its extent is a multiple of 4).
@@ -487,9 +488,9 @@ extern "C" ag_status_t ag_conv2d_transpose_filter_grad_f32(ag_stream_t stream, c
                                 (int)P, N * P, 0.f, gw, (int)N, B, ws, ws_bytes);
 }
 
-// Experiment hook (not part of the operator surface): 0 makes ag_conv2d_transpose_f32 always take
-// the GEMM + col2im path, 1 (default) lets stride-1 calls use the implicit input-gradient GEMM.
-extern "C" void ag_conv_fused_input_grad(int on) { ag::g_fused_input_grad = on != 0; }
+// Test hook (ag_test_hooks.h; not part of the operator surface): 0 makes ag_conv2d_transpose_f32 calls of
+// this thread always take the GEMM + col2im path, 1 (default) lets them use the implicit GEMM.
+extern "C" void ag_test_conv_fused_input_grad(int on) { ag::g_fused_input_grad = on != 0; }
 
 // The two stages of the column-free stride-1 input gradient, for callers that time or schedule
 // them separately.  `scratch` holds ag_conv_input_grad_scratch_floats() floats (0 = this

@@ -24,6 +24,7 @@
 // contiguous range of tiles / images.
 #include <type_traits>
 
+#include "ag_test_hooks.h"
 #include "gemm_shared.h"
 
 namespace ag {
@@ -399,17 +400,18 @@ struct TileCfg {
 };
 
 // Resident blocks per CU of one kernel instantiation, and the CU count (both cached).
+static int query_cus()
+{
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+        return n;
+    return 256;
+}
+
 static int num_cus()
 {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
+    static const int cus = query_cus();  // initialised once, thread-safe (C++11 static)
     return cus;
 }
 
@@ -424,7 +426,8 @@ static int resident_blocks(Kern kern, int threads, int fallback)
     return n;
 }
 
-static int g_grid_scale = 0;  // experiment hook: blocks per CU of the persistent grid (0 = resident count)
+// Test hook (ag_test_hooks.h), per calling thread: blocks per CU of the persistent grid (0 = resident count).
+static thread_local int g_grid_scale = 0;
 
 template <int BM, int BN, int BK, int WM, int WN, int OCC, int STAGES>
 static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
@@ -453,7 +456,7 @@ static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
 #undef AG_GEMM_CASE
 }
 
-static int g_force_cfg = -1;  // experiment hook, see ag_gemm_force_config
+static thread_local int g_force_cfg = -1;  // test hook (ag_test_hooks.h), per calling thread
 
 // Tile configurations {BM, BN}; see launch() for BK, the wave tile and the occupancy target.
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
@@ -890,7 +893,7 @@ ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float 
     return AG_OK;
 }
 
-static int g_force_splits = 0;  // experiment hook, see ag_gemm_force_splits
+static thread_local int g_force_splits = 0;  // test hook (ag_test_hooks.h), per calling thread
 
 // Number of splits for an accumulated-batch GEMM: enough blocks for a few waves over the chip.
 static int choose_splits(int M, int N, int K, int kbatch)
@@ -925,15 +928,11 @@ static int matmul_slices(int M, int N, int K)
 
 using namespace ag;
 
-// Experiment hook (not part of the operator surface): force tile configuration `cfg`
-// (-1 = automatic) for subsequent GEMM calls of this process.
-extern "C" void ag_gemm_force_config(int cfg) { g_force_cfg = cfg; }
-
-// Experiment hook: force the number of splits of accumulated-batch GEMMs (0 = automatic).
-extern "C" void ag_gemm_force_splits(int splits) { g_force_splits = splits; }
-
-// Experiment hook: blocks per CU of the persistent GEMM grid (0 = as many as stay resident).
-extern "C" void ag_gemm_force_grid(int blocks_per_cu) { g_grid_scale = blocks_per_cu; }
+// Test hooks (ag_test_hooks.h; not part of the operator surface).  Each sets a thread-local
+// override that later calls made by the same thread observe.
+extern "C" void ag_test_gemm_force_config(int cfg) { g_force_cfg = cfg; }
+extern "C" void ag_test_gemm_force_splits(int splits) { g_force_splits = splits; }
+extern "C" void ag_test_gemm_force_grid(int blocks_per_cu) { g_grid_scale = blocks_per_cu; }
 
 extern "C" ag_status_t ag_gemm_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K,
                                    float alpha, const float *A, int lda, long long strideA, const float *B,

@@ -186,13 +186,13 @@ def conv2d_transpose(gy, w, pad, stride, dilation=1, out_hw=None, return_cols=Fa
     gcols = _empty((B, xch * kh * kw, yh * yw), gy)
     L = capi.lib()
     if return_cols:  # the caller wants the columns: keep to the GEMM + col2im path
-        L.ag_conv_fused_input_grad(0)
+        L.ag_test_conv_fused_input_grad(0)
     try:
         check(L.ag_conv2d_transpose_f32(_stream(), _ptr(gy), _ptr(w), _ptr(gx), _ptr(gcols), B, ych, yh, yw,
                                         xch, kh, kw, pad, stride, dilation, xh, xw))
     finally:
         if return_cols:
-            L.ag_conv_fused_input_grad(1)
+            L.ag_test_conv_fused_input_grad(1)
     return (gx, gcols) if return_cols else gx
 
 

@@ -46,6 +46,19 @@ def test_ctypes_prototypes_cover_the_header(capi):
     capi.lib()
 
 
+def test_exports_are_the_header_plus_the_test_hooks(capi):
+    """Nothing is exported beyond include/ag_hip.h and the thread-local test hooks of
+    csrc/ag_test_hooks.h, and the hooks are not declared in the public header."""
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True).stdout
+    exported = sorted(l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("ag_"))
+    hooks_h = open(os.path.join(ROOT, "rust-autograd_amd", "csrc", "ag_test_hooks.h")).read()
+    hooks_h = re.sub(r"/\*.*?\*/", "", hooks_h, flags=re.S)
+    hooks = sorted(set(re.findall(r"\b(ag_test_[a-z0-9_]+)\s*\(", hooks_h)))
+    assert hooks == sorted(capi.TEST_HOOKS)
+    assert not [n for n in _declared_functions() if n.startswith("ag_test_")]
+    assert exported == sorted(_declared_functions() + hooks)
+
+
 def test_library_has_gfx950_code_object(capi):
     blob = open(capi.LIB_PATH, "rb").read()
     assert b"gfx950" in blob

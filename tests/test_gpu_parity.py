@@ -191,12 +191,12 @@ def test_gemm_every_tile_configuration(K, rng, cfg):
     a = rng.random((m, k), dtype=np.float32)
     b = rng.random((k, n), dtype=np.float32)
     say("gemm cfg", cfg)
-    L.ag_gemm_force_config(cfg)
+    L.ag_test_gemm_force_config(cfg)
     try:
         got = host(K.matmul(dev(a), dev(b)))
         got_t = host(K.matmul(dev(a.T.copy()), dev(b.T.copy()), True, True))
     finally:
-        L.ag_gemm_force_config(-1)
+        L.ag_test_gemm_force_config(-1)
     truth = a.astype(np.float64) @ b.astype(np.float64)
     assert_close(got, truth, "gemm NN")      # positive inputs: no cancellation, plain bound applies
     assert_close(got_t, truth, "gemm TT")
@@ -216,12 +216,12 @@ def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb):
         b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
         say("gemm direct cfg", cfg, ta, tb, m, n, k, batch)
         c = dev(np.zeros((batch, m, n), np.float32))
-        L.ag_gemm_force_config(cfg)
+        L.ag_test_gemm_force_config(cfg)
         try:
             K.gemm(ta, tb, m, n, k, 1.0, dev(a), a.shape[2], a.shape[1] * a.shape[2], dev(b), b.shape[2],
                    b.shape[1] * b.shape[2], 0.0, c, n, m * n, batch)
         finally:
-            L.ag_gemm_force_config(-1)
+            L.ag_test_gemm_force_config(-1)
         A = a.transpose(0, 2, 1) if ta else a
         Bm = b.transpose(0, 2, 1) if tb else b
         truth = A.astype(np.float64) @ Bm.astype(np.float64)
@@ -249,12 +249,12 @@ def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
         c0 = rng.random((batch, m, n), dtype=np.float32)
         say("gemm folded cfg", cfg, ta, tb, m, n, k, batch, beta)
         c = dev(c0)
-        L.ag_gemm_force_config(cfg)
+        L.ag_test_gemm_force_config(cfg)
         try:
             K.gemm(ta, tb, m, n, k, 2.0, dev(a), a.shape[1], 0, dev(b), b.shape[2], b.shape[1] * b.shape[2], beta, c, n,
                    m * n, batch)
         finally:
-            L.ag_gemm_force_config(-1)
+            L.ag_test_gemm_force_config(-1)
         A = a.T if ta else a
         Bm = b.transpose(0, 2, 1) if tb else b
         truth = 2.0 * (A.astype(np.float64)[None] @ Bm.astype(np.float64)) + beta * c0
@@ -271,11 +271,11 @@ def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg):
     cols = rng.random((imgs, ck, pp), dtype=np.float32)
     c0 = rng.random((kf, ck), dtype=np.float32)
     say("gemm direct batchsum cfg", cfg)
-    L.ag_gemm_force_config(cfg)
+    L.ag_test_gemm_force_config(cfg)
     try:
         got = host(K.gemm_batchsum(0, 1, kf, ck, pp, 0.5, dev(gy), pp, kf * pp, dev(cols), pp, ck * pp, 2.0, dev(c0), ck, imgs))
     finally:
-        L.ag_gemm_force_config(-1)
+        L.ag_test_gemm_force_config(-1)
     want = 0.5 * np.einsum("bkp,bcp->kc", gy.astype(np.float64), cols.astype(np.float64)) + 2.0 * c0
     assert_close(got, want, "direct batchsum")
 
