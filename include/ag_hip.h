@@ -19,8 +19,9 @@
  *     (src/op.rs:66-73) in declaration order; 100 + n is hipError_t n;
  *   - nothing throws or aborts across this boundary;
  *   - functions are re-entrant: the mutable state of the library is the
- *     thread-local error string and caches of device properties that are filled
- *     once under a lock.  The library also exports a few ag_test_* symbols for its own
+ *     thread-local error string, caches of device properties that are filled
+ *     once under a lock, and the fixed scratch array of ag_matmul_f32_noalloc
+ *     (see there).  The library also exports a few ag_test_* symbols for its own
  *     test-suite (rust-autograd_amd/csrc/ag_test_hooks.h); they set thread-local
  *     overrides and are not part of this boundary.
  */
@@ -304,6 +305,20 @@ ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const float *logits, 
 ag_status_t ag_sparse_softmax_xent_grad_f32(ag_stream_t stream, const float *log_softmax,
                                             const float *labels, const float *gy, float *gx,
                                             size_t rows, size_t classes);
+
+/* ---- entry point that allocates nothing ----------------------------------------------------- */
+
+/* ag_matmul_f32 without a workspace argument.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The partial sums of a sliced contraction go to a fixed array
+ * of ag_matmul_f32_static_scratch_bytes() bytes (4 MiB) that every GPU the library runs on holds
+ * until the process ends; a product whose ag_matmul_f32_workspace() exceeds that is refused with
+ * AG_ERR_INVALID_DIMS.  Results are bit-identical to ag_matmul_f32.  Calls that overlap on one
+ * GPU (two streams, two threads) share the array and race: serialise them.  The first call on a
+ * device looks up the array's address there (hipGetSymbolAddress); no call allocates or frees. */
+size_t ag_matmul_f32_static_scratch_bytes(void);
+ag_status_t ag_matmul_f32_noalloc(ag_stream_t stream, int transA, int transB, int M, int N, int K,
+                                  const float *A, int lda, const float *B, int ldb, float *C, int ldc);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

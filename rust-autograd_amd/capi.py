@@ -102,6 +102,8 @@ PROTOTYPES = {
     "ag_conv2d_nocols_with_filter_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32_workspace": (c_sz, [c_i] * 8),
     "ag_conv2d_filter_grad_nocols_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8 + [c_p, c_sz]),
+    "ag_matmul_f32_static_scratch_bytes": (c_sz, []),
+    "ag_matmul_f32_noalloc": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_p, c_i, c_p, c_i, c_p, c_i]),
 }
 
 # Test hooks (csrc/ag_test_hooks.h): thread-local overrides used by the test-suite, not part of the boundary.

@@ -22,6 +22,7 @@
 // writes a partial result that a second fixed-order kernel folds, keeping the result
 // deterministic.  Block ids are permuted so that each XCD (which has its own L2) works on a
 // contiguous range of tiles / images.
+#include <mutex>
 #include <type_traits>
 
 #include "ag_test_hooks.h"
@@ -981,4 +982,59 @@ extern "C" ag_status_t ag_matmul_f32(ag_stream_t stream, int transA, int transB,
     const long long strideB = transB ? Kc : (long long)Kc * ldb;
     return ag_gemm_batchsum_f32(stream, transA, transB, M, N, Kc, 1.f, A, lda, strideA, B, ldb, strideB, 0.f, C, ldc, s, ws,
                                 ws_bytes);
+}
+
+// ---------------------------------------------------------------------------------------------
+// ag_matmul_f32 for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the partial sums of a sliced contraction go to a fixed device
+// array of this library instead of a caller workspace.  Every GPU the library runs on holds its
+// own copy of the array until the process ends; its address on a device is looked up once, with
+// that device current, and only that address (never the array's name, which is a host-side
+// stand-in) is handed to kernels.  Calls that overlap on one GPU share the array and race.
+// ---------------------------------------------------------------------------------------------
+namespace ag {
+
+constexpr size_t kStaticScratchBytes = 4u << 20;  // 4 MiB per GPU
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[kMaxDevices] = {};  // per device, guarded by g_scratch_mutex
+
+static ag_status_t static_scratch(void **out)
+{
+    int dev = -1;
+    if (ag_status_t s = check_hip(hipGetDevice(&dev), "matmul (static scratch): hipGetDevice")) return s;
+    AG_REQUIRE(dev >= 0 && dev < kMaxDevices, AG_ERR_INVALID_DIMS, "matmul (static scratch): device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (ag_status_t s = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)),
+                                      "matmul (static scratch): hipGetSymbolAddress"))
+            return s;
+        AG_REQUIRE(ptr, AG_ERR_INVALID_DIMS, "matmul (static scratch): null symbol address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return AG_OK;
+}
+
+}  // namespace ag
+
+extern "C" size_t ag_matmul_f32_static_scratch_bytes(void) { return ag::kStaticScratchBytes; }
+
+extern "C" ag_status_t ag_matmul_f32_noalloc(ag_stream_t stream, int transA, int transB, int M, int N, int K,
+                                             const float *A, int lda, const float *B, int ldb, float *C, int ldc)
+{
+    const size_t need = ag_matmul_f32_workspace(M, N, K);
+    if (need <= 16)  // not sliced: no scratch involved
+        return ag_matmul_f32(stream, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, nullptr, 0);
+    AG_REQUIRE(need <= ag::kStaticScratchBytes, AG_ERR_INVALID_DIMS,
+               "matmul (no allocation): %d x %d x %d needs %zu bytes of scratch, the fixed array holds %zu; "
+               "use ag_matmul_f32 with a caller workspace",
+               M, N, K, need, ag::kStaticScratchBytes);
+    void *ws = nullptr;
+    if (ag_status_t s = ag::static_scratch(&ws)) return s;
+    // every slot the fold reads is written by this call's GEMM first: nothing needs clearing
+    return ag_matmul_f32(stream, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, ws, need);
 }
