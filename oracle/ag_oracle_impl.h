@@ -315,16 +315,17 @@ ORC_API int FN(orc_maxpool2d_fwd)(const REAL *x, REAL *y, REAL *argmax, int32_t 
                     const int w1 = w0 + size > W ? W : w0 + size;
                     REAL best = -REAL_MAX;
                     size_t best_i = 0;
+                    int found = 0; /* did any element exceed the initial maximum? (none does in an all-NaN window) */
                     for (int h = h0; h < h1; ++h)
                         for (int ww = w0; ww < w1; ++ww) {
                             const size_t i = plane + (size_t)h * W + ww;
                             const REAL v = x[i];
-                            if (v > best) { best = v; best_i = i; }
+                            if (v > best) { best = v; best_i = i; found = 1; }
                         }
                     const size_t o = oplane + (size_t)oy * OW + ox;
                     y[o] = best;
                     argmax[o] = (REAL)best_i;
-                    if (idx_local) idx_local[o] = best_i >= plane ? (int32_t)(best_i - plane) : -1;
+                    if (idx_local) idx_local[o] = found ? (int32_t)(best_i - plane) : -1;
                 }
             }
         }

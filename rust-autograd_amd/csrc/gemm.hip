@@ -217,7 +217,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
     };
 
     // ---- compute stream ----
+    // The MFMAs add to `acc`; after every kChainK elements of k the chain's sum is set aside into
+    // `tot` and the chain restarts from zero (see kChainK).
+    // Tiles whose two accumulator sets would not fit the register file next to the staged loads
+    // (four or more 32 x 32 blocks per wave) keep one chain; long aligned contractions run on the
+    // direct-to-LDS kernel, which chains at every tile size.
+    constexpr bool CHAINING = MI * NI == 1 || (MI * NI == 2 && OCC <= 2);
     f32x16 acc[MI][NI];
+    constexpr int CHAIN = kChainK / BK;  // k tiles per chain
     auto zero_acc = [&]() {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
@@ -299,7 +306,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
         }
     };
 
-    auto run = [&](auto tail_tag) {
+    auto run = [&](auto tail_tag) __attribute__((always_inline)) {
         // Prologue: the first STAGES-1 tiles of the stream go to LDS.
         f_begin();
 #pragma unroll
@@ -315,6 +322,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
         Item ci = decode(cw);
         int c_left = ci.nt;
         zero_acc();
+        // (plain loops, not lambdas: a further closure level keeps the arrays from being promoted to registers)
+        f32x16 tot[CHAINING ? MI : 1][CHAINING ? NI : 1];
+#define AG_FOR_TOT(stmt)                                       \
+    if constexpr (CHAINING) {                                  \
+        _Pragma("unroll") for (int i = 0; i < MI; ++i)         \
+        _Pragma("unroll") for (int j = 0; j < NI; ++j)         \
+        _Pragma("unroll") for (int v = 0; v < 16; ++v) { stmt; } \
+    }
+        bool chained = CHAINING && ci.nt > CHAIN;  // more than one chain: their sums meet in `tot`
+        if (chained) AG_FOR_TOT(tot[i][j][v] = 0.f)
+        int chain_left = CHAIN;
         float4 af[2][MI], bf[2][NI];
         read_frags(0, 0, af[0], bf[0]);
 
@@ -347,17 +365,25 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
             fill = fill + 1 == STAGES ? 0 : fill + 1;
 
             if (item_done) {
+                if (chained) AG_FOR_TOT(acc[i][j][v] += tot[i][j][v])
                 write_out(ci);
                 if (last) break;
                 cw += gridDim.x;
                 ci = decode(cw);
                 c_left = ci.nt;
                 zero_acc();
+                chained = CHAINING && ci.nt > CHAIN;
+                if (chained) AG_FOR_TOT(tot[i][j][v] = 0.f)
+                chain_left = CHAIN;
+            } else if (CHAINING && --chain_left == 0) {
+                AG_FOR_TOT(tot[i][j][v] += acc[i][j][v]; acc[i][j][v] = 0.f)
+                chain_left = CHAIN;
             }
         }
     };
     if (ktail) run(std::true_type{});
     else run(std::false_type{});
+#undef AG_FOR_TOT
 }
 
 // C[m][n] = alpha * sum_s partial[s][m][n] + beta * C[m][n].  A block folds 32 consecutive

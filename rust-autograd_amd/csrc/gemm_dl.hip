@@ -306,7 +306,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         }
     };
     // ---- compute stream ----
-    f32x16 acc[MI][NI];
+    // `acc` is the chain the MFMAs add to.  A chain that ran over the whole contraction would grow a
+    // rounding error like that of any sequential f32 sum; after every kChainK elements of k it is
+    // therefore set aside into `tot` and restarted from zero, which is how a blocked CPU SGEMM
+    // (the reference's OpenBLAS) sums as well.
+    f32x16 acc[MI][NI], tot[MI][NI];
+    constexpr int CHAIN = kChainK / BK;  // k tiles per chain
     auto zero_acc = [&]() {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
@@ -314,6 +319,33 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             for (int j = 0; j < NI; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
+    auto zero_tot = [&]() {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) tot[i][j][v] = 0.f;
+    };
+    auto set_aside = [&]() {  // tot += acc, acc = 0
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    tot[i][j][v] += acc[i][j][v];
+                    acc[i][j][v] = 0.f;
+                }
+    };
+    auto take_back = [&]() {  // acc += tot
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] += tot[i][j][v];
     };
     // Per-lane float indices of the fragments inside a ring slot.
     int a_idx[KA ? KK : MI], b_idx[KB ? KK : NI];
@@ -527,8 +559,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     while (true) {  // work items of this block
         zero_acc();
         int c_left = ci.nt;
+        const bool chained = ci.nt > CHAIN;  // more than one chain: their sums meet in `tot`
+        if (chained) zero_tot();
+        int chain_left = CHAIN;
         const bool last_item = cw + gridDim.x >= total;
-        do {  // k tiles of the item: the accumulators are touched by MFMAs only
+        do {  // k tiles of the item: within a chain the accumulators are touched by MFMAs only
             const bool last = c_left == 1 && last_item;  // nothing follows in the stream
             const float *nxt = cur + TILE == ring_end ? lds : cur + TILE;
 
@@ -553,7 +588,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             second_half(all_issued, cur, nxt, last);
             fill_addr = fill_addr + TILE * 4u == lds_wave + STAGES * TILE * 4u ? lds_wave : fill_addr + TILE * 4u;
             cur = nxt;
+            if (--chain_left == 0 && c_left > 1) {
+                set_aside();
+                chain_left = CHAIN;
+            }
         } while (--c_left != 0);
+        if (chained) take_back();
         const bool counted = write_out(ci);
         if (last_item) break;
         after_epilogue = counted;

@@ -45,6 +45,11 @@ struct GemmParams {
 
 constexpr int kXcds = 8;
 
+// Elements of the contraction that one accumulation chain of the MFMA kernels covers before its sum
+// is set aside and the chain restarts from zero (both GEMM kernels; the length of an OpenBLAS
+// SGEMM k block, so rounding errors grow as they do in the reference's BLAS).
+constexpr int kChainK = 256;
+
 // Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
 // contiguous slice of the logical block range instead.
 __device__ inline unsigned xcd_remap(unsigned id, unsigned total)

@@ -1,0 +1,215 @@
+"""Parity at the benchmark configurations' FULL sizes (through the C ABI, one GPU):
+
+  config 3   4096^3 MatMul in the NN / NT / TN layouts and 64 x 512^3 BatchMatMul with both operand
+             gradients, against numpy's f64 product of the same arrays, plus integer-valued inputs
+             (exact in f32) for equality;
+  config 4   B = 256, 64 -> 128 channels, 56 x 56, 3 x 3, stride 1 AND stride 2: y, gw and gx against
+             the direct definition of the convolution evaluated in f64 on a random sample of output
+             elements (gw: all filters and taps of sampled input channels, each the full sum over the
+             256 images), plus integer-valued inputs for equality; 3 x 3 stride-2 max pooling forward
+             and backward on the full [256,128,56,56] against the oracle, bit for bit;
+  config 5   32 images: dilation-2 convolution and the 4 x 4 stride-2 transposed convolution,
+             forward and both gradients, against the f64 oracle.
+
+The schedules that only exist at these sizes (a dozen rounds of the persistent grid plus the
+narrow-tile tail, the 256-way split fold) are thereby checked against something other than
+themselves.  Bars: tests/bars.py.
+"""
+import numpy as np
+import pytest
+import torch
+
+from bars import assert_contraction, say
+from direct_conv import direct_gw, direct_gx, direct_y
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    import __graft_entry__ as entry
+    entry.load_package()
+    from rust_autograd_amd import kernels
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return kernels
+
+
+@pytest.fixture(scope="module", autouse=True)
+def reference_blas(orc):
+    path = orc.load_openblas()
+    say("oracle BLAS:", path or "built-in blocked GEMM")
+    yield path
+    orc.unload_blas()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.detach().cpu().numpy()
+
+
+# ------------------------------------------------------------------------------------- config 3
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_config3_matmul_4096(K, ta, tb):
+    n = 4096
+    rng = np.random.default_rng(4096 + 2 * ta + tb)
+    a = rng.standard_normal((n, n)).astype(np.float32)
+    b = rng.standard_normal((n, n)).astype(np.float32)
+    say("matmul 4096^3", ta, tb)
+    got = host(K.matmul(dev(a), dev(b), ta, tb))
+    A = (a.T if ta else a).astype(np.float64)
+    Bm = (b.T if tb else b).astype(np.float64)
+    ref32 = (a.T if ta else a) @ (b.T if tb else b)            # numpy's f32 product (OpenBLAS sgemm)
+    assert_contraction(got, A @ Bm, np.abs(A) @ np.abs(Bm), f"matmul 4096^3 ta={ta} tb={tb}", ref32=ref32)
+    del A, Bm
+    ai = rng.integers(-3, 4, (n, n)).astype(np.float32)
+    bi = rng.integers(-3, 4, (n, n)).astype(np.float32)
+    exact = (ai.T if ta else ai) @ (bi.T if tb else bi)         # every partial sum < 2^24: exact in any order
+    assert np.array_equal(host(K.matmul(dev(ai), dev(bi), ta, tb)), exact)
+
+
+def test_config3_batch_matmul_64x512_with_both_gradients(K):
+    rng = np.random.default_rng(64512)
+    a = rng.standard_normal((64, 512, 512)).astype(np.float32)
+    b = rng.standard_normal((64, 512, 512)).astype(np.float32)
+    gy = np.ones((64, 512, 512), np.float32)     # grad() of a sum: dot_ops.rs:697-717 with gy = ones
+    a64, b64, g64 = (v.astype(np.float64) for v in (a, b, gy))
+    say("batch_matmul 64x512^3")
+    z = host(K.batch_matmul(dev(a), dev(b)))
+    assert_contraction(z, a64 @ b64, np.abs(a64) @ np.abs(b64), "batch_matmul z", ref32=a @ b)
+    ga = host(K.batch_matmul(dev(gy), dev(b), False, True))      # gy . b^T
+    assert_contraction(ga, g64 @ b64.transpose(0, 2, 1), g64 @ np.abs(b64).transpose(0, 2, 1), "batch_matmul ga",
+                       ref32=gy @ b.transpose(0, 2, 1))
+    gb = host(K.batch_matmul(dev(a), dev(gy), True, False))      # a^T . gy
+    assert_contraction(gb, a64.transpose(0, 2, 1) @ g64, np.abs(a64).transpose(0, 2, 1) @ g64, "batch_matmul gb",
+                       ref32=a.transpose(0, 2, 1) @ gy)
+    ai = rng.integers(-3, 4, a.shape).astype(np.float32)
+    bi = rng.integers(-3, 4, b.shape).astype(np.float32)
+    assert np.array_equal(host(K.batch_matmul(dev(ai), dev(bi))), ai @ bi)
+    assert np.array_equal(host(K.batch_matmul(dev(ai), dev(bi), True, False)), ai.transpose(0, 2, 1) @ bi)
+    assert np.array_equal(host(K.batch_matmul(dev(ai), dev(bi), False, True)), ai @ bi.transpose(0, 2, 1))
+
+
+# ------------------------------------------------------------------------------------- config 4
+def _conv_paths(K, x, w, gy, pad, stride, dil):
+    """(y, gw, gx) of the operator path the host layer takes for this geometry, and of the column path."""
+    H, W = x.shape[2:]
+    out = {}
+    y, cols = K.conv2d(x, w, pad, stride, dil)
+    gw = K.conv2d_filter_grad(cols, gy, tuple(w.shape))
+    del cols
+    gx = K.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(H, W), return_cols=True)[0]
+    out["columns"] = (y, gw, gx)
+    if stride == 1 and dil == 1:
+        res = K.conv2d_nocols(x, w, pad)
+        staged = K.conv_input_grad_staged(gy, w, pad, (H, W))
+        if res is not None and staged is not None:
+            gw2 = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), pad)
+            out["column-free"] = (res[0], gw2, staged[0])
+    return out
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_config4_conv_b256_against_direct_definition(K, stride):
+    B, C, Kf, H, k, pad = 256, 64, 128, 56, 3, 1
+    OH = (H + 2 * pad - k) // stride + 1
+    rng = np.random.default_rng(256 + stride)
+    sc = np.sqrt(6.0 / Kf)
+    x = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    w = rng.uniform(-sc, sc, (Kf, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kf, OH, OH)).astype(np.float32)
+    n = 8192
+    yi = np.stack([rng.integers(0, B, n), rng.integers(0, Kf, n), rng.integers(0, OH, n), rng.integers(0, OH, n)], 1)
+    xi = np.stack([rng.integers(0, B, n), rng.integers(0, C, n), rng.integers(0, H, n), rng.integers(0, H, n)], 1)
+    # make sure image borders and the last image are in the sample
+    yi[:64, 2] = 0; yi[64:128, 3] = OH - 1; yi[128:192, 0] = B - 1
+    xi[:64, 2] = H - 1; xi[64:128, 3] = 0; xi[128:192, 0] = B - 1
+    chans = np.sort(rng.choice(C, 8, replace=False))
+    say("config 4 B=256 stride", stride, "host truth")
+    y_t, y_a = direct_y(x, w, yi, pad, stride, 1), direct_y(np.abs(x), np.abs(w), yi, pad, stride, 1)
+    gx_t, gx_a = direct_gx(gy, w, xi, pad, stride, 1), direct_gx(np.abs(gy), np.abs(w), xi, pad, stride, 1)
+    gw_t, gw_a = direct_gw(x, gy, chans, k, k, pad, stride, 1), direct_gw(np.abs(x), np.abs(gy), chans, k, k, pad, stride, 1)
+    for name, (y, gw, gx) in _conv_paths(K, dev(x), dev(w), dev(gy), pad, stride, 1).items():
+        say("config 4 B=256 stride", stride, name)
+        yv, gwv, gxv = host(y), host(gw), host(gx)
+        assert_contraction(yv[tuple(yi.T)], y_t, y_a, f"{name} y")
+        assert_contraction(gxv[tuple(xi.T)], gx_t, gx_a, f"{name} gx")
+        assert_contraction(gwv[:, chans], gw_t, gw_a, f"{name} gw")
+    # integer-valued data: every partial sum is an integer below 2^24, so f32 is exact in any order
+    x = rng.integers(-3, 4, x.shape).astype(np.float32)
+    w = rng.integers(-2, 3, w.shape).astype(np.float32)
+    gy = rng.integers(-2, 3, gy.shape).astype(np.float32)
+    y_t, gx_t, gw_t = direct_y(x, w, yi, pad, stride, 1), direct_gx(gy, w, xi, pad, stride, 1), direct_gw(x, gy, chans, k, k, pad, stride, 1)
+    for name, (y, gw, gx) in _conv_paths(K, dev(x), dev(w), dev(gy), pad, stride, 1).items():
+        say("config 4 B=256 stride", stride, name, "integers")
+        assert np.array_equal(host(y)[tuple(yi.T)], y_t), f"{name} y"
+        assert np.array_equal(host(gx)[tuple(xi.T)], gx_t), f"{name} gx"
+        assert np.array_equal(host(gw)[:, chans], gw_t), f"{name} gw"
+
+
+def test_config4_maxpool_full_tensor_bit_exact(K, orc):
+    B, C, H = 256, 128, 56
+    rng = np.random.default_rng(27)
+    x = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    x[3, 5, 10:14, 10:14] = 1.5          # ties inside windows: the first maximum in row-major order wins
+    say("max_pool2d 3x3 s2 on [256,128,56,56]")
+    y, am, il = K.max_pool2d(dev(x), 3, 0, 2)
+    oy, oam, oil = orc.maxpool2d_fwd(x, 3, 0, 2)
+    assert np.array_equal(host(y), oy)
+    assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32)), "f32-encoded argmax (rounded above 2^24)"
+    assert np.array_equal(host(il), oil)
+    gy = rng.standard_normal(oy.shape).astype(np.float32)
+    gx = host(K.max_pool2d_grad(dev(gy), am, il, x.shape, 3, 0, 2))
+    assert np.array_equal(gx.view(np.uint32), orc.maxpool2d_bwd_local(gy, oil, x.shape).view(np.uint32))
+
+
+# ------------------------------------------------------------------------------------- config 5
+def test_config5_dilated_conv_32_images(K, orc):
+    B, C, Kf, H, k, pad, dil = 32, 256, 256, 14, 3, 2, 2
+    rng = np.random.default_rng(55)
+    x = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kf, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kf, H, H)).astype(np.float32)
+    x64, w64, g64 = (v.astype(np.float64) for v in (x, w, gy))
+    say("config 5 dilated, 32 images")
+    y64, cols64 = orc.conv2d_fwd(x64, w64, pad, 1, dil)
+    ya, colsa = orc.conv2d_fwd(np.abs(x64), np.abs(w64), pad, 1, dil)
+    y32, cols32 = orc.conv2d_fwd(x, w, pad, 1, dil)
+    y, cols = K.conv2d(dev(x), dev(w), pad, 1, dil)
+    assert np.array_equal(host(cols), cols32)
+    assert_contraction(host(y), y64, ya, "dilated y", ref32=y32)
+    gw = host(K.conv2d_filter_grad(cols, dev(gy), w.shape))
+    assert_contraction(gw, orc.conv2d_filter_grad(cols64, g64, w.shape), orc.conv2d_filter_grad(colsa, np.abs(g64), w.shape),
+                       "dilated gw", ref32=orc.conv2d_filter_grad(cols32, gy, w.shape))
+    gx = host(K.conv2d_transpose(dev(gy), dev(w), pad, 1, dil, out_hw=(H, H)))
+    assert_contraction(gx, orc.conv2d_transpose(g64, w64, pad, 1, dil, out_hw=(H, H)),
+                       orc.conv2d_transpose(np.abs(g64), np.abs(w64), pad, 1, dil, out_hw=(H, H)), "dilated gx",
+                       ref32=orc.conv2d_transpose(gy, w, pad, 1, dil, out_hw=(H, H)))
+
+
+def test_config5_transposed_conv_32_images(K, orc):
+    B, ych, xch, h, k, pad, stride = 32, 128, 64, 14, 4, 1, 2
+    rng = np.random.default_rng(56)
+    x = rng.standard_normal((B, ych, h, h)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (ych, xch, k, k)).astype(np.float32)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    say("config 5 transposed conv, 32 images")
+    y = K.conv2d_transpose(dev(x), dev(w), pad, stride)                     # reference-reconstructed 28 x 28
+    y64 = orc.conv2d_transpose(x64, w64, pad, stride, 1)
+    assert y64.shape == (B, xch, 28, 28) == tuple(y.shape)
+    assert_contraction(host(y), y64, orc.conv2d_transpose(np.abs(x64), np.abs(w64), pad, stride, 1), "deconv y",
+                       ref32=orc.conv2d_transpose(x, w, pad, stride, 1))
+    gy = rng.standard_normal(y64.shape).astype(np.float32)
+    g64 = gy.astype(np.float64)
+    # gradient w.r.t. the input is a convolution of gy with w (conv2d_transpose.rs:274-300)
+    gx, _ = K.conv2d(dev(gy), dev(w), pad, stride, 1)
+    gx64, _ = orc.conv2d_fwd(g64, w64, pad, stride, 1)
+    assert_contraction(host(gx), gx64, orc.conv2d_fwd(np.abs(g64), np.abs(w64), pad, stride, 1)[0], "deconv gx",
+                       ref32=orc.conv2d_fwd(gy, w, pad, stride, 1)[0])
+    gw = host(K.conv2d_transpose_filter_grad(dev(x), dev(gy), w.shape, pad, stride))
+    assert_contraction(gw, orc.conv2d_transpose_filter_grad(x64, g64, w.shape, pad, stride, 1),
+                       orc.conv2d_transpose_filter_grad(np.abs(x64), np.abs(g64), w.shape, pad, stride, 1), "deconv gw",
+                       ref32=orc.conv2d_transpose_filter_grad(x, gy, w.shape, pad, stride, 1))

@@ -3,8 +3,9 @@
 second-order gradients) are built through libag_host.so, evaluated on the GPU and compared with the
 CPU oracle run stage by stage on the same inputs.
 
-Tolerance for floating point: |got - want| <= 1e-5 + 1e-4 * |want| (contractions are scaled by the
-magnitude of their operands instead, as in test_gpu_parity.py); integer-valued results
+Tolerance for floating point: |got - want| <= 1e-5 + 1e-4 * |want|; contractions: 1e-5 + 2e-5 * the
+magnitude their rounding errors scale with, and the literal bound on 99 % of the elements (the
+kernels themselves are held to the f64 bars of tests/bars.py in test_gpu_parity.py); integer-valued results
 (argmax-driven scatter positions, shapes, the Adam step counter) must be exact.
 """
 import sys
@@ -34,13 +35,25 @@ def G():
     return graph
 
 
-def assert_close(got, want, what, rtol=1e-4, atol=1e-5, scale=None):
+def assert_close(got, want, what, rtol=None, atol=1e-5, scale=None):
+    """Against the f32 oracle run stage by stage.  Without `scale`: the literal bound
+    1e-5 + 1e-4*|want| on every element.  With `scale` (the magnitude rounding errors of the
+    contraction behind `want` scale with): atol + 2e-5 * scale on every element -- two f32 results of
+    the same contraction differ by a few units of roundoff of that magnitude, never by 1e-4 of it --
+    and the literal bound on 99 % of the elements."""
     got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
+    if rtol is None:
+        rtol = 1e-4 if scale is None else 2e-5
     bound = atol + rtol * (np.abs(want) if scale is None else scale)
     err = np.abs(got - want)
     bad = err > bound
+    if scale is not None and err.size:
+        say(f"{what}: worst err {float(err.max()):.3e}, err/scale {float((err / np.maximum(scale, 1e-300)).max()):.3e}, "
+            f"literal {100.0 * float((err <= 1e-5 + 1e-4 * np.abs(want)).mean()):.3f} %")
     assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} outside tolerance, worst {float((err / bound).max()):.2f}x"
+    if scale is not None and err.size:
+        assert float((err <= 1e-5 + 1e-4 * np.abs(want)).mean()) >= 0.99, f"{what}: fewer than 99 % within 1e-5 + 1e-4|want|"
 
 
 def glorot(rng, shape):
@@ -197,7 +210,7 @@ def test_config2_training_steps_with_adam(G, orc, rng):
             got, want = env.array(ids[k]), ref.p[k]
             solid_so_far[k] &= np.abs(og[k]) >= 1e-3 * np.abs(og[k]).max()
             solid = solid_so_far[k]
-            assert_close(got[solid], want[solid], f"param {k} after step {step}", scale=1e-3, rtol=2e-3, atol=1e-7)
+            assert_close(got[solid], want[solid], f"param {k} after step {step}", scale=1e-3, rtol=1e-4, atol=1e-7)
             assert np.abs(got - want).max() <= 2.1e-3
         # Every step is checked from identical state: Adam moves an element by about alpha whatever the
         # size of its gradient, so an element whose gradient is rounding noise can move the other way,
@@ -272,12 +285,12 @@ def test_batch_matmul_and_its_gradients(G, orc, rng, ta, tb):
         except Exception:
             assert isinstance(got, G.OpError), what
             continue
-        assert_close(got, want, what, scale=np.sqrt(max(M, N)), rtol=2e-4)
+        assert_close(got, want, what, scale=np.sqrt(max(M, N)))
     if not ta and not tb:
         gA = np.repeat(bv.astype(np.float64).sum(axis=2)[:, None, :], M, axis=1)
         gB = np.repeat(av.astype(np.float64).sum(axis=1)[:, :, None], N, axis=2)
-        assert_close(gav, gA, "ga analytic", scale=np.sqrt(N), rtol=2e-4)
-        assert_close(gbv, gB, "gb analytic", scale=np.sqrt(M), rtol=2e-4)
+        assert_close(gav, gA, "ga analytic", scale=np.sqrt(N))
+        assert_close(gbv, gB, "gb analytic", scale=np.sqrt(M))
 
 
 # ------------------------------------------------------------------------------- configs 4 / 5 (reduced)
@@ -297,17 +310,17 @@ def test_conv2d_gradients_every_geometry(G, orc, rng, H, pad, stride, dil, k):
     oy, ocols = orc.conv2d_fwd(xv, wv, pad, stride, dil)
     assert_close(yv, oy, "y", scale=1.0)
     gyv = (2 * yv).astype(np.float32)
-    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max())
     # the gradient has x's own extent, also where the transposed-convolution size formula would
     # come out one short (stride 2 on an even extent)
     assert gxv.shape == xv.shape
-    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, stride, dil, out_hw=(H, H)), "gx", scale=np.abs(gxv).max(), rtol=2e-4)
+    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, stride, dil, out_hw=(H, H)), "gx", scale=np.abs(gxv).max())
     # what the reference itself returns (extent rebuilt from gy, conv2d_transpose.rs:55-56) is the
     # top-left crop of that gradient
     ref_like = orc.conv2d_transpose(gyv, wv, pad, stride, dil)
     h = ref_like.shape[2]
     assert h <= H
-    assert_close(gxv[:, :, :h, :h], ref_like, "gx crop", scale=np.abs(gxv).max(), rtol=2e-4)
+    assert_close(gxv[:, :, :h, :h], ref_like, "gx crop", scale=np.abs(gxv).max())
 
 
 def test_conv2d_transpose_upsampling_and_gradients(G, orc, rng):
@@ -326,8 +339,8 @@ def test_conv2d_transpose_upsampling_and_gradients(G, orc, rng):
     gyv = (2 * yv).astype(np.float32)
     # d/dx of a transposed convolution is the forward convolution of gy with the same filter
     ogx, _ = orc.conv2d_fwd(gyv, wv, 1, 2, 1)
-    assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max(), rtol=2e-4)
-    assert_close(gwv, orc.conv2d_transpose_filter_grad(xv, gyv, wv.shape, 1, 2, 1), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max())
+    assert_close(gwv, orc.conv2d_transpose_filter_grad(xv, gyv, wv.shape, 1, 2, 1), "gw", scale=np.abs(gwv).max())
 
 
 def test_max_pool_gradient_and_second_order(G, orc, rng):
@@ -712,8 +725,8 @@ def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, p
     oy, ocols = orc.conv2d_fwd(xv, wv, pad, 1, 1)
     assert_close(yv, oy, "y", scale=1.0)
     gyv = (2 * yv).astype(np.float32)
-    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
-    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, 1, 1, out_hw=(H, H)), "gx", scale=np.abs(gxv).max(), rtol=2e-4)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max())
+    assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, 1, 1, out_hw=(H, H)), "gx", scale=np.abs(gxv).max())
 
 
 def test_conv2d_column_free_second_order(G, orc, rng):
@@ -737,8 +750,8 @@ def test_conv2d_column_free_second_order(G, orc, rng):
     # df/dx = conv_transpose(gy, r) + conv_transpose(2 conv(x, r), w)
     oy, ocols = orc.conv2d_fwd(xv, wv, 1, 1, 1)
     gyv = (2 * oy).astype(np.float32)
-    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max(), rtol=2e-4)
+    assert_close(gwv, orc.conv2d_filter_grad(ocols, gyv, wv.shape), "gw", scale=np.abs(gwv).max())
     oyr, _ = orc.conv2d_fwd(xv, rv, 1, 1, 1)
     want = orc.conv2d_transpose(gyv, rv, 1, 1, 1, out_hw=(H, H)).astype(np.float64) + \
         orc.conv2d_transpose((2 * oyr).astype(np.float32), wv, 1, 1, 1, out_hw=(H, H)).astype(np.float64)
-    assert_close(ggxv, want, "ggx", scale=np.abs(want).max(), rtol=3e-4)
+    assert_close(ggxv, want, "ggx", scale=np.abs(want).max())

@@ -436,3 +436,24 @@ def test_sparse_softmax_xent_matches_torch(orc, rng):
     _allclose(loss.reshape(-1), loss_t.detach().numpy(), rtol=1e-12, atol=1e-12)
     _allclose(lsm, F.log_softmax(lt, dim=1).detach().numpy(), rtol=1e-12, atol=1e-12)
     _allclose(orc.sparse_softmax_xent_grad(lsm, labels, gy), lt.grad.numpy(), rtol=1e-11, atol=1e-12)
+
+
+@pytest.mark.parametrize("pad,stride,dil,k", [(1, 1, 1, 3), (1, 2, 1, 3), (2, 1, 2, 3), (1, 2, 1, 4), (0, 1, 1, 2)])
+def test_direct_definitions_used_by_the_full_size_gpu_tests(orc, rng, pad, stride, dil, k):
+    """tests/direct_conv.py (sampled f64 truth of the B = 256 GPU tests) against the oracle: every
+    output element of a small case."""
+    from direct_conv import direct_gw, direct_gx, direct_y
+    B, C, Kf, H = 3, 5, 4, 11
+    x = rng.standard_normal((B, C, H, H))
+    w = rng.standard_normal((Kf, C, k, k))
+    y, cols = orc.conv2d_fwd(x, w, pad, stride, dil)
+    OH = y.shape[2]
+    gy = rng.standard_normal(y.shape)
+    idx = np.array([(b, f, oy, ox) for b in range(B) for f in range(Kf) for oy in range(OH) for ox in range(OH)])
+    assert np.allclose(direct_y(x, w, idx, pad, stride, dil), y.reshape(-1), rtol=1e-12, atol=1e-12)
+    gx = orc.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(H, H))
+    idx = np.array([(b, c, iy, ix) for b in range(B) for c in range(C) for iy in range(H) for ix in range(H)])
+    assert np.allclose(direct_gx(gy, w, idx, pad, stride, dil), gx.reshape(-1), rtol=1e-12, atol=1e-12)
+    gw = orc.conv2d_filter_grad(cols, gy, w.shape)
+    ch = np.array([1, 3])
+    assert np.allclose(direct_gw(x, gy, ch, k, k, pad, stride, dil), gw[:, ch], rtol=1e-12, atol=1e-12)
