@@ -173,9 +173,11 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch
  * taps.  The filter gradient contracts that copy with the zero-bordered upstream gradient that
  * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images in
  * splits that need the workspace; "same" convolutions only (2*pad == kh-1 == kw-1, K a multiple of
- * 32), so that both copies share one padded plane shape.  A NaN or infinity in x can reach the
- * gradient of the neighbouring channel as well (the contraction runs a few elements past a plane,
- * against border zeros of the gradient). */
+ * 32), so that both copies share one padded plane shape.  The contraction runs a few elements past
+ * a plane, but only over zeros of both operands (the planes are sized for that), so a NaN or
+ * infinity in one channel of x reaches the gradients of that channel only; within the channel it
+ * can reach filter taps that the reference's columns would not pair it with (0 * NaN at a border
+ * position). */
 size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad);
 ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y,
                                      float *xpad, int B, int C, int H, int W, int K, int kh, int kw,
@@ -297,7 +299,9 @@ ag_status_t ag_div_scalar_f32(ag_stream_t stream, const float *a, float s, float
 /* Fill with a constant (zeros / ones / scalar, const_gen_ops.rs:16-90). */
 ag_status_t ag_fill_f32(ag_stream_t stream, float *out, float value, size_t n);
 /* SparseSoftmaxCrossEntropy::compute (xent_ops.rs:63-115): logits [rows,classes], labels [rows]
- * stored as f32 -> loss [rows,1] (output 0) and log_softmax [rows,classes] (output 1). */
+ * stored as f32 -> loss [rows,1] (output 0) and log_softmax [rows,classes] (output 1).  A label that
+ * is negative, not finite or >= classes makes the reference panic (xent_ops.rs:96-104); here that
+ * row's loss, and its gradient row in the function below, are NaN. */
 ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const float *logits, const float *labels,
                                        float *loss, float *log_softmax, size_t rows,
                                        size_t classes);

@@ -250,6 +250,9 @@ __global__ __launch_bounds__(256) void filter_taps_fwd_kernel(const float *__res
     }
 }
 
+// Zeroed floats after the last bordered plane (and before the first one of a bordered input).
+constexpr long long kSlackFloats = 1024;
+
 // Geometry of the implicit (column-free) stride-1 input gradient.
 struct FusedGeom {
     int Hp, Wp;
@@ -265,16 +268,25 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     // its own: a read that runs past the end of a row by up to kw-1-pad elements lands in the left
     // border of the next row, which is just as zero.  The row pitch and the plane (rows added at the
     // bottom) grow until the per-image column range and the plane are multiples of four elements.
-    g->Wp = yw + (kw - 1 - pad);
+    // The implicit filter gradient contracts over the positions of a plane rounded up to its k tile
+    // (32) and reads the other operand up to kh-1 rows and kw-1 elements further: rows are added until
+    // everything it reads past a plane's own data is zero -- the rows below the data, then the top
+    // border of the next plane up to the first data element of its first data row -- so that no value
+    // of a neighbouring plane (which could be a NaN) ever meets one of those zeros.
+    const int top = kh - 1 - pad, left = kw - 1 - pad;
+    g->Wp = yw + left;
     for (;; ++g->Wp) {
         if (g->Wp > xw + kw + 6) return false;
         if (((long long)xh * g->Wp) % 4 != 0) continue;
         g->Hp = xh + kh - 1;
-        while (((long long)g->Hp * g->Wp) % 4 != 0) ++g->Hp;
+        const long long kq = (((long long)xh * g->Wp + 31) / 32) * 32;
+        while (((long long)g->Hp * g->Wp) % 4 != 0 || (long long)(g->Hp - top) * g->Wp - left < kq) ++g->Hp;
         break;
     }
+    // past the last plane the reads run into kSlackFloats zeroed floats
+    if ((long long)(kh - 1) * g->Wp + 2 * (kw - 1) + 32 > kSlackFloats) return false;
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
-    g->gyp_floats = (long long)B * ych * plane + 1024;  // slack: the last taps read a little past a plane
+    g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
     // a tile (64 x 128 for up to 64 channels, else 128 x 256) may straddle two images, not three
     return n_img >= (xch <= 64 ? 128 : 256) && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
@@ -300,7 +312,7 @@ static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w
 // place of the upstream gradient (bordered by `pad`), the C input channels are contracted and the K
 // filters are the output rows.  Leading slack: the implicit filter gradient reads up to one padded
 // row and column before the first plane.
-constexpr long long kFwdLeadFloats = 1024;
+constexpr long long kFwdLeadFloats = kSlackFloats;
 
 static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, FusedGeom *g)
 {
@@ -316,9 +328,9 @@ static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, in
 static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
 {
     // past the end of a plane the next plane's top border (pad rows and pad elements of zeros) or the
-    // zeroed slack follows
+    // zeroed slack follows; fused_geom has sized the plane so that nothing else is reached
     const long long kq = (((long long)OH * g.Wp + 31) / 32) * 32;
-    return kq <= (long long)(g.Hp - pad) * g.Wp ? (int)kq : 0;
+    return kq <= (long long)(g.Hp - pad) * g.Wp - pad ? (int)kq : 0;
 }
 
 }  // namespace ag

@@ -207,6 +207,16 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const float *__restrict_
     }
 }
 
+// A label is an f32 holding a class number (xent_ops.rs:96-104 casts it to usize and panics on a
+// negative, non-finite or too large value: "can't cast to usize" / "Wrong label value").  A kernel
+// cannot panic; such a row's loss and gradient are NaN instead, so the failure shows in the result.
+__device__ inline bool label_of(float lf, size_t classes, size_t *label)
+{
+    const bool ok = lf >= 0.f && lf < (float)classes;  // false for NaN
+    *label = ok ? (size_t)(int)lf : classes;
+    return ok;
+}
+
 // One thread per row (class counts are small): log_softmax = x - (ln(sum exp(x - max)) + max),
 // loss = -log_softmax[label].  xent_ops.rs:63-115, math_ops.rs:540-593.
 __global__ __launch_bounds__(256) void sparse_xent_kernel(const float *__restrict__ logits,
@@ -223,14 +233,15 @@ __global__ __launch_bounds__(256) void sparse_xent_kernel(const float *__restric
         float s = 0.f;
         for (size_t c = 0; c < classes; ++c) s += expf(row[c] - mx);
         const float lse = logf(s) + mx;
-        const size_t label = (size_t)labels[r];
+        size_t label;
+        const bool ok = label_of(labels[r], classes, &label);
         float picked = 0.f;
         for (size_t c = 0; c < classes; ++c) {
             const float v = row[c] - lse;
             lsm[r * classes + c] = v;
             if (c == label) picked = v;
         }
-        loss[r] = -picked;
+        loss[r] = ok ? -picked : __builtin_nanf("");
     }
 }
 
@@ -261,14 +272,15 @@ __global__ __launch_bounds__(256) void sparse_xent_lds_kernel(const float *__res
         float s = 0.f;
         for (unsigned c = 0; c < classes; ++c) s += expf(row[c] - mx);
         const float lse = logf(s) + mx;
-        const size_t label = (size_t)labels[r0 + threadIdx.x];
+        size_t label;
+        const bool ok = label_of(labels[r0 + threadIdx.x], classes, &label);
         float picked = 0.f;
         for (unsigned c = 0; c < classes; ++c) {
             const float v = row[c] - lse;
             row[c] = v;
             if (c == label) picked = v;
         }
-        loss[r0 + threadIdx.x] = -picked;
+        loss[r0 + threadIdx.x] = ok ? -picked : __builtin_nanf("");
     }
     __syncthreads();
     for (unsigned e = threadIdx.x; e < count; e += 256) {
@@ -289,8 +301,10 @@ __global__ __launch_bounds__(256) void sparse_xent_grad_kernel(const float *__re
     {
         const size_t r = i / classes, c = i - r * classes;
         float s = expf(lsm[i]);
-        if (c == (size_t)labels[r]) s -= 1.f;
-        gx[i] = s * gy[r];
+        size_t label;
+        const bool ok = label_of(labels[r], classes, &label);
+        if (c == label) s -= 1.f;
+        gx[i] = ok ? s * gy[r] : __builtin_nanf("");
     }
 }
 

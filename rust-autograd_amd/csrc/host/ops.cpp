@@ -155,6 +155,10 @@ struct Conv2DFilterGrad : Op, ConvHyper {  // conv2d.rs:736-776
     OpError compute(ComputeContext &ctx) const override
     {
         const NdArray cols = ctx.input(0), gy = ctx.input(1), w = ctx.input(2);
+        if (gy.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: gradient must be 4D (got " + shape_str(gy.shape()) + ")");
+        if (w.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: filter must be 4D (got " + shape_str(w.shape()) + ")");
         const int B = (int)gy.shape()[0], K = (int)gy.shape()[1], P = (int)(gy.shape()[2] * gy.shape()[3]);
         const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
         NdArray gw = NdArray::empty(w.shape());
@@ -194,11 +198,16 @@ struct Conv2DWithCols : Op, ConvHyper {  // conv2d.rs:589-629
     OpError compute(ComputeContext &ctx) const override
     {
         const NdArray cols = ctx.input(0), w = ctx.input(1);
+        if (w.ndim() != 4)
+            return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: filter must be 4D (got " + shape_str(w.shape()) + ")");
+        if (cols.ndim() != 1 && cols.ndim() < 3)
+            return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: columns must have at least 3 axes (got " + shape_str(cols.shape()) + ")");
         if (cols.ndim() == 1) {
             // the zero-bordered input of a column-free Conv2D; the third input (only its extents are
             // read) has the shape of the result
             if (ctx.num_inputs() < 3) return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: columns expected");
             const NdArray like = ctx.input(2);
+            if (like.ndim() != 4) return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: 4D result extents expected");
             const int B = (int)like.shape()[0], OH = (int)like.shape()[2], OW = (int)like.shape()[3];
             const int K = (int)w.shape()[0], C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
             const int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
@@ -340,6 +349,10 @@ void Conv2DTranspose::grad(GradientContext &ctx) const
 OpError Conv2DTransposeFilterGrad::compute(ComputeContext &ctx) const
 {
     const NdArray gy = ctx.input(0), x = ctx.input(1), w = ctx.input(2);
+    if (gy.ndim() != 4 || x.ndim() != 4 || w.ndim() != 4)
+        return OpError::make(ErrorKind::IncompatibleShape, "Conv2DTransposeFilterGrad: gradient, input and filter must be 4D (got " +
+                                                               shape_str(gy.shape()) + ", " + shape_str(x.shape()) + ", " +
+                                                               shape_str(w.shape()) + ")");
     const int B = (int)x.shape()[0], ych = (int)x.shape()[1], yh = (int)x.shape()[2], yw = (int)x.shape()[3];
     const int xch = (int)gy.shape()[1], H = (int)gy.shape()[2], W = (int)gy.shape()[3];
     const int kh = (int)w.shape()[2], kw = (int)w.shape()[3];
@@ -567,7 +580,9 @@ std::vector<int> normalize_axes(const std::vector<int> &axes, int rank)
 struct ReduceGradCommon : Op {
     std::vector<int> axes;
     float divide_by_len;  // != 0: additionally divide by the reduced length (ReduceMean::grad, :217-238)
-    ReduceGradCommon(std::vector<int> a, bool mean) : axes(std::move(a)), divide_by_len(mean ? 1.f : 0.f) {}
+    bool should_make_broadcast_dims;  // = !keep_dims of the reduction this is the gradient of (:221-232)
+    ReduceGradCommon(std::vector<int> a, bool mean, bool make_dims)
+        : axes(std::move(a)), divide_by_len(mean ? 1.f : 0.f), should_make_broadcast_dims(make_dims) {}
     const char *name() const override { return "ReduceGradCommon"; }
     OpError compute(ComputeContext &ctx) const override
     {
@@ -589,8 +604,11 @@ struct ReduceGradCommon : Op {
     }
     void grad(GradientContext &ctx) const override
     {
-        // the gradient of a broadcast is the matching sum (:498-511)
-        Tensor s = tensor_ops::reduce_sum(ctx.output_grad(), axes, true);
+        // the gradient of a broadcast is the matching sum, with keep_dims = should_make_broadcast_dims
+        // as the reference has it (:498-511); the division by the reduced length that this op
+        // fuses (a separate Div node in the reference, :231-234) passes through as the mean's 1/len
+        Tensor s = divide_by_len != 0.f ? tensor_ops::reduce_mean(ctx.output_grad(), axes, should_make_broadcast_dims)
+                                        : tensor_ops::reduce_sum(ctx.output_grad(), axes, should_make_broadcast_dims);
         ctx.append_input_grad(s);
         ctx.append_input_grad(std::nullopt);
     }
@@ -630,7 +648,7 @@ struct ReduceSum : Op {
     }
     void grad(GradientContext &ctx) const override
     {
-        const Tensor gx = build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceGradCommon>(axes, mean));
+        const Tensor gx = build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceGradCommon>(axes, mean, !keep_dims));
         ctx.append_input_grad(gx);
     }
 };

@@ -605,6 +605,63 @@ def test_conv2d_column_free_headline_size_matches_columns_path(K):
     assert float((gx - gx_cols).abs().max()) <= 1e-5 + 1e-4 * float(gx_cols.abs().max())
 
 
+def test_conv2d_with_cols_matches_oracle(K, orc, rng):
+    """Conv2DWithCols::compute (conv2d.rs:589-597): the GEMM half of the forward over columns that
+    already exist, called directly through ag_conv2d_with_cols_f32."""
+    for (B, C, Kc, H, W, k, p, s, d) in [(3, 4, 6, 9, 11, 3, 1, 1, 1), (2, 32, 64, 14, 14, 3, 1, 1, 1), (2, 8, 16, 12, 12, 3, 1, 2, 1)]:
+        x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+        w = rng.uniform(-0.3, 0.3, (Kc, C, k, k)).astype(np.float32)
+        w2 = rng.uniform(-0.3, 0.3, (Kc, C, k, k)).astype(np.float32)     # another filter over the same columns
+        say("conv2d_with_cols", (B, C, Kc, H, W, k, p, s, d))
+        oy32, ocols = orc.conv2d_fwd(x, w, p, s, d)
+        OH, OW = oy32.shape[2:]
+        cols = K.im2col(dev(x), k, k, p, p, s, s, d, d)
+        got = host(K.conv2d_with_cols(cols, dev(w2), OH, OW))
+        want32 = orc.conv2d_with_cols(ocols, w2, OH, OW)
+        want64 = orc.conv2d_with_cols(ocols.astype(np.float64), w2.astype(np.float64), OH, OW)
+        wabs = orc.conv2d_with_cols(np.abs(ocols).astype(np.float64), np.abs(w2).astype(np.float64), OH, OW)
+        assert got.shape == want32.shape
+        assert_close_conditioned(got, want64, wabs, "conv2d_with_cols", ref32=want32)
+        # with the forward's own filter it reproduces the forward exactly (same kernel, same operands)
+        y, _ = K.conv2d(dev(x), dev(w), p, s, d)
+        assert np.array_equal(host(K.conv2d_with_cols(cols, dev(w), OH, OW)), host(y))
+
+
+@pytest.mark.parametrize("case", [(3, 64, 64, 14, 14, 3, 1), (2, 64, 128, 56, 56, 3, 1), (2, 32, 32, 16, 16, 5, 2)])
+def test_conv2d_column_free_filter_grad_keeps_a_nan_inside_its_channel(K, orc, rng, case):
+    """The implicit filter gradient contracts a few positions past each plane.  What it reads there
+    must be zeros of both operands: a NaN anywhere in one channel of x -- corners and edges included,
+    first and last image -- may only reach that channel's gradients, as in the reference
+    (conv2d.rs:662-687: gw[:, c] only ever meets the columns of channel c)."""
+    B, C, Kc, H, W, k, p = case
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, H, W)).astype(np.float32)
+    bad = C // 2
+    for b in (0, B - 1):
+        x[b, bad, 0, :] = np.nan
+        x[b, bad, -1, :] = np.nan
+        x[b, bad, :, 0] = np.nan
+        x[b, bad, :, -1] = np.nan
+    say("column-free filter gradient with a NaN channel", case)
+    y, xpad = K.conv2d_nocols(dev(x), dev(w), p)
+    gx, gypad = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+    gw = host(K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p))
+    assert np.isnan(gw[:, bad]).any()
+    others = [c for c in range(C) if c != bad]
+    assert np.isfinite(gw[:, others]).all(), "a NaN left its channel"
+    clean = x.copy()
+    clean[:, bad] = 0.0
+    _, cols64 = orc.conv2d_fwd(clean.astype(np.float64), w.astype(np.float64), p, 1, 1)
+    _, colsabs = orc.conv2d_fwd(np.abs(clean).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1)
+    want = orc.conv2d_filter_grad(cols64, gy.astype(np.float64), w.shape)
+    wabs = orc.conv2d_filter_grad(colsabs, np.abs(gy).astype(np.float64), w.shape)
+    assert_close_conditioned(gw[:, others], want[:, others], wabs[:, others], "gradients of the other channels")
+    # the forward keeps the NaN to the outputs whose windows contain it, like any convolution
+    yv = host(y)
+    assert np.isfinite(yv[1:B - 1]).all()
+
+
 def test_conv2d_column_free_refuses_other_geometries(K, rng):
     L = K.capi.lib()
     assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1) == 0      # C not a multiple of 32
@@ -793,12 +850,15 @@ def test_max_pool_many_ties(K, orc, rng, case):
 
 
 def test_max_pool_nan_window_and_pad_error(K, orc):
-    x = np.zeros((1, 2, 4, 4), dtype=np.float32)
+    x = np.zeros((2, 2, 4, 4), dtype=np.float32)
+    x[0, 0] = np.nan          # the first plane of the tensor: the reference's argmax 0 is ambiguous there
     x[0, 1] = np.nan
+    x[1, 0, :2, :2] = np.nan  # one all-NaN window next to ordinary ones
     say("max_pool NaN")
     y, am, il = K.max_pool2d(dev(x), 2, 0, 2)
     oy, oam, oil = orc.maxpool2d_fwd(x, 2, 0, 2)
     assert np.array_equal(host(y), oy) and np.array_equal(host(am), oam) and np.array_equal(host(il), oil)
+    assert (oil[0] == -1).all() and oil[1, 0, 0, 0] == -1 and (oil[1, 1] >= 0).all()
     with pytest.raises(K.capi.InvalidDims, match="pad must be 0"):
         K.max_pool2d(dev(x), 2, 1, 2)
 
@@ -1038,6 +1098,33 @@ def test_sparse_softmax_cross_entropy_many_rows_and_class_counts(K, orc, rng):
         oloss, olsm = orc.sparse_softmax_xent(logits, labels)
         assert_close(host(loss), oloss, f"xent loss {rows}x{classes}")
         assert_close(host(lsm), olsm, f"log softmax {rows}x{classes}")
+
+
+def test_sparse_softmax_cross_entropy_flags_bad_labels(K, orc, rng):
+    """A negative, non-finite or too large label panics in the reference (xent_ops.rs:96-104); the
+    kernels mark that row with NaN in the loss and in the gradient and leave the other rows alone."""
+    for rows, classes in ((7, 10), (300, 5), (5, 80)):
+        logits = rng.standard_normal((rows, classes)).astype(np.float32)
+        labels = rng.integers(0, classes, rows).astype(np.float32)
+        good = labels.copy()
+        bad_rows = [0, rows // 2, rows - 1, 2]
+        labels[bad_rows[0]] = -1.0
+        labels[bad_rows[1]] = float(classes)
+        labels[bad_rows[2]] = np.nan
+        labels[bad_rows[3]] = np.inf
+        say("xent bad labels", rows, classes)
+        loss, lsm = K.sparse_softmax_cross_entropy(dev(logits), dev(labels))
+        gy = rng.standard_normal((rows, 1)).astype(np.float32)
+        gx = host(K.sparse_softmax_cross_entropy_grad(lsm, dev(labels), dev(gy)))
+        lv = host(loss).reshape(-1)
+        oloss, olsm = orc.sparse_softmax_xent(logits, good)
+        ogx = orc.sparse_softmax_xent_grad(olsm, good, gy)
+        ok = np.ones(rows, bool)
+        ok[bad_rows] = False
+        assert np.isnan(lv[~ok]).all() and np.isnan(gx[~ok]).all()
+        assert_close(lv[ok], oloss.reshape(-1)[ok], "loss of the valid rows")
+        assert_close(gx[ok], ogx[ok], "gradient of the valid rows")
+        assert_close(host(lsm), olsm, "log_softmax does not depend on the labels")
 
 
 def test_sparse_softmax_cross_entropy(K, orc, rng):
