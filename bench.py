@@ -304,7 +304,7 @@ def micro(torch, Kn, capi, dev):
     res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
                           "traffic_bytes": round(TRAFFIC_BYTES["maxpool_fwd"]),
                           "frac_hbm_of_traffic": round(TRAFFIC_BYTES["maxpool_fwd"] / ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "note": "also writes the exact int32 index (95.6 MB, not counted in GB/s) that the backward needs above 2^24 elements"}
+                          "note": "also writes one tap byte per output (23.9 MB, not counted in GB/s): the exact selection that the backward needs above 2^24 elements"}
     ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), None, 256, 128, 56, 56, 3, 0, 2)), 10)
     res["maxpool_fwd_reference_outputs"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
                                             "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),

@@ -213,28 +213,30 @@ ag_status_t ag_conv2d_transpose_filter_grad_f32(ag_stream_t stream, const float 
 
 /* Replaces MaxPool2D::compute -> max_pool_f32 (max_pool2d.rs:166-227, 21-85).  x [B,C,H,W] ->
  * y, argmax [B,C,OH,OW]; argmax holds the flat offset of the first strict maximum inside the whole
- * x tensor converted to f32 by value, as the reference stores it.  idx_local (may be NULL)
- * receives the exact offset inside the (b,c) plane as int32 (-1 when no element exceeded
- * -FLT_MAX), which the backward needs once x has more than 2^24 elements.  pad must be 0: the
- * reference's unsigned `i*stride - pad` is only defined there (max_pool2d.rs:43,53). */
+ * x tensor converted to f32 by value, as the reference stores it.  `taps` (may be NULL; no
+ * counterpart in the reference) receives one byte per output: dy*size + dx of that maximum inside
+ * its window, 255 when no element exceeded -FLT_MAX (an all-NaN window).  It is the exact form of
+ * the selection -- the f32 offset loses its low bits once x has more than 2^24 elements -- and
+ * needs size <= 15.  pad must be 0: the reference's unsigned `i*stride - pad` is only defined
+ * there (max_pool2d.rs:43,53). */
 ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, float *y, float *argmax,
-                                 int32_t *idx_local, int B, int C, int H, int W, int size, int pad,
+                                 uint8_t *taps, int B, int C, int H, int W, int size, int pad,
                                  int stride);
 
 /* Replaces MaxPool2DGrad::compute -> max_pool_grad_f32 (max_pool2d.rs:245-279, 111-135).
  * gy [B,C,OH,OW] -> gx [B,C,H,W] (zero filled, then gx[argmax[i]] += gy[i] in ascending i; done
  * here as a gather that visits the candidate windows of each pixel in that same order, so sums
  * are bit-identical).  (H,W) are explicit; the reference reconstructs them with
- * ag_pool_grad_in_size.  Uses idx_local when it is non-NULL, else the f32 argmax, which is exact
+ * ag_pool_grad_in_size.  Uses `taps` when it is non-NULL, else the f32 argmax, which is exact
  * only while B*C*H*W <= 2^24 (AG_ERR_INVALID_DIMS beyond that). */
 ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy, const float *argmax,
-                                 const int32_t *idx_local, float *gx, int B, int C, int H, int W,
+                                 const uint8_t *taps, float *gx, int B, int C, int H, int W,
                                  int size, int pad, int stride);
 
 /* Replaces MaxPool2DGradGrad::compute -> max_pool_grad_grad_f32 (max_pool2d.rs:297-331, 137-159):
- * ggy[i] = ggx[argmax[i]].  Same idx_local / argmax rule as the backward. */
+ * ggy[i] = ggx[argmax[i]].  Same taps / argmax rule as the backward. */
 ag_status_t ag_maxpool2d_gradgrad_f32(ag_stream_t stream, const float *ggx, const float *argmax,
-                                      const int32_t *idx_local, float *ggy, int B, int C, int H,
+                                      const uint8_t *taps, float *ggy, int B, int C, int H,
                                       int W, int size, int pad, int stride);
 
 /* ---- reductions ----------------------------------------------------------------------------- */

@@ -254,6 +254,17 @@ def maxpool2d_fwd(x, size, pad, stride):
     return y, am, il
 
 
+def maxpool2d_taps(idx_local, W, size, stride):
+    """The exact selection as one byte per output: dy*size + dx of the selected pixel inside its
+    window, 255 where idx_local is -1 (derived from the plane-local index the oracle returns)."""
+    il = np.asarray(idx_local, dtype=np.int64)
+    OH, OW = il.shape[-2:]
+    oy = np.arange(OH).reshape(-1, 1)
+    ox = np.arange(OW).reshape(1, -1)
+    tap = (il // W - oy * stride) * size + (il % W - ox * stride)
+    return np.where(il >= 0, tap, 255).astype(np.uint8)
+
+
 def maxpool2d_bwd(gy, argmax, x_shape):
     gy, argmax = _c(gy), _c(argmax, gy.dtype)
     gx = np.empty(tuple(x_shape), dtype=gy.dtype)

@@ -112,6 +112,7 @@ TEST_HOOKS = {
     "ag_test_gemm_force_splits": (None, [c_i]),
     "ag_test_gemm_force_grid": (None, [c_i]),
     "ag_test_conv_fused_input_grad": (None, [c_i]),
+    "ag_test_pool_chunk_rows": (None, [c_i]),
 }
 
 _lib = None

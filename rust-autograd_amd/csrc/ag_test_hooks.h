@@ -19,6 +19,8 @@ void ag_test_gemm_force_splits(int splits);
 void ag_test_gemm_force_grid(int blocks_per_cu);
 /* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): it may take the implicit GEMM. */
 void ag_test_conv_fused_input_grad(int on);
+/* Output rows per chunk of the stride-2 pooling kernels (0 = automatic). */
+void ag_test_pool_chunk_rows(int rows);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

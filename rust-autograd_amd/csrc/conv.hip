@@ -215,6 +215,61 @@ __global__ __launch_bounds__(256) void pad_border_kernel(const float *__restrict
     }
 }
 
+// The same copy with the divisions replaced by multiplications: grid.y walks the images, so the
+// element counter stays small enough for n / d == umulhi(n, floor(2^32 / d) + 1) to be exact (the
+// host checks the range).  gyp [B][planes][Hp][Wp]; quads_img = planes * Hp * Wp / 4.
+__global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__restrict__ gy, float *__restrict__ gyp,
+                                                              unsigned quads_img, unsigned planes, int OH, int OW, int Wp,
+                                                              int top, int left, unsigned plane_quads, unsigned m_plane,
+                                                              unsigned m_row, int B)
+{
+    const unsigned qi = blockIdx.x * 256u + threadIdx.x;
+    if (qi >= quads_img) return;
+    const unsigned pl = __umulhi(qi, m_plane);
+    const unsigned e0 = (qi - pl * plane_quads) * 4u;
+    int r = (int)__umulhi(e0, m_row), sx = (int)(e0 - (unsigned)r * (unsigned)Wp);
+    // (row, column) of the four elements relative to the image data
+    int oy[4], ox[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        oy[t] = r - top;
+        ox[t] = sx - left;
+        if (++sx == Wp) {
+            sx = 0;
+            ++r;
+        }
+    }
+    for (int b = blockIdx.y; b < B; b += gridDim.y) {
+        const float *src = gy + ((long long)b * planes + pl) * (long long)OH * OW;
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            v[t] = ((unsigned)oy[t] < (unsigned)OH && (unsigned)ox[t] < (unsigned)OW) ? src[oy[t] * OW + ox[t]] : 0.f;
+        st_stream(reinterpret_cast<float4 *>(gyp) + ((long long)b * quads_img + qi), make_float4(v[0], v[1], v[2], v[3]));
+    }
+}
+
+// Launches the bordered copy of `planes` planes per image.
+static void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp, int Wp,
+                              int top, int left)
+{
+    const long long plane_quads = (long long)Hp * Wp / 4, quads_img = plane_quads * planes;
+    // exactness of the two multiply-high divisions: n * (m * d - 2^32) < 2^32 with m * d - 2^32 <= d
+    const bool fast = quads_img * plane_quads < (1LL << 32) && (long long)Hp * Wp * Wp < (1LL << 32) && plane_quads > 1 && Wp > 1;
+    if (fast) {
+        const unsigned m_plane = (unsigned)((1ULL << 32) / (unsigned long long)plane_quads) + 1u;
+        const unsigned m_row = (unsigned)((1ULL << 32) / (unsigned long long)Wp) + 1u;
+        const dim3 grid((unsigned)((quads_img + 255) / 256), (unsigned)(B < 65535 ? B : 65535));
+        hipLaunchKernelGGL(pad_border_fast_kernel, grid, dim3(256), 0, st, src, dst, (unsigned)quads_img, (unsigned)planes, OH, OW,
+                           Wp, top, left, (unsigned)plane_quads, m_plane, m_row, B);
+        return;
+    }
+    const long long quads = quads_img * B;
+    long long blocks = (quads + 255) / 256;
+    if (blocks > 1048576) blocks = 1048576;
+    hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src, dst, quads, OH, OW, Hp, Wp, top, left);
+}
+
 // Zeroes the slack before and after the padded planes: the implicit filter gradient multiplies what
 // it reads there by border zeros of the gradient, which must not meet a NaN bit pattern.
 __global__ void zero_slack_kernel(float *lead, int n_lead, float *tail, int n_tail)
@@ -296,10 +351,7 @@ static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w
                                  int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad)
 {
     const long long quads = (long long)B * ych * g.Hp * g.Wp / 4;
-    long long blocks = (quads + 255) / 256;
-    if (blocks > 1048576) blocks = 1048576;
-    hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, gy, scratch, quads, yh, yw, g.Hp,
-                       g.Wp, kh - 1 - pad, kw - 1 - pad);
+    launch_pad_border(st, gy, scratch, B, ych, yh, yw, g.Hp, g.Wp, kh - 1 - pad, kw - 1 - pad);
     // the implicit filter gradient may read a few elements past the last plane and expects zeros
     hipLaunchKernelGGL(zero_slack_kernel, dim3(4), dim3(256), 0, st, scratch, 0, scratch + quads * 4,
                        (int)(g.gyp_floats - quads * 4));
@@ -358,9 +410,7 @@ extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const fl
     hipStream_t st = as_stream(stream);
     float *xp = xpad + kFwdLeadFloats, *wf = xp + g.gyp_floats;
     const long long quads = (long long)B * C * g.Hp * g.Wp / 4;
-    long long blocks = (quads + 255) / 256;
-    if (blocks > 1048576) blocks = 1048576;
-    hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, x, xp, quads, H, W, g.Hp, g.Wp, pad, pad);
+    launch_pad_border(st, x, xp, B, C, H, W, g.Hp, g.Wp, pad, pad);
     hipLaunchKernelGGL(zero_slack_kernel, dim3(8), dim3(256), 0, st, xpad, (int)kFwdLeadFloats, xp + quads * 4,
                        (int)(g.gyp_floats - quads * 4));
     hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,

@@ -387,9 +387,9 @@ struct PoolHyper {
     int pad, stride, size;
 };
 
-// Outputs of MaxPool2D: [0] y, [1] argmax as f32 (the reference's encoding), [2] exact plane-local
-// int32 indices (bit pattern stored in an f32 array; an addition of this implementation that the
-// backward uses so it stays exact above 2^24 elements).
+// Outputs of MaxPool2D: [0] y, [1] argmax as f32 (the reference's encoding), [2] one tap byte per
+// output (the exact selection inside each window, packed four to an f32 of a rank-1 array; an
+// addition of this implementation that the backward uses so it stays exact above 2^24 elements).
 struct MaxPool2DGradGrad : Op, PoolHyper {  // max_pool2d.rs:297-337
     explicit MaxPool2DGradGrad(PoolHyper h) : PoolHyper(h) {}
     const char *name() const override { return "MaxPool2DGradGrad"; }
@@ -399,7 +399,7 @@ struct MaxPool2DGradGrad : Op, PoolHyper {  // max_pool2d.rs:297-337
         const int B = (int)ggx.shape()[0], C = (int)ggx.shape()[1], H = (int)ggx.shape()[2], W = (int)ggx.shape()[3];
         NdArray ggy = NdArray::empty(argmax.shape());
         const OpError e = from_status(ag_maxpool2d_gradgrad_f32(ctx.stream(), ggx.ptr(), argmax.ptr(),
-                                                                reinterpret_cast<const int32_t *>(idx.ptr()), ggy.ptr(), B, C,
+                                                                reinterpret_cast<const uint8_t *>(idx.ptr()), ggy.ptr(), B, C,
                                                                 H, W, size, pad, stride));
         if (!e.ok()) return e;
         ctx.append_output(ggy);
@@ -436,7 +436,7 @@ struct MaxPool2DGrad : Op, PoolHyper {  // max_pool2d.rs:245-295
         const int xw = in_w >= 0 ? in_w : ag_pool_grad_in_size(yw, size, pad, stride);
         NdArray gx = NdArray::empty({B, C, xh, xw});
         const OpError e = from_status(ag_maxpool2d_bwd_f32(ctx.stream(), gy.ptr(), argmax.ptr(),
-                                                           reinterpret_cast<const int32_t *>(idx.ptr()), gx.ptr(), B, C, xh, xw,
+                                                           reinterpret_cast<const uint8_t *>(idx.ptr()), gx.ptr(), B, C, xh, xw,
                                                            size, pad, stride));
         if (!e.ok()) return e;
         ctx.append_output(gx);
@@ -463,9 +463,10 @@ struct MaxPool2D : Op, PoolHyper {  // max_pool2d.rs:166-243
         const int B = (int)x.shape()[0], C = (int)x.shape()[1], H = (int)x.shape()[2], W = (int)x.shape()[3];
         const int OH = ag_pool_out_size(H, size, pad, stride), OW = ag_pool_out_size(W, size, pad, stride);
         const Shape ys{B, C, std::max(OH, 0), std::max(OW, 0)};
-        NdArray y = NdArray::empty(ys), argmax = NdArray::empty(ys), idx = NdArray::empty(ys);
+        NdArray y = NdArray::empty(ys), argmax = NdArray::empty(ys);
+        NdArray idx = NdArray::empty({(int64_t)((y.len() + 3) / 4 + 1)});
         const OpError e = from_status(ag_maxpool2d_fwd_f32(ctx.stream(), x.ptr(), y.ptr(), argmax.ptr(),
-                                                           reinterpret_cast<int32_t *>(idx.ptr()), B, C, H, W, size, pad, stride));
+                                                           reinterpret_cast<uint8_t *>(idx.ptr()), B, C, H, W, size, pad, stride));
         if (!e.ok()) return e;
         ctx.append_output(y);
         ctx.append_output(argmax);

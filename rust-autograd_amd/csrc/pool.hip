@@ -8,6 +8,7 @@
 #include <cfloat>
 
 #include "ag_internal.h"
+#include "ag_test_hooks.h"
 
 namespace ag {
 
@@ -15,10 +16,26 @@ struct PoolGeom {
     int H, W, OH, OW, size, stride;
 };
 
+// The exact selection of a window travels as ONE BYTE per output: the tap dy*size + dx of the first
+// strict maximum inside the window (row-major, the reference's scan order), kNoTap when no element
+// exceeded the start value (an all-NaN window).  The backward knows the window geometry, so the
+// byte identifies the pixel; it replaces the reference's f32-encoded whole-tensor offset, which is
+// exact only up to 2^24 elements, at a quarter of the bytes.
+constexpr int kNoTap = 255;
+constexpr int kMaxTapSize = 15;  // size*size - 1 must stay below kNoTap
+
+// Plane-local position of the pixel that window (oy, ox) selected, -1 for kNoTap.
+__device__ inline int tap_position(int tap, int oy, int ox, const PoolGeom &g)
+{
+    if (tap == kNoTap) return -1;
+    const int dy = tap / g.size, dx = tap - dy * g.size;
+    return (oy * g.stride + dy) * g.W + ox * g.stride + dx;
+}
+
 __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restrict__ x,
                                                           float *__restrict__ y,
                                                           float *__restrict__ argmax,
-                                                          int32_t *__restrict__ idx_local,
+                                                          uint8_t *__restrict__ taps,
                                                           PoolGeom g, int chunks)
 {
     const int chunk = blockIdx.x % chunks;
@@ -33,13 +50,14 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     // Start value and tie rule of max_pool2d.rs:51-70: most negative finite float, index 0,
     // replaced only by a strictly greater value (NaN never wins).
     float best = -FLT_MAX;
-    int best_local = -1;
+    int best_local = -1, best_tap = kNoTap;
     for (int h = h0; h < h1; ++h)
         for (int w = w0; w < w1; ++w) {
             const float v = xp[h * g.W + w];
             if (v > best) {
                 best = v;
                 best_local = h * g.W + w;
+                best_tap = (h - h0) * g.size + (w - w0);
             }
         }
     const long long out = plane * (long long)g.OH * g.OW + o;
@@ -47,14 +65,14 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float *__restric
     // The reference stores the whole-tensor offset converted to f32 by value (max_pool2d.rs:74-75).
     const unsigned long long flat = best_local >= 0 ? (unsigned long long)(base + best_local) : 0ull;
     argmax[out] = (float)flat;  // round-to-nearest-even, like Rust's `as f32`
-    if (idx_local) idx_local[out] = best_local;
+    if (taps) taps[out] = (uint8_t)best_tap;
 }
 
-// EXACT: selection read from the plane-local int32 buffer; otherwise from the f32 argmax.
+// EXACT: selection read from the tap bytes; otherwise from the f32 argmax.
 template <bool EXACT>
 __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restrict__ gy,
                                                           const float *__restrict__ argmax,
-                                                          const int32_t *__restrict__ idx_local,
+                                                          const uint8_t *__restrict__ taps,
                                                           float *__restrict__ gx, PoolGeom g,
                                                           int chunks)
 {
@@ -75,7 +93,7 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restric
         for (int ox = ox_lo; ox <= ox_hi; ++ox) {
             const long long o = obase + oy * g.OW + ox;
             bool mine;
-            if (EXACT) mine = idx_local[o] == e;
+            if (EXACT) mine = tap_position(taps[o], oy, ox, g) == e;
             else mine = (long long)argmax[o] == flat;
             if (mine) acc += gy[o];
         }
@@ -93,7 +111,7 @@ constexpr int kPoolBandBytes = 8 * 1024;
 // outputs.  256 threads, 256 outputs per round.
 template <int SIZE, int STRIDE>  // 0 = run-time window / stride
 __device__ inline void pool_scan_band(const float *tile, float *__restrict__ y, float *__restrict__ argmax,
-                                      int32_t *__restrict__ idx_local, const PoolGeom &g, long long plane,
+                                      uint8_t *__restrict__ taps, const PoolGeom &g, long long plane,
                                       int oy0, int rows, int iy0)
 {
     const int size = SIZE ? SIZE : g.size, stride = STRIDE ? STRIDE : g.stride;
@@ -101,7 +119,7 @@ __device__ inline void pool_scan_band(const float *tile, float *__restrict__ y, 
     const long long obase = plane * (long long)g.OH * g.OW + (long long)oy0 * g.OW;
     float *const yp = y + obase;
     float *const ap = argmax + obase;
-    int32_t *const ip = idx_local ? idx_local + obase : nullptr;
+    uint8_t *const tp = taps ? taps + obase : nullptr;
     // whole-tensor offsets below 2^32 convert to f32 with one instruction
     const bool small = (unsigned long long)(base + (long long)g.H * g.W) <= 0xffffffffull;
     const int OW = g.OW, W = g.W, n_out = rows * OW;
@@ -112,7 +130,7 @@ __device__ inline void pool_scan_band(const float *tile, float *__restrict__ y, 
         const int first = (r * stride) * W + ox * stride;  // window's first element inside the staged rows
         const float *w0 = tile + first;
         float best = -FLT_MAX;
-        int best_off = -1;
+        int best_off = -1, best_tap = kNoTap;
 #pragma unroll
         for (int dy = 0; dy < size; ++dy)
 #pragma unroll
@@ -121,6 +139,7 @@ __device__ inline void pool_scan_band(const float *tile, float *__restrict__ y, 
                 const bool gt = v > best;
                 best = gt ? v : best;
                 best_off = gt ? dy * W + dx : best_off;
+                best_tap = gt ? dy * size + dx : best_tap;
             }
         const int best_local = best_off >= 0 ? iy0 * W + first + best_off : -1;
         float flat;
@@ -128,7 +147,7 @@ __device__ inline void pool_scan_band(const float *tile, float *__restrict__ y, 
         else flat = best_off >= 0 ? (float)(unsigned long long)(base + best_local) : 0.f;
         st_stream(yp + o, best);
         st_stream(ap + o, flat);
-        if (ip) st_stream(ip + o, best_local);
+        if (tp) tp[o] = (uint8_t)best_tap;
         r += step_r;
         ox += step_x;
         if (ox >= OW) {
@@ -145,7 +164,7 @@ template <int SIZE, int STRIDE>  // 0 = run-time window / stride
 __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__restrict__ x,
                                                               float *__restrict__ y,
                                                               float *__restrict__ argmax,
-                                                              int32_t *__restrict__ idx_local,
+                                                              uint8_t *__restrict__ taps,
                                                               PoolGeom g, int R, int bands, int vec)
 {
     extern __shared__ float tile[];
@@ -167,7 +186,7 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
         for (int e = threadIdx.x; e < n_in; e += 256) tile[e] = xp[e];
     }
     __syncthreads();
-    pool_scan_band<SIZE, STRIDE>(tile, y, argmax, idx_local, g, plane, oy0, rows, iy0);
+    pool_scan_band<SIZE, STRIDE>(tile, y, argmax, taps, g, plane, oy0, rows, iy0);
 }
 
 // LDS-staged backward: one block per (plane, band of IR input rows).  The upstream gradient and
@@ -177,7 +196,7 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
 template <bool EXACT, int SIZE, int STRIDE>  // SIZE/STRIDE 0 = run-time
 __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__restrict__ gy,
                                                               const float *__restrict__ argmax,
-                                                              const int32_t *__restrict__ idx_local,
+                                                              const uint8_t *__restrict__ taps,
                                                               float *__restrict__ gx, PoolGeom g,
                                                               int IR, int bands, int max_orows)
 {
@@ -199,7 +218,8 @@ __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__res
     for (int e = threadIdx.x; e < n_o; e += 256) {
         s_gy[e] = ld_stream(gy + obase + e);
         if (EXACT) {
-            s_idx[e] = ld_stream(idx_local + obase + e);
+            const int orow = e / g.OW;
+            s_idx[e] = tap_position(taps[obase + e], o_lo + orow, e - orow * g.OW, g);
         } else {
             // whole-tensor offset -> plane-local (exact below 2^24 elements); other planes never match
             const long long a = (long long)argmax[obase + e] - xbase;
@@ -253,16 +273,18 @@ __global__ __launch_bounds__(256) void maxpool_bwd_lds_kernel(const float *__res
 template <bool EXACT>
 __global__ __launch_bounds__(256) void maxpool_gradgrad_kernel(const float *__restrict__ ggx,
                                                                const float *__restrict__ argmax,
-                                                               const int32_t *__restrict__ idx_local,
-                                                               float *__restrict__ ggy,
+                                                               const uint8_t *__restrict__ taps,
+                                                               float *__restrict__ ggy, PoolGeom g,
                                                                long long plane_x, long long plane_y,
                                                                long long total_y)
 {
     for (long long o = blockIdx.x * 256LL + threadIdx.x; o < total_y; o += gridDim.x * 256LL) {
         long long src;
         if (EXACT) {
-            const int32_t l = idx_local[o];
-            src = l >= 0 ? (o / plane_y) * plane_x + l : 0;  // index 0 when nothing beat the start value
+            const long long plane = o / plane_y;
+            const int in_plane = (int)(o - plane * plane_y), oy = in_plane / g.OW;
+            const int l = tap_position(taps[o], oy, in_plane - oy * g.OW, g);
+            src = l >= 0 ? plane * plane_x + l : 0;  // index 0 when nothing beat the start value
         } else {
             src = (long long)argmax[o];
         }
@@ -303,7 +325,7 @@ static ag_status_t pool_geom(const char *who, int B, int C, int H, int W, int si
 template <bool EXACT, int SIZE, int LPR>
 __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__restrict__ gy,
                                                              const float *__restrict__ argmax,
-                                                             const int32_t *__restrict__ idx_local,
+                                                             const uint8_t *__restrict__ taps,
                                                              float *__restrict__ gx, PoolGeom g, int rows_per_chunk,
                                                              int chunks, unsigned groups_total)
 {
@@ -327,7 +349,7 @@ __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__rest
         // gradient and selected plane-local position of outputs (oy, 2q) and (oy, 2q+1)
         struct Out {
             float ga, gb;
-            long long ia, ib;
+            int ia, ib;
         };
         auto load_out = [&](int oy) {
             Out o;
@@ -335,19 +357,24 @@ __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__rest
             o.ga = va ? gy[at] : 0.f;
             o.gb = vb ? gy[at + 1] : 0.f;
             if (EXACT) {
-                o.ia = va ? (long long)idx_local[at] : -1;
-                o.ib = vb ? (long long)idx_local[at + 1] : -1;
+                // tap -> pixel: window (oy, ox) starts at (2*oy, 2*ox).  (Plain loads: a cache line of
+                // gradients or taps serves several consecutive rows of the walk.)
+                const int ta = va ? (int)taps[at] : kNoTap, tb = vb ? (int)taps[at + 1] : kNoTap;
+                o.ia = ta != kNoTap ? (2 * oy + ta / SIZE) * W + 4 * q + ta % SIZE : -1;
+                o.ib = tb != kNoTap ? (2 * oy + tb / SIZE) * W + 4 * q + 2 + tb % SIZE : -1;
             } else {
                 // whole-tensor offsets as stored by the forward pass; made plane-local here
-                o.ia = va ? (long long)argmax[at] - base : -1;
-                o.ib = vb ? (long long)argmax[at + 1] - base : -1;
+                const long long hw = (long long)g.H * W;
+                const long long da = va ? (long long)argmax[at] - base : -1, db = vb ? (long long)argmax[at + 1] - base : -1;
+                o.ia = da >= 0 && da < hw ? (int)da : -1;
+                o.ib = db >= 0 && db < hw ? (int)db : -1;
             }
             return o;
         };
         // Adds what window row `o` (with the neighbour's second window `pg`, `pi`) gives to the
         // four pixels of input row iy, pixel by pixel in ascending ox.
-        auto add_row = [&](float (&acc)[4], const Out &o, float pg, long long pi, int iy) {
-            const long long r = (long long)iy * W + 4 * q;
+        auto add_row = [&](float (&acc)[4], const Out &o, float pg, int pi, int iy) {
+            const int r = iy * W + 4 * q;
             if (SIZE == 3) {
                 acc[0] = pi == r ? acc[0] + pg : acc[0];
                 acc[0] = o.ia == r ? acc[0] + o.ga : acc[0];
@@ -362,11 +389,13 @@ __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__rest
                 acc[3] = o.ib == r + 3 ? acc[3] + o.gb : acc[3];
             }
         };
-        auto neighbour = [&](const Out &o, float &pg, long long &pi) {
+        auto neighbour = [&](const Out &o, float &pg, int &pi) {
             pg = __shfl_up(o.gb, 1, LPR);
-            const int lo = __shfl_up((int)(o.ib & 0xffffffffll), 1, LPR), hi = __shfl_up((int)(o.ib >> 32), 1, LPR);
-            pi = q > 0 ? (((long long)hi << 32) | (unsigned)lo) : -1;
-            if (q == 0) pg = 0.f;
+            pi = __shfl_up(o.ib, 1, LPR);
+            if (q == 0) {
+                pg = 0.f;
+                pi = -1;
+            }
         };
         auto store_row = [&](int iy, const float (&acc)[4]) {
             if (active) st_stream(reinterpret_cast<float4 *>(gxp + iy * W), make_float4(acc[0], acc[1], acc[2], acc[3]));
@@ -378,7 +407,7 @@ __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__rest
         if (SIZE == 3 && oy0 > 0 && oy0 < oy1) {
             const Out above = load_out(oy0 - 1);
             float pg;
-            long long pi;
+            int pi;
             neighbour(above, pg, pi);
             add_row(carry, above, pg, pi, 2 * oy0);
         }
@@ -389,7 +418,7 @@ __global__ __launch_bounds__(256) void maxpool_bwd_s2_kernel(const float *__rest
             nxt.ia = nxt.ib = -1;
             if (oy + 1 < oy1) nxt = load_out(oy + 1);
             float pg = 0.f;
-            long long pi = -1;
+            int pi = -1;
             if (SIZE == 3) neighbour(cur, pg, pi);
             float a0[4] = {carry[0], carry[1], carry[2], carry[3]}, a1[4] = {0.f, 0.f, 0.f, 0.f};
             add_row(a0, cur, pg, pi, 2 * oy);
@@ -421,9 +450,16 @@ static int lanes_per_row(int W)
     return W4 <= 4 ? 4 : W4 <= 8 ? 8 : W4 <= 16 ? 16 : W4 <= 32 ? 32 : 64;
 }
 
-// Output rows per chunk: short chunks give more independent streams, long ones re-read fewer
-// halo rows; nine rows of a 27-row plane measured well.
-static int pool_chunk_rows(int OH) { return OH <= 12 ? OH : (OH + (OH + 8) / 9 - 1) / ((OH + 8) / 9); }
+static thread_local int g_chunk_rows = 0;  // test hook (ag_test_hooks.h), per calling thread
+// Output rows per chunk of the stride-2 backward.  Short chunks win by a wide margin although each
+// re-reads the window row above it (one byte and one float per output): 256 x 128 planes of
+// 56 x 56 take 0.120 ms as whole planes, 0.113 with 9 rows, 0.103 with 3 and 0.082-0.091 with 2
+// (one row: 0.096-0.114).
+static int pool_chunk_rows(int OH)
+{
+    if (g_chunk_rows > 0) return g_chunk_rows < OH ? g_chunk_rows : OH;
+    return OH < 2 ? OH : 2;
+}
 
 constexpr long long kExactFloatIndexLimit = 1LL << 24;
 
@@ -431,14 +467,20 @@ constexpr long long kExactFloatIndexLimit = 1LL << 24;
 
 using namespace ag;
 
+// Test hook (ag_test_hooks.h; not part of the operator surface): output rows per chunk of the
+// stride-2 pooling kernels for later calls of this thread (0 = automatic).
+extern "C" void ag_test_pool_chunk_rows(int rows) { ag::g_chunk_rows = rows; }
+
 extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, float *y,
-                                            float *argmax, int32_t *idx_local, int B, int C, int H,
+                                            float *argmax, uint8_t *taps, int B, int C, int H,
                                             int W, int size, int pad, int stride)
 {
     PoolGeom g;
     if ((long long)B * C == 0) return AG_OK;
     if (ag_status_t s = pool_geom("max_pool2d", B, C, H, W, size, pad, stride, &g)) return s;
     AG_REQUIRE(x && y && argmax, AG_ERR_INVALID_DIMS, "max_pool2d: null pointer");
+    AG_REQUIRE(!taps || size <= kMaxTapSize, AG_ERR_INVALID_DIMS,
+               "max_pool2d: a tap byte addresses windows of up to %d x %d (got %d)", kMaxTapSize, kMaxTapSize, size);
     if (g.OH <= 0 || g.OW <= 0) return AG_OK;
     const long long row_bytes = (long long)W * 4;
     if (row_bytes * size <= kPoolLdsBytes) {
@@ -455,7 +497,7 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
         const int vec = (W % 4 == 0) && aligned16(x);
 #define AG_POOL_FWD(SZ, ST)                                                                                   \
     hipLaunchKernelGGL((maxpool_fwd_lds_kernel<SZ, ST>), dim3((unsigned)blocks), dim3(256), lds, as_stream(stream), \
-                       x, y, argmax, idx_local, g, R, bands, vec)
+                       x, y, argmax, taps, g, R, bands, vec)
         if (size == 3 && stride == 2) AG_POOL_FWD(3, 2);
         else if (size == 2 && stride == 2) AG_POOL_FWD(2, 2);
         else AG_POOL_FWD(0, 0);
@@ -465,21 +507,23 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
         const long long blocks = (long long)B * C * chunks;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
         hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), x, y,
-                           argmax, idx_local, g, chunks);
+                           argmax, taps, g, chunks);
     }
     return check_launch("max_pool2d");
 }
 
 extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy, const float *argmax,
-                                            const int32_t *idx_local, float *gx, int B, int C, int H,
+                                            const uint8_t *taps, float *gx, int B, int C, int H,
                                             int W, int size, int pad, int stride)
 {
     PoolGeom g;
     if ((long long)B * C == 0) return AG_OK;
     if (ag_status_t s = pool_geom("max_pool2d_grad", B, C, H, W, size, pad, stride, &g)) return s;
-    AG_REQUIRE(gy && gx && (argmax || idx_local), AG_ERR_INVALID_DIMS, "max_pool2d_grad: null pointer");
-    AG_REQUIRE(idx_local || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
-               "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the int32 plane-local indices",
+    AG_REQUIRE(gy && gx && (argmax || taps), AG_ERR_INVALID_DIMS, "max_pool2d_grad: null pointer");
+    AG_REQUIRE(!taps || size <= kMaxTapSize, AG_ERR_INVALID_DIMS,
+               "max_pool2d_grad: a tap byte addresses windows of up to %d x %d (got %d)", kMaxTapSize, kMaxTapSize, size);
+    AG_REQUIRE(taps || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
+               "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the tap bytes",
                (long long)B * C * H * W);
     if (stride == 2 && (size == 2 || size == 3) && W % 4 == 0 && W <= 256 && aligned16(gx) && g.OH > 0 && g.OW > 0 &&
         (long long)B * C * g.OH < 0x7fffffffLL && (long long)H * W < 0x7fffffffLL) {
@@ -490,7 +534,7 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
         if (blocks > 1048576) blocks = 1048576;
 #define AG_POOL_BWD_S2(EX, SZ, LP)                                                                            \
     hipLaunchKernelGGL((maxpool_bwd_s2_kernel<EX, SZ, LP>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), \
-                       gy, argmax, idx_local, gx, g, rpc, chunks, (unsigned)groups)
+                       gy, argmax, taps, gx, g, rpc, chunks, (unsigned)groups)
 #define AG_POOL_BWD_S2_LPR(EX, SZ)                      \
     switch (lpr) {                                      \
         case 4: AG_POOL_BWD_S2(EX, SZ, 4); break;       \
@@ -499,7 +543,7 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
         case 32: AG_POOL_BWD_S2(EX, SZ, 32); break;     \
         default: AG_POOL_BWD_S2(EX, SZ, 64); break;     \
     }
-        if (idx_local) {
+        if (taps) {
             if (size == 3) { AG_POOL_BWD_S2_LPR(true, 3) } else { AG_POOL_BWD_S2_LPR(true, 2) }
         } else {
             if (size == 3) { AG_POOL_BWD_S2_LPR(false, 3) } else { AG_POOL_BWD_S2_LPR(false, 2) }
@@ -525,9 +569,9 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
         const size_t lds = (size_t)max_orows * orow_bytes;
 #define AG_POOL_BWD(EX, SZ, ST)                                                                               \
     hipLaunchKernelGGL((maxpool_bwd_lds_kernel<EX, SZ, ST>), dim3((unsigned)blocks), dim3(256), lds,               \
-                       as_stream(stream), gy, argmax, idx_local, gx, g, IR, bands, max_orows)
+                       as_stream(stream), gy, argmax, taps, gx, g, IR, bands, max_orows)
         const bool s32 = size == 3 && stride == 2, s22 = size == 2 && stride == 2;
-        if (idx_local) {
+        if (taps) {
             if (s32) AG_POOL_BWD(true, 3, 2);
             else if (s22) AG_POOL_BWD(true, 2, 2);
             else AG_POOL_BWD(true, 0, 0);
@@ -542,36 +586,38 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
     const int chunks = (H * W + 255) / 256;
     const long long blocks = (long long)B * C * chunks;
     AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);
-    if (idx_local)
+    if (taps)
         hipLaunchKernelGGL(maxpool_bwd_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), gy, argmax, idx_local, gx, g, chunks);
+                           as_stream(stream), gy, argmax, taps, gx, g, chunks);
     else
         hipLaunchKernelGGL(maxpool_bwd_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), gy, argmax, idx_local, gx, g, chunks);
+                           as_stream(stream), gy, argmax, taps, gx, g, chunks);
     return check_launch("max_pool2d_grad");
 }
 
 extern "C" ag_status_t ag_maxpool2d_gradgrad_f32(ag_stream_t stream, const float *ggx,
-                                                 const float *argmax, const int32_t *idx_local,
+                                                 const float *argmax, const uint8_t *taps,
                                                  float *ggy, int B, int C, int H, int W, int size,
                                                  int pad, int stride)
 {
     PoolGeom g;
     if ((long long)B * C == 0) return AG_OK;
     if (ag_status_t s = pool_geom("max_pool2d_grad_grad", B, C, H, W, size, pad, stride, &g)) return s;
-    AG_REQUIRE(ggx && ggy && (argmax || idx_local), AG_ERR_INVALID_DIMS, "max_pool2d_grad_grad: null pointer");
-    AG_REQUIRE(idx_local || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
-               "max_pool2d_grad_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the int32 plane-local indices",
+    AG_REQUIRE(ggx && ggy && (argmax || taps), AG_ERR_INVALID_DIMS, "max_pool2d_grad_grad: null pointer");
+    AG_REQUIRE(!taps || size <= kMaxTapSize, AG_ERR_INVALID_DIMS,
+               "max_pool2d_grad_grad: a tap byte addresses windows of up to %d x %d (got %d)", kMaxTapSize, kMaxTapSize, size);
+    AG_REQUIRE(taps || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
+               "max_pool2d_grad_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the tap bytes",
                (long long)B * C * H * W);
     const long long plane_y = (long long)g.OH * g.OW, total_y = plane_y * B * C;
     if (total_y == 0) return AG_OK;
     long long blocks = (total_y + 255) / 256;
     if (blocks > 262144) blocks = 262144;
-    if (idx_local)
+    if (taps)
         hipLaunchKernelGGL(maxpool_gradgrad_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), ggx, argmax, idx_local, ggy, (long long)H * W, plane_y, total_y);
+                           as_stream(stream), ggx, argmax, taps, ggy, g, (long long)H * W, plane_y, total_y);
     else
         hipLaunchKernelGGL(maxpool_gradgrad_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
-                           as_stream(stream), ggx, argmax, idx_local, ggy, (long long)H * W, plane_y, total_y);
+                           as_stream(stream), ggx, argmax, taps, ggy, g, (long long)H * W, plane_y, total_y);
     return check_launch("max_pool2d_grad_grad");
 }

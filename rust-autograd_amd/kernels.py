@@ -263,35 +263,35 @@ def conv2d_transpose_filter_grad(x, gy, w_shape, pad, stride, dilation=1):
 
 # ------------------------------------------------------------------------------------------ pooling
 def max_pool2d(x, pool_size, pad, stride):
-    """MaxPool2D::compute: returns (y, argmax as f32, exact plane-local int32 index)."""
+    """MaxPool2D::compute: returns (y, argmax as f32, tap bytes = exact selection inside each window)."""
     x = _f32(x, "max_pool2d")
     B, Cc, H, W = x.shape
     L = capi.lib()
     OH, OW = L.ag_pool_out_size(H, pool_size, pad, stride), L.ag_pool_out_size(W, pool_size, pad, stride)
     y = _empty((B, Cc, max(OH, 0), max(OW, 0)), x)
     am = torch.empty_like(y)
-    il = torch.empty(y.shape, dtype=torch.int32, device=x.device)
+    il = torch.empty(y.shape, dtype=torch.uint8, device=x.device)
     check(L.ag_maxpool2d_fwd_f32(_stream(), _ptr(x), _ptr(y), _ptr(am), _ptr(il), B, Cc, H, W, pool_size, pad,
                                  stride))
     return y, am, il
 
 
-def max_pool2d_grad(gy, argmax, idx_local, x_shape, pool_size, pad, stride):
+def max_pool2d_grad(gy, argmax, taps, x_shape, pool_size, pad, stride):
     gy = _f32(gy, "max_pool2d_grad")
     B, Cc, H, W = x_shape
     gx = _empty(x_shape, gy)
-    check(capi.lib().ag_maxpool2d_bwd_f32(_stream(), _ptr(gy), _ptr(argmax), _ptr(idx_local), _ptr(gx), B, Cc, H,
+    check(capi.lib().ag_maxpool2d_bwd_f32(_stream(), _ptr(gy), _ptr(argmax), _ptr(taps), _ptr(gx), B, Cc, H,
                                           W, pool_size, pad, stride))
     return gx
 
 
-def max_pool2d_grad_grad(ggx, argmax, idx_local, pool_size, pad, stride):
+def max_pool2d_grad_grad(ggx, argmax, taps, pool_size, pad, stride):
     ggx = _f32(ggx, "max_pool2d_grad_grad")
     B, Cc, H, W = ggx.shape
     L = capi.lib()
     OH, OW = L.ag_pool_out_size(H, pool_size, pad, stride), L.ag_pool_out_size(W, pool_size, pad, stride)
     ggy = _empty((B, Cc, OH, OW), ggx)
-    check(L.ag_maxpool2d_gradgrad_f32(_stream(), _ptr(ggx), _ptr(argmax), _ptr(idx_local), _ptr(ggy), B, Cc, H, W,
+    check(L.ag_maxpool2d_gradgrad_f32(_stream(), _ptr(ggx), _ptr(argmax), _ptr(taps), _ptr(ggy), B, Cc, H, W,
                                       pool_size, pad, stride))
     return ggy
 

@@ -794,14 +794,18 @@ def test_max_pool_reference_vector(K, golden):
     y, am, il = K.max_pool2d(dev(x), g["size"], g["pad"], g["stride"])
     assert host(y).reshape(-1).tolist() == [float(v) for v in g["expected_output"]]
     assert host(am).reshape(-1).tolist() == [float(v) for v in g["expected_argmax"]]
-    assert host(il).reshape(-1).tolist() == g["expected_argmax"]
+    # the same selection as one tap byte per window: pixel 3 = (1,0) is tap 1*2+0 of window (0,0), ...
+    want_taps = [(i // g["xw"] - o // 2) * g["size"] + (i % g["xw"] - o % 2) for o, i in enumerate(g["expected_argmax"])]
+    assert host(il).reshape(-1).tolist() == want_taps
 
 
 POOL_CASES = [(2, 3, 6, 6, 2, 2), (2, 3, 7, 9, 3, 2), (1, 2, 8, 8, 3, 1), (3, 32, 28, 28, 2, 2),
               (2, 16, 56, 56, 3, 2), (1, 1, 5, 7, 2, 3), (1, 3, 33, 65, 3, 2),
               # stride-2 register kernels: one lane group per plane, 4 .. 64 lanes per row, chunked rows
               (2, 3, 8, 4, 2, 2), (1, 2, 64, 64, 3, 2), (1, 2, 30, 128, 3, 2), (1, 1, 9, 256, 2, 2),
-              (5, 3, 40, 12, 3, 2), (1, 1, 4, 4, 3, 2), (7, 1, 5, 8, 3, 2), (3, 2, 27, 20, 2, 2)]
+              (5, 3, 40, 12, 3, 2), (1, 1, 4, 4, 3, 2), (7, 1, 5, 8, 3, 2), (3, 2, 27, 20, 2, 2),
+              # other windows: the tap byte through the staged and the direct kernels
+              (2, 2, 17, 19, 5, 3), (1, 2, 20, 24, 4, 4), (1, 1, 3, 9000, 3, 2), (1, 2, 16, 16, 15, 1)]
 
 
 @pytest.mark.parametrize("case", POOL_CASES)
@@ -814,13 +818,13 @@ def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
     oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, stride)
     assert np.array_equal(host(y), oy)
     assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32)), "argmax must be bit-exact"
-    assert np.array_equal(host(il), oil)
+    assert np.array_equal(host(il), orc.maxpool2d_taps(oil, W, size, stride))
     gy = rng.standard_normal(oy.shape).astype(np.float32)
     ogx, skipped = orc.maxpool2d_bwd(gy, oam, x.shape)
     assert skipped == 0
     say("max_pool bwd (f32 argmax)", case)
     gx_f = host(K.max_pool2d_grad(dev(gy), am, None, x.shape, size, 0, stride))
-    say("max_pool bwd (int32 index)", case)
+    say("max_pool bwd (tap bytes)", case)
     gx_i = host(K.max_pool2d_grad(dev(gy), am, il, x.shape, size, 0, stride))
     assert np.array_equal(gx_f.view(np.uint32), ogx.view(np.uint32))
     assert np.array_equal(gx_i.view(np.uint32), ogx.view(np.uint32))
@@ -829,6 +833,27 @@ def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
     for idx in (None, il):
         ggy = host(K.max_pool2d_grad_grad(dev(ggx), am, idx, size, 0, stride))
         assert np.array_equal(ggy, orc.maxpool2d_gradgrad(ggx, oam, oy.shape))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 1000])
+def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows):
+    """The stride-2 backward walks chunks of output rows; whatever their length (one row, odd
+    lengths, the whole plane) the result is the reference's, bit for bit."""
+    L = K.capi.lib()
+    for (B, C, H, W, size) in [(2, 3, 56, 56, 3), (1, 2, 28, 28, 2), (1, 2, 11, 8, 3), (3, 1, 9, 12, 2)]:
+        x = rng.integers(0, 4, (B, C, H, W)).astype(np.float32)   # many ties
+        y, am, taps = K.max_pool2d(dev(x), size, 0, 2)
+        oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, 2)
+        gy = rng.standard_normal(oy.shape).astype(np.float32)
+        ogx, _ = orc.maxpool2d_bwd(gy, oam, x.shape)
+        say("max_pool bwd chunk rows", rows, (B, C, H, W, size))
+        L.ag_test_pool_chunk_rows(rows)
+        try:
+            got = [host(K.max_pool2d_grad(dev(gy), am, idx, x.shape, size, 0, 2)) for idx in (None, taps)]
+        finally:
+            L.ag_test_pool_chunk_rows(0)
+        for gx in got:
+            assert np.array_equal(gx.view(np.uint32), ogx.view(np.uint32))
 
 
 @pytest.mark.parametrize("case", [(2, 4, 56, 56, 3, 2), (2, 4, 28, 28, 2, 2), (1, 3, 21, 16, 3, 2)])
@@ -840,7 +865,7 @@ def test_max_pool_many_ties(K, orc, rng, case):
     say("max_pool ties", case)
     y, am, il = K.max_pool2d(dev(x), size, 0, stride)
     oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, stride)
-    assert np.array_equal(host(y), oy) and np.array_equal(host(il), oil)
+    assert np.array_equal(host(y), oy) and np.array_equal(host(il), orc.maxpool2d_taps(oil, W, size, stride))
     assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32))
     gy = rng.standard_normal(oy.shape).astype(np.float32)
     ogx, _ = orc.maxpool2d_bwd(gy, oam, x.shape)
@@ -857,15 +882,23 @@ def test_max_pool_nan_window_and_pad_error(K, orc):
     say("max_pool NaN")
     y, am, il = K.max_pool2d(dev(x), 2, 0, 2)
     oy, oam, oil = orc.maxpool2d_fwd(x, 2, 0, 2)
-    assert np.array_equal(host(y), oy) and np.array_equal(host(am), oam) and np.array_equal(host(il), oil)
+    assert np.array_equal(host(y), oy) and np.array_equal(host(am), oam)
+    assert np.array_equal(host(il), orc.maxpool2d_taps(oil, 4, 2, 2))
+    assert (host(il)[0] == 255).all() and host(il)[1, 0, 0, 0] == 255
     assert (oil[0] == -1).all() and oil[1, 0, 0, 0] == -1 and (oil[1, 1] >= 0).all()
     with pytest.raises(K.capi.InvalidDims, match="pad must be 0"):
         K.max_pool2d(dev(x), 2, 1, 2)
 
 
+def test_max_pool_tap_bytes_need_a_window_of_at_most_15(K):
+    x = torch.zeros(1, 1, 20, 20, device="cuda")
+    with pytest.raises(K.capi.InvalidDims, match="tap byte"):
+        K.max_pool2d(x, 16, 0, 1)
+
+
 def test_max_pool_above_2_pow_24_elements(K, orc, rng):
     """33.5 M elements: the f32 argmax is the rounded offset (bit-exact with the reference's
-    encoding), the int32 plane index is exact, the backward refuses the f32 indices and is
+    encoding), the tap bytes are exact, the backward refuses the f32 indices and is
     bit-exact with the exact-index oracle."""
     B, C, H, W = 2, 64, 512, 512
     x = rng.standard_normal((B, C, H, W)).astype(np.float32)
@@ -874,7 +907,7 @@ def test_max_pool_above_2_pow_24_elements(K, orc, rng):
     oy, oam, oil = orc.maxpool2d_fwd(x, 2, 0, 2)
     assert np.array_equal(host(y), oy)
     assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32))
-    assert np.array_equal(host(il), oil)
+    assert np.array_equal(host(il), orc.maxpool2d_taps(oil, W, 2, 2))
     gy = rng.standard_normal(oy.shape).astype(np.float32)
     with pytest.raises(K.capi.InvalidDims, match="2\\^24"):
         K.max_pool2d_grad(dev(gy), am, None, x.shape, 2, 0, 2)
