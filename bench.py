@@ -208,8 +208,8 @@ def main():
     L = capi.lib()
     st, ptr, chk = Kn._stream, Kn._ptr, capi.check
     T = Timer(torch)
-    fgeom = (Bn, C, H, W, K, KH, KH, PAD)                # forward / filter gradient
-    igeom = (Bn, K, OH, OH, C, KH, KH, PAD, H, W)        # input gradient
+    fgeom = (Bn, C, H, W, K, KH, KH, PAD, STRIDE, 1)                # forward / filter gradient
+    igeom = (Bn, K, OH, OH, C, KH, KH, PAD, STRIDE, 1, H, W)        # input gradient
     n_xpad, n_gypad = L.ag_conv2d_nocols_scratch_floats(*fgeom), L.ag_conv_input_grad_scratch_floats(*igeom)
     assert n_xpad > 0 and n_gypad > 0, "the headline geometry takes the column-free path"
     xpad = torch.empty(n_xpad, device=dev)

@@ -148,56 +148,64 @@ ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const f
                                     float *gcols, int B, int ych, int yh, int yw, int xch, int kh,
                                     int kw, int pad, int stride, int dilation, int xh, int xw);
 
-/* The two stages of the stride-1, dilation-1 input gradient that ag_conv2d_transpose_f32 runs
- * when the geometry allows it (no counterpart in the reference, which always materialises the
- * columns): `prepare` writes a zero-bordered copy of gy and the filter in tap-major order into
- * `scratch`; `gemm` accumulates gx over the kh*kw taps in one contraction that reads them.
- * ag_conv_input_grad_scratch_floats returns the scratch size in floats, or 0 when the geometry
- * is not supported (then use ag_conv2d_transpose_f32). */
+/* The two stages of the column-free input gradient that ag_conv2d_transpose_f32 runs when the
+ * geometry allows it (no counterpart in the reference, which always materialises the columns):
+ * `prepare` writes a zero-bordered copy of gy and the filter in tap-major order into `scratch`;
+ * `gemm` accumulates gx over the filter taps in implicit GEMMs that read them -- one for stride 1;
+ * for stride 2 one per parity of the pixel position, whose results (kept in `scratch`) a copy
+ * kernel interleaves into gx.  dilation must be 1.  ag_conv_input_grad_scratch_floats returns the
+ * scratch size in floats, or 0 when the geometry is not supported (then use
+ * ag_conv2d_transpose_f32). */
 size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int yw, int xch, int kh, int kw,
-                                         int pad, int xh, int xw);
+                                         int pad, int stride, int dilation, int xh, int xw);
 ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w,
                                            float *scratch, int B, int ych, int yh, int yw, int xch,
-                                           int kh, int kw, int pad, int xh, int xw);
-ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch, float *gx, int B,
+                                           int kh, int kw, int pad, int stride, int dilation, int xh,
+                                           int xw);
+ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, float *gx, int B,
                                         int ych, int yh, int yw, int xch, int kh, int kw, int pad,
-                                        int xh, int xw);
+                                        int stride, int dilation, int xh, int xw);
 
-/* Column-free stride-1, dilation-1 convolution: forward and filter gradient without the im2col
- * columns.  No counterpart in the reference, which always materialises them (Conv2D::compute ->
- * fast_im2col_gemm_fused_kernel, conv2d.rs:25-112; conv2d_filter_grad_impl, conv2d.rs:631-734); the
- * results are those of ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32 within the floating-point
- * tolerance (other summation order).  The forward writes a zero-bordered copy of x into `xpad`
- * (ag_conv2d_nocols_scratch_floats() floats; 0 = geometry not supported: square window, C a multiple
- * of 32, planes of at least 128 or 256 padded elements) and runs one implicit GEMM over the filter
- * taps.  The filter gradient contracts that copy with the zero-bordered upstream gradient that
- * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images in
- * splits that need the workspace; "same" convolutions only (2*pad == kh-1 == kw-1, K a multiple of
- * 32), so that both copies share one padded plane shape.  The contraction runs a few elements past
- * a plane, but only over zeros of both operands (the planes are sized for that), so a NaN or
- * infinity in one channel of x reaches the gradients of that channel only; within the channel it
- * can reach filter taps that the reference's columns would not pair it with (0 * NaN at a border
- * position). */
-size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad);
+/* Column-free convolution (stride 1 or 2, dilation 1): forward and filter gradient without the
+ * im2col columns.  No counterpart in the reference, which always materialises them (Conv2D::compute
+ * -> fast_im2col_gemm_fused_kernel, conv2d.rs:25-112; conv2d_filter_grad_impl, conv2d.rs:631-734);
+ * the results are those of ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32 within the floating-point
+ * tolerance (other summation order).  The forward writes a rearranged copy of x into `xpad`
+ * (ag_conv2d_nocols_scratch_floats() floats; 0 = geometry not supported: C a multiple of 32, planes
+ * of at least 128 padded elements, ...) -- the zero-bordered input for stride 1, its four phase
+ * planes x'[2i+a][2j+b] for stride 2 -- and runs one implicit GEMM over the filter taps.  The filter
+ * gradient contracts that copy with the zero-bordered upstream gradient that
+ * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images
+ * in splits that need the workspace; for stride 1 "same" convolutions only (2*pad == kh-1 == kw-1,
+ * K a multiple of 32), so that both copies share one padded plane shape.  The contraction runs a
+ * few elements past a plane, but only over zeros of both operands (the planes are sized for that),
+ * so a NaN or infinity in one channel of x reaches the gradients of that channel only; within the
+ * channel it can reach filter taps that the reference's columns would not pair it with (0 * NaN at
+ * a border position). */
+size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad,
+                                       int stride, int dilation);
 ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y,
                                      float *xpad, int B, int C, int H, int W, int K, int kh, int kw,
-                                     int pad);
-/* The two stages of ag_conv2d_fwd_nocols_f32 (bordered copy of x and tap-major filter; the GEMM). */
+                                     int pad, int stride, int dilation);
+/* The two stages of ag_conv2d_fwd_nocols_f32 (rearranged copy of x and tap-major filter; the GEMM). */
 ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, const float *w, float *xpad,
-                                         int B, int C, int H, int W, int K, int kh, int kw, int pad);
+                                         int B, int C, int H, int W, int K, int kh, int kw, int pad,
+                                         int stride, int dilation);
 ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C,
-                                      int H, int W, int K, int kh, int kw, int pad);
-/* The forward GEMM over an existing bordered copy with another filter: what Conv2DWithCols
+                                      int H, int W, int K, int kh, int kw, int pad, int stride,
+                                      int dilation);
+/* The forward GEMM over an existing rearranged copy with another filter: what Conv2DWithCols
  * (conv2d.rs:589-629) becomes when its "columns" input is such a copy.  wf: K*C*kh*kw floats. */
 ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, const float *xpad, const float *w,
                                              float *wf, float *y, int B, int C, int H, int W, int K,
-                                             int kh, int kw, int pad);
+                                             int kh, int kw, int pad, int stride, int dilation);
 /* 0 = geometry not supported by the column-free filter gradient. */
 size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw,
-                                                  int pad);
+                                                  int pad, int stride, int dilation);
 ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, const float *xpad, const float *gypad,
                                              float *gw, int B, int C, int H, int W, int K, int kh,
-                                             int kw, int pad, void *ws, size_t ws_bytes);
+                                             int kw, int pad, int stride, int dilation, void *ws,
+                                             size_t ws_bytes);
 
 /* Replaces Conv2DTransposeFilterGrad::compute -> conv2d_transpose_filter_grad_impl
  * (conv2d_transpose.rs:433-451, 303-431).  x [B,ych,yh,yw] (input of the transposed conv),

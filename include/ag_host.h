@@ -61,6 +61,9 @@ int agh_variable(agh_ctx *ctx, int var_id);
 int agh_placeholder(agh_ctx *ctx, const char *name, const int64_t *shape, int rank); /* -1 = unknown extent */
 int agh_scalar(agh_ctx *ctx, float value);
 int agh_conv2d(agh_ctx *ctx, int x, int w, int pad, int stride, int dilation);           /* conv2d / dilated_conv2d */
+/* the same operator made to materialise the im2col columns as its second output, like the reference,
+ * whatever the geometry (the default takes the column-free path for large stride-1 / stride-2 cases) */
+int agh_conv2d_with_columns(agh_ctx *ctx, int x, int w, int pad, int stride, int dilation);
 int agh_conv2d_transpose(agh_ctx *ctx, int x, int w, int pad, int stride, int dilation); /* (dilated_)conv2d_transpose */
 int agh_max_pool2d(agh_ctx *ctx, int x, int pool_size, int pad, int stride);
 int agh_matmul(agh_ctx *ctx, int a, int b);

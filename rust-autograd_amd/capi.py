@@ -92,16 +92,16 @@ PROTOTYPES = {
     "ag_fill_f32": (c_i, [c_p, c_p, c_f, c_sz]),
     "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
-    "ag_conv_input_grad_scratch_floats": (C.c_size_t, [c_i] * 10),
-    "ag_conv_input_grad_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 10),
-    "ag_conv_input_grad_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 10),
-    "ag_conv2d_nocols_scratch_floats": (c_sz, [c_i] * 8),
-    "ag_conv2d_fwd_nocols_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
-    "ag_conv2d_nocols_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8),
-    "ag_conv2d_nocols_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 8),
-    "ag_conv2d_nocols_with_filter_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 8),
-    "ag_conv2d_filter_grad_nocols_f32_workspace": (c_sz, [c_i] * 8),
-    "ag_conv2d_filter_grad_nocols_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 8 + [c_p, c_sz]),
+    "ag_conv_input_grad_scratch_floats": (C.c_size_t, [c_i] * 12),
+    "ag_conv_input_grad_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 12),
+    "ag_conv_input_grad_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 12),
+    "ag_conv2d_nocols_scratch_floats": (c_sz, [c_i] * 10),
+    "ag_conv2d_fwd_nocols_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 10),
+    "ag_conv2d_nocols_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 10),
+    "ag_conv2d_nocols_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 10),
+    "ag_conv2d_nocols_with_filter_f32": (c_i, [c_p, c_p, c_p, c_p, c_p] + [c_i] * 10),
+    "ag_conv2d_filter_grad_nocols_f32_workspace": (c_sz, [c_i] * 10),
+    "ag_conv2d_filter_grad_nocols_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 10 + [c_p, c_sz]),
     "ag_matmul_f32_static_scratch_bytes": (c_sz, []),
     "ag_matmul_f32_noalloc": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_p, c_i, c_p, c_i, c_p, c_i]),
 }

@@ -3,7 +3,7 @@
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 out="$here/../libag_hip.so"
-srcs=(common.hip im2col.hip gemm.hip gemm_dl.hip conv.hip pool.hip reduce.hip adam.hip elementwise.hip)
+srcs=(common.hip im2col.hip gemm.hip gemm_dl.hip conv.hip conv_s2.hip pool.hip reduce.hip adam.hip elementwise.hip)
 flags=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -fvisibility=hidden
        -Xclang -target-feature -Xclang -packed-fp32-ops
        -I"$here/../../include" -I"$here" -Wall -Wno-unused-function "$@")

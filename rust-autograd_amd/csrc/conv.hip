@@ -4,6 +4,7 @@
 // task per image, and one split-accumulation GEMM instead of an image-sequential beta=1 loop.
 #include "ag_internal.h"
 #include "ag_test_hooks.h"
+#include "conv_shared.h"
 #include "gemm_shared.h"
 
 using namespace ag;
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__res
 }
 
 // Launches the bordered copy of `planes` planes per image.
-static void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp, int Wp,
+void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp, int Wp,
                               int top, int left)
 {
     const long long plane_quads = (long long)Hp * Wp / 4, quads_img = plane_quads * planes;
@@ -387,13 +388,24 @@ static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
 
 }  // namespace ag
 
-// ---- column-free stride-1 convolution: forward and filter gradient ------------------------------
-// No counterpart of these three in the reference, which always materialises the columns
-// (conv2d.rs:25-112, 631-734); they compute the same y and gw from a zero-bordered copy of x.
-// `xpad`: ag_conv2d_nocols_scratch_floats() floats, written by the forward and read by the filter
-// gradient.  0 floats = geometry not supported (use ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32).
-extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad)
+// ---- column-free convolution: forward and filter gradient ---------------------------------------
+// No counterpart of these in the reference, which always materialises the columns
+// (conv2d.rs:25-112, 631-734); they compute the same y and gw from a rearranged copy of x: the
+// zero-bordered input for stride 1, its four phase planes for stride 2 (conv_s2.hip).  dilation must
+// be 1.  `xpad`: ag_conv2d_nocols_scratch_floats() floats, written by the forward and read by the
+// filter gradient.  0 floats = geometry not supported (use ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32).
+namespace ag {
+static bool nocols_mode(int stride, int dilation) { return dilation == 1 && (stride == 1 || stride == 2); }
+}  // namespace ag
+
+extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad, int stride,
+                                                  int dilation)
 {
+    if (!nocols_mode(stride, dilation)) return 0;
+    if (stride == 2) {
+        S2Geom g2;
+        return s2_geom(B, C, H, W, K, kh, kw, pad, &g2) ? (size_t)(g2.xph_floats + g2.wf_floats) : 0;
+    }
     FusedGeom g;
     if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g)) return 0;
     return (size_t)(kFwdLeadFloats + g.gyp_floats + g.wr_floats);
@@ -401,13 +413,21 @@ extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, in
 
 // The two stages of the forward, for callers that time or schedule them separately.
 extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, const float *w, float *xpad, int B,
-                                                    int C, int H, int W, int K, int kh, int kw, int pad)
+                                                    int C, int H, int W, int K, int kh, int kw, int pad, int stride, int dilation)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv2d (column-free): stride %d / dilation %d not supported",
+               stride, dilation);
+    AG_REQUIRE(x && w && xpad, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    hipStream_t st = as_stream(stream);
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, C, H, W, K, kh, kw, pad, &g2) && aligned16(xpad), AG_ERR_INVALID_DIMS,
+                   "conv2d (column-free): geometry not supported");
+        return s2_fwd_prepare(st, x, w, xpad, g2, B, C, H, W, K, kh, kw, pad);
+    }
     FusedGeom g;
     AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
-    AG_REQUIRE(x && w && xpad, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
-    hipStream_t st = as_stream(stream);
     float *xp = xpad + kFwdLeadFloats, *wf = xp + g.gyp_floats;
     const long long quads = (long long)B * C * g.Hp * g.Wp / 4;
     launch_pad_border(st, x, xp, B, C, H, W, g.Hp, g.Wp, pad, pad);
@@ -419,34 +439,53 @@ extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const fl
 }
 
 extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C, int H, int W,
-                                                 int K, int kh, int kw, int pad)
+                                                 int K, int kh, int kw, int pad, int stride, int dilation)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv2d (column-free): stride %d / dilation %d not supported",
+               stride, dilation);
+    AG_REQUIRE(xpad && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, C, H, W, K, kh, kw, pad, &g2) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
+                   "conv2d (column-free): geometry not supported");
+        return s2_fwd_gemm(as_stream(stream), xpad, xpad + g2.xph_floats, y, g2, B, C, K, kh, kw);
+    }
     FusedGeom g;
     AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
-    AG_REQUIRE(xpad && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
     const float *xp = xpad + kFwdLeadFloats;
     return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1,
                                 kh, kw, g.Hp, g.Wp);
 }
 
 extern "C" ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y, float *xpad,
-                                                int B, int C, int H, int W, int K, int kh, int kw, int pad)
+                                                int B, int C, int H, int W, int K, int kh, int kw, int pad, int stride,
+                                                int dilation)
 {
-    if (ag_status_t s = ag_conv2d_nocols_prepare_f32(stream, x, w, xpad, B, C, H, W, K, kh, kw, pad)) return s;
-    return ag_conv2d_nocols_gemm_f32(stream, xpad, y, B, C, H, W, K, kh, kw, pad);
+    if (ag_status_t s = ag_conv2d_nocols_prepare_f32(stream, x, w, xpad, B, C, H, W, K, kh, kw, pad, stride, dilation)) return s;
+    return ag_conv2d_nocols_gemm_f32(stream, xpad, y, B, C, H, W, K, kh, kw, pad, stride, dilation);
 }
 
-// The forward GEMM over an existing bordered copy with another filter (Conv2DWithCols, conv2d.rs:
-// 589-629, when the "columns" it is given are a bordered input): `wf` receives K*C*kh*kw floats.
+// The forward GEMM over an existing rearranged copy with another filter (Conv2DWithCols, conv2d.rs:
+// 589-629, when the "columns" it is given are such a copy): `wf` receives K*C*kh*kw floats.
 extern "C" ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, const float *xpad, const float *w, float *wf,
-                                                        float *y, int B, int C, int H, int W, int K, int kh, int kw, int pad)
+                                                        float *y, int B, int C, int H, int W, int K, int kh, int kw, int pad,
+                                                        int stride, int dilation)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv2d (column-free): stride %d / dilation %d not supported",
+               stride, dilation);
+    AG_REQUIRE(xpad && w && wf && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
+    hipStream_t st = as_stream(stream);
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, C, H, W, K, kh, kw, pad, &g2) && aligned16(xpad) && aligned16(y) && aligned16(wf), AG_ERR_INVALID_DIMS,
+                   "conv2d (column-free): geometry not supported");
+        if (ag_status_t s = s2_fwd_filter(st, w, wf, g2, C, K, kh, kw)) return s;
+        return s2_fwd_gemm(st, xpad, wf, y, g2, B, C, K, kh, kw);
+    }
     FusedGeom g;
     AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y) && aligned16(wf),
                AG_ERR_INVALID_DIMS, "conv2d (column-free): geometry not supported");
-    AG_REQUIRE(xpad && w && wf && y, AG_ERR_INVALID_DIMS, "conv2d (column-free): null pointer");
-    hipStream_t st = as_stream(stream);
     hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
                        kh * kw);
     if (ag_status_t s = check_launch("conv2d")) return s;
@@ -454,11 +493,17 @@ extern "C" ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, cons
                                 g.Hp, g.Wp);
 }
 
-// gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the first
-// B*K*Hp*Wp floats of its scratch); the geometry must be a "same" convolution (2*pad == k-1) so
-// that x and gy share one padded plane shape.
-extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw, int pad)
+// gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the start
+// of its scratch).  Stride 1: the geometry must be a "same" convolution (2*pad == k-1) so that x
+// and gy share one padded plane shape.
+extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw, int pad,
+                                                             int stride, int dilation)
 {
+    if (!nocols_mode(stride, dilation)) return 0;
+    if (stride == 2) {
+        S2Geom g2;
+        return s2_geom(B, C, H, W, K, kh, kw, pad, &g2) ? s2_filter_grad_workspace(g2, B, C, K, kh, kw) : 0;
+    }
     FusedGeom g, gg;
     const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
     if (2 * pad != kh - 1 || 2 * pad != kw - 1 || K % 4 != 0 || !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) ||
@@ -470,9 +515,18 @@ extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H
 }
 
 extern "C" ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, const float *xpad, const float *gypad, float *gw,
-                                                        int B, int C, int H, int W, int K, int kh, int kw, int pad, void *ws,
-                                                        size_t ws_bytes)
+                                                        int B, int C, int H, int W, int K, int kh, int kw, int pad, int stride,
+                                                        int dilation, void *ws, size_t ws_bytes)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS,
+               "conv2d_filter_grad (column-free): stride %d / dilation %d not supported", stride, dilation);
+    AG_REQUIRE(gw, AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): null output");
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, C, H, W, K, kh, kw, pad, &g2) && aligned16(xpad) && aligned16(gypad), AG_ERR_INVALID_DIMS,
+                   "conv2d_filter_grad (column-free): geometry not supported");
+        return s2_filter_grad(as_stream(stream), xpad, gypad, gw, g2, B, C, K, kh, kw, ws, ws_bytes);
+    }
     FusedGeom g, gg;
     const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
     AG_REQUIRE(2 * pad == kh - 1 && 2 * pad == kw - 1 && K % 4 == 0 && C >= 1 &&
@@ -482,7 +536,6 @@ extern "C" ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, cons
     const int kq = filter_grad_positions(g, OH, pad);
     AG_REQUIRE(kq > 0 && (long long)C * g.Hp * g.Wp < (1LL << 30), AG_ERR_INVALID_DIMS,
                "conv2d_filter_grad (column-free): plane too small or too many channels");
-    AG_REQUIRE(gw, AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): null output");
     return gemm_conv_filter_grad(as_stream(stream), gypad, xpad + kFwdLeadFloats, gw, ws, ws_bytes, B, K, C, kh, kw, pad, g.Hp,
                                  g.Wp, kq);
 }
@@ -514,6 +567,14 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
         if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad)) return s;
         return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
                                     fg.Wp);
+    }
+    // Stride 2: four parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
+    // is large enough to serve as their scratch.
+    S2Geom g2;
+    if (stride == 2 && dilation == 1 && g_fused_input_grad && s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh &&
+        g2.OW == yw && g2.gyp_floats + g2.wf_floats + g2.gxp_floats <= (long long)B * M * P && aligned16(gcols) && aligned16(gx)) {
+        if (ag_status_t s = s2_igrad_prepare(as_stream(stream), gy, w, gcols, g2, B, xch, ych, kh, kw, pad)) return s;
+        return s2_igrad_gemm(as_stream(stream), gcols, gx, g2, B, xch, ych, xh, xw);
     }
     // gcols_b[M x P] = w^T[M x ych] * gy_b[ych x P]               conv2d_transpose.rs:114-116,167-182
     if (ag_status_t s = ag_gemm_f32(stream, 1, 0, (int)M, (int)P, ych, 1.f, w, (int)M, 0, gy, (int)P,
@@ -558,25 +619,50 @@ extern "C" void ag_test_conv_fused_input_grad(int on) { ag::g_fused_input_grad =
 // them separately.  `scratch` holds ag_conv_input_grad_scratch_floats() floats (0 = this
 // geometry takes the GEMM + col2im path and the staged entry points refuse it).
 extern "C" size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad,
-                                                    int xh, int xw)
+                                                    int stride, int dilation, int xh, int xw)
 {
+    if (!nocols_mode(stride, dilation)) return 0;
+    if (stride == 2) {
+        S2Geom g2;
+        if (!s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) || g2.OH != yh || g2.OW != yw) return 0;
+        return (size_t)(g2.gyp_floats + g2.wf_floats + g2.gxp_floats);
+    }
     FusedGeom g;
     return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) ? (size_t)(g.gyp_floats + g.wr_floats) : 0;
 }
 
 extern "C" ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w, float *scratch,
                                                       int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad,
-                                                      int xh, int xw)
+                                                      int stride, int dilation, int xh, int xw)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv_input_grad_prepare: stride %d / dilation %d not supported",
+               stride, dilation);
+    AG_REQUIRE(gy && w && scratch, AG_ERR_INVALID_DIMS, "conv_input_grad_prepare: null pointer");
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh && g2.OW == yw && aligned16(scratch),
+                   AG_ERR_INVALID_DIMS, "conv_input_grad_prepare: geometry not supported by the column-free path");
+        return s2_igrad_prepare(as_stream(stream), gy, w, scratch, g2, B, xch, ych, kh, kw, pad);
+    }
     FusedGeom g;
     AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch), AG_ERR_INVALID_DIMS,
                "conv_input_grad_prepare: geometry not supported by the column-free path");
     return fused_prepare(as_stream(stream), gy, w, scratch, g, B, ych, yh, yw, xch, kh, kw, pad);
 }
 
-extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, const float *scratch, float *gx, int B, int ych,
-                                                   int yh, int yw, int xch, int kh, int kw, int pad, int xh, int xw)
+extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, float *gx, int B, int ych,
+                                                   int yh, int yw, int xch, int kh, int kw, int pad, int stride, int dilation,
+                                                   int xh, int xw)
 {
+    AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: stride %d / dilation %d not supported",
+               stride, dilation);
+    AG_REQUIRE(scratch && gx, AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: null pointer");
+    if (stride == 2) {
+        S2Geom g2;
+        AG_REQUIRE(s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh && g2.OW == yw && aligned16(scratch) && aligned16(gx),
+                   AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: geometry not supported by the column-free path");
+        return s2_igrad_gemm(as_stream(stream), scratch, gx, g2, B, xch, ych, xh, xw);
+    }
     FusedGeom g;
     AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch) && aligned16(gx),
                AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: geometry not supported by the column-free path");

@@ -1,0 +1,276 @@
+// Column-free stride-2 convolution: forward, filter gradient and input gradient as implicit GEMMs.
+// No counterpart in the reference, which materialises the im2col columns for every stride
+// (conv2d.rs:25-112, 631-734; conv2d_transpose.rs:89-247); the index arithmetic restated here is
+// that of conv_ops/mod.rs:89-112 (x index = o*stride - pad + k) and its adjoint (:198-219).
+//
+// A stride-2 window reads x'[2*oy + ky][2*ox + kx] (x' = x with a zero border of `pad`).  Splitting
+// x' into its four PHASE planes x'_{a,b}[i][j] = x'[2i+a][2j+b] turns that into the unit-stride read
+// x'_{ky&1,kx&1}[oy + (ky>>1)][ox + (kx>>1)], so
+//   forward          y  = sum over taps and channels of w * phase plane shifted by (ky>>1, kx>>1)  -- one GEMM;
+//   filter gradient  gw[k][c][ky][kx] = sum over images and positions q of gy'[k][q] * x'_{..}[c][q + shift]  -- one GEMM;
+//   input gradient   the pixels of one parity (iy&1, ix&1) of gx only meet the taps with ky = iy + pad and
+//                    kx = ix + pad (mod 2): four unit-stride input-gradient GEMMs, one per parity, over ONE
+//                    zero-bordered copy of gy; their results (parity-planar) are interleaved into gx by a copy kernel.
+// All planes share one row pitch Wc, so the bordered gy serves the filter gradient as well.
+#include "ag_internal.h"
+#include "conv_shared.h"
+#include "gemm_shared.h"
+
+namespace ag {
+
+static long long round_up32(long long v) { return (v + 31) / 32 * 32; }
+
+bool s2_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, S2Geom *g)
+{
+    if (B < 1 || C < 1 || K < 1 || H < 1 || W < 1 || kh < 2 || kw < 2 || pad < 0 || pad > kh - 1 || pad > kw - 1) return false;
+    if (C % 32 != 0 || K % 32 != 0) return false;
+    if (H + 2 * pad < kh || W + 2 * pad < kw) return false;
+    g->OH = (H + 2 * pad - kh) / 2 + 1;
+    g->OW = (W + 2 * pad - kw) / 2 + 1;
+    // parities of the input gradient: which taps they meet and how far they reach into gy
+    int T = 0, L = 0, reach_h = 0, reach_w = 0;
+    for (int a = 0; a < 2; ++a) {
+        const int alpha = (a + pad) & 1;
+        g->kh_a[a] = (kh - alpha + 1) / 2;
+        g->kw_b[a] = (kw - alpha + 1) / 2;
+        g->d_a[a] = (a + pad) >> 1;
+        g->H_a[a] = (H - a + 1) / 2;
+        g->W_b[a] = (W - a + 1) / 2;
+        T = T > g->kh_a[a] - 1 - g->d_a[a] ? T : g->kh_a[a] - 1 - g->d_a[a];
+        L = L > g->kw_b[a] - 1 - g->d_a[a] ? L : g->kw_b[a] - 1 - g->d_a[a];
+        L = L > g->d_a[a] ? L : g->d_a[a];  // a read past the end of a row lands in the next row's left border
+        reach_h = reach_h > g->H_a[a] + g->d_a[a] ? reach_h : g->H_a[a] + g->d_a[a];
+        reach_w = reach_w > g->W_b[a] + g->d_a[a] ? reach_w : g->W_b[a] + g->d_a[a];
+    }
+    g->T = T;
+    g->L = L;
+    // common row pitch: wide enough for the phase planes and for the bordered gy; every per-image column
+    // range that a GEMM folds along n (OH*Wc forward, H_a*Wc input gradient) a multiple of four elements
+    int Wc = g->OW + (kw - 1) / 2;
+    if (Wc < L + g->OW) Wc = L + g->OW;
+    if (Wc < reach_w) Wc = reach_w;
+    const int first = Wc;
+    for (;; ++Wc) {
+        if (Wc > first + 8) return false;
+        if (((long long)g->OH * Wc) % 4 == 0 && ((long long)g->H_a[0] * Wc) % 4 == 0 &&
+            (g->H_a[1] == 0 || ((long long)g->H_a[1] * Wc) % 4 == 0))
+            break;
+    }
+    g->Wc = Wc;
+    g->kq = (int)round_up32((long long)g->OH * Wc);
+    // phase planes of x': every tap of every output lies inside, and so does everything the filter
+    // gradient reads while its positions run up to kq (against zeros of gy')
+    g->Hpp = g->OH + (kh - 1) / 2;
+    while (((long long)g->Hpp * Wc) % 4 != 0 || (long long)g->Hpp * Wc < g->kq + (long long)((kh - 1) / 2) * Wc + (kw - 1) / 2) ++g->Hpp;
+    g->pp = (long long)g->Hpp * Wc;
+    // bordered gy: rows for the deepest reach of the input gradient and for the kq positions of the filter gradient
+    g->Hp = T + (g->OH > reach_h ? g->OH : reach_h);
+    while (((long long)g->Hp * Wc) % 4 != 0 || (long long)g->Hp * Wc < (long long)T * Wc + L + g->kq) ++g->Hp;
+    g->xph_floats = (long long)B * C * 4 * g->pp + kS2Slack;
+    g->wf_floats = (long long)K * C * kh * kw;
+    g->gyp_floats = (long long)B * K * g->Hp * Wc + kS2Slack;
+    g->gxp_floats = (long long)B * C * H * W;
+    if (g->pp / 4 >= 32768) return false;  // range of the multiply-high divisions of the phase split
+    // 128-column tiles may straddle two images, not three; 32-bit offsets inside one image
+    if ((long long)g->OH * Wc < 128 || (long long)g->H_a[0] * Wc < 128 || (g->H_a[1] > 0 && (long long)g->H_a[1] * Wc < 128)) return false;
+    if ((long long)B * g->Hpp * Wc >= 0x7fffffffLL || (long long)C * 4 * g->pp >= (1LL << 30) ||
+        (long long)K * g->Hp * Wc >= (1LL << 30))
+        return false;
+    return true;
+}
+
+// xph[b][c][a][b'][i][j] = x'[2i+a][2j+b'] = x[b][c][2i+a-pad][2j+b'-pad], zero outside x.  One thread per four
+// consecutive elements of a phase plane; grid.y walks the (image, channel) planes.
+__global__ __launch_bounds__(256) void phase_split_kernel(const float *__restrict__ x, float *__restrict__ xph, int planes,
+                                                          int H, int W, int pad, int Wc, unsigned quads_phase, unsigned m_phase,
+                                                          unsigned m_row)
+{
+    const unsigned qi = blockIdx.x * 256u + threadIdx.x;  // quad inside the four phase planes of one channel
+    if (qi >= 4u * quads_phase) return;
+    const unsigned ph = __umulhi(qi, m_phase);
+    const unsigned e0 = (qi - ph * quads_phase) * 4u;
+    int i = (int)__umulhi(e0, m_row), j = (int)(e0 - (unsigned)i * (unsigned)Wc);
+    const int a = (int)(ph >> 1), b = (int)(ph & 1);
+    int off[4];
+    bool in[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int r = 2 * i + a - pad, s = 2 * j + b - pad;
+        in[t] = (unsigned)r < (unsigned)H && (unsigned)s < (unsigned)W;
+        off[t] = r * W + s;
+        if (++j == Wc) {
+            j = 0;
+            ++i;
+        }
+    }
+    for (int pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+        const float *src = x + (long long)pl * H * W;
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v[t] = in[t] ? src[off[t]] : 0.f;
+        st_stream(reinterpret_cast<float4 *>(xph) + ((long long)pl * 4 * quads_phase + qi), make_float4(v[0], v[1], v[2], v[3]));
+    }
+}
+
+__global__ void s2_zero_kernel(float *p, int n)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+// wf[k][tap][c] = w[k][c][tap]: the filter as the k-contiguous left operand of the stride-2 forward GEMM.
+__global__ __launch_bounds__(256) void s2_filter_fwd_kernel(const float *__restrict__ w, float *__restrict__ wf, int K, int C,
+                                                            int taps)
+{
+    const int total = K * C * taps;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int c = e % C, tap = e / C % taps, k = e / (C * taps);
+        wf[e] = w[((long long)k * C + c) * taps + tap];
+    }
+}
+
+// The four sub-filters of the input gradient, one per output parity (a, b), back to back:
+// wr_ab[c][m*kw_b + n][k] = w[k][c][2m + alpha_a][2n + alpha_b]  (k fastest).
+__global__ __launch_bounds__(256) void s2_filter_parity_kernel(const float *__restrict__ w, float *__restrict__ wr, int K, int C,
+                                                               int kh, int kw, int pad)
+{
+    const int total = K * C * kh * kw;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        // destination element e: find its parity block
+        int rest = e, a = 0, b = 0, kha = 0, kwb = 0;
+        for (int ph = 0; ph < 4; ++ph) {
+            a = ph >> 1;
+            b = ph & 1;
+            kha = (kh - ((a + pad) & 1) + 1) / 2;
+            kwb = (kw - ((b + pad) & 1) + 1) / 2;
+            const int size = C * kha * kwb * K;
+            if (rest < size) break;
+            rest -= size;
+        }
+        const int k = rest % K, tap = rest / K % (kha * kwb), c = rest / (K * kha * kwb);
+        const int m = tap / kwb, n = tap - m * kwb;
+        const int ky = 2 * m + ((a + pad) & 1), kx = 2 * n + ((b + pad) & 1);
+        wr[e] = w[(((long long)k * C + c) * kh + ky) * kw + kx];
+    }
+}
+
+// gx[pl][2i+a][2j+b] = gxp_ab[pl][i][j]: four consecutive pixels of a row per thread (W % 4 == 0), or one.
+__global__ __launch_bounds__(256) void s2_interleave_kernel(const float *__restrict__ gxp, float *__restrict__ gx, long long planes,
+                                                            int H, int W, int H0, int H1, int W0, int W1, int vec)
+{
+    const long long o00 = 0, o01 = planes * H0 * W0, o10 = o01 + planes * H0 * W1, o11 = o10 + planes * H1 * W0;
+    if (vec) {
+        const long long quads = planes * H * (W / 4);
+        for (long long q = blockIdx.x * 256LL + threadIdx.x; q < quads; q += gridDim.x * 256LL) {
+            const int xq = (int)(q % (W / 4));
+            const long long t = q / (W / 4);
+            const int iy = (int)(t % H);
+            const long long pl = t / H;
+            const int i = iy >> 1, j = 2 * xq;
+            const float *e, *o;  // even and odd columns of this row
+            if (iy & 1) {
+                e = gxp + o10 + (pl * H1 + i) * W0 + j;
+                o = gxp + o11 + (pl * H1 + i) * W1 + j;
+            } else {
+                e = gxp + o00 + (pl * H0 + i) * W0 + j;
+                o = gxp + o01 + (pl * H0 + i) * W1 + j;
+            }
+            st_stream(reinterpret_cast<float4 *>(gx) + q, make_float4(e[0], o[0], e[1], o[1]));
+        }
+    } else {
+        const long long total = planes * H * W;
+        for (long long q = blockIdx.x * 256LL + threadIdx.x; q < total; q += gridDim.x * 256LL) {
+            const int ix = (int)(q % W);
+            const long long t = q / W;
+            const int iy = (int)(t % H);
+            const long long pl = t / H;
+            const int i = iy >> 1, j = ix >> 1;
+            const int Ha = (iy & 1) ? H1 : H0, Wb = (ix & 1) ? W1 : W0;
+            const long long base = (iy & 1) ? ((ix & 1) ? o11 : o10) : ((ix & 1) ? o01 : o00);
+            gx[q] = gxp[base + (pl * Ha + i) * Wb + j];
+        }
+    }
+}
+
+static unsigned magic(unsigned d) { return (unsigned)((1ULL << 32) / d) + 1u; }
+
+ag_status_t s2_fwd_prepare(hipStream_t st, const float *x, const float *w, float *xpad, const S2Geom &g, int B, int C, int H,
+                           int W, int K, int kh, int kw, int pad)
+{
+    const unsigned quads_phase = (unsigned)(g.pp / 4);
+    const long long planes = (long long)B * C;
+    const dim3 grid((4 * quads_phase + 255) / 256, (unsigned)(planes < 65535 ? planes : 65535));
+    hipLaunchKernelGGL(phase_split_kernel, grid, dim3(256), 0, st, x, xpad, (int)planes, H, W, pad, g.Wc, quads_phase,
+                       magic(quads_phase), magic((unsigned)g.Wc));
+    hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, xpad + planes * 4 * g.pp, (int)kS2Slack);
+    hipLaunchKernelGGL(s2_filter_fwd_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
+                       xpad + g.xph_floats, K, C, kh * kw);
+    return check_launch("conv2d");
+}
+
+ag_status_t s2_fwd_filter(hipStream_t st, const float *w, float *wf, const S2Geom &g, int C, int K, int kh, int kw)
+{
+    hipLaunchKernelGGL(s2_filter_fwd_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C, kh * kw);
+    return check_launch("conv2d");
+}
+
+ag_status_t s2_fwd_gemm(hipStream_t st, const float *xph, const float *wf, float *y, const S2Geom &g, int B, int C, int K, int kh,
+                        int kw)
+{
+    return gemm_conv_fwd_stride2(st, wf, xph, y, B, K, C, g.OH, g.OW, kh, kw, g.Hpp, g.Wc);
+}
+
+// Scratch of the input gradient: zero-bordered gy, the four parity filters, the parity-planar result.
+ag_status_t s2_igrad_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const S2Geom &g, int B, int C, int K,
+                             int kh, int kw, int pad)
+{
+    launch_pad_border(st, gy, scratch, B, K, g.OH, g.OW, g.Hp, g.Wc, g.T, g.L);
+    hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, scratch + (long long)B * K * g.Hp * g.Wc, (int)kS2Slack);
+    hipLaunchKernelGGL(s2_filter_parity_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
+                       scratch + g.gyp_floats, K, C, kh, kw, pad);
+    return check_launch("conv2d_transpose");
+}
+
+ag_status_t s2_igrad_gemm(hipStream_t st, float *scratch, float *gx, const S2Geom &g, int B, int C, int K, int H, int W)
+{
+    const float *gyp = scratch;
+    const float *wr = scratch + g.gyp_floats;
+    float *gxp = scratch + g.gyp_floats + g.wf_floats;
+    long long out_off = 0;
+    for (int a = 0; a < 2; ++a)
+        for (int b = 0; b < 2; ++b) {
+            const int kha = g.kh_a[a], kwb = g.kw_b[b], Ha = g.H_a[a], Wb = g.W_b[b];
+            const long long wsize = (long long)C * kha * kwb * K;
+            if (Ha > 0 && Wb > 0) {
+                // this parity's own borders inside the shared copy
+                const int top = kha - 1 - g.d_a[a], left = kwb - 1 - g.d_a[b];
+                const float *origin = gyp + (long long)(g.T - top) * g.Wc + (g.L - left);
+                if (ag_status_t s = gemm_conv_input_grad(st, wr, origin, gxp + out_off, B, C, K, Ha, Wb, kha, kwb, g.Hp, g.Wc))
+                    return s;
+            }
+            wr += wsize;
+            out_off += (long long)B * C * Ha * Wb;
+        }
+    const long long planes = (long long)B * C;
+    const int vec = (W % 4 == 0) && aligned16(gx);
+    long long blocks = ((vec ? planes * H * (W / 4) : planes * H * W) + 255) / 256;
+    if (blocks > 1048576) blocks = 1048576;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(s2_interleave_kernel, dim3((unsigned)blocks), dim3(256), 0, st, gxp, gx, planes, H, W, g.H_a[0], g.H_a[1],
+                       g.W_b[0], g.W_b[1], vec);
+    return check_launch("conv2d_transpose");
+}
+
+size_t s2_filter_grad_workspace(const S2Geom &, int B, int C, int K, int kh, int kw)
+{
+    return gemm_conv_filter_grad_stride2_workspace(B, K, C, kh * kw);
+}
+
+ag_status_t s2_filter_grad(hipStream_t st, const float *xph, const float *gyp, float *gw, const S2Geom &g, int B, int C, int K,
+                           int kh, int kw, void *ws, size_t ws_bytes)
+{
+    // positions are counted from the first gradient value of a bordered plane
+    return gemm_conv_filter_grad_stride2(st, gyp + ((long long)g.T * g.Wc + g.L), xph, gw, ws, ws_bytes, B, K, C, kh, kw, g.Hp,
+                                         g.Hpp, g.Wc, g.kq);
+}
+
+}  // namespace ag

@@ -716,8 +716,9 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (fold) p.N = c.N * c.batch;
     p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
+    p.conv_phase = 0;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
-    p.rows_plane = 0;
+    p.rows_plane = p.rows_phase = 0;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * (fold ? 1 : c.batch) * p.splits;
@@ -793,24 +794,28 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
 // Implicit input gradient of a stride-1 convolution on the direct-to-LDS kernel (see the conv_*
 // fields of GemmParams): gx[b][c] = sum over taps and filters of wr[c][tap][k] * gyp[b][k] shifted.
 // wr [C][kh*kw*Kf] (k fastest), gyp [B][Kf][Hp][Wp] zero-bordered, gx [B][C][H][W].
-ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
-                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp)
+// `phase` != 0: stride-2 forward over four phase planes of `phase` elements per contracted channel.
+static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
+                                      int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
     p.M = C; p.K = Kf;
     p.n_img = H * Wp;
     p.N = B * p.n_img;
-    p.lda = (long long)kh * kw * Kf; p.ldb = (long long)Hp * Wp; p.ldc = (long long)H * W;
-    p.sA = 0; p.sB = (long long)Kf * Hp * Wp; p.sC = (long long)C * H * W;
+    const long long chan = phase != 0 ? 4LL * phase : (long long)Hp * Wp;  // elements per contracted channel of B
+    p.lda = (long long)kh * kw * Kf; p.ldb = chan; p.ldc = (long long)H * W;
+    p.sA = 0; p.sB = (long long)Kf * chan; p.sC = (long long)C * H * W;
     p.sAk = Kf; p.sBk = 0;
     p.kbatch = kh * kw; p.kb_per_split = p.kbatch; p.splits = 1; p.sCsplit = 0;
     p.alpha = 1.f; p.beta = 0.f;
     p.n_off = 0;
     p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
+    p.conv_phase = phase;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
-    p.rows_plane = 0;
-    const int cfg = C <= 64 ? kDirectCfg64 : 14;  // 64 x 128 or 128 x 256
+    p.rows_plane = p.rows_phase = 0;
+    // 64 x 128 for up to 64 output rows, else 128 x 256, or 128 x 128 when an image has fewer than 256 columns
+    const int cfg = C <= 64 ? kDirectCfg64 : (p.n_img >= 256 ? 14 : 13);
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n;
@@ -857,6 +862,18 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     return AG_OK;
 }
 
+ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp)
+{
+    return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0);
+}
+
+ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
+                                  int OH, int OW, int kh, int kw, int Hpp, int Wpp)
+{
+    return conv_implicit_gemm(st, wf, xph, y, B, K, C, OH, OW, kh, kw, Hpp, Wpp, (unsigned)(Hpp * Wpp));
+}
+
 constexpr int kConvFilterGradCfg = 17;  // 128 x 192 tiles, both operands k-contiguous
 
 static int conv_filter_grad_splits(int B, int Kf, int C, int taps, int kq)
@@ -876,18 +893,20 @@ size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq)
     return splits > 1 ? sizeof(float) * (size_t)splits * Kf * C * taps : 16;
 }
 
-ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
-                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq)
+// a_plane / b_plane: elements per row of A (one filter's gradient plane) and per channel of B; phase != 0: B is
+// split into four phase planes per channel (stride 2).
+static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const float *xp, float *gw, void *ws, size_t ws_bytes,
+                                         int B, int Kf, int C, int kh, int kw, int Wp, int kq, long long a_plane,
+                                         long long b_plane, unsigned phase)
 {
     const int taps = kh * kw;
-    const long long plane = (long long)Hp * Wp;
     GemmParams p;
-    p.A = gyp + ((long long)pad * Wp + pad);  // positions are counted from the first gradient value
+    p.A = a;
     p.B = xp;
     p.M = Kf; p.N = C * taps; p.K = kq;
-    p.lda = plane; p.ldb = plane; p.ldc = p.N;
+    p.lda = a_plane; p.ldb = b_plane; p.ldc = p.N;
     p.sA = p.sB = p.sC = 0;
-    p.sAk = (long long)Kf * plane; p.sBk = (long long)C * plane;
+    p.sAk = (long long)Kf * a_plane; p.sBk = (long long)C * b_plane;
     p.kbatch = B;
     p.splits = conv_filter_grad_splits(B, Kf, C, taps, kq);
     p.kb_per_split = (int)cdiv(B, p.splits);
@@ -896,7 +915,8 @@ ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float 
     p.alpha = 1.f; p.beta = 0.f;
     p.n_img = 0; p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
-    p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)plane;
+    p.conv_phase = 0;
+    p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)b_plane; p.rows_phase = phase;
     p.C = gw;
     if (p.splits > 1) {
         const size_t need = sizeof(float) * (size_t)p.splits * p.M * p.N;
@@ -918,6 +938,28 @@ ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float 
         return check_launch("conv2d_filter_grad");
     }
     return AG_OK;
+}
+
+ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
+                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq)
+{
+    const long long plane = (long long)Hp * Wp;
+    // positions are counted from the first gradient value
+    return conv_filter_grad_gemm(st, gyp + ((long long)pad * Wp + pad), xp, gw, ws, ws_bytes, B, Kf, C, kh, kw, Wp, kq, plane,
+                                 plane, 0);
+}
+
+size_t gemm_conv_filter_grad_stride2_workspace(int B, int Kf, int C, int taps)
+{
+    return gemm_conv_filter_grad_workspace(B, Kf, C, taps, 0);
+}
+
+ag_status_t gemm_conv_filter_grad_stride2(hipStream_t st, const float *gyq, const float *xph, float *gw, void *ws,
+                                          size_t ws_bytes, int B, int Kf, int C, int kh, int kw, int Hq, int Hpp, int Wpp, int kq)
+{
+    const long long pp = (long long)Hpp * Wpp;
+    return conv_filter_grad_gemm(st, gyq, xph, gw, ws, ws_bytes, B, Kf, C, kh, kw, Wpp, kq, (long long)Hq * Wpp, 4 * pp,
+                                 (unsigned)pp);
 }
 
 static thread_local int g_force_splits = 0;  // test hook (ag_test_hooks.h), per calling thread

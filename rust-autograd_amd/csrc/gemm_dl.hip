@@ -84,7 +84,10 @@ struct DirectTile {
     }
     // k-contiguous rows that are (channel, tap) pairs of a zero-bordered input (implicit filter
     // gradient): row n starts (n / taps) * plane + ky * wp + kx elements after the origin.
-    __device__ inline void init_conv_rows(int row0, int rows, int taps, int kw, int wp, unsigned plane, int wave, int lane)
+    // `phase` != 0 (stride 2): the input is split into four phase planes of `phase` elements each and
+    // tap (ky, kx) reads phase (ky&1, kx&1) shifted by (ky>>1) rows and (kx>>1) elements.
+    __device__ inline void init_conv_rows(int row0, int rows, int taps, int kw, int wp, unsigned plane, unsigned phase,
+                                          int wave, int lane)
     {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
@@ -93,7 +96,9 @@ struct DirectTile {
             const int row = min(row0 + r, rows - 1);
             const int ch = row / taps, tap = row - ch * taps;
             const int ky = tap / kw, kx = tap - ky * kw;
-            off[i] = ((unsigned)ch * plane + (unsigned)(ky * wp + kx + c * 4)) * 4u;
+            const unsigned shift = phase != 0 ? (unsigned)((ky & 1) * 2 + (kx & 1)) * phase + (unsigned)((ky >> 1) * wp + (kx >> 1))
+                                              : (unsigned)(ky * wp + kx);
+            off[i] = ((unsigned)ch * plane + shift + (unsigned)(c * 4)) * 4u;
         }
     }
     // Folded batch (m/n-contiguous operand only): the tile starts at column r0 of one batch and
@@ -248,8 +253,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     LoadA ldr_a;
     LoadB ldr_b;
     const float *pa = nullptr, *pb = nullptr;  // origin of the next k tile to fetch
-    int fkt = 0, f_left = 0, f_kx = 0;
-    const int conv_first_shift = p.conv_wp != 0 ? (p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1) : 0;
+    const float *pb_group = nullptr;           // stride-2 forward: B origin of the current group of 32 channels
+    int fkt = 0, f_left = 0, f_kx = 0, f_ky = 0;
+    const int conv_first_shift =
+        p.conv_wp != 0 && p.conv_phase == 0 ? (p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1) : 0;
     Cursor fcur = first;
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
@@ -258,15 +265,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
             ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
         } else if (KB && p.rows_taps != 0) {
-            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, wave, lane);
+            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, wave, lane);
         } else {
             ldr_b.init(ldb, it.n0, p.N, wave, lane);
         }
         pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
         pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
-        if (p.conv_wp != 0) {  // first tap (0, 0): the largest shift
+        if (p.conv_wp != 0) {  // first tap (0, 0): the largest shift (input gradient), or phase (0, 0) unshifted
+            pb_group = pb;
             pb += conv_first_shift;
-            f_kx = 0;
+            f_kx = f_ky = 0;
         }
         fkt = 0;
         f_left = it.nt;
@@ -278,6 +286,22 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             if (f_valid) {
                 cursor_next(fcur);
                 f_begin();
+            }
+        } else if (p.conv_phase != 0) {
+            // Stride-2 forward: all taps of one group of 32 channels in natural order, then the next group.
+            if (++fkt == p.kbatch) {
+                fkt = 0;
+                f_kx = f_ky = 0;
+                pa += BK - (long long)(p.kbatch - 1) * p.sAk;
+                pb_group += step_b;
+                pb = pb_group;
+            } else {
+                pa += p.sAk;
+                if (++f_kx == p.conv_kw) {
+                    f_kx = 0;
+                    ++f_ky;
+                }
+                pb = pb_group + (long long)((f_ky & 1) * 2 + (f_kx & 1)) * p.conv_phase + (f_ky >> 1) * p.conv_wp + (f_kx >> 1);
             }
         } else if (p.conv_wp != 0) {
             // Implicit input gradient: for one group of 32 filters all taps are visited in turn

@@ -35,12 +35,19 @@ struct GemmParams {
     // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
     // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
     int conv_wp, conv_w, conv_kw;
+    // Stride-2 forward (conv_phase != 0): B holds the four phase planes of the zero-bordered input,
+    // [batch][K][2][2][Hpp][conv_wp] with phase (a, b) = elements (2i+a, 2j+b), conv_phase elements
+    // each; tap (ky, kx), visited in natural order, reads phase (ky&1, kx&1) shifted by
+    // (ky>>1)*conv_wp + (kx>>1) elements.
+    unsigned conv_phase;
     // Implicit filter gradient of a stride-1 convolution (direct-to-LDS kernel, k-contiguous B): row n
     // of B is (channel n / rows_taps, tap n % rows_taps) of a zero-bordered input [..][C][Hp][rows_wp]
     // and starts (channel * rows_plane + ky * rows_wp + kx) elements after B; the contraction runs
     // over the flattened padded plane.  0 = rows of B are ldb apart.
     int rows_taps, rows_kw, rows_wp;
     unsigned rows_plane;
+    unsigned rows_phase;  // != 0: stride-2 filter gradient, row (channel, ky, kx) starts at
+                          // channel*rows_plane + ((ky&1)*2 + (kx&1))*rows_phase + (ky>>1)*rows_wp + (kx>>1)
 };
 
 constexpr int kXcds = 8;
@@ -73,6 +80,16 @@ ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float 
                                   int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq);
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
                                  int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
+// Stride-2 forward over phase planes (see GemmParams::conv_phase): wf [K][kh*kw][C] in natural tap
+// order, xph [B][C][4][Hpp][Wpp], y [B][K][OH][OW].
+ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
+                                  int OH, int OW, int kh, int kw, int Hpp, int Wpp);
+// Stride-2 filter gradient: gw[k][c][ky][kx] = sum over images and positions q of
+// gyq[b][k][q] * xph[b][c][phase(ky,kx)][q + (ky>>1)*Wpp + (kx>>1)]; gyq [B][K][Hq][Wpp] holds gy at row
+// pitch Wpp with zeros elsewhere; kq (a multiple of 32) positions.
+size_t gemm_conv_filter_grad_stride2_workspace(int B, int Kf, int C, int taps);
+ag_status_t gemm_conv_filter_grad_stride2(hipStream_t st, const float *gyq, const float *xph, float *gw, void *ws,
+                                          size_t ws_bytes, int B, int Kf, int C, int kh, int kw, int Hq, int Hpp, int Wpp, int kq);
 // Direct-to-LDS configuration with a 64-row tile (64 x 128, two blocks per CU), used by the implicit input gradient.
 constexpr int kDirectCfg64 = 19;
 

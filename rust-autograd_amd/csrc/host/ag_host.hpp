@@ -303,6 +303,9 @@ class Evaluator {  // src/evaluation.rs:100-181
 namespace tensor_ops {
 Tensor conv2d(Tensor x, Tensor w, int pad, int stride);                                   // :2733
 Tensor dilated_conv2d(Tensor x, Tensor w, int pad, int stride, int dilate);               // :2763
+// The same operator made to write the im2col columns as its second output like the reference,
+// whatever the geometry (by default large stride-1 / stride-2 convolutions take the column-free path).
+Tensor conv2d_with_columns(Tensor x, Tensor w, int pad, int stride, int dilate);
 Tensor conv2d_transpose(Tensor x, Tensor w, int pad, int stride);                         // :2799
 Tensor dilated_conv2d_transpose(Tensor x, Tensor w, int pad, int stride, int dilate);     // :2834
 Tensor max_pool2d(Tensor x, int pool_size, int pad, int stride);                          // :2869

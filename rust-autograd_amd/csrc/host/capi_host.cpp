@@ -145,6 +145,11 @@ int agh_conv2d(agh_ctx *c, int x, int w, int pad, int stride, int dilation)
     return guard([&] { return tensor_ops::dilated_conv2d(T(c, x), T(c, w), pad, stride, dilation).id; });
 }
 
+int agh_conv2d_with_columns(agh_ctx *c, int x, int w, int pad, int stride, int dilation)
+{
+    return guard([&] { return tensor_ops::conv2d_with_columns(T(c, x), T(c, w), pad, stride, dilation).id; });
+}
+
 int agh_conv2d_transpose(agh_ctx *c, int x, int w, int pad, int stride, int dilation)
 {
     return guard([&] { return tensor_ops::dilated_conv2d_transpose(T(c, x), T(c, w), pad, stride, dilation).id; });

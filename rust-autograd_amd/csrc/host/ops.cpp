@@ -162,21 +162,34 @@ struct Conv2DFilterGrad : Op, ConvHyper {  // conv2d.rs:736-776
         const int B = (int)gy.shape()[0], K = (int)gy.shape()[1], P = (int)(gy.shape()[2] * gy.shape()[3]);
         const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
         NdArray gw = NdArray::empty(w.shape());
-        if (cols.ndim() == 1) {  // the zero-bordered input of a column-free Conv2D (stride 1, dilation 1)
+        if (cols.ndim() == 1) {  // the rearranged input of a column-free Conv2D (stride 1 or 2, dilation 1)
             const int C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
             const int OH = (int)gy.shape()[2], OW = (int)gy.shape()[3];
-            const int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
-            const size_t n_gyp = ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, H, W);
-            const size_t nb = ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad);
-            if (n_gyp == 0 || nb == 0 || cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad))
-                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: the bordered input does not match gy and the filter");
+            // extents of x: from the optional fourth input (only its shape is read), else what a unit
+            // stride implies
+            int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
+            bool have_extents = false;
+            if (ctx.num_inputs() > 3) {
+                const NdArray like = ctx.input(3);  // (an input may be taken once)
+                if (like.ndim() == 4) {
+                    H = (int)like.shape()[2];
+                    W = (int)like.shape()[3];
+                    have_extents = true;
+                }
+            }
+            if (!have_extents && stride != 1)
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: the input's extents are needed for stride 2");
+            const size_t n_gyp = ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, stride, dilation, H, W);
+            const size_t nb = ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad, stride, dilation);
+            if (n_gyp == 0 || nb == 0 || cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad, stride, dilation))
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DFilterGrad: the rearranged input does not match gy and the filter");
             NdArray gyp = NdArray::empty({(int64_t)n_gyp});
-            OpError e = from_status(
-                ag_conv_input_grad_prepare_f32(ctx.stream(), gy.ptr(), w.ptr(), gyp.ptr(), B, K, OH, OW, C, kh, kw, pad, H, W));
+            OpError e = from_status(ag_conv_input_grad_prepare_f32(ctx.stream(), gy.ptr(), w.ptr(), gyp.ptr(), B, K, OH, OW, C, kh, kw,
+                                                                   pad, stride, dilation, H, W));
             if (!e.ok()) return e;
             NdArray ws = workspace(nb);
             e = from_status(ag_conv2d_filter_grad_nocols_f32(ctx.stream(), cols.ptr(), gyp.ptr(), gw.ptr(), B, C, H, W, K, kh, kw,
-                                                             pad, ws.ptr(), ws.len() * 4));
+                                                             pad, stride, dilation, ws.ptr(), ws.len() * 4));
             if (!e.ok()) return e;
             ctx.append_output(gw);
             return OpError::none();
@@ -210,13 +223,24 @@ struct Conv2DWithCols : Op, ConvHyper {  // conv2d.rs:589-629
             if (like.ndim() != 4) return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: 4D result extents expected");
             const int B = (int)like.shape()[0], OH = (int)like.shape()[2], OW = (int)like.shape()[3];
             const int K = (int)w.shape()[0], C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
-            const int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
-            if (cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad))
-                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: the bordered input does not match the filter");
+            int H = OH + kh - 1 - 2 * pad, W = OW + kw - 1 - 2 * pad;
+            bool have_extents = false;
+            if (ctx.num_inputs() > 3) {  // extents of x (needed for stride 2)
+                const NdArray xl = ctx.input(3);  // (an input may be taken once)
+                if (xl.ndim() == 4) {
+                    H = (int)xl.shape()[2];
+                    W = (int)xl.shape()[3];
+                    have_extents = true;
+                }
+            }
+            if (!have_extents && stride != 1)
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: the input's extents are needed for stride 2");
+            if (cols.len() != ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad, stride, dilation))
+                return OpError::make(ErrorKind::IncompatibleShape, "Conv2DWithCols: the rearranged input does not match the filter");
             NdArray y = NdArray::empty({B, K, OH, OW});
             NdArray wf = NdArray::empty(w.shape());
             const OpError e = from_status(ag_conv2d_nocols_with_filter_f32(ctx.stream(), cols.ptr(), w.ptr(), wf.ptr(), y.ptr(), B, C,
-                                                                           H, W, K, kh, kw, pad));
+                                                                           H, W, K, kh, kw, pad, stride, dilation));
             if (!e.ok()) return e;
             ctx.append_output(y);
             return OpError::none();
@@ -235,7 +259,9 @@ struct Conv2DWithCols : Op, ConvHyper {  // conv2d.rs:589-629
 };
 
 struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
-    explicit Conv2D(ConvHyper h) : ConvHyper(h) {}
+    // true: always write the im2col columns as output 1, like the reference (no column-free path)
+    bool materialise_columns;
+    explicit Conv2D(ConvHyper h, bool columns = false) : ConvHyper(h), materialise_columns(columns) {}
     const char *name() const override { return "Conv2D"; }
     OpError compute(ComputeContext &ctx) const override
     {
@@ -260,12 +286,13 @@ struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
         // input (rank 1) instead of the columns.
         // (small problems are launch-bound and the column path has fewer launches: from 64 MB of columns on)
         const bool large = (long long)B * C * kh * kw * OH * OW >= (16LL << 20);
-        const size_t n_xpad = (large && stride == 1 && dilation == 1) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad) : 0;
-        if (n_xpad > 0 && ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad) > 0 &&
-            ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, H, W) > 0) {
+        const size_t n_xpad =
+            (large && !materialise_columns) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad, stride, dilation) : 0;
+        if (n_xpad > 0 && ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad, stride, dilation) > 0 &&
+            ag_conv_input_grad_scratch_floats(B, K, OH, OW, C, kh, kw, pad, stride, dilation, H, W) > 0) {
             NdArray xpad = NdArray::empty({(int64_t)n_xpad});
-            const OpError e = from_status(
-                ag_conv2d_fwd_nocols_f32(ctx.stream(), x.ptr(), w.ptr(), y.ptr(), xpad.ptr(), B, C, H, W, K, kh, kw, pad));
+            const OpError e = from_status(ag_conv2d_fwd_nocols_f32(ctx.stream(), x.ptr(), w.ptr(), y.ptr(), xpad.ptr(), B, C, H, W, K,
+                                                                   kh, kw, pad, stride, dilation));
             if (!e.ok()) return e;
             ctx.append_output(y);
             ctx.append_output(xpad);
@@ -290,6 +317,7 @@ struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
                               .append_input(cols, false)
                               .append_input(gy, false)
                               .append_input(w, false)
+                              .append_input(tensor_ops::stop_gradient(x), false)  // extents of x only
                               .append_backprop_input(x)
                               .append_backprop_input(gy)
                               .build(std::make_unique<Conv2DFilterGrad>(ConvHyper{pad, stride, dilation}));
@@ -308,6 +336,7 @@ void Conv2DWithCols::grad(GradientContext &ctx) const
                           .append_input(cols, false)
                           .append_input(gy, false)
                           .append_input(w, false)
+                          .append_input(tensor_ops::stop_gradient(x0), false)  // extents of x only
                           .append_backprop_input(x0)
                           .append_backprop_input(gy)
                           .build(std::make_unique<Conv2DFilterGrad>(ConvHyper{pad, stride, dilation}));
@@ -326,6 +355,7 @@ void Conv2DFilterGrad::grad(GradientContext &ctx) const
                            .append_input(cols, false)
                            .append_input(ggw, false)
                            .append_input(tensor_ops::stop_gradient(gy), false)  // extents of the result
+                           .append_input(tensor_ops::stop_gradient(x0), false)  // extents of x
                            .append_backprop_input(x0)
                            .append_backprop_input(ggw)
                            .build(std::make_unique<Conv2DWithCols>(ConvHyper{pad, stride, dilation}));
@@ -1053,6 +1083,10 @@ Tensor dilated_conv2d(Tensor x, Tensor w, int pad, int stride, int dilate)
     return build(x.graph, {x, w}, std::make_unique<Conv2D>(ConvHyper{pad, stride, dilate}));
 }
 Tensor conv2d(Tensor x, Tensor w, int pad, int stride) { return dilated_conv2d(x, w, pad, stride, 1); }
+Tensor conv2d_with_columns(Tensor x, Tensor w, int pad, int stride, int dilate)
+{
+    return build(x.graph, {x, w}, std::make_unique<Conv2D>(ConvHyper{pad, stride, dilate}, true));
+}
 
 Tensor dilated_conv2d_transpose(Tensor x, Tensor w, int pad, int stride, int dilate)
 {

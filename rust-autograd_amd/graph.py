@@ -40,6 +40,7 @@ PROTOTYPES = {
     "agh_placeholder": (_i, [_p, _s, _lp, _i]),
     "agh_scalar": (_i, [_p, _f]),
     "agh_conv2d": (_i, [_p, _i, _i, _i, _i, _i]),
+    "agh_conv2d_with_columns": (_i, [_p, _i, _i, _i, _i, _i]),
     "agh_conv2d_transpose": (_i, [_p, _i, _i, _i, _i, _i]),
     "agh_max_pool2d": (_i, [_p, _i, _i, _i, _i]),
     "agh_matmul": (_i, [_p, _i, _i]),
@@ -253,11 +254,14 @@ class Context:
         return self._t(lib().agh_scalar(self._h, float(v)))
 
     # -- tensor_ops ---------------------------------------------------------------------------
-    def conv2d(self, x, w, pad, stride):
-        return self._t(lib().agh_conv2d(self._h, x.id, w.id, pad, stride, 1))
+    def conv2d(self, x, w, pad, stride, columns=False):
+        """columns=True: materialise the im2col columns like the reference, whatever the geometry."""
+        fn = lib().agh_conv2d_with_columns if columns else lib().agh_conv2d
+        return self._t(fn(self._h, x.id, w.id, pad, stride, 1))
 
-    def dilated_conv2d(self, x, w, pad, stride, dilation):
-        return self._t(lib().agh_conv2d(self._h, x.id, w.id, pad, stride, dilation))
+    def dilated_conv2d(self, x, w, pad, stride, dilation, columns=False):
+        fn = lib().agh_conv2d_with_columns if columns else lib().agh_conv2d
+        return self._t(fn(self._h, x.id, w.id, pad, stride, dilation))
 
     def conv2d_transpose(self, x, w, pad, stride):
         return self._t(lib().agh_conv2d_transpose(self._h, x.id, w.id, pad, stride, 1))

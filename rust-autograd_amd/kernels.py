@@ -196,52 +196,55 @@ def conv2d_transpose(gy, w, pad, stride, dilation=1, out_hw=None, return_cols=Fa
     return (gx, gcols) if return_cols else gx
 
 
-def conv2d_nocols(x, w, pad):
-    """Column-free stride-1 forward: (y, xpad) or None when the geometry is not supported.  `xpad`
-    (the zero-bordered input) is what conv2d_filter_grad_nocols reads instead of the columns."""
+def conv2d_nocols(x, w, pad, stride=1, dilation=1):
+    """Column-free forward (stride 1 or 2): (y, xpad) or None when the geometry is not supported.
+    `xpad` (the rearranged input) is what conv2d_filter_grad_nocols reads instead of the columns."""
     x, w = _f32(x, "conv2d"), _f32(w, "conv2d")
     B, Cc, H, W = x.shape
     Kf, C2, kh, kw = w.shape
     if Cc != C2:
         raise capi.IncompatibleShape(f"conv2d: Number of input channels ({Cc}) must match second filter dim ({C2})")
     L = capi.lib()
-    n = L.ag_conv2d_nocols_scratch_floats(B, Cc, H, W, Kf, kh, kw, pad)
+    n = L.ag_conv2d_nocols_scratch_floats(B, Cc, H, W, Kf, kh, kw, pad, stride, dilation)
     if n == 0:
         return None
     xpad = torch.empty(n, dtype=torch.float32, device=x.device)
-    y = _empty((B, Kf, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1), x)
-    check(L.ag_conv2d_fwd_nocols_f32(_stream(), _ptr(x), _ptr(w), _ptr(y), _ptr(xpad), B, Cc, H, W, Kf, kh, kw, pad))
+    OH, OW = conv_out_size(H, kh, pad, stride, dilation), conv_out_size(W, kw, pad, stride, dilation)
+    y = _empty((B, Kf, OH, OW), x)
+    check(L.ag_conv2d_fwd_nocols_f32(_stream(), _ptr(x), _ptr(w), _ptr(y), _ptr(xpad), B, Cc, H, W, Kf, kh, kw, pad,
+                                     stride, dilation))
     return y, xpad
 
 
-def conv_input_grad_staged(gy, w, pad, x_hw):
-    """The two stages of the column-free stride-1 input gradient: (gx, scratch); the scratch starts
-    with the zero-bordered gy that conv2d_filter_grad_nocols takes.  None when not supported."""
+def conv_input_grad_staged(gy, w, pad, x_hw, stride=1, dilation=1):
+    """The two stages of the column-free input gradient (stride 1 or 2): (gx, scratch); the scratch
+    starts with the zero-bordered gy that conv2d_filter_grad_nocols takes.  None when not supported."""
     gy, w = _f32(gy, "conv2d_transpose"), _f32(w, "conv2d_transpose")
     B, ych, yh, yw = gy.shape
     _, xch, kh, kw = w.shape
     xh, xw = x_hw
     L = capi.lib()
-    n = L.ag_conv_input_grad_scratch_floats(B, ych, yh, yw, xch, kh, kw, pad, xh, xw)
+    geom = (B, ych, yh, yw, xch, kh, kw, pad, stride, dilation, xh, xw)
+    n = L.ag_conv_input_grad_scratch_floats(*geom)
     if n == 0:
         return None
     scratch = torch.empty(n, dtype=torch.float32, device=gy.device)
     gx = _empty((B, xch, xh, xw), gy)
-    check(L.ag_conv_input_grad_prepare_f32(_stream(), _ptr(gy), _ptr(w), _ptr(scratch), B, ych, yh, yw, xch, kh, kw, pad, xh, xw))
-    check(L.ag_conv_input_grad_gemm_f32(_stream(), _ptr(scratch), _ptr(gx), B, ych, yh, yw, xch, kh, kw, pad, xh, xw))
+    check(L.ag_conv_input_grad_prepare_f32(_stream(), _ptr(gy), _ptr(w), _ptr(scratch), *geom))
+    check(L.ag_conv_input_grad_gemm_f32(_stream(), _ptr(scratch), _ptr(gx), *geom))
     return gx, scratch
 
 
-def conv2d_filter_grad_nocols(xpad, gypad, x_shape, w_shape, pad):
-    """Column-free filter gradient of a "same" stride-1 convolution from the zero-bordered copies of
-    x (conv2d_nocols) and gy (conv_input_grad_staged)."""
+def conv2d_filter_grad_nocols(xpad, gypad, x_shape, w_shape, pad, stride=1, dilation=1):
+    """Column-free filter gradient from the rearranged copies of x (conv2d_nocols) and gy
+    (conv_input_grad_staged): "same" convolutions for stride 1, any supported geometry for stride 2."""
     B, Cc, H, W = x_shape
     Kf, _, kh, kw = w_shape
     L = capi.lib()
     gw = _empty(w_shape, xpad)
-    ws = _ws(L.ag_conv2d_filter_grad_nocols_f32_workspace(B, Cc, H, W, Kf, kh, kw, pad), xpad)
-    check(L.ag_conv2d_filter_grad_nocols_f32(_stream(), _ptr(xpad), _ptr(gypad), _ptr(gw), B, Cc, H, W, Kf, kh, kw, pad,
-                                             _ptr(ws), ws.numel()))
+    geom = (B, Cc, H, W, Kf, kh, kw, pad, stride, dilation)
+    ws = _ws(L.ag_conv2d_filter_grad_nocols_f32_workspace(*geom), xpad)
+    check(L.ag_conv2d_filter_grad_nocols_f32(_stream(), _ptr(xpad), _ptr(gypad), _ptr(gw), *geom, _ptr(ws), ws.numel()))
     return gw
 
 

@@ -113,3 +113,21 @@ def test_validation_errors_map_to_op_error_variants(capi):
     # empty problems are accepted without touching the device
     assert L.ag_im2col_f32(null, null, null, 0, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 0
     assert L.ag_gemm_f32(null, 0, 0, 0, 4, 4, 1.0, null, 4, 0, null, 4, 0, 0.0, null, 4, 0, 1) == 0
+
+
+def test_column_free_geometry_support_is_decided_on_the_host(capi):
+    """Which geometries the implicit (column-free) convolution takes is pure host arithmetic."""
+    L = capi.lib()
+    # the headline (stride 1) and its stride-2 variant at B = 256
+    assert L.ag_conv2d_nocols_scratch_floats(256, 64, 56, 56, 128, 3, 3, 1, 1, 1) > 0
+    assert L.ag_conv2d_nocols_scratch_floats(256, 64, 56, 56, 128, 3, 3, 1, 2, 1) > 0
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(256, 64, 56, 56, 128, 3, 3, 1, 2, 1) > 0
+    assert L.ag_conv_input_grad_scratch_floats(256, 128, 28, 28, 64, 3, 3, 1, 2, 1, 56, 56) > 0
+    assert L.ag_conv_input_grad_scratch_floats(256, 128, 28, 28, 64, 3, 3, 1, 2, 1, 55, 55) > 0   # the reference's reconstructed extent
+    # the 4x4 stride-2 transposed convolution of configuration 5 is the input-gradient form
+    assert L.ag_conv_input_grad_scratch_floats(32, 128, 14, 14, 64, 4, 4, 1, 2, 1, 28, 28) > 0
+    # not taken: dilation, stride 3, channel counts that are not multiples of 32, a gradient of the wrong extent
+    assert L.ag_conv2d_nocols_scratch_floats(32, 256, 14, 14, 256, 3, 3, 2, 1, 2) == 0
+    assert L.ag_conv2d_nocols_scratch_floats(8, 64, 56, 56, 128, 3, 3, 1, 3, 1) == 0
+    assert L.ag_conv2d_nocols_scratch_floats(8, 48, 56, 56, 128, 3, 3, 1, 2, 1) == 0
+    assert L.ag_conv_input_grad_scratch_floats(8, 128, 27, 27, 64, 3, 3, 1, 2, 1, 56, 56) == 0

@@ -729,6 +729,34 @@ def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, p
     assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, 1, 1, out_hw=(H, H)), "gx", scale=np.abs(gxv).max())
 
 
+@pytest.mark.parametrize("H", [32, 33])
+def test_conv2d_stride2_column_free_through_the_graph_and_the_column_switch(G, orc, rng, H):
+    # stride 2 at a size where Conv2D goes column-free: the kept second output is the phase-split input
+    # (rank 1), the filter gradient reads x's extents from its extra input (28 outputs fit both 55 and 56
+    # input rows), and `columns=True` makes the same operator keep the reference's columns instead
+    B, Cin, Cout, k, pad = 240, 32, 64, 3, 1   # 17.7 M column elements: above the size from which Conv2D goes column-free
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = glorot(rng, (Cout, Cin, k, k))
+    oy, ocols = orc.conv2d_fwd(xv, wv, pad, 2, 1)
+    gyv = (2 * oy).astype(np.float32)
+    ogw = orc.conv2d_filter_grad(ocols, gyv, wv.shape)
+    ogx = orc.conv2d_transpose(gyv, wv, pad, 2, 1, out_hw=(H, H))
+    for columns in (False, True):
+        env = G.VariableEnvironment()
+        c = env.context()
+        x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+        y = c.conv2d(x, w, pad, 2, columns=columns)
+        gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+        say(f"stride-2 conv through the graph H={H} columns={columns}")
+        yv, gxv, gwv, kept = c.eval([y, gx, gw, c.nth_tensor(y, 1)], {"x": xv, "w": wv})
+        assert (kept.ndim == 1) == (not columns)
+        if columns:
+            assert np.array_equal(kept.reshape(ocols.shape), ocols)
+        assert_close(yv, oy, "y", scale=1.0)
+        assert_close(gwv, ogw, "gw", scale=np.abs(ogw).max())
+        assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max())
+
+
 def test_conv2d_column_free_second_order(G, orc, rng):
     # the gradient of the filter gradient: w.r.t. x (Conv2DTranspose of the incoming gradient) and
     # w.r.t. gy (Conv2DWithCols, here over the bordered input)

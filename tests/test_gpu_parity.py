@@ -573,7 +573,7 @@ def test_conv2d_column_free_random_geometries_exact(K):
         staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
         if staged is not None:
             assert np.array_equal(host(staged[0]), host(gx_cols)), (B, C, Kc, H, W, k, p)
-        if res is not None and staged is not None and L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p) > 0:
+        if res is not None and staged is not None and L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, 1) > 0:
             ran_bwd += 1
             gw = K.conv2d_filter_grad_nocols(res[1], staged[1], x.shape, w.shape, p)
             assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape))), (B, C, Kc, H, W, k, p)
@@ -662,14 +662,102 @@ def test_conv2d_column_free_filter_grad_keeps_a_nan_inside_its_channel(K, orc, r
     assert np.isfinite(yv[1:B - 1]).all()
 
 
+S2_CASES = [  # B, C, K (filters), H, W, k, pad: stride-2 convolutions without columns
+    (2, 64, 128, 56, 56, 3, 1),   # the headline's stride-2 variant, 2 of 256 images
+    (3, 32, 64, 28, 28, 3, 1),
+    (2, 64, 32, 55, 57, 3, 1),    # odd extents: the parities of the input gradient differ in size
+    (2, 32, 32, 30, 26, 4, 1),    # 4x4 window of the transposed convolution: four taps per parity
+    (2, 32, 64, 29, 31, 3, 0),    # no padding
+    (2, 32, 32, 40, 36, 5, 2),    # 5x5
+    (5, 32, 160, 24, 24, 3, 1),   # more than 128 filters: two row tiles; tiles straddle images
+]
+
+
+@pytest.mark.parametrize("case", S2_CASES)
+def test_conv2d_stride2_column_free(K, orc, rng, case):
+    """Stride 2 without the im2col columns: the forward over the four phase planes of the bordered
+    input, the filter gradient over the same planes and a bordered gy, the input gradient as four
+    parity GEMMs interleaved afterwards.  Against the f64 oracle (with the f32 oracle's error as the
+    yardstick) and, on integer-valued data, bit for bit against the column path."""
+    B, C, Kc, H, W, k, p = case
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    y32, cols32 = orc.conv2d_fwd(x, w, p, 2, 1)
+    OH, OW = y32.shape[2:]
+    gy = rng.standard_normal((B, Kc, OH, OW)).astype(np.float32)
+    x64, w64, g64 = (v.astype(np.float64) for v in (x, w, gy))
+    say("stride-2 column-free forward", case)
+    res = K.conv2d_nocols(dev(x), dev(w), p, 2)
+    assert res is not None, "geometry expected to be supported"
+    y, xph = res
+    y64, cols64 = orc.conv2d_fwd(x64, w64, p, 2, 1)
+    yabs, colsabs = orc.conv2d_fwd(np.abs(x64), np.abs(w64), p, 2, 1)
+    assert tuple(y.shape) == y64.shape
+    assert_close_conditioned(host(y), y64, yabs, "stride-2 forward", ref32=y32)
+    say("stride-2 column-free input gradient", case)
+    staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 2)
+    assert staged is not None
+    gx, scratch = staged
+    gx64 = orc.conv2d_transpose(g64, w64, p, 2, 1, out_hw=(H, W))
+    gxabs = orc.conv2d_transpose(np.abs(g64), np.abs(w64), p, 2, 1, out_hw=(H, W))
+    assert_close_conditioned(host(gx), gx64, gxabs, "stride-2 input gradient",
+                             ref32=orc.conv2d_transpose(gy, w, p, 2, 1, out_hw=(H, W)))
+    say("stride-2 column-free filter gradient", case)
+    gw = host(K.conv2d_filter_grad_nocols(xph, scratch, x.shape, w.shape, p, 2))
+    gw64 = orc.conv2d_filter_grad(cols64, g64, w.shape)
+    gwabs = orc.conv2d_filter_grad(colsabs, np.abs(g64), w.shape)
+    assert_close_conditioned(gw, gw64, gwabs, "stride-2 filter gradient", ref32=orc.conv2d_filter_grad(cols32, gy, w.shape))
+    assert np.array_equal(gw, host(K.conv2d_filter_grad_nocols(xph, scratch, x.shape, w.shape, p, 2)))   # deterministic
+    # the operator entry point takes the same route when the columns' buffer it is handed is large enough
+    # to serve as scratch (else GEMM + col2im), at the true input size and at the size the reference
+    # reconstructs (conv2d_transpose.rs:55-56: a crop when H is even)
+    gx_op = host(K.conv2d_transpose(dev(gy), dev(w), p, 2, 1, out_hw=(H, W)))
+    if K.capi.lib().ag_conv_input_grad_scratch_floats(B, Kc, OH, OW, C, k, k, p, 2, 1, H, W) <= B * C * k * k * OH * OW:
+        assert np.array_equal(gx_op, host(gx))
+    assert_close_conditioned(gx_op, gx64, gxabs, "input gradient through ag_conv2d_transpose_f32")
+    rh, rw = orc.conv_transpose_out_size(OH, k, p, 2, 1), orc.conv_transpose_out_size(OW, k, p, 2, 1)
+    gx_ref = host(K.conv2d_transpose(dev(gy), dev(w), p, 2, 1))
+    assert gx_ref.shape[2:] == (rh, rw)
+    assert_close_conditioned(gx_ref, gx64[:, :, :rh, :rw], gxabs[:, :, :rh, :rw], "input gradient at the reference's size")
+    # integer-valued data: every partial sum is exact, so the results equal the column path's bit for bit
+    xi = rng.integers(-3, 4, x.shape).astype(np.float32)
+    wi = rng.integers(-2, 3, w.shape).astype(np.float32)
+    gi = rng.integers(-2, 3, gy.shape).astype(np.float32)
+    yi, xphi = K.conv2d_nocols(dev(xi), dev(wi), p, 2)
+    yc, colsi = K.conv2d(dev(xi), dev(wi), p, 2, 1)
+    assert np.array_equal(host(yi), host(yc))
+    gxi, scri = K.conv_input_grad_staged(dev(gi), dev(wi), p, (H, W), 2)
+    assert np.array_equal(host(gxi), host(K.conv2d_transpose(dev(gi), dev(wi), p, 2, 1, out_hw=(H, W), return_cols=True)[0]))
+    assert np.array_equal(host(K.conv2d_filter_grad_nocols(xphi, scri, x.shape, w.shape, p, 2)),
+                          host(K.conv2d_filter_grad(colsi, dev(gi), w.shape)))
+
+
+def test_conv2d_stride2_filter_grad_keeps_a_nan_inside_its_channel(K, rng):
+    B, C, Kc, H, W, k, p = 2, 64, 64, 28, 28, 3, 1
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, 14, 14)).astype(np.float32)
+    bad = 17
+    x[:, bad, 0, :] = np.nan
+    x[:, bad, -1, :] = np.nan
+    x[:, bad, :, 0] = np.nan
+    x[:, bad, :, -1] = np.nan
+    say("stride-2 filter gradient with a NaN channel")
+    _, xph = K.conv2d_nocols(dev(x), dev(w), p, 2)
+    _, scratch = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 2)
+    gw = host(K.conv2d_filter_grad_nocols(xph, scratch, x.shape, w.shape, p, 2))
+    assert np.isnan(gw[:, bad]).any()
+    assert np.isfinite(np.delete(gw, bad, axis=1)).all(), "a NaN left its channel"
+
+
 def test_conv2d_column_free_refuses_other_geometries(K, rng):
     L = K.capi.lib()
-    assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1) == 0      # C not a multiple of 32
-    assert L.ag_conv2d_nocols_scratch_floats(2, 32, 4, 4, 32, 3, 3, 1) == 0       # plane too small
+    assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1, 1, 1) == 0      # C not a multiple of 32
+    assert L.ag_conv2d_nocols_scratch_floats(2, 32, 4, 4, 32, 3, 3, 1, 1, 1) == 0       # plane too small
     assert K.conv2d_nocols(dev(np.zeros((2, 3, 28, 28), np.float32)), dev(np.zeros((32, 3, 3, 3), np.float32)), 1) is None
-    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 32, 3, 3, 0) >= 0
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 32, 3, 3, 0, 1, 1) >= 0
     x = dev(np.zeros(4096, np.float32))
-    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 32, 3, 3, 0, None, 0)
+    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 32, 3, 3, 0, 1, 1, None, 0)
     assert rc == 4 and b"geometry not supported" in L.ag_last_error()
 
 
@@ -710,7 +798,7 @@ def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
     """ag_conv_input_grad_{scratch_floats,prepare,gemm}: the two stages a caller may launch itself."""
     L = K.capi.lib()
     B, C, Kc, H, W, k, p = 3, 24, 64, 20, 28, 3, 1
-    geom = (B, Kc, H, W, C, k, k, p, H, W)
+    geom = (B, Kc, H, W, C, k, k, p, 1, 1, H, W)
     n = L.ag_conv_input_grad_scratch_floats(*geom)
     assert n > B * Kc * (H + 2) * (W + 2)
     gy = rng.standard_normal((B, Kc, H, W)).astype(np.float32)
@@ -725,11 +813,13 @@ def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
     oabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, 1, out_hw=(H, W))
     assert_close_conditioned(host(gx), o64, oabs, "staged input grad")
     # geometries the column-free path does not take report 0 and are refused
-    assert L.ag_conv_input_grad_scratch_floats(B, 48, H, W, C, k, k, p, H, W) == 0          # filters not a multiple of 32
-    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 8, 8) == 0           # fewer than 128 columns per image
+    assert L.ag_conv_input_grad_scratch_floats(B, 48, H, W, C, k, k, p, 1, 1, H, W) == 0          # filters not a multiple of 32
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 1, 1, 8, 8) == 0           # fewer than 128 columns per image
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, H, W, C, k, k, p, 1, 2, H, W) == 0          # dilation
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, H, W, C, k, k, p, 3, 1, H, W) == 0          # stride 3
     with pytest.raises(K.capi.InvalidDims, match="not supported"):
         K.check(L.ag_conv_input_grad_prepare_f32(K._stream(), K._ptr(gyd), K._ptr(wd), K._ptr(scratch), B, 48, H, W,
-                                                 C, k, k, p, H, W))
+                                                 C, k, k, p, 1, 1, H, W))
 
 
 def test_conv2d_all_ones_closed_form(K):
