@@ -395,21 +395,34 @@ def other_conv_configs(torch, Kn, dev, g):
     """Operator-level conv2d forward + both gradients at the remaining convolution configurations
     (stride-2 variant of the headline; dilated and transposed convolutions of configuration 5)."""
     out = {}
+    L = Kn.capi.lib()
 
     def conv_case(name, Bn, Cc, Kf, Hh, k, pad, stride, dil):
+        """Forward, filter gradient and input gradient the way the host Conv2D operator runs them:
+        column-free where the library supports the geometry, over materialised columns otherwise."""
         x = torch.randn(Bn, Cc, Hh, Hh, device=dev, generator=g)
         w = torch.randn(Kf, Cc, k, k, device=dev, generator=g) * 0.05
         y, cols = Kn.conv2d(x, w, pad, stride, dil)
         gy = torch.randn_like(y)
+        del cols
+        free = Kn.conv2d_nocols(x, w, pad, stride, dil) is not None and \
+            Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil) is not None and \
+            L.ag_conv2d_filter_grad_nocols_f32_workspace(Bn, Cc, Hh, Hh, Kf, k, k, pad, stride, dil) > 0
 
         def step():
-            yy, cc = Kn.conv2d(x, w, pad, stride, dil)
-            Kn.conv2d_filter_grad(cc, gy, tuple(w.shape))
-            Kn.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(Hh, Hh))
+            if free:
+                yy, xp = Kn.conv2d_nocols(x, w, pad, stride, dil)
+                gx, scratch = Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil)
+                Kn.conv2d_filter_grad_nocols(xp, scratch, tuple(x.shape), tuple(w.shape), pad, stride, dil)
+            else:
+                yy, cc = Kn.conv2d(x, w, pad, stride, dil)
+                Kn.conv2d_filter_grad(cc, gy, tuple(w.shape))
+                Kn.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(Hh, Hh))
 
         ms = time_events(torch, step, 8)
         flop = 3 * 2.0 * Bn * Kf * y.shape[2] * y.shape[3] * Cc * k * k
-        out[name] = {"ms": round(ms, 4), "images/s": round(Bn / ms * 1e3, 1), "TFLOP/s": round(flop / ms / 1e9, 2)}
+        out[name] = {"ms": round(ms, 4), "images/s": round(Bn / ms * 1e3, 1), "TFLOP/s": round(flop / ms / 1e9, 2),
+                     "frac_mfma": round(flop / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4), "path": "column-free" if free else "columns"}
 
     conv_case("conv2d_fwd_bwd_stride2_B256_64to128_56x56", 256, 64, 128, 56, 3, 1, 2, 1)
     conv_case("conv2d_fwd_bwd_dilated_B32_256to256_14x14", 32, 256, 256, 14, 3, 2, 1, 2)
@@ -425,7 +438,9 @@ def other_conv_configs(torch, Kn, dev, g):
         Kn.conv2d_transpose_filter_grad(x, go, tuple(w.shape), 1, 2)
 
     ms = time_events(torch, tstep, 8)
-    out["conv2d_transpose_fwd_bwd_B32_128to64_14to28"] = {"ms": round(ms, 4), "images/s": round(32 / ms * 1e3, 1)}
+    tflop = 3 * 2.0 * 32 * 128 * 14 * 14 * 64 * 16
+    out["conv2d_transpose_fwd_bwd_B32_128to64_14to28"] = {"ms": round(ms, 4), "images/s": round(32 / ms * 1e3, 1),
+                                                          "TFLOP/s": round(tflop / ms / 1e9, 2)}
     return out
 
 

@@ -569,9 +569,12 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
                                     fg.Wp);
     }
     // Stride 2: four parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
-    // is large enough to serve as their scratch.
+    // is large enough to serve as their scratch.  Only from 2^24 column elements on: below that the
+    // seven launches cost more than GEMM + col2im (the 4x4 stride-2 transposed convolution
+    // [32,128,14,14] -> [32,64,28,28] takes 0.23 ms this way against 0.15 ms over columns).
     S2Geom g2;
-    if (stride == 2 && dilation == 1 && g_fused_input_grad && s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh &&
+    if (stride == 2 && dilation == 1 && g_fused_input_grad && (long long)B * M * P >= (1LL << 24) &&
+        s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh &&
         g2.OW == yw && g2.gyp_floats + g2.wf_floats + g2.gxp_floats <= (long long)B * M * P && aligned16(gcols) && aligned16(gx)) {
         if (ag_status_t s = s2_igrad_prepare(as_stream(stream), gy, w, gcols, g2, B, xch, ych, kh, kw, pad)) return s;
         return s2_igrad_gemm(as_stream(stream), gcols, gx, g2, B, xch, ych, xh, xw);

@@ -103,12 +103,14 @@ def _conv_paths(K, x, w, gy, pad, stride, dil):
     del cols
     gx = K.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(H, W), return_cols=True)[0]
     out["columns"] = (y, gw, gx)
-    if stride == 1 and dil == 1:
-        res = K.conv2d_nocols(x, w, pad)
-        staged = K.conv_input_grad_staged(gy, w, pad, (H, W))
-        if res is not None and staged is not None:
-            gw2 = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), pad)
-            out["column-free"] = (res[0], gw2, staged[0])
+    res = K.conv2d_nocols(x, w, pad, stride, dil)
+    staged = K.conv_input_grad_staged(gy, w, pad, (H, W), stride, dil)
+    if res is not None and staged is not None:
+        gw2 = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), pad, stride, dil)
+        out["column-free"] = (res[0], gw2, staged[0])
+        del res, staged
+        # the input gradient through the operator entry point, which picks the column-free route itself
+        out["column-free, operator entry"] = (out["column-free"][0], gw2, K.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(H, W)))
     return out
 
 
@@ -121,6 +123,7 @@ def test_config4_conv_b256_against_direct_definition(K, stride):
     x = rng.standard_normal((B, C, H, H)).astype(np.float32)
     w = rng.uniform(-sc, sc, (Kf, C, k, k)).astype(np.float32)
     gy = rng.standard_normal((B, Kf, OH, OH)).astype(np.float32)
+    assert stride == 1 or K.conv2d_nocols(dev(x[:2]), dev(w), pad, stride) is not None, "stride 2 is expected to be column-free too"
     n = 8192
     yi = np.stack([rng.integers(0, B, n), rng.integers(0, Kf, n), rng.integers(0, OH, n), rng.integers(0, OH, n)], 1)
     xi = np.stack([rng.integers(0, B, n), rng.integers(0, C, n), rng.integers(0, H, n), rng.integers(0, H, n)], 1)
