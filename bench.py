@@ -37,26 +37,84 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 # headline workload
 B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 
-# HBM bytes per launch at the headline shape, measured with two rocprofv3 --pmc passes over this
-# script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
-# reads for the --pmc-calibration copy kernel (1 GiB in, 1 GiB out): FETCH_SIZE reads 0.5 of the
-# true bytes on this GPU (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
-KIB = 1024.0
-TRAFFIC_BYTES = {
+# HBM bytes per launch at the headline shape come from the tracked counter summaries under profiles/:
+# two rocprofv3 --pmc passes over this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled
+# by what the same counter reads for the --pmc-calibration copy kernel in the same pass (1 GiB in, 1 GiB out).
+# Each entry: summary file, then (kernel name, statistic) pairs whose scaled fetch + write are added up.
+# pad_border_fast_kernel runs twice per step (x with 64 channels, gy with 128): min is the x call, max the gy call.
+CALIBRATION_KERNEL = "ag::ew_vec_kernel<ag::ScaleF<false> >"
+CALIBRATION_KIB = float(1 << 20)
+_STEP, _POOL, _COLS = ("profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt", "profiles/maxpool_c4_hbm_traffic.txt",
+                       "profiles/conv2d_columns_c4_hbm_traffic.txt")
+_DL = "ag::gemm_dl_kernel<%s>"
+PROFILE_TRAFFIC = {
     # the step (column-free)
-    "gemm_fwd": ((158390.0 + 5455.7) * 2.0 + 392641.7 + 15116.0) * KIB,                  # implicit GEMM over bordered x + narrow-tile tail
-    "gemm_filter_grad": ((327022.7 + 36883.4) * 2.0 + 73730.3 + 288.0) * KIB,            # implicit GEMM + fold of the split partials
-    "gemm_input_grad": (232756.5 * 2.0 + 201655.9) * KIB,                                # implicit GEMM over bordered gy
-    "fwd_prepare": ((155175.4 * 2.0 + 328320.0) * 2 / 3 + 445.5 * 2.0 + 288.0) * KIB,    # pad_border averages x (64 ch) and gy (128 ch)
-    "input_grad_prepare": ((155175.4 * 2.0 + 328320.0) * 4 / 3 + 1165.0 * 2.0 + 288.0) * KIB,
-    # per-kernel section (column-materialising operators)
-    "gemm_fwd_columns": ((898691.8 + 19691.6) * 2.0 + 393230.8 + 8192.0) * KIB,          # whole rounds + narrow-tile tail
-    "gemm_filter_grad_columns": ((1116520.0 + 36883.5) * 2.0 + 73729.8 + 288.0) * KIB,   # GEMM + fold of the split partials
-    "im2col": (112667.1 * 2.0 + 1806374.2) * KIB,
-    "col2im": (919260.8 * 2.0 + 200704.0) * KIB,
-    "maxpool_fwd": (198682.5 * 2.0 + 301828.7) * KIB,   # x in; y, f32 index and int32 index out
-    "maxpool_bwd": (113241.7 * 2.0 + 418113.7) * KIB,   # gy and int32 index in (rows shared by two chunks read twice); gx out
+    "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false", "avg")]),
+    "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_kernel", "avg")]),
+    "gemm_input_grad": (_STEP, [(_DL % "64, 128, 32, 32, 64, 3, true, false", "avg")]),
+    "fwd_prepare": (_STEP, [("ag::pad_border_fast_kernel", "min"), ("ag::zero_slack_kernel", "min"), ("ag::filter_taps_fwd_kernel", "avg")]),
+    "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max"), ("ag::zero_slack_kernel", "max"), ("ag::filter_taps_kernel", "avg")]),
+    # per-kernel section: pooling, and the column-materialising operators
+    "maxpool_fwd": (_POOL, [("ag::maxpool_fwd_lds_kernel<3, 2>", "avg")]),
+    "maxpool_bwd": (_POOL, [("ag::maxpool_bwd_s2_kernel<true, 3, 16>", "avg")]),
+    "im2col": (_COLS, [("ag::im2col_same_kernel<3, 3, 1, 16>", "avg")]),
+    "col2im": (_COLS, [("ag::col2im_same_kernel<3, 3, 1, 16>", "avg")]),
+    "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false", "avg")]),
+    "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_kernel", "avg")]),
+    "gemm_input_grad_columns": (_COLS, [(_DL % "192, 128, 32, 96, 32, 3, false, false", "avg")]),
 }
+_profile_cache = {}
+_profile_strict = True   # False under --only: the passes that produce the summaries cannot depend on them
+
+
+def _profile_table(path):
+    """{counter: {kernel: {"avg","min","max"}}} of one summary file (lines as rocpd_summary.py prints them)."""
+    import re
+    if path not in _profile_cache:
+        table = {}
+        pat = re.compile(r"^(FETCH_SIZE|WRITE_SIZE)\s+n=\s*\d+\s+avg=\s*([\d.]+)\s+min=\s*([\d.]+)\s+max=\s*([\d.]+)\s+(.*\S)\s*$")
+        with open(os.path.join(ROOT, path)) as f:
+            for line in f:
+                m = pat.match(line)
+                if m:
+                    table.setdefault(m.group(1), {})[m.group(5)] = {"avg": float(m.group(2)), "min": float(m.group(3)),
+                                                                    "max": float(m.group(4))}
+        _profile_cache[path] = table
+    return _profile_cache[path]
+
+
+def profile_traffic(key):
+    """(HBM bytes per launch, summary file) of one benchmark entry, from the tracked counter summary.
+    Raises when the file or one of the kernel names the entry is made of is missing: a figure from kernels
+    that no longer exist must not be reported."""
+    path, parts = PROFILE_TRAFFIC[key]
+    table = _profile_table(path)
+    total = 0.0
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        rows = table.get(counter, {})
+        if CALIBRATION_KERNEL not in rows:
+            raise RuntimeError(f"{path}: no {counter} line of the calibration kernel {CALIBRATION_KERNEL}")
+        factor = CALIBRATION_KIB / rows[CALIBRATION_KERNEL]["avg"]
+        for kernel, stat in parts:
+            if kernel not in rows:
+                raise RuntimeError(f"{path}: no {counter} line of {kernel} (entry {key}): re-run the counter passes "
+                                   f"the file names after changing which kernels an entry launches")
+            total += rows[kernel][stat] * factor * 1024.0
+    return total, path
+
+
+def traffic_fields(key, ms=None):
+    """JSON fields of one entry's measured HBM traffic (and, given its duration, the fraction of HBM peak)."""
+    try:
+        nbytes = profile_traffic(key)[0]
+    except (RuntimeError, OSError):
+        if _profile_strict:
+            raise
+        return {}
+    out = {"traffic_bytes": round(nbytes)}
+    if ms is not None:
+        out["frac_hbm_of_traffic"] = round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)
+    return out
 
 
 def parse():
@@ -67,9 +125,11 @@ def parse():
     ap.add_argument("--batch", type=int, default=B, help="images per step (headline: 256)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
-    ap.add_argument("--cpu-images", type=int, default=32, help="images in the CPU baseline sample")
-    ap.add_argument("--pool-only", action="store_true",
-                    help="run only the two pooling kernels of the per-kernel section, three times each (for counter passes)")
+    ap.add_argument("--cpu-images", type=int, default=B, help="images per step of the CPU baseline (default: the whole batch)")
+    ap.add_argument("--only", choices=("pool", "columns", "config1", "config2"),
+                    help="run only one part of the per-kernel section (for profiler passes): the two pooling kernels, "
+                         "the column-materialising convolution kernels, or the steps of configuration 1 / 2 "
+                         "through the host operator layer")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch one plain copy kernel (ag_scale_f32 by 1.0) over 2^28 floats, "
                          "so that a rocprofv3 --pmc run of this command holds a kernel of known traffic "
@@ -160,10 +220,19 @@ def cpu_baseline(images):
         dt = time.perf_counter() - t0
         if dt > 8.0 or reps >= 20:
             break
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {
         "value": round(images * reps / dt, 2), "unit": "images/s", "cores": cores, "kind": "port",
-        "sample": f"{images} of {B} images of the same conv2d fwd+bwd workload, {reps} repetitions, "
-                  f"BLAS: {blas or 'none (built-in loops, not OpenBLAS)'}",
+        "sample": f"{images} of {B} images per step of the same conv2d fwd+bwd workload, {reps} timed steps after one warm-up, "
+                  f"{cores} threads on {model}; BLAS: {blas or 'none (built-in loops, not OpenBLAS)'}",
     }
 
 
@@ -185,15 +254,21 @@ def main():
     OH = Kn.conv_out_size(H, KH, PAD, STRIDE, DIL)
     P, CK = OH * OH, C * KH * KH
 
-    if args.pool_only:
-        xp_ = torch.randn(256, 128, 56, 56, device=dev)
-        yp_, am_, il_ = Kn.max_pool2d(xp_, 3, 0, 2)
-        for _ in range(2):
-            Kn.max_pool2d(xp_, 3, 0, 2)
-        for _ in range(3):
-            Kn.max_pool2d_grad(yp_, am_, il_, tuple(xp_.shape), 3, 0, 2)
+    if args.only:
+        global _profile_strict
+        _profile_strict = False
+        g = torch.Generator(device=dev)
+        g.manual_seed(99)
+        if args.only == "pool":
+            res = micro_pool(torch, Kn, capi, dev, g, iters=3, only=True)
+        elif args.only == "columns":
+            res = micro_columns(torch, Kn, capi, dev, g, iters=3)
+        else:
+            res = graph_steps(which=args.only)
+        if args.pmc_calibration:
+            calibration_copy(torch, Kn, capi, dev)
         torch.cuda.synchronize()
-        print(json.dumps({"pool_only": True, "launches": 3}))
+        print(json.dumps({"only": args.only, "kernels": res}))
         return
 
     g = torch.Generator(device=dev)
@@ -229,11 +304,7 @@ def main():
         T.run("gemm_input_grad", lambda: chk(L.ag_conv_input_grad_gemm_f32(st(), ptr(gypad), ptr(gx), *igeom)))
 
     if args.pmc_calibration:
-        src = torch.ones(1 << 28, device=dev)
-        dst = torch.empty_like(src)
-        chk(L.ag_scale_f32(st(), ptr(src), 1.0, ptr(dst), src.numel()))
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch, Kn, capi, dev)
 
     for _ in range(args.warmup):
         step()
@@ -258,15 +329,15 @@ def main():
         kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
     if Bn == B:
         for name in kernels:
-            if name in TRAFFIC_BYTES:
-                kernels[name]["traffic_bytes"] = round(TRAFFIC_BYTES[name])
+            kernels[name]["traffic_bytes"] = round(profile_traffic(name)[0])
     gemm_ms = sum(per[n] for n in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"))
     gemm_tf = 3 * gemm_flop / (gemm_ms * 1e-3) / 1e12
     dominant = max(("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"), key=lambda n: per[n])
     dom_tf = gemm_flop / (per[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(dom_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4),
-                "traffic": round(TRAFFIC_BYTES[dominant]) if Bn == B and dominant in TRAFFIC_BYTES else None,
+                "traffic": round(profile_traffic(dominant)[0]) if Bn == B else None,
+                "traffic_source": profile_traffic(dominant)[1] if Bn == B else None,
                 "gemm_phase_TFLOP/s": round(gemm_tf, 2),
                 "gemm_phase_frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)}
 
@@ -287,12 +358,26 @@ def main():
     print(json.dumps(out))
 
 
+def calibration_copy(torch, Kn, capi, dev):
+    """One plain copy kernel of known traffic: 2^28 floats read, 2^28 floats written."""
+    src = torch.ones(1 << 28, device=dev)
+    dst = torch.empty_like(src)
+    capi.check(capi.lib().ag_scale_f32(Kn._stream(), Kn._ptr(src), 1.0, Kn._ptr(dst), src.numel()))
+    torch.cuda.synchronize()
+
+
 def micro(torch, Kn, capi, dev):
     """Per-kernel microbenchmarks at the shapes of the other configurations (median of 10)."""
-    res = {}
     g = torch.Generator(device=dev)
     g.manual_seed(99)
+    res = micro_pool(torch, Kn, capi, dev, g)
+    res.update(micro_columns(torch, Kn, capi, dev, g))
+    res.update(micro_rest(torch, Kn, capi, dev, g))
+    return res
 
+
+def micro_pool(torch, Kn, capi, dev, g, iters=10, only=False):
+    res = {}
     # max_pool2d 3x3 stride 2 on the conv output [256,128,56,56], forward and argmax backward
     x = torch.randn(256, 128, 56, 56, device=dev, generator=g)
     y, am, il = Kn.max_pool2d(x, 3, 0, 2)
@@ -300,21 +385,25 @@ def micro(torch, Kn, capi, dev):
     by = 4.0 * (x.numel() + 2 * y.numel())
     Lp = capi.lib()
     sp, pp, cp = Kn._stream, Kn._ptr, capi.check
-    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), pp(il), 256, 128, 56, 56, 3, 0, 2)), 10)
+    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), pp(il), 256, 128, 56, 56, 3, 0, 2)), iters)
     res["maxpool_fwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "traffic_bytes": round(TRAFFIC_BYTES["maxpool_fwd"]),
-                          "frac_hbm_of_traffic": round(TRAFFIC_BYTES["maxpool_fwd"] / ms / 1e6 / HBM_PEAK_GBS, 4),
+                          **traffic_fields("maxpool_fwd", ms),
                           "note": "also writes one tap byte per output (23.9 MB, not counted in GB/s): the exact selection that the backward needs above 2^24 elements"}
-    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), None, 256, 128, 56, 56, 3, 0, 2)), 10)
+    if only:
+        ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), iters)
+        return res
+    ms = time_events(torch, lambda: cp(Lp.ag_maxpool2d_fwd_f32(sp(), pp(x), pp(y), pp(am), None, 256, 128, 56, 56, 3, 0, 2)), iters)
     res["maxpool_fwd_reference_outputs"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
                                             "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
                                             "note": "y and the f32-encoded argmax only, the reference's two outputs"}
-    ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), 10)
+    ms = time_events(torch, lambda: Kn.max_pool2d_grad(gy, am, il, tuple(x.shape), 3, 0, 2), iters)
     res["maxpool_bwd"] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
-                          "traffic_bytes": round(TRAFFIC_BYTES["maxpool_bwd"]),
-                          "frac_hbm_of_traffic": round(TRAFFIC_BYTES["maxpool_bwd"] / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    del x, y, am, il, gy
+                          **traffic_fields("maxpool_bwd", ms)}
+    return res
 
+
+def micro_columns(torch, Kn, capi, dev, g, iters=10):
+    res = {}
     # the column-materialising operators (what the reference does per image): im2col + W . cols, gy . cols^T summed
     # over images, W^T . gy + col2im
     Bn, Cc, Kf, Hh = 256, 64, 128, 56
@@ -331,28 +420,33 @@ def micro(torch, Kn, capi, dev):
     wsf = torch.empty(max(16, L.ag_conv2d_filter_grad_f32_workspace(Bn, CKk, Pp, Kf)), dtype=torch.uint8, device=dev)
     cb = 4.0 * (gc.numel() + gxx.numel())
     gf = 2.0 * Kf * Pp * CKk * Bn
-    ms = time_events(torch, lambda: chk(L.ag_im2col_f32(st(), ptr(xx), ptr(gc), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1)), 10)
+    ms = time_events(torch, lambda: chk(L.ag_im2col_f32(st(), ptr(xx), ptr(gc), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1)), iters)
     res["im2col"] = {"ms": round(ms, 4), "GB/s": round(cb / ms / 1e6, 1), "frac_hbm": round(cb / ms / 1e6 / HBM_PEAK_GBS, 4),
-                     "traffic_bytes": round(TRAFFIC_BYTES["im2col"])}
+                     **traffic_fields("im2col")}
     ms = time_events(torch, lambda: chk(L.ag_gemm_f32(st(), 0, 0, Kf, Pp, CKk, 1.0, ptr(wt), CKk, 0, ptr(gc), Pp, CKk * Pp, 0.0,
-                                                      ptr(yy), Pp, Kf * Pp, Bn)), 10)
+                                                      ptr(yy), Pp, Kf * Pp, Bn)), iters)
     res["gemm_fwd_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(gf / ms / 1e9, 2), "frac_mfma": round(gf / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
-                               "traffic_bytes": round(TRAFFIC_BYTES["gemm_fwd_columns"])}
+                               **traffic_fields("gemm_fwd_columns")}
     ms = time_events(torch, lambda: chk(L.ag_gemm_batchsum_f32(st(), 0, 1, Kf, CKk, Pp, 1.0, ptr(gyy), Pp, Kf * Pp, ptr(gc), Pp,
-                                                               CKk * Pp, 0.0, ptr(gww), CKk, Bn, ptr(wsf), wsf.numel())), 10)
+                                                               CKk * Pp, 0.0, ptr(gww), CKk, Bn, ptr(wsf), wsf.numel())), iters)
     res["gemm_filter_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(gf / ms / 1e9, 2),
                                        "frac_mfma": round(gf / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
-                                       "traffic_bytes": round(TRAFFIC_BYTES["gemm_filter_grad_columns"])}
+                                       **traffic_fields("gemm_filter_grad_columns")}
     del xx, yy, gww, wsf
     ms = time_events(torch, lambda: chk(L.ag_gemm_f32(st(), 1, 0, CKk, Pp, Kf, 1.0, ptr(wt), CKk, 0, ptr(gyy), Pp, Kf * Pp,
-                                                      0.0, ptr(gc), Pp, CKk * Pp, Bn)), 10)
+                                                      0.0, ptr(gc), Pp, CKk * Pp, Bn)), iters)
     tf = 2.0 * Kf * Pp * CKk * Bn / ms / 1e9
-    res["gemm_input_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
-    ms = time_events(torch, lambda: chk(L.ag_col2im_f32(st(), ptr(gc), ptr(gxx), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1, Hh, Hh)), 10)
+    res["gemm_input_grad_columns"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4),
+                                      **traffic_fields("gemm_input_grad_columns")}
+    ms = time_events(torch, lambda: chk(L.ag_col2im_f32(st(), ptr(gc), ptr(gxx), Bn, Cc, Hh, Hh, 3, 3, 1, 1, 1, 1, 1, 1, Hh, Hh)), iters)
     res["col2im"] = {"ms": round(ms, 4), "GB/s": round(cb / ms / 1e6, 1), "frac_hbm": round(cb / ms / 1e6 / HBM_PEAK_GBS, 4),
-                     "traffic_bytes": round(TRAFFIC_BYTES["col2im"])}
-    del wt, gyy, gc, gxx
+                     **traffic_fields("col2im")}
+    return res
 
+
+def micro_rest(torch, Kn, capi, dev, g, iters=10):
+    res = {}
+    Bn, Kf, Hh = 256, 128, 56
     # reduce_sum (to scalar) and Adam on 2^26 elements
     n = 1 << 26
     a = torch.randn(n, device=dev, generator=g)
@@ -444,7 +538,7 @@ def other_conv_configs(torch, Kn, dev, g):
     return out
 
 
-def graph_steps():
+def graph_steps(which=None):
     """Configurations 1 and 2 end to end through the host operator layer (graph build, evaluation,
     gradients, Adam), host arrays fed every step as the reference's examples do.  These steps are
     tens of MFLOP: launch- and copy-latency bound, reported as wall-clock time only."""
@@ -496,6 +590,8 @@ def graph_steps():
         adam.update([v[k] for k in names], grads, c, {"x": x2, "y": y2})
 
     for name, step, images in (("config1_conv_block_step", c1_step, 64), ("config2_cnn_adam_step", c2_step, 128)):
+        if which is not None and not name.startswith(which):
+            continue
         for _ in range(3):
             step()
         ts = []
