@@ -157,12 +157,12 @@ class Timer:
         return out
 
     def totals(self):
+        """Median duration per name over the timed steps."""
         self.torch.cuda.synchronize()
-        tot, cnt = {}, {}
+        per = {}
         for name, a, b in self.pending:
-            tot[name] = tot.get(name, 0.0) + a.elapsed_time(b)
-            cnt[name] = cnt.get(name, 0) + 1
-        return {k: tot[k] / cnt[k] for k in tot}
+            per.setdefault(name, []).append(a.elapsed_time(b))
+        return {k: sorted(v)[len(v) // 2] for k, v in per.items()}
 
 
 def time_events(torch, fn, iters, warm=3):

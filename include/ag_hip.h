@@ -278,6 +278,18 @@ ag_status_t ag_adam_update_f32(ag_stream_t stream, float *param, const float *gr
                                float *v, float *t, size_t n, float alpha, float eps, float b1,
                                float b2);
 
+/* The AdamOp::compute of `count` parameters (one optimizer step: Adam::compute builds one AdamOp
+ * per parameter, optimizers/adam.rs:116-154) in one launch plus one for the step counters.  The
+ * six tables are host arrays of `count` entries (device pointers, element counts); they are read
+ * before the call returns.  Per element the arithmetic is ag_adam_update_f32's, so the results
+ * equal `count` separate calls.  No two entries may share param, m, v or t
+ * (AG_ERR_INVALID_DIMS); count is at most ag_adam_update_multi_max(). */
+int ag_adam_update_multi_max(void);
+ag_status_t ag_adam_update_multi_f32(ag_stream_t stream, int count, float *const *params,
+                                     const float *const *grads, float *const *ms, float *const *vs,
+                                     float *const *ts, const size_t *ns, float alpha, float eps,
+                                     float b1, float b2);
+
 /* ---- elementwise and loss glue met on either side of the operators above -------------------- */
 
 /* ReLU::compute, x.max(0) (activation_ops.rs:154-159). */

@@ -80,6 +80,8 @@ PROTOTYPES = {
     "ag_reduce_sum_f32": (c_i, [c_p, c_p, c_p, c_p, c_i, c_p, c_i, c_i, c_p, c_sz]),
     "ag_broadcast_grad_f32": (c_i, [c_p, c_p, c_p, c_p, c_i, c_p, c_i]),
     "ag_adam_update_f32": (c_i, [c_p] * 6 + [c_sz] + [c_f] * 4),
+    "ag_adam_update_multi_max": (c_i, []),
+    "ag_adam_update_multi_f32": (c_i, [c_p, c_i] + [c_p] * 6 + [c_f] * 4),
     "ag_relu_f32": (c_i, [c_p, c_p, c_p, c_sz]),
     "ag_relu_grad_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),
     "ag_add_bias_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz]),

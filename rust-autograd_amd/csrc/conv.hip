@@ -20,6 +20,64 @@ static ag_status_t conv_dims(const char *who, int B, int C, int H, int W, int K,
     return AG_OK;
 }
 
+namespace ag {
+
+// Forward product of a thin first layer, y_b[K x P] = w[K x CK] . cols_b[CK x P] with CK <= 16 (e.g. the
+// 1 -> 32 channel 3x3 convolution of the small CNN: CK = 9).  A tiled GEMM spends its time on a k-tile that is
+// mostly padding; here the kernel is the HBM-bound copy it should be: a thread holds the CK column values of four
+// neighbouring positions in registers and writes one 128-bit result per filter for a pair of filters
+// (the filter taps, padded to 16 per filter with zeros, sit in LDS).  Products are added in tap order.
+constexpr int kThinFwdMaxCK = 16, kThinFwdGroup = 2;
+
+__global__ __launch_bounds__(256) void thin_fwd_kernel(const float *__restrict__ cols, const float *__restrict__ w,
+                                                       float *__restrict__ y, int CK, int P4, int K, long long quads)
+{
+    __shared__ float s_w[kThinFwdGroup * kThinFwdMaxCK];
+    const int k0 = blockIdx.y * kThinFwdGroup;
+    if (threadIdx.x < kThinFwdGroup * kThinFwdMaxCK) {
+        const int k = k0 + threadIdx.x / kThinFwdMaxCK, j = threadIdx.x % kThinFwdMaxCK;
+        s_w[threadIdx.x] = (k < K && j < CK) ? w[k * CK + j] : 0.f;
+    }
+    __syncthreads();
+    const long long q = blockIdx.x * 256ll + threadIdx.x;
+    if (q >= quads) return;
+    const long long b = q / P4;
+    const int p4 = (int)(q - b * P4);
+    const float4 *cb = reinterpret_cast<const float4 *>(cols) + b * CK * (long long)P4 + p4;
+    float4 c[kThinFwdMaxCK];
+#pragma unroll
+    for (int j = 0; j < kThinFwdMaxCK; ++j) c[j] = j < CK ? cb[(long long)j * P4] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 *yb = reinterpret_cast<float4 *>(y) + (b * K + k0) * (long long)P4 + p4;
+#pragma unroll
+    for (int g = 0; g < kThinFwdGroup; ++g) {
+        if (k0 + g >= K) break;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < kThinFwdMaxCK; ++j) {
+            const float wv = s_w[g * kThinFwdMaxCK + j];
+            acc.x = fmaf(wv, c[j].x, acc.x);
+            acc.y = fmaf(wv, c[j].y, acc.y);
+            acc.z = fmaf(wv, c[j].z, acc.z);
+            acc.w = fmaf(wv, c[j].w, acc.w);
+        }
+        yb[(long long)g * P4] = acc;
+    }
+}
+
+// Takes the product when it fits the kernel; false = the caller runs the GEMM.
+static bool thin_fwd(hipStream_t st, const float *cols, const float *w, float *y, int B, long long CK, long long P, int K)
+{
+    if (CK < 1 || CK > kThinFwdMaxCK || P % 4 != 0 || P < 64 || K < 1 || B < 1) return false;
+    if (!aligned16(cols) || !aligned16(y)) return false;
+    const long long quads = (long long)B * (P / 4), blocks = (quads + 255) / 256, groups = (K + kThinFwdGroup - 1) / kThinFwdGroup;
+    if (blocks > kMaxGridX || groups > 65535) return false;
+    hipLaunchKernelGGL(thin_fwd_kernel, dim3((unsigned)blocks, (unsigned)groups), dim3(256), 0, st, cols, w, y, (int)CK,
+                       (int)(P / 4), K, quads);
+    return true;
+}
+
+}  // namespace ag
+
 extern "C" ag_status_t ag_conv2d_fwd_f32(ag_stream_t stream, const float *x, const float *w, float *y,
                                          float *cols, int B, int C, int H, int W, int K, int kh, int kw,
                                          int pad, int stride, int dilation)
@@ -34,6 +92,7 @@ extern "C" ag_status_t ag_conv2d_fwd_f32(ag_stream_t stream, const float *x, con
     if (ag_status_t s = ag_im2col_f32(stream, x, cols, B, C, H, W, kh, kw, pad, pad, stride, stride, dilation,
                                       dilation))
         return s;
+    if (w && y && cols && ag::thin_fwd(as_stream(stream), cols, w, y, B, CK, P, K)) return check_launch("conv2d");
     return ag_gemm_f32(stream, 0, 0, K, (int)P, (int)CK, 1.f, w, (int)CK, 0, cols, (int)P, CK * P, 0.f, y,
                        (int)P, (long long)K * P, B);
 }
@@ -41,6 +100,8 @@ extern "C" ag_status_t ag_conv2d_fwd_f32(ag_stream_t stream, const float *x, con
 extern "C" ag_status_t ag_conv2d_with_cols_f32(ag_stream_t stream, const float *cols, const float *w,
                                                float *y, int B, int CK, int P, int K)
 {
+    if (w && y && cols && B >= 0 && CK >= 0 && P >= 0 && K >= 0 && ag::thin_fwd(as_stream(stream), cols, w, y, B, CK, P, K))
+        return check_launch("conv2d_with_cols");
     return ag_gemm_f32(stream, 0, 0, K, P, CK, 1.f, w, CK, 0, cols, P, (long long)CK * P, 0.f, y, P,
                        (long long)K * P, B);
 }

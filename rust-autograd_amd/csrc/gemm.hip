@@ -532,6 +532,8 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
         // The cheapest tile among those that give the chip at least half a round of blocks: padded
         // area over efficiency, counted in whole rounds of the persistent grid while there are few
         // of them (264 blocks on 256 CUs take two rounds, 200 take one).
+        // up to 64 output rows: the 128-row tiles would spend half of their matrix work on padding
+        if (M <= 64 && cdiv(N, kCfgs[kDirectCfg64].bn) * zcount >= direct_grid(num_cus()) / 2) return kDirectCfg64;
         int best = -1;
         double best_cost = 1e300;
         for (int c = 0; c < 6; ++c) {

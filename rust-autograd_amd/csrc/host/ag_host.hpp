@@ -64,6 +64,11 @@ class NdArray {
     static NdArray filled(const Shape &shape, float value);
     static NdArray from_host(const Shape &shape, const float *data);
     static NdArray scalar(float v) { return filled({}, v); }
+    // A 0-dimensional 0.0 that every caller shares (the reference's NdArray::zeros(vec![]) of an op
+    // without a result, src/op.rs:290-294); nothing writes to it.
+    static NdArray shared_zero();
+    // Identity of the allocation behind the array (views of one allocation compare equal).
+    const void *allocation() const { return block_.get(); }
 
     const Shape &shape() const { return shape_; }
     int ndim() const { return (int)shape_.size(); }
@@ -127,6 +132,26 @@ struct TensorInternal {  // src/tensor.rs:408-441
 // ---------------------------------------------------------------------------------------------
 // Op and its contexts                                                     src/op.rs:90-434
 // ---------------------------------------------------------------------------------------------
+// In-place Adam updates of one evaluation, collected so that they go out as one launch over all
+// parameters instead of one per AdamOp node.  The evaluator flushes the batch before any node that
+// reads an array the batch writes, so every node sees what it would have seen had each update run
+// at its own node.
+struct AdamJob {
+    NdArray p, g, m, v, t;
+    float alpha, eps, b1, b2;
+};
+class DeferredUpdates {
+  public:
+    void add(AdamJob job);                     // flushes first if the job touches an array of the batch
+    bool writes(const NdArray &a) const;       // is `a` one of the batch's param / m / v / t arrays?
+    bool reads(const NdArray &a) const;        // is `a` one of the batch's gradient arrays?
+    bool empty() const { return jobs_.empty(); }
+    void flush();
+
+  private:
+    std::vector<AdamJob> jobs_;
+};
+
 class ComputeContext {
   public:
     enum class InputKind { NonVariable, RdOnlyVariable, RdWrVariable };
@@ -135,7 +160,8 @@ class ComputeContext {
         InputKind kind;
         bool taken = false;
     };
-    explicit ComputeContext(std::vector<Input> xs) : xs_(std::move(xs)) {}
+    explicit ComputeContext(std::vector<Input> xs, DeferredUpdates *deferred = nullptr)
+        : xs_(std::move(xs)), deferred_(deferred) {}
 
     // Each input may be grabbed once; variable inputs registered with allow_mut must be grabbed
     // with input_mut (src/op.rs:206-259).
@@ -146,7 +172,9 @@ class ComputeContext {
     void append_output(NdArray y) { ys_.push_back(std::move(y)); }
     // A view of an input: copied first when any input is a variable (src/op.rs:273-287).
     void append_output_view(const NdArray &y);
-    void append_empty_output() { ys_.push_back(NdArray::zeros({})); }  // src/op.rs:290-294
+    void append_empty_output() { ys_.push_back(NdArray::shared_zero()); }  // src/op.rs:290-294
+    // An Adam update: joins the evaluation's batch, or runs at once when there is none.
+    void adam_update(AdamJob job);
 
     std::vector<NdArray> &outputs() { return ys_; }
     void *stream() const { return current_stream(); }
@@ -154,6 +182,7 @@ class ComputeContext {
   private:
     std::vector<Input> xs_;
     std::vector<NdArray> ys_;
+    DeferredUpdates *deferred_;
 };
 
 class GradientContext {

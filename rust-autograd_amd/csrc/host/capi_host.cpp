@@ -1,4 +1,7 @@
 // extern "C" wrapper of the host operator layer (see include/ag_host.h).
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <exception>
 
@@ -295,11 +298,23 @@ int agh_eval(agh_ctx *c, const int *tensors, int n, const char *const *feed_name
     return guard([&] {
         std::vector<Tensor> ts;
         for (int i = 0; i < n; ++i) ts.push_back(T(c, tensors[i]));
+        static const bool timing = [] {
+            const char *e = std::getenv("AG_HOST_TRACE");
+            return e && std::string(e) == "time";
+        }();
+        const auto t0 = std::chrono::steady_clock::now();
         std::vector<std::pair<std::string, NdArray>> feeds;
         for (int i = 0; i < n_feeds; ++i)
             feeds.emplace_back(feed_names[i], NdArray::from_host(to_shape(feed_shapes[i], feed_ranks[i]), feed_data[i]));
+        const auto t1 = std::chrono::steady_clock::now();
         c->results = c->ctx.eval(ts, feeds);
+        const auto t2 = std::chrono::steady_clock::now();
         synchronize();
+        if (timing) {
+            const auto t3 = std::chrono::steady_clock::now();
+            auto us = [](auto a, auto b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+            std::fprintf(stderr, "[ag_host] eval: feeds %.1f us, enqueue %.1f us, wait %.1f us\n", us(t0, t1), us(t1, t2), us(t2, t3));
+        }
         return 0;
     });
 }

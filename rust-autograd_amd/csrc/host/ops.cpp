@@ -1055,8 +1055,8 @@ struct AdamOp : Op {
         NdArray m = ctx.input_mut(2), v = ctx.input_mut(3), p = ctx.input_mut(0);
         if (g.len() != p.len() || m.len() != p.len() || v.len() != p.len())
             return OpError::make(ErrorKind::IncompatibleShape, "AdamOp: parameter, gradient and moment shapes differ");
-        const OpError e = from_status(ag_adam_update_f32(ctx.stream(), p.ptr(), g.ptr(), m.ptr(), v.ptr(), t.ptr(), p.len(), alpha, eps, b1, b2));
-        if (!e.ok()) return e;
+        if (t.len() < 1) return OpError::make(ErrorKind::IncompatibleShape, "AdamOp: empty step counter");
+        ctx.adam_update(AdamJob{p, g, m, v, t, alpha, eps, b1, b2});
         ctx.append_empty_output();
         return OpError::none();
     }

@@ -3,6 +3,8 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <stdexcept>
 
@@ -110,24 +112,100 @@ NdArray NdArray::filled(const Shape &shape, float value)
 
 NdArray NdArray::zeros(const Shape &shape) { return filled(shape, 0.f); }
 
+NdArray NdArray::shared_zero()
+{
+    static const NdArray zero = zeros({});
+    return zero;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host-to-device uploads go through a page-locked staging ring: the caller's array is copied into
+// it on the host and the DMA is enqueued without waiting, so a feed costs a memcpy instead of a
+// pageable-memory transfer plus a device synchronisation.  The caller's buffer is free for reuse
+// when upload() returns.  Arrays larger than the ring take the synchronous path.
+// ---------------------------------------------------------------------------------------------
+namespace {
+class StagingRing {
+  public:
+    static constexpr size_t kBytes = 16u << 20;
+    ~StagingRing()
+    {
+        if (base_) (void)hipHostFree(base_);
+        if (drained_) (void)hipEventDestroy(drained_);
+    }
+    // Device-to-host through the same ring; returns after the data has arrived in `dst`.
+    void download(void *dst, const void *src, size_t bytes)
+    {
+        hipStream_t st = static_cast<hipStream_t>(current_stream());
+        if (bytes > kBytes) {
+            check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, st), "hipMemcpy D2H");
+            synchronize();
+            return;
+        }
+        std::lock_guard<std::mutex> lk(mu_);
+        reserve();
+        // the synchronisation below drains every earlier transfer, so the whole ring is free
+        check(hipMemcpyAsync(base_, src, bytes, hipMemcpyDeviceToHost, st), "hipMemcpy D2H");
+        synchronize();
+        used_ = 0;
+        pending_ = false;
+        std::memcpy(dst, base_, bytes);
+    }
+    void upload(void *dst, const void *src, size_t bytes)
+    {
+        hipStream_t st = static_cast<hipStream_t>(current_stream());
+        if (bytes > kBytes) {
+            check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st), "hipMemcpy H2D");
+            synchronize();
+            return;
+        }
+        std::lock_guard<std::mutex> lk(mu_);
+        reserve();
+        const size_t need = (bytes + 255) / 256 * 256;
+        if (used_ + need > kBytes) {
+            // wrap: every transfer enqueued so far must have left the ring
+            if (pending_) check(hipEventSynchronize(drained_), "hipEventSynchronize");
+            used_ = 0;
+            pending_ = false;
+        }
+        char *slot = static_cast<char *>(base_) + used_;
+        std::memcpy(slot, src, bytes);
+        check(hipMemcpyAsync(dst, slot, bytes, hipMemcpyHostToDevice, st), "hipMemcpy H2D");
+        check(hipEventRecord(drained_, st), "hipEventRecord");
+        used_ += need;
+        pending_ = true;
+    }
+
+  private:
+    void reserve()
+    {
+        if (base_) return;
+        check(hipHostMalloc(&base_, kBytes, hipHostMallocDefault), "hipHostMalloc");
+        check(hipEventCreateWithFlags(&drained_, hipEventDisableTiming), "hipEventCreate");
+    }
+    std::mutex mu_;
+    void *base_ = nullptr;
+    hipEvent_t drained_ = nullptr;
+    size_t used_ = 0;
+    bool pending_ = false;
+};
+StagingRing &staging()
+{
+    static StagingRing r;
+    return r;
+}
+}  // namespace
+
 NdArray NdArray::from_host(const Shape &shape, const float *data)
 {
     NdArray a = empty(shape);
-    if (a.len())
-        check(hipMemcpyAsync(a.ptr(), data, a.len() * sizeof(float), hipMemcpyHostToDevice,
-                             static_cast<hipStream_t>(current_stream())),
-              "hipMemcpy H2D");
-    synchronize();  // the host buffer may be reused by the caller
+    if (a.len()) staging().upload(a.ptr(), data, a.len() * sizeof(float));
     return a;
 }
 
 void NdArray::copy_from_host(const float *data)
 {
-    if (len())
-        check(hipMemcpyAsync(ptr(), data, len() * sizeof(float), hipMemcpyHostToDevice,
-                             static_cast<hipStream_t>(current_stream())),
-              "hipMemcpy H2D");
-    synchronize();
+    if (len()) staging().upload(ptr(), data, len() * sizeof(float));
 }
 
 NdArray NdArray::reshaped(const Shape &shape) const
@@ -151,11 +229,8 @@ NdArray NdArray::deep_copy() const
 std::vector<float> NdArray::to_host() const
 {
     std::vector<float> out(len());
-    if (len())
-        check(hipMemcpyAsync(out.data(), ptr(), len() * sizeof(float), hipMemcpyDeviceToHost,
-                             static_cast<hipStream_t>(current_stream())),
-              "hipMemcpy D2H");
-    synchronize();
+    if (len()) staging().download(out.data(), ptr(), len() * sizeof(float));
+    else synchronize();
     return out;
 }
 
@@ -187,6 +262,68 @@ NdArray ComputeContext::input_mut(size_t i)
                     ") cannot be called twice");
     x.taken = true;
     return x.array;
+}
+
+void ComputeContext::adam_update(AdamJob job)
+{
+    if (deferred_) {
+        deferred_->add(std::move(job));
+        return;
+    }
+    DeferredUpdates one;
+    one.add(std::move(job));
+    one.flush();
+}
+
+bool DeferredUpdates::writes(const NdArray &a) const
+{
+    const void *id = a.allocation();
+    for (const AdamJob &j : jobs_)
+        if (id == j.p.allocation() || id == j.m.allocation() || id == j.v.allocation() || id == j.t.allocation()) return true;
+    return false;
+}
+
+bool DeferredUpdates::reads(const NdArray &a) const
+{
+    for (const AdamJob &j : jobs_)
+        if (a.allocation() == j.g.allocation()) return true;
+    return false;
+}
+
+void DeferredUpdates::add(AdamJob job)
+{
+    bool clash = false;
+    for (const AdamJob &j : jobs_) {
+        // another optimizer's coefficients, or a gradient that the batch is about to overwrite / a
+        // parameter that the batch still reads as a gradient
+        clash |= j.alpha != job.alpha || j.eps != job.eps || j.b1 != job.b1 || j.b2 != job.b2;
+        clash |= job.p.allocation() == j.g.allocation() || job.m.allocation() == j.g.allocation() ||
+                 job.v.allocation() == j.g.allocation() || job.t.allocation() == j.g.allocation();
+    }
+    clash |= writes(job.p) || writes(job.g) || writes(job.m) || writes(job.v) || writes(job.t);
+    if (clash || (int)jobs_.size() == ag_adam_update_multi_max()) flush();
+    jobs_.push_back(std::move(job));
+}
+
+void DeferredUpdates::flush()
+{
+    if (jobs_.empty()) return;
+    std::vector<float *> p, m, v, t;
+    std::vector<const float *> g;
+    std::vector<size_t> n;
+    for (const AdamJob &j : jobs_) {
+        p.push_back(j.p.ptr());
+        g.push_back(j.g.ptr());
+        m.push_back(j.m.ptr());
+        v.push_back(j.v.ptr());
+        t.push_back(j.t.ptr());
+        n.push_back(j.p.len());
+    }
+    const AdamJob &h = jobs_.front();
+    const ag_status_t st = ag_adam_update_multi_f32(current_stream(), (int)jobs_.size(), p.data(), g.data(), m.data(),
+                                                    v.data(), t.data(), n.data(), h.alpha, h.eps, h.b1, h.b2);
+    jobs_.clear();
+    if (st != AG_OK) throw std::runtime_error(ag_last_error());
 }
 
 void ComputeContext::append_output_view(const NdArray &y)
@@ -325,12 +462,38 @@ const NdArray *find_placeholder(const std::vector<std::pair<std::string, NdArray
         }
     throw Panic("Placeholder unfilled: " + n.placeholder_name);
 }
+
+// AG_HOST_TRACE=1 in the environment lists every evaluated node on stderr (op, inputs, output shapes)
+bool trace_enabled()
+{
+    static const bool on = [] {
+        const char *e = std::getenv("AG_HOST_TRACE");
+        return e && std::string(e) == "1";
+    }();
+    return on;
+}
+
+void trace_node(const TensorInternal &n, const std::vector<NdArray> &outputs, const OpError &status)
+{
+    std::string line = "[ag_host] #" + std::to_string(n.id) + " " + n.op->name() + "(";
+    for (size_t i = 0; i < n.incoming_nodes.size(); ++i)
+        line += (i ? ", #" : "#") + std::to_string(n.incoming_nodes[i].id);
+    line += ") ->";
+    for (const NdArray &y : outputs) {
+        line += " [";
+        for (size_t i = 0; i < y.shape().size(); ++i) line += (i ? "," : "") + std::to_string(y.shape()[i]);
+        line += "]";
+    }
+    if (!status.ok()) line += " error: " + status.message;
+    std::fprintf(stderr, "%s\n", line.c_str());
+}
 }  // namespace
 
 std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
                                       const std::vector<std::pair<std::string, NdArray>> &feeds)
 {
     std::unordered_map<TensorID, StorageEntry> storage;  // every output lives until eval returns
+    DeferredUpdates deferred;                            // in-place optimizer updates, batched
     auto would_not_visit = [&](const TensorInternal &n) {
         return n.is_placeholder || n.is_variable() || storage.count(n.id) != 0;
     };
@@ -367,12 +530,20 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
             }
             StorageEntry entry;
             if (status.ok()) {
-                ComputeContext cc(std::move(inputs));
+                if (!deferred.empty())
+                    for (const ComputeContext::Input &x : inputs)
+                        if (deferred.writes(x.array) ||
+                            (x.kind == ComputeContext::InputKind::RdWrVariable && deferred.reads(x.array))) {
+                            deferred.flush();
+                            break;
+                        }
+                ComputeContext cc(std::move(inputs), &deferred);
                 status = n.op->compute(cc);
                 if (status.ok()) {
                     if (cc.outputs().empty()) throw Panic("Bad op implementation: empty return value");
                     entry.outputs = std::move(cc.outputs());
                 }
+                if (trace_enabled()) trace_node(n, entry.outputs, status);
             }
             entry.error = status;
             storage.emplace(id, std::move(entry));
@@ -382,6 +553,7 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
                 if (!would_not_visit(node(in.id))) dfs.emplace_back(in.id, false);
         }
     }
+    deferred.flush();
     std::vector<EvalResult> ret;
     for (const Tensor &t : tensors) {
         const TensorInternal &n = node(t.id);

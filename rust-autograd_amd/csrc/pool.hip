@@ -100,6 +100,42 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float *__restric
     gx[flat] = acc;
 }
 
+// 2 x 2 windows at stride 2 over a plane with even extents: the windows tile the plane, so every input
+// pixel belongs to exactly one window and each thread writes the four pixels of its own window
+// (two 8-byte stores; a wave's stores cover two whole input rows of contiguous memory).
+template <bool EXACT>
+__global__ __launch_bounds__(256) void maxpool_bwd_tile2_kernel(const float *__restrict__ gy,
+                                                                const float *__restrict__ argmax,
+                                                                const uint8_t *__restrict__ taps,
+                                                                float *__restrict__ gx, PoolGeom g,
+                                                                long long outputs)
+{
+    const long long o = blockIdx.x * 256ll + threadIdx.x;
+    if (o >= outputs) return;
+    const int per_plane = g.OH * g.OW;
+    const long long plane = o / per_plane;
+    const int e = (int)(o - plane * per_plane);
+    const int oy = e / g.OW, ox = e - oy * g.OW;
+    const long long xbase = plane * (long long)g.H * g.W;
+    int tap;  // 0..3 = dy * 2 + dx, anything else = none
+    if (EXACT) {
+        tap = taps[o];
+    } else {
+        // whole-tensor offset -> tap inside this window (exact below 2^24 elements)
+        const long long a = (long long)argmax[o] - xbase - (long long)(2 * oy) * g.W - 2 * ox;
+        tap = a == 0 ? 0 : a == 1 ? 1 : a == g.W ? 2 : a == g.W + 1 ? 3 : kNoTap;
+    }
+    const float v = gy[o];
+    float2 top, bottom;
+    top.x = tap == 0 ? v : 0.f;
+    top.y = tap == 1 ? v : 0.f;
+    bottom.x = tap == 2 ? v : 0.f;
+    bottom.y = tap == 3 ? v : 0.f;
+    float *row = gx + xbase + (long long)(2 * oy) * g.W + 2 * ox;
+    *reinterpret_cast<float2 *>(row) = top;
+    *reinterpret_cast<float2 *>(row + g.W) = bottom;
+}
+
 constexpr int kPoolLdsBytes = 32 * 1024;
 // A plane that does not fit half of that is cut into bands of at most this many staged bytes:
 // eight resident blocks per CU measured better than fewer, larger ones (112x112 planes: 0.242 ms
@@ -525,6 +561,18 @@ extern "C" ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy,
     AG_REQUIRE(taps || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
                "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the tap bytes",
                (long long)B * C * H * W);
+    if (size == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && W % 4 != 0 && (reinterpret_cast<uintptr_t>(gx) & 7) == 0 &&
+        g.OH > 0 && g.OW > 0) {
+        const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);
+        if (taps)
+            hipLaunchKernelGGL(maxpool_bwd_tile2_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), gy,
+                               argmax, taps, gx, g, outputs);
+        else
+            hipLaunchKernelGGL(maxpool_bwd_tile2_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), gy,
+                               argmax, taps, gx, g, outputs);
+        return check_launch("max_pool2d_grad");
+    }
     if (stride == 2 && (size == 2 || size == 3) && W % 4 == 0 && W <= 256 && aligned16(gx) && g.OH > 0 && g.OW > 0 &&
         (long long)B * C * g.OH < 0x7fffffffLL && (long long)H * W < 0x7fffffffLL) {
         const int rpc = pool_chunk_rows(g.OH), chunks = (g.OH + rpc - 1) / rpc;

@@ -352,6 +352,19 @@ def adam_update(param, grad, m, v, t, alpha=1e-3, eps=1e-8, b1=0.9, b2=0.999):
                                         param.numel(), alpha, eps, b1, b2))
 
 
+def adam_update_multi(params, grads, ms, vs, ts, alpha=1e-3, eps=1e-8, b1=0.9, b2=0.999):
+    """One optimizer step over several parameters (one AdamOp::compute each in the reference) as one launch."""
+    import ctypes as C
+    n = len(params)
+    assert len(grads) == len(ms) == len(vs) == len(ts) == n
+    for a in (*params, *grads, *ms, *vs, *ts):
+        assert a.is_cuda and a.dtype == torch.float32 and a.is_contiguous()
+    table = lambda xs: (C.c_void_p * max(n, 1))(*[x.data_ptr() for x in xs])
+    sizes = (C.c_size_t * max(n, 1))(*[p.numel() for p in params])
+    check(capi.lib().ag_adam_update_multi_f32(_stream(), n, table(params), table(grads), table(ms), table(vs), table(ts),
+                                              sizes, alpha, eps, b1, b2))
+
+
 def relu(x):
     x = _f32(x, "relu")
     y = torch.empty_like(x)

@@ -13,6 +13,7 @@ C_TO_RUST = {
     "ag_status_t": "AgStatus", "ag_stream_t": "AgStream", "int": "c_int", "long long": "c_longlong", "size_t": "usize",
     "float": "f32", "void": "()",
     "const float *": "*const f32", "float *": "*mut f32", "const float *const *": "*const *const f32",
+    "float *const *": "*const *mut f32", "const size_t *": "*const usize",
     "void *": "*mut c_void", "const void *": "*const c_void", "const int *": "*const c_int", "int *": "*mut c_int",
     "uint8_t *": "*mut u8", "const uint8_t *": "*const u8", "const char *": "*const c_char",
 }

@@ -48,6 +48,8 @@ extern "C" {
     pub fn ag_reduce_sum_f32(stream: AgStream, x: *const f32, out: *mut f32, shape: *const c_int, rank: c_int, axes: *const c_int, n_axes: c_int, mean: c_int, ws: *mut c_void, ws_bytes: usize) -> AgStatus;
     pub fn ag_broadcast_grad_f32(stream: AgStream, gy: *const f32, gx: *mut f32, shape: *const c_int, rank: c_int, axes: *const c_int, n_axes: c_int) -> AgStatus;
     pub fn ag_adam_update_f32(stream: AgStream, param: *mut f32, grad: *const f32, m: *mut f32, v: *mut f32, t: *mut f32, n: usize, alpha: f32, eps: f32, b1: f32, b2: f32) -> AgStatus;
+    pub fn ag_adam_update_multi_max() -> c_int;
+    pub fn ag_adam_update_multi_f32(stream: AgStream, count: c_int, params: *const *mut f32, grads: *const *const f32, ms: *const *mut f32, vs: *const *mut f32, ts: *const *mut f32, ns: *const usize, alpha: f32, eps: f32, b1: f32, b2: f32) -> AgStatus;
     pub fn ag_relu_f32(stream: AgStream, x: *const f32, y: *mut f32, n: usize) -> AgStatus;
     pub fn ag_relu_grad_f32(stream: AgStream, x: *const f32, gy: *const f32, gx: *mut f32, n: usize) -> AgStatus;
     pub fn ag_add_bias_f32(stream: AgStream, x: *const f32, bias: *const f32, y: *mut f32, rows: usize, cols: usize) -> AgStatus;

@@ -462,6 +462,37 @@ def test_variables_are_shared_between_contexts_and_updated_in_place(G, orc, rng)
     assert np.abs(env.array(wid) - (wv - 1.0)).max() < 0.05
 
 
+def test_batched_adam_updates_keep_the_evaluation_order(G, orc, rng):
+    """The AdamOp nodes of one evaluation go out as one launch, but a node that reads a variable after its
+    AdamOp ran must see the updated array, exactly as if every update had run at its own node.  The evaluator
+    visits the last requested tensor first (src/evaluation.rs:267-272), so in [read, update] the update runs
+    before the read and in [update, read] after it."""
+    for update_first in (True, False):
+        env = G.VariableEnvironment()
+        wv = rng.random((6, 5), dtype=np.float32) + 1.0
+        bv = rng.random((1, 5), dtype=np.float32) + 1.0
+        wid, bid = env.set("w", wv), env.set("b", bv)
+        adam = G.Adam(env, [wid, bid], alpha=0.25)
+        c = env.context()
+        w, b = c.variable(wid), c.variable(bid)
+        gw, gb = c.grad([c.sum_all(c.mul(w, w)) + c.sum_all(c.mul(b, b))], [w, b])
+        update = adam.get_update_op([w, b], [gw, gb], c)
+        read = c.mul(w, w)
+        wanted = [read, update] if update_first else [update, read]
+        out = c.eval(wanted)
+        got = out[0] if update_first else out[1]
+        p, m, v, t = wv.copy(), np.zeros_like(wv), np.zeros_like(wv), np.ones(1, np.float32)
+        orc.adam(p, (wv + wv).astype(np.float32), m, v, t, alpha=0.25)
+        assert_close(env.array(wid), p, "w after the step")
+        if update_first:
+            assert np.array_equal(got, env.array(wid) ** 2), "the read ran after the update and sees the new array"
+        else:
+            assert np.array_equal(got, wv * wv), "the read ran before the update and sees the old array"
+        pb, mb, vb = bv.copy(), np.zeros_like(bv), np.zeros_like(bv)
+        orc.adam(pb, (bv + bv).astype(np.float32), mb, vb, np.ones(1, np.float32), alpha=0.25)
+        assert_close(env.array(bid), pb, "b after the step")
+
+
 # ------------------------------------------------------------------------------- the reference's own gradient tests
 def check_theoretical_grads(G, env, c, objective, gradients, var_ids, eps=1e-2, tol=2e-2):
     """src/test_helper.rs:9-140: the analytic gradients of sum_all(objective) w.r.t. shared variables

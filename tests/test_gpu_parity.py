@@ -894,6 +894,8 @@ POOL_CASES = [(2, 3, 6, 6, 2, 2), (2, 3, 7, 9, 3, 2), (1, 2, 8, 8, 3, 1), (3, 32
               # stride-2 register kernels: one lane group per plane, 4 .. 64 lanes per row, chunked rows
               (2, 3, 8, 4, 2, 2), (1, 2, 64, 64, 3, 2), (1, 2, 30, 128, 3, 2), (1, 1, 9, 256, 2, 2),
               (5, 3, 40, 12, 3, 2), (1, 1, 4, 4, 3, 2), (7, 1, 5, 8, 3, 2), (3, 2, 27, 20, 2, 2),
+              # 2x2 windows tiling an even plane whose width is not a multiple of four: one thread per window
+              (4, 64, 14, 14, 2, 2), (3, 5, 6, 2, 2, 2), (1, 2, 10, 30, 2, 2),
               # other windows: the tap byte through the staged and the direct kernels
               (2, 2, 17, 19, 5, 3), (1, 2, 20, 24, 4, 4), (1, 1, 3, 9000, 3, 2), (1, 2, 16, 16, 15, 1)]
 
@@ -1132,6 +1134,45 @@ def test_adam_matches_oracle_over_steps(K, orc, rng, n):
     assert np.array_equal(host(md).view(np.uint32), m.view(np.uint32))
     assert np.array_equal(host(vd).view(np.uint32), v.view(np.uint32))
     assert_close(host(pd), p, "adam param")
+
+
+def test_adam_several_parameters_in_one_launch(K, rng):
+    """ag_adam_update_multi_f32 against one ag_adam_update_f32 per parameter: bit-identical param, m, v and t
+    over three steps; sizes with partial quads, one element, an empty parameter and a misaligned one."""
+    sizes = [25088, 1, 0, 4099, 288, 31360, 10, 7]
+    def fresh():
+        r = np.random.default_rng(3)
+        ps = [dev(r.standard_normal(n + 1).astype(np.float32)) for n in sizes]
+        ps = [p[1:] if i == 3 else p[:n] for i, (p, n) in enumerate(zip(ps, sizes))]   # parameter 3 is only 4-byte aligned
+        ms = [torch.zeros(n, device="cuda") for n in sizes]
+        vs = [torch.zeros(n, device="cuda") for n in sizes]
+        ts = [torch.full((1,), float(1 + i), device="cuda") for i in range(len(sizes))]  # different step counts
+        return ps, ms, vs, ts
+    a, b = fresh(), fresh()
+    assert a[0][3].data_ptr() % 16 != 0
+    for step in range(3):
+        gs = [dev(rng.standard_normal(n).astype(np.float32)) for n in sizes]
+        say("adam multi", step)
+        K.adam_update_multi(a[0], gs, a[1], a[2], a[3])
+        for p, g, m, v, t in zip(b[0], gs, b[1], b[2], b[3]):
+            K.adam_update(p, g, m, v, t)
+    for xs, ys in zip(a, b):
+        for x, y in zip(xs, ys):
+            assert np.array_equal(host(x).view(np.uint32), host(y).view(np.uint32))
+    assert [float(t) for t in a[3]] == [4.0 + i for i in range(len(sizes))]
+
+
+def test_adam_multi_rejects_shared_arrays_and_too_many(K):
+    p = torch.zeros(8, device="cuda")
+    g, m, v, t = (torch.zeros(8, device="cuda") for _ in range(4))
+    t2 = torch.ones(1, device="cuda")
+    with pytest.raises(K.capi.InvalidDims, match="share an array"):
+        K.adam_update_multi([p, p], [g, g], [m, torch.zeros(8, device="cuda")], [v, torch.zeros(8, device="cuda")], [t, t2])
+    many = K.capi.lib().ag_adam_update_multi_max() + 1
+    xs = lambda: [torch.zeros(4, device="cuda") for _ in range(many)]
+    with pytest.raises(K.capi.InvalidDims, match="at most"):
+        K.adam_update_multi(xs(), xs(), xs(), xs(), xs())
+    K.adam_update_multi([], [], [], [], [])
 
 
 def test_adam_first_step_closed_form(K, rng):

@@ -20,6 +20,8 @@ COMPATIBLE = {
     "const float*": {"*const f32"},
     "float*": {"*mut f32"},
     "const float*const*": {"*const *const f32"},
+    "float*const*": {"*const *mut f32"},
+    "const size_t*": {"*const usize"},
     "void*": {"*mut c_void"},
     "const int*": {"*const c_int", "*const i32"},
     "uint8_t*": {"*mut u8"},
