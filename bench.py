@@ -41,7 +41,8 @@ B, C, K, H, W, KH, PAD, STRIDE, DIL = 256, 64, 128, 56, 56, 3, 1, 1, 1
 # two rocprofv3 --pmc passes over this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled
 # by what the same counter reads for the --pmc-calibration copy kernel in the same pass (1 GiB in, 1 GiB out).
 # Each entry: summary file, then (kernel name, statistic) pairs whose scaled fetch + write are added up.
-# pad_border_fast_kernel runs twice per step (x with 64 channels, gy with 128): min is the x call, max the gy call.
+# pad_border_fast_kernel runs twice per step (x with 64 channels, gy with 128): min is the x call, max the gy call
+# (the same launch zeroes the slack around the planes and rewrites the filter in tap order).
 CALIBRATION_KERNEL = "ag::ew_vec_kernel<ag::ScaleF<false> >"
 CALIBRATION_KIB = float(1 << 20)
 _STEP, _POOL, _COLS = ("profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt", "profiles/maxpool_c4_hbm_traffic.txt",
@@ -52,8 +53,8 @@ PROFILE_TRAFFIC = {
     "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false", "avg")]),
     "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_kernel", "avg")]),
     "gemm_input_grad": (_STEP, [(_DL % "64, 128, 32, 32, 64, 3, true, false", "avg")]),
-    "fwd_prepare": (_STEP, [("ag::pad_border_fast_kernel", "min"), ("ag::zero_slack_kernel", "min"), ("ag::filter_taps_fwd_kernel", "avg")]),
-    "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max"), ("ag::zero_slack_kernel", "max"), ("ag::filter_taps_kernel", "avg")]),
+    "fwd_prepare": (_STEP, [("ag::pad_border_fast_kernel", "min")]),
+    "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max")]),
     # per-kernel section: pooling, and the column-materialising operators
     "maxpool_fwd": (_POOL, [("ag::maxpool_fwd_lds_kernel<3, 2>", "avg")]),
     "maxpool_bwd": (_POOL, [("ag::maxpool_bwd_s2_kernel<true, 3, 16>", "avg")]),

@@ -27,6 +27,20 @@ constexpr int kWave = 64;  // CDNA wavefront width
 // Largest grid.x HIP accepts.
 constexpr long long kMaxGridX = 2147483647LL;
 
+constexpr int kXcds = 8;
+
+#if defined(__HIPCC__)
+// Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
+// contiguous slice of the logical block range instead, so that blocks which touch neighbouring
+// memory share an L2 (partial cache lines at the seams of their outputs merge there).
+__device__ inline unsigned xcd_remap(unsigned id, unsigned total)
+{
+    const unsigned per = total / kXcds, rem = total % kXcds;
+    const unsigned xcd = id % kXcds, pos = id / kXcds;
+    return xcd * per + (xcd < rem ? xcd : rem) + pos;
+}
+#endif
+
 #if defined(__HIPCC__)
 // Streaming (non-temporal) accesses for data that is touched once: they do not displace the
 // operands other kernels keep in L2 and measured ~10 % faster than plain accesses on MI355X.

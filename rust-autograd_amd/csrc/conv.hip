@@ -277,14 +277,59 @@ __global__ __launch_bounds__(256) void pad_border_kernel(const float *__restrict
     }
 }
 
+// wr[c][tap][k] = w[k][c][tap]  (tap = ky*kw + kx): the filter as the k-contiguous left operand of
+// the implicit input-gradient GEMM.  Element e of wr.
+__device__ inline float filter_tap(const float *__restrict__ w, int e, int Kf, int C, int taps)
+{
+    const int k = e % Kf, tap = e / Kf % taps, c = e / (Kf * taps);
+    return w[((long long)k * C + c) * taps + tap];
+}
+
+// wf[k][tap'][c] = w[k][c][taps - 1 - tap']: the filter as the left operand of the implicit forward
+// GEMM.  The GEMM visits its taps from the largest shift to none (the order the input gradient
+// needs), so a correlation lists them reversed.  Element e of wf.
+__device__ inline float filter_tap_fwd(const float *__restrict__ w, int e, int C, int taps)
+{
+    const int c = e % C, tap = e / C % taps, k = e / (C * taps);
+    return w[((long long)k * C + c) * taps + (taps - 1 - tap)];
+}
+
+// The small jobs that accompany a bordered copy (see pad_border_fast_kernel).
+struct PrepareExtras {
+    float *lead;     // n_lead floats to zero before the planes
+    int n_lead;
+    float *tail;     // n_tail floats to zero after them
+    int n_tail;
+    const float *w;  // filter [Kf][C][taps] ...
+    float *wt;       // ... rewritten here (nullptr: not asked for)
+    int Kf, C, taps;
+    int fwd;         // 1: forward order (filter_tap_fwd), 0: input-gradient order (filter_tap)
+};
+
 // The same copy with the divisions replaced by multiplications: grid.y walks the images, so the
 // element counter stays small enough for n / d == umulhi(n, floor(2^32 / d) + 1) to be exact (the
 // host checks the range).  gyp [B][planes][Hp][Wp]; quads_img = planes * Hp * Wp / 4.
+// The last row of the grid (blockIdx.y == gridDim.y - 1) copies nothing: it does the two small jobs that go with
+// every bordered copy -- zeroing the slack around the planes and writing the filter in the tap order of the
+// implicit GEMM -- so that preparing an operand is one launch.
 __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__restrict__ gy, float *__restrict__ gyp,
                                                               unsigned quads_img, unsigned planes, int OH, int OW, int Wp,
                                                               int top, int left, unsigned plane_quads, unsigned m_plane,
-                                                              unsigned m_row, int B)
+                                                              unsigned m_row, int B, PrepareExtras ex)
 {
+    const unsigned ny = gridDim.y - 1;
+    if (blockIdx.y == ny) {
+        const int tid = (int)(blockIdx.x * 256u + threadIdx.x), nth = (int)(gridDim.x * 256u);
+        for (int i = tid; i < ex.n_lead + ex.n_tail; i += nth) {
+            if (i < ex.n_lead) ex.lead[i] = 0.f;
+            else ex.tail[i - ex.n_lead] = 0.f;
+        }
+        if (ex.wt) {
+            const int total = ex.Kf * ex.C * ex.taps;
+            for (int e = tid; e < total; e += nth) ex.wt[e] = ex.fwd ? filter_tap_fwd(ex.w, e, ex.C, ex.taps) : filter_tap(ex.w, e, ex.Kf, ex.C, ex.taps);
+        }
+        return;
+    }
     const unsigned qi = blockIdx.x * 256u + threadIdx.x;
     if (qi >= quads_img) return;
     const unsigned pl = __umulhi(qi, m_plane);
@@ -301,7 +346,7 @@ __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__res
             ++r;
         }
     }
-    for (int b = blockIdx.y; b < B; b += gridDim.y) {
+    for (int b = blockIdx.y; b < B; b += ny) {
         const float *src = gy + ((long long)b * planes + pl) * (long long)OH * OW;
         float v[4];
 #pragma unroll
@@ -311,9 +356,10 @@ __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__res
     }
 }
 
-// Launches the bordered copy of `planes` planes per image.
-void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp, int Wp,
-                              int top, int left)
+// Launches the bordered copy of `planes` planes per image.  With `extras` the same launch also zeroes the slack
+// and rewrites the filter when it can (returns true); otherwise the caller launches those itself.
+static bool launch_pad_border_with(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp,
+                                   int Wp, int top, int left, const PrepareExtras *extras)
 {
     const long long plane_quads = (long long)Hp * Wp / 4, quads_img = plane_quads * planes;
     // exactness of the two multiply-high divisions: n * (m * d - 2^32) < 2^32 with m * d - 2^32 <= d
@@ -321,15 +367,26 @@ void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int 
     if (fast) {
         const unsigned m_plane = (unsigned)((1ULL << 32) / (unsigned long long)plane_quads) + 1u;
         const unsigned m_row = (unsigned)((1ULL << 32) / (unsigned long long)Wp) + 1u;
-        const dim3 grid((unsigned)((quads_img + 255) / 256), (unsigned)(B < 65535 ? B : 65535));
+        // one grid row per image (at most 65534) plus the row of the small jobs
+        const dim3 grid((unsigned)((quads_img + 255) / 256), (unsigned)(B < 65534 ? B : 65534) + 1u);
+        const bool fits = extras && (!extras->wt || (long long)extras->Kf * extras->C * extras->taps < 0x7fffffffLL);
+        PrepareExtras ex = {};
+        if (fits) ex = *extras;
         hipLaunchKernelGGL(pad_border_fast_kernel, grid, dim3(256), 0, st, src, dst, (unsigned)quads_img, (unsigned)planes, OH, OW,
-                           Wp, top, left, (unsigned)plane_quads, m_plane, m_row, B);
-        return;
+                           Wp, top, left, (unsigned)plane_quads, m_plane, m_row, B, ex);
+        return fits;
     }
     const long long quads = quads_img * B;
     long long blocks = (quads + 255) / 256;
     if (blocks > 1048576) blocks = 1048576;
     hipLaunchKernelGGL(pad_border_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src, dst, quads, OH, OW, Hp, Wp, top, left);
+    return false;
+}
+
+void launch_pad_border(hipStream_t st, const float *src, float *dst, int B, int planes, int OH, int OW, int Hp, int Wp,
+                       int top, int left)
+{
+    launch_pad_border_with(st, src, dst, B, planes, OH, OW, Hp, Wp, top, left, nullptr);
 }
 
 // Zeroes the slack before and after the padded planes: the implicit filter gradient multiplies what
@@ -342,29 +399,20 @@ __global__ void zero_slack_kernel(float *lead, int n_lead, float *tail, int n_ta
     }
 }
 
-// wr[c][tap][k] = w[k][c][tap]  (tap = ky*kw + kx): the filter as the k-contiguous left operand of
-// the implicit input-gradient GEMM.
+// The filter in input-gradient order (filter_tap) as a launch of its own.
 __global__ __launch_bounds__(256) void filter_taps_kernel(const float *__restrict__ w, float *__restrict__ wr, int Kf,
                                                           int C, int taps)
 {
     const int total = Kf * C * taps;
-    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
-        const int k = e % Kf, tap = e / Kf % taps, c = e / (Kf * taps);
-        wr[e] = w[((long long)k * C + c) * taps + tap];
-    }
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) wr[e] = filter_tap(w, e, Kf, C, taps);
 }
 
-// wf[k][tap'][c] = w[k][c][taps - 1 - tap']: the filter as the left operand of the implicit forward
-// GEMM.  The GEMM visits its taps from the largest shift to none (the order the input gradient
-// needs), so a correlation lists them reversed.
+// The filter in forward order (filter_tap_fwd) as a launch of its own.
 __global__ __launch_bounds__(256) void filter_taps_fwd_kernel(const float *__restrict__ w, float *__restrict__ wf, int Kf,
                                                               int C, int taps)
 {
     const int total = Kf * C * taps;
-    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
-        const int c = e % C, tap = e / C % taps, k = e / (C * taps);
-        wf[e] = w[((long long)k * C + c) * taps + (taps - 1 - tap)];
-    }
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) wf[e] = filter_tap_fwd(w, e, C, taps);
 }
 
 // Zeroed floats after the last bordered plane (and before the first one of a bordered input).
@@ -413,12 +461,14 @@ static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w
                                  int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad)
 {
     const long long quads = (long long)B * ych * g.Hp * g.Wp / 4;
-    launch_pad_border(st, gy, scratch, B, ych, yh, yw, g.Hp, g.Wp, kh - 1 - pad, kw - 1 - pad);
     // the implicit filter gradient may read a few elements past the last plane and expects zeros
-    hipLaunchKernelGGL(zero_slack_kernel, dim3(4), dim3(256), 0, st, scratch, 0, scratch + quads * 4,
-                       (int)(g.gyp_floats - quads * 4));
-    hipLaunchKernelGGL(filter_taps_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w,
-                       scratch + g.gyp_floats, ych, xch, kh * kw);
+    const PrepareExtras ex = {scratch, 0, scratch + quads * 4, (int)(g.gyp_floats - quads * 4), w, scratch + g.gyp_floats,
+                              ych, xch, kh * kw, 0};
+    if (!launch_pad_border_with(st, gy, scratch, B, ych, yh, yw, g.Hp, g.Wp, kh - 1 - pad, kw - 1 - pad, &ex)) {
+        hipLaunchKernelGGL(zero_slack_kernel, dim3(4), dim3(256), 0, st, ex.lead, ex.n_lead, ex.tail, ex.n_tail);
+        hipLaunchKernelGGL(filter_taps_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w,
+                           scratch + g.gyp_floats, ych, xch, kh * kw);
+    }
     return check_launch("conv2d_transpose");
 }
 
@@ -491,11 +541,12 @@ extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const fl
                "conv2d (column-free): geometry not supported");
     float *xp = xpad + kFwdLeadFloats, *wf = xp + g.gyp_floats;
     const long long quads = (long long)B * C * g.Hp * g.Wp / 4;
-    launch_pad_border(st, x, xp, B, C, H, W, g.Hp, g.Wp, pad, pad);
-    hipLaunchKernelGGL(zero_slack_kernel, dim3(8), dim3(256), 0, st, xpad, (int)kFwdLeadFloats, xp + quads * 4,
-                       (int)(g.gyp_floats - quads * 4));
-    hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
-                       kh * kw);
+    const PrepareExtras ex = {xpad, (int)kFwdLeadFloats, xp + quads * 4, (int)(g.gyp_floats - quads * 4), w, wf, K, C, kh * kw, 1};
+    if (!launch_pad_border_with(st, x, xp, B, C, H, W, g.Hp, g.Wp, pad, pad, &ex)) {
+        hipLaunchKernelGGL(zero_slack_kernel, dim3(8), dim3(256), 0, st, ex.lead, ex.n_lead, ex.tail, ex.n_tail);
+        hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
+                           kh * kw);
+    }
     return check_launch("conv2d");
 }
 

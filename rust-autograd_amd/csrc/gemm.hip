@@ -489,7 +489,8 @@ static thread_local int g_force_cfg = -1;  // test hook (ag_test_hooks.h), per c
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
                                 {128, 128}, {192, 128}, {256, 128}, {128, 256}, {64, 64}, {128, 64},
                                 {128, 128}, {192, 128}, {128, 64},
-                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}, {64, 128}};
+                                {128, 128}, {128, 256}, {256, 128}, {192, 128}, {128, 192}, {128, 64}, {64, 128},
+                                {32, 128}, {64, 64}};
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 static void launch(hipStream_t st, int cfg, int la, int lb, const GemmParams &p)
 {
@@ -522,9 +523,11 @@ static long long cdiv(long long a, long long b) { return (a + b - 1) / b; }
 // block fall back to 64 x 64 tiles of the register-staged kernel.
 // `tail_split`: the launch will be cut into whole rounds plus a narrow-tile tail (folded batch with
 // one row of tiles), so a partly filled last round costs nothing here.
-static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bool direct, bool tail_split = false)
+// `a_kcontig`: A is k-contiguous (not transposed), which the 32-row tile needs.
+static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bool direct, bool tail_split = false,
+                      bool a_kcontig = false)
 {
-    if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg;
+    if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg == kDirectCfg32 && !a_kcontig ? kDirectCfg64 : g_force_cfg;
     if (direct) {
         // 128x256, 256x128, 192x128, 128x192, 128x128, and 64x128 (two blocks per CU) for outputs of up to 64 rows
         static const int dl[] = {14, 15, 16, 17, 13, kDirectCfg64};
@@ -532,8 +535,14 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
         // The cheapest tile among those that give the chip at least half a round of blocks: padded
         // area over efficiency, counted in whole rounds of the persistent grid while there are few
         // of them (264 blocks on 256 CUs take two rounds, 200 take one).
-        // up to 64 output rows: the 128-row tiles would spend half of their matrix work on padding
-        if (M <= 64 && cdiv(N, kCfgs[kDirectCfg64].bn) * zcount >= direct_grid(num_cus()) / 2) return kDirectCfg64;
+        // up to 64 (32) output rows: taller tiles would spend half of their matrix work on padding; a
+        // problem that gives the chip fewer than two 64 x 128 blocks per CU takes 64 x 64 tiles instead
+        const long long wide = cdiv(N, 128) * zcount, cus2 = direct_grid(num_cus());
+        if (M <= 32 && a_kcontig && wide >= cus2 / 2) return kDirectCfg32;
+        if (M <= 64 && wide >= cus2 / 2) return wide < 2 * cus2 ? kDirectCfg64Narrow : kDirectCfg64;
+        // fewer 128 x 128 tiles than CUs: 64 x 64 tiles (two or three blocks per CU) use the whole chip
+        if (!accumulate && cdiv(M, 128) * cdiv(N, 128) * zcount < cus2 && cdiv(M, 64) * cdiv(N, 64) * zcount >= cus2 / 2)
+            return kDirectCfg64Narrow;
         int best = -1;
         double best_cost = 1e300;
         for (int c = 0; c < 6; ++c) {
@@ -655,7 +664,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         // only when the body really lands on the direct-to-LDS kernel (enough tiles for it)
         const int eff_splits = splits < 1 ? 1 : (int)cdiv(c.kbatch, cdiv(c.kbatch, splits));
         if (direct_ok(body) &&
-            choose_cfg(body.M, body.N, body.K, (long long)body.batch * eff_splits, body.kbatch > 1, true) >= kFirstDirectCfg) {
+            choose_cfg(body.M, body.N, body.K, (long long)body.batch * eff_splits, body.kbatch > 1, true, false, !body.transA) >=
+                kFirstDirectCfg) {
             GemmCall rest = c;
             rest.K = c.K % 32;
             rest.beta = 1.f;
@@ -711,7 +721,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
                           !c.transB && c.N % 4 == 0 && (long long)c.N * c.batch < 0x7fffffffLL &&
                           c.sB < (1LL << 30) && c.sB % 4 == 0;
     int cfg = choose_cfg(c.M, foldable ? c.N * c.batch : c.N, c.K, foldable ? 1 : (long long)c.batch * p.splits,
-                         c.kbatch > 1, direct_ok(c), foldable && g_force_cfg < 0);
+                         c.kbatch > 1, direct_ok(c), foldable && g_force_cfg < 0, !c.transA);
     if (cfg >= kFirstDirectCfg && !direct_ok(c)) cfg = 0;  // a forced configuration that cannot run
     const bool fold = foldable && cfg >= kFirstDirectCfg && c.N >= kCfgs[cfg].bn;
     p.n_img = fold ? c.N : 0;
@@ -816,8 +826,11 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.conv_phase = phase;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
-    // 64 x 128 for up to 64 output rows, else 128 x 256, or 128 x 128 when an image has fewer than 256 columns
-    const int cfg = C <= 64 ? kDirectCfg64 : (p.n_img >= 256 ? 14 : 13);
+    // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
+    // CU); else 128 x 256, or 128 x 128 when an image has fewer than 256 columns
+    const int cfg = C <= 32   ? kDirectCfg32
+                    : C <= 64 ? (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64 ? kDirectCfg64Narrow : kDirectCfg64)
+                              : (p.n_img >= 256 ? 14 : 13);
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n;

@@ -632,7 +632,7 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
 {
     constexpr int NT = (BM / WM) * (BN / WN) * 64;
 #define AG_GEMM_DL_CASE(KA_, KB_)                                                                     \
-    if (ka == KA_ && kb == KB_) {                                                                     \
+    if constexpr ((KA_ || BM % 64 == 0) && (KB_ || BN % 64 == 0)) if (ka == KA_ && kb == KB_) {      \
         auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_>;                                 \
         long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \
         if (g >= p.total_blocks) g = p.total_blocks;        /* one item per block */                 \
@@ -657,6 +657,10 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
         case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
         case 18: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        // small problems: tiles that still give every CU a block or two
+        // (32 rows only with a k-contiguous A: an m-contiguous tile is swizzled in groups of 64 rows)
+        case 20: launch_dl<32, 128, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
+        case 21: launch_dl<64, 64, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
         default: launch_dl<64, 128, 32, 32, 64, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
     }
 }

@@ -50,21 +50,10 @@ struct GemmParams {
                           // channel*rows_plane + ((ky&1)*2 + (kx&1))*rows_phase + (ky>>1)*rows_wp + (kx>>1)
 };
 
-constexpr int kXcds = 8;
-
 // Elements of the contraction that one accumulation chain of the MFMA kernels covers before its sum
 // is set aside and the chain restarts from zero (both GEMM kernels; the length of an OpenBLAS
 // SGEMM k block, so rounding errors grow as they do in the reference's BLAS).
 constexpr int kChainK = 256;
-
-// Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
-// contiguous slice of the logical block range instead.
-__device__ inline unsigned xcd_remap(unsigned id, unsigned total)
-{
-    const unsigned per = total / kXcds, rem = total % kXcds;
-    const unsigned xcd = id % kXcds, pos = id / kXcds;
-    return xcd * per + (xcd < rem ? xcd : rem) + pos;
-}
 
 // Launches direct-to-LDS configuration `cfg` (kFirstDirectCfg ..); `ka` / `kb`: the operand is
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
@@ -92,5 +81,7 @@ ag_status_t gemm_conv_filter_grad_stride2(hipStream_t st, const float *gyq, cons
                                           size_t ws_bytes, int B, int Kf, int C, int kh, int kw, int Hq, int Hpp, int Wpp, int kq);
 // Direct-to-LDS configuration with a 64-row tile (64 x 128, two blocks per CU), used by the implicit input gradient.
 constexpr int kDirectCfg64 = 19;
+constexpr int kDirectCfg32 = 20;        // 32 x 128, k-contiguous A only
+constexpr int kDirectCfg64Narrow = 21;  // 64 x 64
 
 }  // namespace ag

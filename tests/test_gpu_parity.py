@@ -194,7 +194,7 @@ def test_gemm_every_tile_configuration(K, rng, cfg):
     assert_close(got_t, truth, "gemm TT")
 
 
-DIRECT_CFGS = list(range(13, 20))  # operand tiles loaded from global memory straight into LDS
+DIRECT_CFGS = list(range(13, 22))  # operand tiles loaded from global memory straight into LDS
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
