@@ -448,6 +448,13 @@ def micro_columns(torch, Kn, capi, dev, g, iters=10):
 def micro_rest(torch, Kn, capi, dev, g, iters=10):
     res = {}
     Bn, Kf, Hh = 256, 128, 56
+    # a plain copy (ag_scale_f32 by 1.0) of 2^28 floats: what a streaming kernel with one read and one write stream reaches
+    src = torch.ones(1 << 28, device=dev)
+    dst = torch.empty_like(src)
+    ms = time_events(torch, lambda: capi.check(capi.lib().ag_scale_f32(Kn._stream(), Kn._ptr(src), 1.0, Kn._ptr(dst), src.numel())), 10)
+    res["copy_2^28"] = {"ms": round(ms, 4), "GB/s": round(8.0 * src.numel() / ms / 1e6, 1),
+                        "frac_hbm": round(8.0 * src.numel() / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del src, dst
     # reduce_sum (to scalar) and Adam on 2^26 elements
     n = 1 << 26
     a = torch.randn(n, device=dev, generator=g)

@@ -29,6 +29,9 @@ constexpr long long kMaxGridX = 2147483647LL;
 
 constexpr int kXcds = 8;
 
+// Compute units of the current device (queried once per process; 256 when the query fails).
+int device_cus();
+
 #if defined(__HIPCC__)
 // Hardware hands consecutive workgroup ids to the XCDs round-robin; give XCD x the x-th
 // contiguous slice of the logical block range instead, so that blocks which touch neighbouring

@@ -49,3 +49,17 @@ int ag_pool_grad_in_size(int y, int size, int pad, int stride)
 }
 
 }  // extern "C"
+
+namespace ag {
+int device_cus()
+{
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            return n;
+        return 256;
+    }();
+    return cus;
+}
+}  // namespace ag

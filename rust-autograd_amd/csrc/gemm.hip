@@ -427,20 +427,7 @@ struct TileCfg {
 };
 
 // Resident blocks per CU of one kernel instantiation, and the CU count (both cached).
-static int query_cus()
-{
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-        return n;
-    return 256;
-}
-
-static int num_cus()
-{
-    static const int cus = query_cus();  // initialised once, thread-safe (C++11 static)
-    return cus;
-}
+static int num_cus() { return device_cus(); }
 
 // Blocks of the direct-to-LDS kernel's persistent grid: one per CU, a multiple of the XCD count.
 static long long direct_grid(int cus) { return cus >= kXcds ? cus - cus % kXcds : kXcds; }

@@ -215,9 +215,26 @@ __global__ __launch_bounds__(256) void maxpool_fwd_lds_kernel(const float *__res
     const float *xp = x + base + (long long)iy0 * g.W;
     const int n_in = in_rows * g.W;
     if (vec) {
+        // Four loads are in flight per thread before the first LDS write.  Written as a plain copy loop
+        // the compiler waits for every load before it issues the next, and a block pays the memory
+        // latency once per 4 KB instead of once per 16 KB (measured: 0.1135 -> 0.108 ms on the
+        // [256,128,56,56] 3x3 stride-2 case, whose planes take three loads per thread).
         const float4 *x4 = reinterpret_cast<const float4 *>(xp);
         float4 *t4 = reinterpret_cast<float4 *>(tile);
-        for (int e = threadIdx.x; e < n_in / 4; e += 256) t4[e] = ld_stream(x4 + e);
+        const int n4 = n_in / 4;
+        for (int e0 = 0; e0 < n4; e0 += 1024) {
+            float4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int e = e0 + j * 256 + threadIdx.x;
+                if (e < n4) v[j] = ld_stream(x4 + e);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int e = e0 + j * 256 + threadIdx.x;
+                if (e < n4) t4[e] = v[j];
+            }
+        }
     } else {
         for (int e = threadIdx.x; e < n_in; e += 256) tile[e] = xp[e];
     }
