@@ -310,13 +310,18 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    T.enabled = True
+    # the timed region: exactly `steps` steps, nothing but the step's own launches on the stream
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
+    # per-kernel durations: the same steps again with an event pair around every entry (the event
+    # records cost a few microseconds each on the stream, so they stay out of the timed region)
+    T.enabled = True
+    for _ in range(args.steps):
+        step()
     per = T.totals()
 
     gemm_flop = 2.0 * K * P * CK * Bn            # identical for the three contractions

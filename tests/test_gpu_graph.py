@@ -462,6 +462,27 @@ def test_variables_are_shared_between_contexts_and_updated_in_place(G, orc, rng)
     assert np.abs(env.array(wid) - (wv - 1.0)).max() < 0.05
 
 
+def test_feeds_and_read_backs_of_any_size_cross_the_staging_ring_intact(G, rng):
+    """Host arrays travel through a 16 MiB page-locked ring: many small feeds wrap it several times, a feed larger
+    than the ring takes the synchronous path, and the caller's buffer may be overwritten as soon as eval returns."""
+    env = G.VariableEnvironment()
+    c = env.context()
+    x = c.placeholder("x", [-1, 1024])
+    y = c.relu(x)
+    buf = np.empty((300, 1024), np.float32)                     # 1.2 MB per feed: the ring wraps every 13 feeds
+    for i in range(40):
+        buf[:] = rng.random((300, 1024), dtype=np.float32) + 0.5
+        want = buf.copy()
+        (got,) = c.eval([y], {"x": buf})
+        buf[:] = -1.0                                           # reuse of the caller's buffer must not reach the device
+        assert np.array_equal(got, want), f"feed {i}"
+    big = rng.random((5000, 1024), dtype=np.float32) + 0.5      # 20.5 MB > the ring
+    (got,) = c.eval([y], {"x": big})
+    assert np.array_equal(got, big)
+    wid = env.set("w", big)                                     # variables are uploaded the same way
+    assert np.array_equal(env.array(wid), big)
+
+
 def test_batched_adam_updates_keep_the_evaluation_order(G, orc, rng):
     """The AdamOp nodes of one evaluation go out as one launch, but a node that reads a variable after its
     AdamOp ran must see the updated array, exactly as if every update had run at its own node.  The evaluator
