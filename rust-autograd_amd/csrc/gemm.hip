@@ -418,6 +418,89 @@ __global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__restric
     }
 }
 
+// The same fold over four consecutive elements per thread (128 per block) with 128-bit loads, four
+// of them in flight per chain: per element the additions are the ones of splitk_fold_kernel in the
+// same order, so the two kernels give identical results.  Needs total, split_stride and N
+// multiples of four, ldc a multiple of four and 16-byte aligned partials and C.
+__global__ __launch_bounds__(256) void splitk_fold_vec_kernel(const float *__restrict__ partial, int splits,
+                                                              long long split_stride, float *__restrict__ C,
+                                                              int M, int N, long long ldc, float alpha,
+                                                              float beta)
+{
+    __shared__ float4 part[8][32];
+    const long long quads = (long long)M * N / 4, stride4 = split_stride / 4;
+    const float4 *p4 = reinterpret_cast<const float4 *>(partial);
+    const int q_in = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    for (long long q0 = blockIdx.x * 32LL; q0 < quads; q0 += gridDim.x * 32LL) {
+        const long long q = q0 + q_in;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (q < quads) {
+            int sidx = grp;
+            for (; sidx + 24 < splits; sidx += 32) {
+                float4 v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = p4[(sidx + 8 * u) * stride4 + q];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    acc.x += v[u].x;
+                    acc.y += v[u].y;
+                    acc.z += v[u].z;
+                    acc.w += v[u].w;
+                }
+            }
+            for (; sidx < splits; sidx += 8) {
+                const float4 v = p4[sidx * stride4 + q];
+                acc.x += v.x;
+                acc.y += v.y;
+                acc.z += v.z;
+                acc.w += v.w;
+            }
+        }
+        part[grp][q_in] = acc;
+        __syncthreads();
+        if (grp == 0 && q < quads) {
+            float4 sum = part[0][q_in];
+#pragma unroll
+            for (int g = 1; g < 8; ++g) {
+                sum.x += part[g][q_in].x;
+                sum.y += part[g][q_in].y;
+                sum.z += part[g][q_in].z;
+                sum.w += part[g][q_in].w;
+            }
+            const long long e = q * 4;
+            const int m = (int)(e / N), n = (int)(e - (long long)m * N);
+            float4 *dst = reinterpret_cast<float4 *>(C + m * ldc + n);
+            float4 r = make_float4(alpha * sum.x, alpha * sum.y, alpha * sum.z, alpha * sum.w);
+            if (beta != 0.f) {
+                const float4 old = *dst;
+                r.x += beta * old.x;
+                r.y += beta * old.y;
+                r.z += beta * old.z;
+                r.w += beta * old.w;
+            }
+            *dst = r;
+        }
+        __syncthreads();
+    }
+}
+
+// Launches the fold that suits the operands.
+static void launch_fold(hipStream_t st, const float *ws, int splits, long long split_stride, float *C, int M, int N,
+                        long long ldc, float alpha, float beta)
+{
+    const long long total = (long long)M * N;
+    const bool vec = total % 4 == 0 && N % 4 == 0 && ldc % 4 == 0 && split_stride % 4 == 0 && aligned16(ws) && aligned16(C);
+    if (vec) {
+        const long long blocks = (total / 4 + 31) / 32;
+        hipLaunchKernelGGL(splitk_fold_vec_kernel, dim3((unsigned)(blocks > 16384 ? 16384 : blocks)), dim3(256), 0, st, ws,
+                           splits, split_stride, C, M, N, ldc, alpha, beta);
+    } else {
+        const long long blocks = (total + 31) / 32;
+        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(blocks > 16384 ? 16384 : blocks)), dim3(256), 0, st, ws,
+                           splits, split_stride, C, M, N, ldc, alpha, beta);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side: configuration choice and launch
 // ---------------------------------------------------------------------------------------------
@@ -673,9 +756,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
                 // rest split: fold everything onto beta * C; rest not split: it has written
                 // alpha * rest + beta * C, the body's partial sums are added on top
                 const long long total = (long long)c.M * c.N;
-                hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
-                                   dim3(256), 0, st, static_cast<const float *>(ws), s_rest > 1 ? s_body + s_rest : s_body, total,
-                                   c.C, c.M, c.N, c.ldc, c.alpha, s_rest > 1 ? c.beta : 1.f);
+                launch_fold(st, static_cast<const float *>(ws), s_rest > 1 ? s_body + s_rest : s_body, total, c.C, c.M, c.N,
+                            c.ldc, c.alpha, s_rest > 1 ? c.beta : 1.f);
                 return check_launch(who);
             }
             if (ag_status_t s = run_gemm(st, who, body, ws, ws_bytes, splits)) return s;
@@ -782,9 +864,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     }
     if (p.splits > 1 && partials_only < 0) {
         const long long total = (long long)c.M * c.N;
-        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
-                           dim3(256), 0, st, static_cast<const float *>(ws), p.splits, p.sCsplit, real_c, c.M,
-                           c.N, c.ldc, c.alpha, c.beta);
+        launch_fold(st, static_cast<const float *>(ws), p.splits, p.sCsplit, real_c, c.M, c.N, c.ldc, c.alpha, c.beta);
         return check_launch(who);
     }
     return AG_OK;
@@ -934,9 +1014,7 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     if (ag_status_t s = check_launch("conv2d_filter_grad")) return s;
     if (p.splits > 1) {
         const long long total = (long long)p.M * p.N;
-        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)(cdiv(total, 32) > 16384 ? 16384 : cdiv(total, 32))),
-                           dim3(256), 0, st, static_cast<const float *>(ws), p.splits, p.sCsplit, gw, p.M, p.N,
-                           (long long)p.N, 1.f, 0.f);
+        launch_fold(st, static_cast<const float *>(ws), p.splits, p.sCsplit, gw, p.M, p.N, (long long)p.N, 1.f, 0.f);
         return check_launch("conv2d_filter_grad");
     }
     return AG_OK;

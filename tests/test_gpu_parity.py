@@ -272,6 +272,26 @@ def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg):
     assert_close(got, want, "direct batchsum")
 
 
+def test_split_fold_vector_and_scalar_forms_agree_bit_for_bit(K, rng):
+    """The fold of the split partial sums has a 128-bit form and a scalar form (unaligned or odd-sized outputs);
+    per element they add the same partials in the same order, so an output that is merely shifted by one float
+    in memory must come out with identical bits."""
+    kf, ck, pp, imgs = 64, 288, 196, 128
+    gy = rng.standard_normal((imgs, kf, pp)).astype(np.float32)
+    cols = rng.standard_normal((imgs, ck, pp)).astype(np.float32)
+    dgy, dcols = dev(gy), dev(cols)
+    say("fold forms")
+    aligned = torch.zeros(kf * ck + 4, device="cuda")
+    K.gemm_batchsum(0, 1, kf, ck, pp, 1.0, dgy, pp, kf * pp, dcols, pp, ck * pp, 0.0, aligned[:kf * ck], ck, imgs)
+    shifted = torch.zeros(kf * ck + 4, device="cuda")
+    K.gemm_batchsum(0, 1, kf, ck, pp, 1.0, dgy, pp, kf * pp, dcols, pp, ck * pp, 0.0, shifted[1:kf * ck + 1], ck, imgs)
+    assert shifted[1:].data_ptr() % 16 != 0
+    assert np.array_equal(host(aligned[:kf * ck]).view(np.uint32), host(shifted[1:kf * ck + 1]).view(np.uint32))
+    want = np.einsum("bkp,bcp->kc", gy.astype(np.float64), cols.astype(np.float64)).reshape(-1)
+    absdot = np.einsum("bkp,bcp->kc", np.abs(gy).astype(np.float64), np.abs(cols).astype(np.float64)).reshape(-1)
+    assert np.all(np.abs(host(aligned[:kf * ck]) - want) <= 2e-6 * absdot)
+
+
 def test_gemm_leading_dims_alpha_beta_batch(K, rng):
     m, n, k, batch = 45, 70, 52, 3
     lda, ldb, ldc = k + 4, n + 8, n + 3
