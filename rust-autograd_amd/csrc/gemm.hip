@@ -330,7 +330,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
         _Pragma("unroll") for (int j = 0; j < NI; ++j)         \
         _Pragma("unroll") for (int v = 0; v < 16; ++v) { stmt; } \
     }
-        bool chained = CHAINING && ci.nt > CHAIN;  // more than one chain: their sums meet in `tot`
+        bool chained = CHAINING && ci.nt > CHAIN + CHAIN / 4;  // more than one chain: their sums meet in `tot`
         if (chained) AG_FOR_TOT(tot[i][j][v] = 0.f)
         int chain_left = CHAIN;
         float4 af[2][MI], bf[2][NI];
@@ -372,10 +372,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, OCC) void gemm_mfma_ker
                 ci = decode(cw);
                 c_left = ci.nt;
                 zero_acc();
-                chained = CHAINING && ci.nt > CHAIN;
+                chained = CHAINING && ci.nt > CHAIN + CHAIN / 4;
                 if (chained) AG_FOR_TOT(tot[i][j][v] = 0.f)
                 chain_left = CHAIN;
-            } else if (CHAINING && --chain_left == 0) {
+            } else if (CHAINING && --chain_left == 0 && c_left > CHAIN / 4) {
+                // (a remainder of up to a quarter chain joins the chain before it)
                 AG_FOR_TOT(tot[i][j][v] += acc[i][j][v]; acc[i][j][v] = 0.f)
                 chain_left = CHAIN;
             }

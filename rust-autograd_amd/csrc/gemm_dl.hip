@@ -583,7 +583,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     while (true) {  // work items of this block
         zero_acc();
         int c_left = ci.nt;
-        const bool chained = ci.nt > CHAIN;  // more than one chain: their sums meet in `tot`
+        const bool chained = ci.nt > CHAIN + CHAIN / 4;  // more than one chain: their sums meet in `tot`
         if (chained) zero_tot();
         int chain_left = CHAIN;
         const bool last_item = cw + gridDim.x >= total;
@@ -612,7 +612,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             second_half(all_issued, cur, nxt, last);
             fill_addr = fill_addr + TILE * 4u == lds_wave + STAGES * TILE * 4u ? lds_wave : fill_addr + TILE * 4u;
             cur = nxt;
-            if (--chain_left == 0 && c_left > 1) {
+            if (--chain_left == 0 && c_left - 1 > CHAIN / 4) {
+                // (a remainder of up to a quarter chain joins the chain before it: the 576-element
+                // contractions of a 3x3 convolution over 64 channels stay one chain)
                 set_aside();
                 chain_left = CHAIN;
             }

@@ -51,9 +51,10 @@ struct GemmParams {
 };
 
 // Elements of the contraction that one accumulation chain of the MFMA kernels covers before its sum
-// is set aside and the chain restarts from zero (both GEMM kernels; the length of an OpenBLAS
-// SGEMM k block, so rounding errors grow as they do in the reference's BLAS).
-constexpr int kChainK = 256;
+// is set aside and the chain restarts from zero (both GEMM kernels).  OpenBLAS blocks its SGEMM
+// contraction the same way; with 512 the error against an f64 result is 1.08 times OpenBLAS's at
+// 4096^3 (256: 0.76 times, for twice the set-aside work; one chain of 4096: 6 times).
+constexpr int kChainK = 512;
 
 // Launches direct-to-LDS configuration `cfg` (kFirstDirectCfg ..); `ka` / `kb`: the operand is
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
