@@ -34,19 +34,21 @@ __global__ __launch_bounds__(256) void thin_fwd_kernel(const float *__restrict__
 {
     __shared__ float s_w[kThinFwdGroup * kThinFwdMaxCK];
     const int k0 = blockIdx.y * kThinFwdGroup;
+    const long long q = blockIdx.x * 256ll + threadIdx.x;
+    const bool active = q < quads;
+    const long long b = active ? q / P4 : 0;
+    const int p4 = active ? (int)(q - b * P4) : 0;
+    // the column loads go out before the filter taps are staged: both round trips overlap
+    const float4 *cb = reinterpret_cast<const float4 *>(cols) + b * CK * (long long)P4 + p4;
+    float4 c[kThinFwdMaxCK];
+#pragma unroll
+    for (int j = 0; j < kThinFwdMaxCK; ++j) c[j] = (active && j < CK) ? cb[(long long)j * P4] : make_float4(0.f, 0.f, 0.f, 0.f);
     if (threadIdx.x < kThinFwdGroup * kThinFwdMaxCK) {
         const int k = k0 + threadIdx.x / kThinFwdMaxCK, j = threadIdx.x % kThinFwdMaxCK;
         s_w[threadIdx.x] = (k < K && j < CK) ? w[k * CK + j] : 0.f;
     }
     __syncthreads();
-    const long long q = blockIdx.x * 256ll + threadIdx.x;
-    if (q >= quads) return;
-    const long long b = q / P4;
-    const int p4 = (int)(q - b * P4);
-    const float4 *cb = reinterpret_cast<const float4 *>(cols) + b * CK * (long long)P4 + p4;
-    float4 c[kThinFwdMaxCK];
-#pragma unroll
-    for (int j = 0; j < kThinFwdMaxCK; ++j) c[j] = j < CK ? cb[(long long)j * P4] : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!active) return;
     float4 *yb = reinterpret_cast<float4 *>(y) + (b * K + k0) * (long long)P4 + p4;
 #pragma unroll
     for (int g = 0; g < kThinFwdGroup; ++g) {

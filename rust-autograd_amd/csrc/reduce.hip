@@ -311,6 +311,49 @@ __global__ __launch_bounds__(256) void fold_cols_kernel(const float *__restrict_
     }
 }
 
+// x [outer][len][inner] -> out [outer][inner] in ONE pass for inner a multiple of four: a block takes 32
+// column quads and splits the rows over its eight groups of 32 lanes (eight 128-bit loads in flight per
+// lane); the group sums meet in LDS and are added in group order, so the result is deterministic.
+// Compared with a thread per column plus a second pass over split partial sums this needs one launch,
+// writes no partials, and has eight times the lanes per column.
+__global__ __launch_bounds__(256) void fold_cols_groups_kernel(const float *__restrict__ x, float *__restrict__ out,
+                                                               size_t outer, size_t len, size_t inner4, float scale,
+                                                               int apply_scale)
+{
+    __shared__ float4 part[8][32];
+    const unsigned c = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const size_t col = blockIdx.x * 32ull + c;
+    const size_t chunk = (len + 7) / 8;
+    const size_t r0 = (size_t)g * chunk < len ? (size_t)g * chunk : len, r1 = r0 + chunk < len ? r0 + chunk : len;
+    for (size_t o = blockIdx.y; o < outer; o += gridDim.y) {
+        float4 acc0 = vec_zero<float4>(), acc1 = vec_zero<float4>();
+        if (col < inner4) {
+            const float4 *p = reinterpret_cast<const float4 *>(x) + (o * len + r0) * inner4 + col;
+            size_t r = r0;
+            constexpr int U = 8;
+            for (; r + U <= r1; r += U) {
+                float4 v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[u] = ld_stream(p + u * inner4);
+                acc0 = vadd(acc0, vadd(vadd(v[0], v[1]), vadd(v[2], v[3])));
+                acc1 = vadd(acc1, vadd(vadd(v[4], v[5]), vadd(v[6], v[7])));
+                p += U * inner4;
+            }
+            for (; r < r1; ++r, p += inner4) acc0 = vadd(acc0, ld_stream(p));
+        }
+        part[g][c] = vadd(acc0, acc1);
+        __syncthreads();
+        if (g == 0 && col < inner4) {
+            float4 sum = part[0][c];
+#pragma unroll
+            for (int g2 = 1; g2 < 8; ++g2) sum = vadd(sum, part[g2][c]);
+            if (apply_scale) sum = vscale(sum, scale);
+            reinterpret_cast<float4 *>(out)[o * inner4 + col] = sum;
+        }
+        __syncthreads();
+    }
+}
+
 __global__ __launch_bounds__(256) void scale_copy_kernel(const float *__restrict__ x,
                                                          float *__restrict__ out, size_t n, float scale,
                                                          int apply_scale)
@@ -590,6 +633,10 @@ static void run_stream(hipStream_t st, const StreamPlan &pl, const float *x, siz
             if (vec) hipLaunchKernelGGL((fold_rows_split_kernel<true>), grid, block, 0, st, cur, part, s.len, s.splits, s.chunk);
             else hipLaunchKernelGGL((fold_rows_split_kernel<false>), grid, block, 0, st, cur, part, s.len, s.splits, s.chunk);
             launch_fold_rows(st, part, dst, s.outer, s.splits, scale, sc);
+        } else if (s.inner % 4 == 0 && s.len >= 16 && aligned16(cur) && aligned16(dst)) {
+            const size_t inner4 = s.inner / 4;
+            const dim3 grid((unsigned)ceil_div(inner4, 32), (unsigned)(s.outer < 65535 ? s.outer : 65535));
+            hipLaunchKernelGGL(fold_cols_groups_kernel, grid, dim3(256), 0, st, cur, dst, s.outer, s.len, inner4, scale, sc);
         } else if (s.splits > 1) {
             launch_fold_cols(st, cur, part, s.outer, s.len, s.inner, s.splits, s.chunk, 1.f, 0);
             launch_fold_cols(st, part, dst, s.outer, s.splits, s.inner, 1, s.splits, scale, sc);
