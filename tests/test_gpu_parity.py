@@ -449,6 +449,8 @@ CONV_CASES = [  # B, C, K, H, W, k, pad, stride, dil
     (2, 64, 128, 56, 56, 3, 1, 2, 1),  # north star stride-2 variant
     (2, 256, 256, 14, 14, 3, 2, 1, 2), # config 5 dilated, 2 of 32 images
     (2, 5, 7, 9, 11, 2, 0, 1, 1),      # ragged
+    (3, 1, 5, 12, 12, 3, 1, 1, 1),     # thin first layer: C*k*k = 9, an odd number of filters (the kernel takes pairs)
+    (2, 1, 7, 9, 9, 4, 2, 1, 1),       # thin first layer at its limit: C*k*k = 16, 10x10 outputs
 ]
 
 
