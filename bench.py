@@ -51,7 +51,7 @@ _DL = "ag::gemm_dl_kernel<%s>"
 PROFILE_TRAFFIC = {
     # the step (column-free)
     "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false", "avg")]),
-    "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_kernel", "avg")]),
+    "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
     "gemm_input_grad": (_STEP, [(_DL % "64, 128, 32, 32, 64, 3, true, false", "avg")]),
     "fwd_prepare": (_STEP, [("ag::pad_border_fast_kernel", "min")]),
     "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max")]),
@@ -61,7 +61,7 @@ PROFILE_TRAFFIC = {
     "im2col": (_COLS, [("ag::im2col_same_kernel<3, 3, 1, 16>", "avg")]),
     "col2im": (_COLS, [("ag::col2im_same_kernel<3, 3, 1, 16>", "avg")]),
     "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false", "avg")]),
-    "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_kernel", "avg")]),
+    "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
     "gemm_input_grad_columns": (_COLS, [(_DL % "192, 128, 32, 96, 32, 3, false, false", "avg")]),
 }
 _profile_cache = {}
@@ -131,6 +131,9 @@ def parse():
                     help="run only one part of the per-kernel section (for profiler passes): the two pooling kernels, "
                          "the column-materialising convolution kernels, or the steps of configuration 1 / 2 "
                          "through the host operator layer")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="leave the HBM-traffic fields out (for the profiler passes that produce the summaries those "
+                         "fields are read from)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch one plain copy kernel (ag_scale_f32 by 1.0) over 2^28 floats, "
                          "so that a rocprofv3 --pmc run of this command holds a kernel of known traffic "
@@ -255,8 +258,8 @@ def main():
     OH = Kn.conv_out_size(H, KH, PAD, STRIDE, DIL)
     P, CK = OH * OH, C * KH * KH
 
+    global _profile_strict
     if args.only:
-        global _profile_strict
         _profile_strict = False
         g = torch.Generator(device=dev)
         g.manual_seed(99)
@@ -333,7 +336,8 @@ def main():
     for name, nbytes in (("fwd_prepare", 4.0 * (x.numel() + n_xpad)), ("input_grad_prepare", 4.0 * (gy.numel() + n_gypad))):
         gbs = nbytes / (per[name] * 1e-3) / 1e9
         kernels[name] = {"ms": round(per[name], 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
-    if Bn == B:
+    with_traffic = Bn == B and not args.no_traffic
+    if with_traffic:
         for name in kernels:
             kernels[name]["traffic_bytes"] = round(profile_traffic(name)[0])
     gemm_ms = sum(per[n] for n in ("gemm_fwd", "gemm_filter_grad", "gemm_input_grad"))
@@ -342,8 +346,8 @@ def main():
     dom_tf = gemm_flop / (per[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(dom_tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_tf / FP32_MFMA_PEAK_TFLOPS, 4),
-                "traffic": round(profile_traffic(dominant)[0]) if Bn == B else None,
-                "traffic_source": profile_traffic(dominant)[1] if Bn == B else None,
+                "traffic": round(profile_traffic(dominant)[0]) if with_traffic else None,
+                "traffic_source": profile_traffic(dominant)[1] if with_traffic else None,
                 "gemm_phase_TFLOP/s": round(gemm_tf, 2),
                 "gemm_phase_frac": round(gemm_tf / FP32_MFMA_PEAK_TFLOPS, 4)}
 
