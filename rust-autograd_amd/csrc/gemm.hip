@@ -614,6 +614,10 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
         // fewer 128 x 128 tiles than CUs: 64 x 64 tiles (two or three blocks per CU) use the whole chip
         if (!accumulate && cdiv(M, 128) * cdiv(N, 128) * zcount < cus2 && cdiv(M, 64) * cdiv(N, 64) * zcount >= cus2 / 2)
             return kDirectCfg64Narrow;
+        // a short contraction over a few rounds of tiles: the prologue and epilogue of a tile weigh as much as
+        // its k loop, and two 64 x 128 blocks per CU overlap the one's with the other's (M = 2304, N = 32 x 196,
+        // K = 256: 71 us against 89 us with 256 x 128 tiles)
+        if (!accumulate && K <= 512 && M >= 64 && cdiv(M, 128) * cdiv(N, 128) * zcount < 8 * cus2) return kDirectCfg64;
         int best = -1;
         double best_cost = 1e300;
         for (int c = 0; c < 6; ++c) {

@@ -141,6 +141,37 @@ __global__ __launch_bounds__(256) void col2im_gather_kernel(const float *__restr
     gx[plane * HW + e] = acc;
 }
 
+// The same for a 3 x 3 filter at stride 1 and any dilation: the nine tap addresses are computed and their
+// loads issued together (absent taps read nothing and add 0.0, which leaves the sum unchanged), then
+// added in (ky, kx) ascending order.  The run-time loops of the general kernel issue one load at a time.
+__global__ __launch_bounds__(256) void col2im_gather3_kernel(const float *__restrict__ cols, float *__restrict__ gx,
+                                                             ConvGeom g, int chunks)
+{
+    const int chunk = blockIdx.x % chunks;
+    const long long plane = blockIdx.x / chunks;
+    const int HW = g.H * g.W;
+    const int e = chunk * 256 + threadIdx.x;
+    if (e >= HW) return;
+    const int iy = e / g.W, ix = e - iy * g.W;
+    const long long P = (long long)g.OH * g.OW;
+    const float *cp = cols + plane * 9 * P;
+    float v[9];
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int oy = iy + g.ph - ky * g.dh;
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            const int ox = ix + g.pw - kx * g.dw;
+            const bool in = (unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW;
+            v[ky * 3 + kx] = in ? cp[(long long)(ky * 3 + kx) * P + oy * g.OW + ox] : 0.f;
+        }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) acc += v[t];
+    gx[plane * HW + e] = acc;
+}
+
 // 16 bytes that are only 4-byte aligned (the hardware handles the misalignment).
 struct __attribute__((packed, aligned(4))) Float4U {
     float x, y, z, w;
@@ -604,8 +635,12 @@ extern "C" ag_status_t ag_col2im_f32(ag_stream_t stream, const float *cols, floa
         const int chunks = (H * W + 255) / 256;
         const long long blocks = planes * chunks;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "col2im: too many tiles (%lld)", blocks);
-        hipLaunchKernelGGL(col2im_gather_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cols,
-                           gx, g, chunks);
+        if (kh == 3 && kw == 3 && sh == 1 && sw == 1)
+            hipLaunchKernelGGL(col2im_gather3_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cols, gx, g,
+                               chunks);
+        else
+            hipLaunchKernelGGL(col2im_gather_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cols,
+                               gx, g, chunks);
     }
     return check_launch("col2im");
 }
