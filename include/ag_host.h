@@ -104,6 +104,16 @@ int agh_adam_update_op(agh_adam *adam, agh_ctx *ctx, const int *params, const in
  * the next agh_eval; agh_result_* read them.  Returns 0, or -1 if evaluation panicked. */
 int agh_eval(agh_ctx *ctx, const int *tensors, int n, const char *const *feed_names, const float *const *feed_data,
              const int64_t *const *feed_shapes, const int *feed_ranks, int n_feeds);
+/* The same evaluation without waiting for the device: the work is enqueued and the call returns.  The
+ * statuses of the results are known (operator errors are found on the host while the work is enqueued);
+ * agh_result_read and every other read of device data wait as needed.  For steps whose results are not
+ * read, Optimizer::update above all (optimizers/mod.rs:63-81 only unwraps them): the host builds the next
+ * graph while the device runs this one.  Feed buffers may be reused when the call returns. */
+int agh_eval_nowait(agh_ctx *ctx, const int *tensors, int n, const char *const *feed_names,
+                    const float *const *feed_data, const int64_t *const *feed_shapes, const int *feed_ranks,
+                    int n_feeds);
+/* Waits until the device has finished everything enqueued so far. */
+int agh_synchronize(void);
 int agh_result_status(agh_ctx *ctx, int i); /* 0 = Ok, 1..5 = OpError variant, 100 = HIP error */
 const char *agh_result_message(agh_ctx *ctx, int i);
 int agh_result_shape(agh_ctx *ctx, int i, int64_t *shape_out, int max_rank); /* returns the rank */

@@ -292,8 +292,8 @@ int agh_adam_update_op(agh_adam *adam, agh_ctx *c, const int *params, const int 
     });
 }
 
-int agh_eval(agh_ctx *c, const int *tensors, int n, const char *const *feed_names, const float *const *feed_data,
-             const int64_t *const *feed_shapes, const int *feed_ranks, int n_feeds)
+static int eval_impl(agh_ctx *c, const int *tensors, int n, const char *const *feed_names, const float *const *feed_data,
+                     const int64_t *const *feed_shapes, const int *feed_ranks, int n_feeds, bool wait)
 {
     return guard([&] {
         std::vector<Tensor> ts;
@@ -309,12 +309,32 @@ int agh_eval(agh_ctx *c, const int *tensors, int n, const char *const *feed_name
         const auto t1 = std::chrono::steady_clock::now();
         c->results = c->ctx.eval(ts, feeds);
         const auto t2 = std::chrono::steady_clock::now();
-        synchronize();
+        if (wait) synchronize();
         if (timing) {
             const auto t3 = std::chrono::steady_clock::now();
             auto us = [](auto a, auto b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
             std::fprintf(stderr, "[ag_host] eval: feeds %.1f us, enqueue %.1f us, wait %.1f us\n", us(t0, t1), us(t1, t2), us(t2, t3));
         }
+        return 0;
+    });
+}
+
+int agh_eval(agh_ctx *c, const int *tensors, int n, const char *const *feed_names, const float *const *feed_data,
+             const int64_t *const *feed_shapes, const int *feed_ranks, int n_feeds)
+{
+    return eval_impl(c, tensors, n, feed_names, feed_data, feed_shapes, feed_ranks, n_feeds, true);
+}
+
+int agh_eval_nowait(agh_ctx *c, const int *tensors, int n, const char *const *feed_names, const float *const *feed_data,
+                    const int64_t *const *feed_shapes, const int *feed_ranks, int n_feeds)
+{
+    return eval_impl(c, tensors, n, feed_names, feed_data, feed_shapes, feed_ranks, n_feeds, false);
+}
+
+int agh_synchronize(void)
+{
+    return guard([&] {
+        synchronize();
         return 0;
     });
 }

@@ -67,6 +67,8 @@ PROTOTYPES = {
     "agh_adam_free": (None, [_p]),
     "agh_adam_update_op": (_i, [_p, _p, _ip, _ip, _i]),
     "agh_eval": (_i, [_p, _ip, _i, C.POINTER(_s), C.POINTER(_fp), C.POINTER(_lp), _ip, _i]),
+    "agh_eval_nowait": (_i, [_p, _ip, _i, C.POINTER(_s), C.POINTER(_fp), C.POINTER(_lp), _ip, _i]),
+    "agh_synchronize": (_i, []),
     "agh_result_status": (_i, [_p, _i]),
     "agh_result_message": (_s, [_p, _i]),
     "agh_result_shape": (_i, [_p, _i, _lp, _i]),
@@ -342,7 +344,7 @@ class Context:
         return lib().agh_num_nodes(self._h)
 
     # -- evaluation ---------------------------------------------------------------------------
-    def eval(self, tensors, feeds=None):
+    def _evaluate(self, entry, tensors, feeds):
         feeds = feeds or {}
         ids, n = _ints(t.id for t in tensors)
         arrays = [_f32(a) for a in feeds.values()]
@@ -352,7 +354,11 @@ class Context:
         shapes_keep = [_shape(a.shape)[0] for a in arrays]
         shapes = (_lp * max(nf, 1))(*[C.cast(s, _lp) for s in shapes_keep])
         ranks, _ = _ints(a.ndim for a in arrays)
-        _check(lib().agh_eval(self._h, ids, n, names, data, shapes, ranks, nf))
+        _check(entry(self._h, ids, n, names, data, shapes, ranks, nf))
+        return n
+
+    def eval(self, tensors, feeds=None):
+        n = self._evaluate(lib().agh_eval, tensors, feeds)
         out = []
         buf = (C.c_int64 * 8)()
         for i in range(n):
@@ -365,6 +371,22 @@ class Context:
             _check(lib().agh_result_read(self._h, i, a.ctypes.data_as(_fp), a.size))
             out.append(a)
         return out
+
+    def run(self, tensors, feeds=None):
+        """Evaluates `tensors` for their effects (optimizer updates) without waiting for the device and without
+        reading anything back: returns None per tensor, or its OpError.  The next graph can be built while the
+        device works; reading a variable (or any eval) waits as needed."""
+        n = self._evaluate(lib().agh_eval_nowait, tensors, feeds)
+        out = []
+        for i in range(n):
+            st = lib().agh_result_status(self._h, i)
+            out.append(OpError(st, lib().agh_result_message(self._h, i).decode()) if st != 0 else None)
+        return out
+
+
+def synchronize():
+    """Waits until the device has finished everything enqueued so far."""
+    _check(lib().agh_synchronize())
 
 
 class Adam:
@@ -388,6 +410,7 @@ class Adam:
         return ctx._t(lib().agh_adam_update_op(self._h, ctx._h, pi, gi, n))
 
     def update(self, params, grads, ctx, feeds=None):
-        r = ctx.eval([self.get_update_op(params, grads, ctx)], feeds)[0]
+        """Optimizer::update (optimizers/mod.rs:63-81): runs the updates; the call does not wait for the device."""
+        r = ctx.run([self.get_update_op(params, grads, ctx)], feeds)[0]
         if isinstance(r, OpError):
             raise r

@@ -483,6 +483,38 @@ def test_feeds_and_read_backs_of_any_size_cross_the_staging_ring_intact(G, rng):
     assert np.array_equal(env.array(wid), big)
 
 
+def test_updates_that_do_not_wait_for_the_device_equal_waiting_ones(G, rng):
+    """Optimizer::update returns once its work is enqueued.  Forty steps in a row, each fed from one host buffer
+    that is overwritten as soon as update() returns, must leave the variables with exactly the bits of the same
+    forty steps run through eval() (which waits and reads the result back) — the graph of step n+1 is built and
+    its feeds are copied while the device still runs step n."""
+    def train(waiting):
+        r = np.random.default_rng(11)
+        env = G.VariableEnvironment()
+        wid = env.set("w", r.standard_normal((8, 1, 3, 3)).astype(np.float32) * 0.3)
+        bid = env.set("b", np.zeros((1, 8, 1, 1), np.float32))
+        adam = G.Adam(env, [wid, bid], alpha=0.01)
+        buf = np.empty((16, 1, 12, 12), np.float32)
+        for step in range(40):
+            buf[:] = r.standard_normal(buf.shape).astype(np.float32)
+            c = env.context()
+            w, b = c.variable(wid), c.variable(bid)
+            x = c.placeholder("x", [-1, 1, 12, 12])
+            loss = c.sum_all(c.max_pool2d(c.relu(c.conv2d(x, w, 1, 1) + b), 2, 0, 2))
+            gw, gb = c.grad([loss], [w, b])
+            if waiting:
+                out = c.eval([adam.get_update_op([w, b], [gw, gb], c)], {"x": buf})
+                assert not isinstance(out[0], G.OpError)
+            else:
+                adam.update([w, b], [gw, gb], c, {"x": buf})
+            buf[:] = np.nan                                     # the device must not see this
+        return env.array(wid), env.array(bid)
+    w1, b1 = train(waiting=True)
+    w2, b2 = train(waiting=False)
+    assert np.isfinite(w1).all() and np.array_equal(w1.view(np.uint32), w2.view(np.uint32))
+    assert np.array_equal(b1.view(np.uint32), b2.view(np.uint32))
+
+
 def test_batched_adam_updates_keep_the_evaluation_order(G, orc, rng):
     """The AdamOp nodes of one evaluation go out as one launch, but a node that reads a variable after its
     AdamOp ran must see the updated array, exactly as if every update had run at its own node.  The evaluator
