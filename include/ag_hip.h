@@ -305,6 +305,11 @@ ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const float *bia
  * examples/cnn_mnist.rs).  bshape[i] must be shape[i] or 1; rank <= 8. */
 ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
                                  const int *shape, const int *bshape, int rank);
+/* That AddOp followed by ReLU::compute (activation_ops.rs:154-159) in one pass, y = max(x + b, 0):
+ * the conv-bias-activation step of examples/cnn_mnist.rs.  The sum is rounded to f32 before the
+ * maximum, so the result has the bits of ag_add_broadcast_f32 followed by ag_relu_f32. */
+ag_status_t ag_add_broadcast_relu_f32(ag_stream_t stream, const float *x, const float *b, float *y,
+                                      const int *shape, const int *bshape, int rank);
 /* MaybeReduceSum for that operand: out[c] = sum_r gy[r][c], r ascending (binary_ops.rs:39-105). */
 ag_status_t ag_bias_grad_f32(ag_stream_t stream, const float *gy, float *out, size_t rows,
                              size_t cols);

@@ -86,6 +86,7 @@ PROTOTYPES = {
     "ag_relu_grad_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),
     "ag_add_bias_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz]),
     "ag_add_broadcast_f32": (c_i, [c_p, c_p, c_p, c_p, C.POINTER(c_i), C.POINTER(c_i), c_i]),
+    "ag_add_broadcast_relu_f32": (c_i, [c_p, c_p, c_p, c_p, C.POINTER(c_i), C.POINTER(c_i), c_i]),
     "ag_bias_grad_f32": (c_i, [c_p, c_p, c_p, c_sz, c_sz]),
     "ag_add_n_f32": (c_i, [c_p, c_p, c_i, c_p, c_sz]),
     "ag_mul_f32": (c_i, [c_p, c_p, c_p, c_p, c_sz]),

@@ -142,8 +142,11 @@ struct BroadcastGeom {
 // ADD: y = x + b (AddOp, binary_ops.rs:147-166, 304-346); otherwise y = b (ReduceGradCommon,
 // reduction_ops.rs:459-512).  I = unsigned when the result has fewer than 2^32 elements.  `vec`
 // needs an innermost merged extent that is a multiple of 4.
-template <bool ADD, typename I>
+// MODE 0: y = broadcast(b); 1: y = x + broadcast(b); 2: y = relu(x + broadcast(b)), the sum rounded to f32 first,
+// so the result has the bits of the two operations run one after the other.
+template <int MODE, typename I>
 struct BroadcastF {
+    static __device__ float fin(float v) { return MODE == 2 ? ReluF::f(v) : v; }
     const float *x, *b;
     float *y;
     BroadcastGeom g;
@@ -156,7 +159,7 @@ struct BroadcastF {
             rest = q;
         }
         bi += rest * g.bstride[0];
-        y[i] = ADD ? x[i] + b[bi] : b[bi];
+        y[i] = MODE != 0 ? fin(x[i] + b[bi]) : b[bi];
     }
     __device__ void vec(size_t q4) const
     {
@@ -177,9 +180,9 @@ struct BroadcastF {
         } else {
             bv = *reinterpret_cast<const float4 *>(b + bi);
         }
-        if (ADD) {
+        if (MODE != 0) {
             const float4 v = ld_stream(as4(x) + q4);
-            bv = make_float4(v.x + bv.x, v.y + bv.y, v.z + bv.z, v.w + bv.w);
+            bv = make_float4(fin(v.x + bv.x), fin(v.y + bv.y), fin(v.z + bv.z), fin(v.w + bv.w));
         }
         st_stream(as4(y) + q4, bv);
     }
@@ -363,14 +366,14 @@ static ag_status_t make_broadcast_geom(const char *who, const int *shape, const 
     return AG_OK;
 }
 
-template <bool ADD>
+template <int MODE>
 static ag_status_t launch_broadcast(const char *name, ag_stream_t stream, const float *x, const float *b, float *y,
                                     const BroadcastGeom &g, size_t n)
 {
     const int last = g.rank - 1;
-    const bool vec = g.dims[last] % 4 == 0 && aligned16(y) && (!ADD || aligned16(x)) && (g.bstride[last] == 0 || aligned16(b));
-    if (n <= 0xffffffffu) return ew_launch(name, stream, n, vec, BroadcastF<ADD, unsigned>{x, b, y, g});
-    return ew_launch(name, stream, n, vec, BroadcastF<ADD, size_t>{x, b, y, g});
+    const bool vec = g.dims[last] % 4 == 0 && aligned16(y) && (MODE == 0 || aligned16(x)) && (g.bstride[last] == 0 || aligned16(b));
+    if (n <= 0xffffffffu) return ew_launch(name, stream, n, vec, BroadcastF<MODE, unsigned>{x, b, y, g});
+    return ew_launch(name, stream, n, vec, BroadcastF<MODE, size_t>{x, b, y, g});
 }
 
 extern "C" ag_status_t ag_relu_f32(ag_stream_t stream, const float *x, float *y, size_t n)
@@ -396,7 +399,7 @@ extern "C" ag_status_t ag_add_bias_f32(ag_stream_t stream, const float *x, const
     size_t n;
     if (ag_status_t s = make_broadcast_geom("add", shape, bshape, 2, &g, &n)) return s;
     if (n == 0) return AG_OK;
-    return launch_broadcast<true>("add", stream, x, bias, y, g, n);
+    return launch_broadcast<1>("add", stream, x, bias, y, g, n);
 }
 
 extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, const float *b, float *y,
@@ -408,7 +411,19 @@ extern "C" ag_status_t ag_add_broadcast_f32(ag_stream_t stream, const float *x, 
     if (ag_status_t s = make_broadcast_geom("add", shape, bshape, rank, &g, &n)) return s;
     if (n == 0) return AG_OK;
     AG_REQUIRE(x && b && y, AG_ERR_INVALID_DIMS, "add: null pointer");
-    return launch_broadcast<true>("add", stream, x, b, y, g, n);
+    return launch_broadcast<1>("add", stream, x, b, y, g, n);
+}
+
+extern "C" ag_status_t ag_add_broadcast_relu_f32(ag_stream_t stream, const float *x, const float *b, float *y,
+                                                 const int *shape, const int *bshape, int rank)
+{
+    AG_REQUIRE(rank >= 1, AG_ERR_INVALID_DIMS, "add+relu: rank %d not in 1..8", rank);
+    BroadcastGeom g{};
+    size_t n;
+    if (ag_status_t s = make_broadcast_geom("add+relu", shape, bshape, rank, &g, &n)) return s;
+    if (n == 0) return AG_OK;
+    AG_REQUIRE(x && b && y, AG_ERR_INVALID_DIMS, "add+relu: null pointer");
+    return launch_broadcast<2>("add+relu", stream, x, b, y, g, n);
 }
 
 extern "C" ag_status_t ag_broadcast_grad_f32(ag_stream_t stream, const float *gy, float *gx,
@@ -423,7 +438,7 @@ extern "C" ag_status_t ag_broadcast_grad_f32(ag_stream_t stream, const float *gy
     if (ag_status_t s = make_broadcast_geom("reduce_grad", shape, bshape, rank, &g, &n)) return s;
     if (n == 0) return AG_OK;
     AG_REQUIRE(gy && gx, AG_ERR_INVALID_DIMS, "reduce_grad: null pointer");
-    return launch_broadcast<false>("reduce_grad", stream, nullptr, gy, gx, g, n);
+    return launch_broadcast<0>("reduce_grad", stream, nullptr, gy, gx, g, n);
 }
 
 extern "C" ag_status_t ag_bias_grad_f32(ag_stream_t stream, const float *gy, float *out, size_t rows,

@@ -882,6 +882,43 @@ struct AddOp : Op {  // binary_ops.rs:147-166, 304-346
     }
 };
 
+// AddOp followed by ReLU as one node: what tensor_ops::relu builds when its argument is an AddOp node, with
+// that node's two operands as inputs.  The value is relu(a + b) bit for bit; the AddOp node stays in the graph and
+// is evaluated only if something else asks for it.  The gradient is the mask taken from this node's own OUTPUT
+// (y > 0 exactly where a + b > 0), handed to both operands the way AddOp::grad does.
+struct AddReLU : Op {
+    const char *name() const override { return "AddReLU"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray a = ctx.input(0), b = ctx.input(1);
+        std::vector<int> bshape;
+        if (a.shape() == b.shape()) {
+            bshape.assign(a.shape().begin(), a.shape().end());
+        } else if (broadcasts_over_rows(a.shape(), b.shape())) {
+            bshape.assign(a.shape().begin(), a.shape().end());
+            bshape[0] = 1;
+        } else if (!broadcasts_along_axes(a.shape(), b.shape(), &bshape)) {
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "AddOp: unsupported broadcast " + shape_str(a.shape()) + " + " + shape_str(b.shape()));
+        }
+        if (a.shape().empty() || a.shape().size() > 8)
+            return OpError::make(ErrorKind::IncompatibleShape, "AddOp: rank " + std::to_string(a.shape().size()) + " not in 1..8");
+        NdArray y = NdArray::empty(a.shape());
+        const std::vector<int> shape(a.shape().begin(), a.shape().end());
+        const OpError e = from_status(ag_add_broadcast_relu_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), shape.data(),
+                                                                bshape.data(), (int)shape.size()));
+        if (!e.ok()) return e;
+        ctx.append_output(y);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        const Tensor g = build(ctx.graph(), {ctx.output(), ctx.output_grad()}, std::make_unique<ReLUGrad>());
+        ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(0)}, std::make_unique<MaybeReduceSum>()));
+        ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(1)}, std::make_unique<MaybeReduceSum>()));
+    }
+};
+
 struct MulOp : Op {  // binary_ops.rs:209-237 (same-shape operands)
     const char *name() const override { return "MulOp"; }
     OpError compute(ComputeContext &ctx) const override
@@ -1112,7 +1149,16 @@ Tensor reduce_mean(Tensor x, const std::vector<int> &axes, bool keep_dims)
     return build(x.graph, {x}, std::make_unique<ReduceSum>(axes, keep_dims, true));
 }
 Tensor sum_all(Tensor x) { return build(x.graph, {x}, std::make_unique<ReduceSumToScalar>()); }
-Tensor relu(Tensor x) { return build(x.graph, {x}, std::make_unique<ReLU>()); }
+Tensor relu(Tensor x)
+{
+    // relu(a + b): one fused node over a and b (the bias-activation step after a convolution)
+    const TensorInternal &n = x.graph->node(x.id);
+    if (dynamic_cast<const AddOp *>(n.op.get()) && n.incoming_nodes.size() == 2 && n.incoming_nodes[0].array_selector == 0 &&
+        n.incoming_nodes[1].array_selector == 0 && !n.incoming_nodes[0].allow_mut && !n.incoming_nodes[1].allow_mut)
+        return build(x.graph, {x.graph->tensor(n.incoming_nodes[0].id), x.graph->tensor(n.incoming_nodes[1].id)},
+                     std::make_unique<AddReLU>());
+    return build(x.graph, {x}, std::make_unique<ReLU>());
+}
 Tensor add(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<AddOp>()); }
 Tensor mul(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<MulOp>()); }
 

@@ -398,6 +398,18 @@ def add_broadcast(x, b):
     return y
 
 
+def add_broadcast_relu(x, b):
+    """relu(x + b) in one pass, b as for add_broadcast."""
+    x, b = _f32(x, "add+relu"), _f32(b, "add+relu")
+    if x.dim() != b.dim():
+        raise capi.IncompatibleShape(f"add+relu: operands of rank {x.dim()} and {b.dim()}")
+    y = torch.empty_like(x)
+    shape = (C.c_int * max(x.dim(), 1))(*x.shape)
+    bshape = (C.c_int * max(x.dim(), 1))(*b.shape)
+    check(capi.lib().ag_add_broadcast_relu_f32(_stream(), _ptr(x), _ptr(b), _ptr(y), shape, bshape, x.dim()))
+    return y
+
+
 def bias_grad(gy):
     gy = _f32(gy, "reduce_sum")
     out = _empty((1, gy.shape[1]), gy)

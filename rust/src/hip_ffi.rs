@@ -54,6 +54,7 @@ extern "C" {
     pub fn ag_relu_grad_f32(stream: AgStream, x: *const f32, gy: *const f32, gx: *mut f32, n: usize) -> AgStatus;
     pub fn ag_add_bias_f32(stream: AgStream, x: *const f32, bias: *const f32, y: *mut f32, rows: usize, cols: usize) -> AgStatus;
     pub fn ag_add_broadcast_f32(stream: AgStream, x: *const f32, b: *const f32, y: *mut f32, shape: *const c_int, bshape: *const c_int, rank: c_int) -> AgStatus;
+    pub fn ag_add_broadcast_relu_f32(stream: AgStream, x: *const f32, b: *const f32, y: *mut f32, shape: *const c_int, bshape: *const c_int, rank: c_int) -> AgStatus;
     pub fn ag_bias_grad_f32(stream: AgStream, gy: *const f32, out: *mut f32, rows: usize, cols: usize) -> AgStatus;
     pub fn ag_add_n_f32(stream: AgStream, xs: *const *const f32, count: c_int, out: *mut f32, n: usize) -> AgStatus;
     pub fn ag_mul_f32(stream: AgStream, a: *const f32, b: *const f32, out: *mut f32, n: usize) -> AgStatus;

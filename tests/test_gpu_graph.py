@@ -483,6 +483,31 @@ def test_feeds_and_read_backs_of_any_size_cross_the_staging_ring_intact(G, rng):
     assert np.array_equal(env.array(wid), big)
 
 
+def test_relu_of_a_sum_is_one_node_with_the_values_and_gradients_of_two(G, orc, rng):
+    """relu(a + b) is built as one fused node over a and b.  Its value, and the gradients that reach a and the
+    broadcast b through it, must have exactly the bits of the unfused graph (relu applied to the sum through an
+    identity, which hides the AddOp from the fusion)."""
+    env = G.VariableEnvironment()
+    av = rng.standard_normal((6, 5, 4, 4)).astype(np.float32)
+    bv = rng.standard_normal((1, 5, 1, 1)).astype(np.float32)
+    aid, bid = env.set("a", av), env.set("b", bv)
+    c = env.context()
+    a, b = c.variable(aid), c.variable(bid)
+    fused = c.relu(a + b)
+    assert fused.op_name == "AddReLU" and fused.num_inputs == 2
+    plain = c.relu(c.reshape(a + b, [6, 5, 4, 4]))
+    assert plain.op_name == "ReLU"
+    wts = c.placeholder("wts", [6, 5, 4, 4])
+    gf = c.grad([c.sum_all(c.mul(fused, wts))], [a, b])
+    gp = c.grad([c.sum_all(c.mul(plain, wts))], [a, b])
+    wv = rng.standard_normal((6, 5, 4, 4)).astype(np.float32)
+    yf, yp, gfa, gfb, gpa, gpb = c.eval([fused, plain, *gf, *gp], {"wts": wv})
+    want = np.maximum(av + bv, 0)
+    assert np.array_equal(yf, want) and np.array_equal(yp, want)
+    assert np.array_equal(gfa.view(np.uint32), gpa.view(np.uint32)) and np.array_equal(gfa, wv * (av + bv > 0))
+    assert gfb.shape == (1, 5, 1, 1) and np.array_equal(gfb.view(np.uint32), gpb.view(np.uint32))
+
+
 def test_updates_that_do_not_wait_for_the_device_equal_waiting_ones(G, rng):
     """Optimizer::update returns once its work is enqueued.  Forty steps in a row, each fed from one host buffer
     that is overwritten as soon as update() returns, must leave the variables with exactly the bits of the same

@@ -1239,6 +1239,21 @@ def test_add_with_an_operand_broadcast_along_its_unit_axes(K, rng, shape, bshape
     assert np.array_equal(host(K.add_broadcast(dev(x), dev(b))), x + b)
 
 
+@pytest.mark.parametrize("shape,bshape", [((4, 32, 28, 28), (1, 32, 28, 28)), ((3, 5, 7, 6), (1, 5, 1, 1)), ((37, 10), (1, 10)),
+                                          ((5, 9), (5, 9)), ((2, 3, 5), (1, 1, 1)), ((6, 1027), (1, 1027))])
+def test_add_and_relu_in_one_pass_has_the_bits_of_the_two_operations(K, rng, shape, bshape):
+    x = rng.standard_normal(shape).astype(np.float32)
+    b = rng.standard_normal(bshape).astype(np.float32)
+    x.reshape(-1)[::7] = np.nan                                  # max(NaN, 0) is 0 in the reference (f32::max)
+    say("add+relu", shape, bshape)
+    fused = host(K.add_broadcast_relu(dev(x), dev(b)))
+    two = host(K.relu(K.add_broadcast(dev(x), dev(b))))
+    assert np.array_equal(fused.view(np.uint32), two.view(np.uint32))
+    want = x + b
+    want = np.where(want > 0, want, np.float32(0)).astype(np.float32)
+    assert np.array_equal(fused, want)
+
+
 def test_add_broadcast_rejects_other_extents(K, rng):
     from rust_autograd_amd import capi
     x, b = dev(np.zeros((4, 3), np.float32)), dev(np.zeros((2, 3), np.float32))
