@@ -79,36 +79,77 @@ bool s2_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, S2Geom 
     return true;
 }
 
-// xph[b][c][a][b'][i][j] = x'[2i+a][2j+b'] = x[b][c][2i+a-pad][2j+b'-pad], zero outside x.  One thread per four
-// consecutive elements of a phase plane; grid.y walks the (image, channel) planes.
-__global__ __launch_bounds__(256) void phase_split_kernel(const float *__restrict__ x, float *__restrict__ xph, int planes,
-                                                          int H, int W, int pad, int Wc, unsigned quads_phase, unsigned m_phase,
-                                                          unsigned m_row)
+// xph[b][c][a][b'][i][j] = x'[2i+a][2j+b'] = x[b][c][2i+a-pad][2j+b'-pad], zero outside x; grid.y walks the
+// (image, channel) planes.  One thread per four consecutive elements of BOTH column phases of a row phase a: the
+// eight inputs x[2i+a-pad][2j-pad .. 2j+7-pad] are neighbours in memory (two 16-byte loads that need only
+// 4-byte alignment when the quad lies inside one row and inside the image), the even ones go to phase (a,0) and
+// the odd ones to phase (a,1).  A wave then uses every byte of the cache lines it touches; with a thread per
+// phase each line was fetched twice, by threads far apart in the grid.
+struct __attribute__((packed, aligned(4))) F4U {
+    float x, y, z, w;
+};
+
+// The last `extra_rows` rows of the grid split nothing: they zero the slack after the planes and write the filter as the
+// k-contiguous left operand of the forward GEMM, wf[k][tap][c] = w[k][c][tap], so that the preparation is one launch.
+__global__ __launch_bounds__(256) void phase_split_pair_kernel(const float *__restrict__ x, float *__restrict__ xph, int planes,
+                                                               int H, int W, int pad, int Wc, unsigned quads_phase,
+                                                               unsigned m_phase, unsigned m_row, float *__restrict__ slack,
+                                                               int n_slack, const float *__restrict__ w,
+                                                               float *__restrict__ wf, int K, int C, int taps,
+                                                               unsigned extra_rows)
 {
-    const unsigned qi = blockIdx.x * 256u + threadIdx.x;  // quad inside the four phase planes of one channel
-    if (qi >= 4u * quads_phase) return;
-    const unsigned ph = __umulhi(qi, m_phase);
-    const unsigned e0 = (qi - ph * quads_phase) * 4u;
+    const unsigned ny = gridDim.y - extra_rows;
+    if (blockIdx.y >= ny) {
+        const int tid = (int)(((blockIdx.y - ny) * gridDim.x + blockIdx.x) * 256u + threadIdx.x);
+        const int nth = (int)(extra_rows * gridDim.x * 256u);
+        for (int e = tid; e < n_slack; e += nth) slack[e] = 0.f;
+        const int total = K * C * taps;
+        for (int e = tid; e < total; e += nth) {
+            const int c = e % C, tap = e / C % taps, k = e / (C * taps);
+            wf[e] = w[((long long)k * C + c) * taps + tap];
+        }
+        return;
+    }
+    const unsigned qi = blockIdx.x * 256u + threadIdx.x;  // quad inside the two row phases of one channel
+    if (qi >= 2u * quads_phase) return;
+    const unsigned a = __umulhi(qi, m_phase);
+    const unsigned q = qi - a * quads_phase;
+    const unsigned e0 = q * 4u;
     int i = (int)__umulhi(e0, m_row), j = (int)(e0 - (unsigned)i * (unsigned)Wc);
-    const int a = (int)(ph >> 1), b = (int)(ph & 1);
-    int off[4];
-    bool in[4];
+    const int r0 = 2 * i + (int)a - pad, s0 = 2 * j - pad;
+    const bool fast = j + 3 < Wc && (unsigned)r0 < (unsigned)H && s0 >= 0 && s0 + 7 < W;
+    int off[8];
+    bool in[8];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const int r = 2 * i + a - pad, s = 2 * j + b - pad;
-        in[t] = (unsigned)r < (unsigned)H && (unsigned)s < (unsigned)W;
-        off[t] = r * W + s;
+        const int r = 2 * i + (int)a - pad;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int sx = 2 * j + b - pad;
+            in[2 * t + b] = (unsigned)r < (unsigned)H && (unsigned)sx < (unsigned)W;
+            off[2 * t + b] = r * W + sx;
+        }
         if (++j == Wc) {
             j = 0;
             ++i;
         }
     }
-    for (int pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const long long phase_pair = 2LL * quads_phase;  // float4 units of the two column phases of one row phase
+    for (int pl = blockIdx.y; pl < planes; pl += ny) {
         const float *src = x + (long long)pl * H * W;
-        float v[4];
+        float v[8];
+        if (fast) {
+            const F4U lo = *reinterpret_cast<const F4U *>(src + off[0]);
+            const F4U hi = *reinterpret_cast<const F4U *>(src + off[0] + 4);
+            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+            v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+        } else {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) v[t] = in[t] ? src[off[t]] : 0.f;
-        st_stream(reinterpret_cast<float4 *>(xph) + ((long long)pl * 4 * quads_phase + qi), make_float4(v[0], v[1], v[2], v[3]));
+            for (int t = 0; t < 8; ++t) v[t] = in[t] ? src[off[t]] : 0.f;
+        }
+        float4 *dst = reinterpret_cast<float4 *>(xph) + ((long long)pl * 2 + a) * phase_pair + q;
+        st_stream(dst, make_float4(v[0], v[2], v[4], v[6]));
+        st_stream(dst + quads_phase, make_float4(v[1], v[3], v[5], v[7]));
     }
 }
 
@@ -198,12 +239,15 @@ ag_status_t s2_fwd_prepare(hipStream_t st, const float *x, const float *w, float
 {
     const unsigned quads_phase = (unsigned)(g.pp / 4);
     const long long planes = (long long)B * C;
-    const dim3 grid((4 * quads_phase + 255) / 256, (unsigned)(planes < 65535 ? planes : 65535));
-    hipLaunchKernelGGL(phase_split_kernel, grid, dim3(256), 0, st, x, xpad, (int)planes, H, W, pad, g.Wc, quads_phase,
-                       magic(quads_phase), magic((unsigned)g.Wc));
-    hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, xpad + planes * 4 * g.pp, (int)kS2Slack);
-    hipLaunchKernelGGL(s2_filter_fwd_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
-                       xpad + g.xph_floats, K, C, kh * kw);
+    // one grid row per (image, channel) plane, plus enough rows for a thread per filter element (256 blocks at most)
+    const unsigned gx_blocks = (2 * quads_phase + 255) / 256;
+    unsigned extra_rows = (unsigned)((g.wf_floats + 255) / 256 + gx_blocks - 1) / gx_blocks;
+    if (extra_rows * gx_blocks > 256) extra_rows = (256 + gx_blocks - 1) / gx_blocks;
+    if (extra_rows < 1) extra_rows = 1;
+    const dim3 grid(gx_blocks, (unsigned)(planes < 65535 - extra_rows ? planes : 65535 - extra_rows) + extra_rows);
+    hipLaunchKernelGGL(phase_split_pair_kernel, grid, dim3(256), 0, st, x, xpad, (int)planes, H, W, pad, g.Wc, quads_phase,
+                       magic(quads_phase), magic((unsigned)g.Wc), xpad + planes * 4 * g.pp, (int)kS2Slack, w,
+                       xpad + g.xph_floats, K, C, kh * kw, extra_rows);
     return check_launch("conv2d");
 }
 

@@ -868,7 +868,6 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         if (ag_status_t s = check_launch(who)) return s;
     }
     if (p.splits > 1 && partials_only < 0) {
-        const long long total = (long long)c.M * c.N;
         launch_fold(st, static_cast<const float *>(ws), p.splits, p.sCsplit, real_c, c.M, c.N, c.ldc, c.alpha, c.beta);
         return check_launch(who);
     }
@@ -1018,7 +1017,6 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     launch_direct(st, cfg, true, true, p, num_cus(), g_grid_scale);
     if (ag_status_t s = check_launch("conv2d_filter_grad")) return s;
     if (p.splits > 1) {
-        const long long total = (long long)p.M * p.N;
         launch_fold(st, static_cast<const float *>(ws), p.splits, p.sCsplit, gw, p.M, p.N, (long long)p.N, 1.f, 0.f);
         return check_launch("conv2d_filter_grad");
     }
