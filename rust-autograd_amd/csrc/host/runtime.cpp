@@ -20,39 +20,55 @@ namespace host {
 // hipMalloc after the first step.
 // ---------------------------------------------------------------------------------------------
 struct DeviceBlock {
-    void *ptr = nullptr;
+    void *ptr = nullptr;   // what the array uses
+    void *base = nullptr;  // what hipMalloc returned
     size_t bytes = 0;
     ~DeviceBlock();
 };
 
 namespace {
+// Large blocks start a rotating multiple of 4 KiB into their allocation.  hipMalloc hands out addresses with the
+// same low 21 bits, and an elementwise kernel that streams several such arrays in lockstep (Adam: param, grad, m, v)
+// then sends all of its streams to the same DRAM banks at the same time: 0.354 ms against 0.313 ms for the Adam
+// update of 2^26 elements with the arrays 4 KiB apart modulo 2 MiB.
+constexpr size_t kStaggerFrom = (size_t)1 << 20, kStaggerStep = 4096, kStaggerSlots = 16;
+
 struct Arena {
+    struct Free {
+        void *base, *ptr;
+    };
     std::mutex mu;
-    std::multimap<size_t, void *> free_blocks;
+    std::multimap<size_t, Free> free_blocks;
+    size_t next_slot = 0;
     ~Arena()
     {
-        for (auto &kv : free_blocks) (void)hipFree(kv.second);
+        for (auto &kv : free_blocks) (void)hipFree(kv.second.base);
     }
     static size_t round_up(size_t bytes)
     {
         const size_t q = bytes < (1u << 20) ? 256 : (1u << 16);
         return (bytes + q - 1) / q * q;
     }
-    void *take(size_t bytes)
+    bool take(size_t bytes, Free *out)
     {
         std::lock_guard<std::mutex> lk(mu);
         auto it = free_blocks.lower_bound(bytes);
         if (it != free_blocks.end() && it->first <= bytes + bytes / 8) {
-            void *p = it->second;
+            *out = it->second;
             free_blocks.erase(it);
-            return p;
+            return true;
         }
-        return nullptr;
+        return false;
     }
-    void give(size_t bytes, void *p)
+    size_t stagger()
     {
         std::lock_guard<std::mutex> lk(mu);
-        free_blocks.emplace(bytes, p);
+        return (next_slot++ % kStaggerSlots) * kStaggerStep;
+    }
+    void give(size_t bytes, Free f)
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        free_blocks.emplace(bytes, f);
     }
 };
 Arena &arena()
@@ -68,8 +84,15 @@ std::shared_ptr<DeviceBlock> allocate(size_t bytes)
 {
     auto blk = std::make_shared<DeviceBlock>();
     blk->bytes = Arena::round_up(bytes ? bytes : 4);
-    blk->ptr = arena().take(blk->bytes);
-    if (!blk->ptr) check(hipMalloc(&blk->ptr, blk->bytes), "hipMalloc");
+    Arena::Free f;
+    if (arena().take(blk->bytes, &f)) {
+        blk->base = f.base;
+        blk->ptr = f.ptr;
+        return blk;
+    }
+    const bool large = blk->bytes >= kStaggerFrom;
+    check(hipMalloc(&blk->base, blk->bytes + (large ? kStaggerStep * kStaggerSlots : 0)), "hipMalloc");
+    blk->ptr = static_cast<char *>(blk->base) + (large ? arena().stagger() : 0);
     return blk;
 }
 size_t product(const Shape &s)
@@ -82,7 +105,7 @@ size_t product(const Shape &s)
 
 DeviceBlock::~DeviceBlock()
 {
-    if (ptr) arena().give(bytes, ptr);
+    if (base) arena().give(bytes, Arena::Free{base, ptr});
 }
 
 void *current_stream() { return nullptr; }  // the null stream: every op is ordered on it
