@@ -194,6 +194,49 @@ __global__ __launch_bounds__(256) void s2_filter_parity_kernel(const float *__re
     }
 }
 
+// The pair form of the input gradient (even W): for a row parity a, the two column parities b of a channel are
+// rows 2c + b of ONE product whose taps are the union of the two parities' column shifts (parity b reads gy shifted
+// by d_b - n columns for its tap n; the union is smin .. smax, visited from smax down), with zeros where a parity
+// has no tap at a shift.  The GEMM's epilogue then writes gx[c][2i+a][2j .. 2j+1] as one 8-byte store, so no
+// parity-planar intermediate and no interleaving pass exist; the price is the zero taps (3 x 3, pad 1: 12 instead of
+// 9 tap-products per channel pair) on tiles of 128 rows instead of 64.
+struct S2Pair {
+    int smax, kwp;           // largest column shift, number of shifts in the union
+    long long floats[2];     // elements of the merged filter of row parity a
+};
+
+static bool s2_pair(const S2Geom &g, int C, int K, int W, S2Pair *pr)
+{
+    if (W % 2 != 0 || g.W_b[0] != g.W_b[1] || g.W_b[0] < 1 || g.kw_b[0] < 1 || g.kw_b[1] < 1) return false;
+    const int smax = g.d_a[0] > g.d_a[1] ? g.d_a[0] : g.d_a[1];
+    const int lo0 = g.d_a[0] - g.kw_b[0] + 1, lo1 = g.d_a[1] - g.kw_b[1] + 1;
+    const int smin = lo0 < lo1 ? lo0 : lo1;
+    if (g.L + smin < 0) return false;
+    pr->smax = smax;
+    pr->kwp = smax - smin + 1;
+    for (int a = 0; a < 2; ++a) pr->floats[a] = 2LL * C * g.kh_a[a] * pr->kwp * K;
+    // the merged filters take the place of the parity filters and of the parity-planar result
+    return pr->floats[0] + pr->floats[1] <= g.wf_floats + g.gxp_floats && pr->floats[0] + pr->floats[1] < 0x7fffffffLL;
+}
+
+// wp_a[2c + b][m * kwp + n'][k] = w[k][c][2m + alpha_a][2n + alpha_b] with n = n' - (smax - d_b), or 0 when parity b
+// has no tap n there; the filters of a = 0 and a = 1 back to back.
+__global__ __launch_bounds__(256) void s2_filter_pair_kernel(const float *__restrict__ w, float *__restrict__ wp, int K, int C,
+                                                             int kh, int kw, int pad, int smax, int kwp, int size0, int total)
+{
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int a = e >= size0, rest = a ? e - size0 : e;
+        const int alpha_a = (a + pad) & 1, kha = (kh - alpha_a + 1) / 2;
+        const int k = rest % K, tap = rest / K % (kha * kwp), row = rest / (K * kha * kwp);
+        const int c = row >> 1, b = row & 1;
+        const int alpha_b = (b + pad) & 1, kwb = (kw - alpha_b + 1) / 2, d_b = (b + pad) >> 1;
+        const int m = tap / kwp, n = tap - m * kwp - (smax - d_b);
+        float v = 0.f;
+        if (n >= 0 && n < kwb) v = w[(((long long)k * C + c) * kh + 2 * m + alpha_a) * kw + 2 * n + alpha_b];
+        wp[e] = v;
+    }
+}
+
 // gx[pl][2i+a][2j+b] = gxp_ab[pl][i][j]: four consecutive pixels of a row per thread (W % 4 == 0), or one.
 __global__ __launch_bounds__(256) void s2_interleave_kernel(const float *__restrict__ gxp, float *__restrict__ gx, long long planes,
                                                             int H, int W, int H0, int H1, int W0, int W1, int vec)
@@ -269,8 +312,15 @@ ag_status_t s2_igrad_prepare(hipStream_t st, const float *gy, const float *w, fl
 {
     launch_pad_border(st, gy, scratch, B, K, g.OH, g.OW, g.Hp, g.Wc, g.T, g.L);
     hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, scratch + (long long)B * K * g.Hp * g.Wc, (int)kS2Slack);
-    hipLaunchKernelGGL(s2_filter_parity_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
-                       scratch + g.gyp_floats, K, C, kh, kw, pad);
+    S2Pair pr;
+    if (s2_pair(g, C, K, g.W_b[0] + g.W_b[1], &pr)) {
+        const int total = (int)(pr.floats[0] + pr.floats[1]);
+        hipLaunchKernelGGL(s2_filter_pair_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, scratch + g.gyp_floats,
+                           K, C, kh, kw, pad, pr.smax, pr.kwp, (int)pr.floats[0], total);
+    } else {
+        hipLaunchKernelGGL(s2_filter_parity_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
+                           scratch + g.gyp_floats, K, C, kh, kw, pad);
+    }
     return check_launch("conv2d_transpose");
 }
 
@@ -278,6 +328,24 @@ ag_status_t s2_igrad_gemm(hipStream_t st, float *scratch, float *gx, const S2Geo
 {
     const float *gyp = scratch;
     const float *wr = scratch + g.gyp_floats;
+    S2Pair pr;
+    if (s2_pair(g, C, K, W, &pr)) {
+        // (the prepare step has written the merged filters, so there is no falling back to the parity form here)
+        AG_REQUIRE((reinterpret_cast<uintptr_t>(gx) & 7) == 0, AG_ERR_INVALID_DIMS,
+                   "conv2d_transpose (column-free, stride 2): the output must be 8-byte aligned");
+        for (int a = 0; a < 2; ++a) {
+            if (g.H_a[a] > 0) {
+                const int top = g.kh_a[a] - 1 - g.d_a[a];
+                // the first shift the GEMM visits is the largest: origin + (kwp - 1) = L + smax
+                const float *origin = gyp + (long long)(g.T - top) * g.Wc + (g.L + pr.smax - (pr.kwp - 1));
+                if (ag_status_t s = gemm_conv_input_grad_pair(st, wr, origin, gx, B, C, K, g.H_a[a], g.W_b[0], g.kh_a[a], pr.kwp,
+                                                              g.Hp, g.Wc, a, H, W))
+                    return s;
+            }
+            wr += pr.floats[a];
+        }
+        return AG_OK;
+    }
     float *gxp = scratch + g.gyp_floats + g.wf_floats;
     long long out_off = 0;
     for (int a = 0; a < 2; ++a)

@@ -802,6 +802,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     if (fold) p.N = c.N * c.batch;
     p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
+    p.conv_pair_w = p.conv_pair_a = 0;
     p.conv_phase = 0;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
@@ -878,8 +879,11 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
 // fields of GemmParams): gx[b][c] = sum over taps and filters of wr[c][tap][k] * gyp[b][k] shifted.
 // wr [C][kh*kw*Kf] (k fastest), gyp [B][Kf][Hp][Wp] zero-bordered, gx [B][C][H][W].
 // `phase` != 0: stride-2 forward over four phase planes of `phase` elements per contracted channel.
+// `pair_w` != 0: the pair form of the stride-2 input gradient (C counts the 2 x channels rows; the output planes are
+// pair_h x pair_w and receive row parity pair_a).
 static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
-                                      int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase)
+                                      int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase, int pair_w = 0,
+                                      int pair_a = 0, int pair_h = 0)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
@@ -895,6 +899,11 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.n_off = 0;
     p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
     p.conv_phase = phase;
+    p.conv_pair_w = pair_w; p.conv_pair_a = pair_a;
+    if (pair_w != 0) {
+        p.ldc = (long long)pair_h * pair_w;
+        p.sC = (long long)(C / 2) * pair_h * pair_w;
+    }
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
     // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
@@ -954,6 +963,12 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
     return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0);
 }
 
+ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,
+                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout)
+{
+    return conv_implicit_gemm(st, wr, gyp, gx, B, 2 * C, Kf, Ha, Wb, kh, kw, Hp, Wp, 0, Wout, a, Hout);
+}
+
 ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
                                   int OH, int OW, int kh, int kw, int Hpp, int Wpp)
 {
@@ -1001,6 +1016,7 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     p.alpha = 1.f; p.beta = 0.f;
     p.n_img = 0; p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
+    p.conv_pair_w = p.conv_pair_a = 0;
     p.conv_phase = 0;
     p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)b_plane; p.rows_phase = phase;
     p.C = gw;

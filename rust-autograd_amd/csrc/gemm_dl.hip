@@ -457,7 +457,25 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 }
                 const int iy = col / p.conv_wp, ix = col - iy * p.conv_wp;
                 ok[j] = in_range && ix < p.conv_w;
-                dst0[j] = Cb + img + iy * p.conv_w + ix;
+                dst0[j] = p.conv_pair_w != 0 ? Cb + img + (long long)(2 * iy + p.conv_pair_a) * p.conv_pair_w + 2 * ix
+                                             : Cb + img + iy * p.conv_w + ix;
+            }
+            if (p.conv_pair_w != 0) {
+                // rows come in (channel, parity) pairs: a lane's values v, v + 1 (v even) are the two column
+                // parities of one channel at neighbouring addresses
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
+#pragma unroll
+                        for (int j = 0; j < NI; ++j)
+                            if (ok[j] && row < p.M) {
+                                float2 *dst = reinterpret_cast<float2 *>(dst0[j] + (long long)(row >> 1) * ldc);
+                                *dst = make_float2(alpha * acc[i][j][v], alpha * acc[i][j][v + 1]);
+                            }
+                    }
+                return false;
             }
             // rows outermost: the segments of one output row leave back to back, so the cache lines
             // they share are completed before they can be evicted

@@ -35,6 +35,11 @@ struct GemmParams {
     // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
     // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
     int conv_wp, conv_w, conv_kw;
+    // Stride-2 input gradient, both column parities of row parity conv_pair_a in one product
+    // (conv_pair_w != 0): row m of the result is (channel m / 2, column parity m % 2), column (i, j)
+    // is pixel (2i + conv_pair_a, 2j + m % 2) of an output plane conv_pair_w wide, so the two parities
+    // of a channel leave as one 8-byte store.  ldc / sC are the plane / image strides of that output.
+    int conv_pair_w, conv_pair_a;
     // Stride-2 forward (conv_phase != 0): B holds the four phase planes of the zero-bordered input,
     // [batch][K][2][2][Hpp][conv_wp] with phase (a, b) = elements (2i+a, 2j+b), conv_phase elements
     // each; tap (ky, kx), visited in natural order, reads phase (ky&1, kx&1) shifted by
@@ -72,6 +77,10 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
                                  int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
 // Stride-2 forward over phase planes (see GemmParams::conv_phase): wf [K][kh*kw][C] in natural tap
 // order, xph [B][C][4][Hpp][Wpp], y [B][K][OH][OW].
+// The pair form of the implicit input gradient (see GemmParams::conv_pair_w): wr [2C][kh*kw*Kf], gyp bordered
+// upstream gradient, gx [B][C][Hout][Wout] receives rows 2i + a, i < Ha, and columns 2j + b, j < Wb.
+ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,
+                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout);
 ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
                                   int OH, int OW, int kh, int kw, int Hpp, int Wpp);
 // Stride-2 filter gradient: gw[k][c][ky][kx] = sum over images and positions q of

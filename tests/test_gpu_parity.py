@@ -698,8 +698,9 @@ S2_CASES = [  # B, C, K (filters), H, W, k, pad: stride-2 convolutions without c
 @pytest.mark.parametrize("case", S2_CASES)
 def test_conv2d_stride2_column_free(K, orc, rng, case):
     """Stride 2 without the im2col columns: the forward over the four phase planes of the bordered
-    input, the filter gradient over the same planes and a bordered gy, the input gradient as four
-    parity GEMMs interleaved afterwards.  Against the f64 oracle (with the f32 oracle's error as the
+    input, the filter gradient over the same planes and a bordered gy, the input gradient by output parity
+    (even W: the two column parities of a row in one GEMM that stores them side by side; odd W: four parity GEMMs
+    interleaved afterwards).  Against the f64 oracle (with the f32 oracle's error as the
     yardstick) and, on integer-valued data, bit for bit against the column path."""
     B, C, Kc, H, W, k, p = case
     x = rng.standard_normal((B, C, H, W)).astype(np.float32)
