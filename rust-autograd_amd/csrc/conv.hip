@@ -682,10 +682,11 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
         return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
                                     fg.Wp);
     }
-    // Stride 2: four parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
+    // Stride 2: parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
     // is large enough to serve as their scratch.  Only from 2^24 column elements on: below that the
-    // seven launches cost more than GEMM + col2im (the 4x4 stride-2 transposed convolution
-    // [32,128,14,14] -> [32,64,28,28] takes 0.23 ms this way against 0.15 ms over columns).
+    // launches and the short contractions cost more than GEMM + col2im (the 4x4 stride-2 transposed
+    // convolution [32,128,14,14] -> [32,64,28,28] with both gradients takes 0.21 ms this way against
+    // 0.13 ms over columns).
     S2Geom g2;
     if (stride == 2 && dilation == 1 && g_fused_input_grad && (long long)B * M * P >= (1LL << 24) &&
         s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh &&
