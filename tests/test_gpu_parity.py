@@ -362,6 +362,31 @@ def test_matmul_long_contraction_few_tiles(K, rng, m, n, k, ta, tb):
     assert np.array_equal(host(K.matmul(dev(ai), dev(bi), ta, tb)), exact.astype(np.float32))
 
 
+@pytest.mark.parametrize("m,n,k,ta", [(128, 10, 3136, False), (33, 7, 1025, False), (128, 16, 2048, False), (65, 1, 4096, False),
+                                      (3136, 10, 128, True), (1030, 3, 17, True), (2048, 16, 512, True), (1024, 1, 16, True)])
+def test_matmul_with_a_handful_of_columns(K, rng, m, n, k, ta):
+    """N <= 16 (the classifier layer of the small CNN and its weight gradient): a few output tiles that are mostly
+    padding, long or short contractions.  Same bars as every contraction, exact on small integers, deterministic,
+    and the no-allocation entry agrees bit for bit."""
+    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    say(f"matmul skinny {m}x{n}x{k} ta={ta}")
+    A = (a.T if ta else a).astype(np.float64)
+    got = host(K.matmul(dev(a), dev(b), ta, False))
+    assert_close_conditioned(got, A @ b.astype(np.float64), np.abs(A) @ np.abs(b).astype(np.float64), "skinny matmul",
+                             ref32=(a.T if ta else a) @ b)
+    assert np.array_equal(got, host(K.matmul(dev(a), dev(b), ta, False)))
+    ai = rng.integers(-3, 4, size=a.shape).astype(np.float32)
+    bi = rng.integers(-3, 4, size=b.shape).astype(np.float32)
+    exact = (ai.T if ta else ai).astype(np.int64) @ bi.astype(np.int64)
+    assert np.array_equal(host(K.matmul(dev(ai), dev(bi), ta, False)), exact.astype(np.float32))
+    L = K.capi.lib()
+    c = torch.empty(m, n, device="cuda")
+    da, db = dev(a), dev(b)
+    K.capi.check(L.ag_matmul_f32_noalloc(K._stream(), int(ta), 0, m, n, k, K._ptr(da), a.shape[1], K._ptr(db), n, K._ptr(c), n))
+    assert np.array_equal(host(c), got)
+
+
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_long_k_with_a_tail(K, rng, ta, tb):
     """K = 32 q + r: whole k tiles on the direct-to-LDS kernel, the remaining r accumulated on top."""
