@@ -153,7 +153,9 @@ ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const f
  * `prepare` writes a zero-bordered copy of gy and the filter in tap-major order into `scratch`;
  * `gemm` accumulates gx over the filter taps in implicit GEMMs that read them -- one for stride 1;
  * for stride 2 one per parity of the pixel position, whose results (kept in `scratch`) a copy
- * kernel interleaves into gx.  dilation must be 1.  ag_conv_input_grad_scratch_floats returns the
+ * kernel interleaves into gx.  Stride 1 takes any dilation (the taps are read `dilation` rows and
+ * elements apart in the bordered copy); stride 2 requires dilation 1.
+ * ag_conv_input_grad_scratch_floats returns the
  * scratch size in floats, or 0 when the geometry is not supported (then use
  * ag_conv2d_transpose_f32). */
 size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int yw, int xch, int kh, int kw,
@@ -166,7 +168,8 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, floa
                                         int ych, int yh, int yw, int xch, int kh, int kw, int pad,
                                         int stride, int dilation, int xh, int xw);
 
-/* Column-free convolution (stride 1 or 2, dilation 1): forward and filter gradient without the
+/* Column-free convolution (stride 1 with any dilation, or stride 2 with dilation 1): forward and
+ * filter gradient without the
  * im2col columns.  No counterpart in the reference, which always materialises them (Conv2D::compute
  * -> fast_im2col_gemm_fused_kernel, conv2d.rs:25-112; conv2d_filter_grad_impl, conv2d.rs:631-734);
  * the results are those of ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32 within the floating-point
@@ -176,7 +179,8 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, floa
  * planes x'[2i+a][2j+b] for stride 2 -- and runs one implicit GEMM over the filter taps.  The filter
  * gradient contracts that copy with the zero-bordered upstream gradient that
  * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images
- * in splits that need the workspace; for stride 1 "same" convolutions only (2*pad == kh-1 == kw-1,
+ * in splits that need the workspace; for stride 1 "same" convolutions only
+ * (2*pad == dilation*(kh-1) == dilation*(kw-1),
  * K a multiple of 32), so that both copies share one padded plane shape.  The contraction runs a
  * few elements past a plane, but only over zeros of both operands (the planes are sized for that),
  * so a NaN or infinity in one channel of x reaches the gradients of that channel only; within the

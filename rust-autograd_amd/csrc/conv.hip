@@ -427,10 +427,12 @@ struct FusedGeom {
 };
 
 // False when the geometry does not allow the implicit path.
-static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad, int xh, int xw, FusedGeom *g)
+// `dil`: the filter taps are dil apart; borders and reach follow the filter's extent ekh = dil*(kh-1)+1.
+static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad, int xh, int xw, FusedGeom *g, int dil = 1)
 {
-    if (pad > kh - 1 || pad > kw - 1 || ych % 32 != 0 || B < 1 || xch < 1) return false;
-    if (yh != xh + 2 * pad - kh + 1 || yw != xw + 2 * pad - kw + 1 || yh < 1 || yw < 1) return false;
+    const int ekh = dil * (kh - 1) + 1, ekw = dil * (kw - 1) + 1;
+    if (dil < 1 || pad > ekh - 1 || pad > ekw - 1 || ych % 32 != 0 || B < 1 || xch < 1) return false;
+    if (yh != xh + 2 * pad - ekh + 1 || yw != xw + 2 * pad - ekw + 1 || yh < 1 || yw < 1) return false;
     // A padded row holds the left border (kw-1-pad zeros) and the data; it needs no right border of
     // its own: a read that runs past the end of a row by up to kw-1-pad elements lands in the left
     // border of the next row, which is just as zero.  The row pitch and the plane (rows added at the
@@ -440,33 +442,35 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     // everything it reads past a plane's own data is zero -- the rows below the data, then the top
     // border of the next plane up to the first data element of its first data row -- so that no value
     // of a neighbouring plane (which could be a NaN) ever meets one of those zeros.
-    const int top = kh - 1 - pad, left = kw - 1 - pad;
+    const int top = ekh - 1 - pad, left = ekw - 1 - pad;
     g->Wp = yw + left;
     for (;; ++g->Wp) {
-        if (g->Wp > xw + kw + 6) return false;
+        if (g->Wp > xw + ekw + 6) return false;
         if (((long long)xh * g->Wp) % 4 != 0) continue;
-        g->Hp = xh + kh - 1;
+        g->Hp = xh + ekh - 1;
         const long long kq = (((long long)xh * g->Wp + 31) / 32) * 32;
         while (((long long)g->Hp * g->Wp) % 4 != 0 || (long long)(g->Hp - top) * g->Wp - left < kq) ++g->Hp;
         break;
     }
     // past the last plane the reads run into kSlackFloats zeroed floats
-    if ((long long)(kh - 1) * g->Wp + 2 * (kw - 1) + 32 > kSlackFloats) return false;
+    if ((long long)(ekh - 1) * g->Wp + 2 * (ekw - 1) + 32 > kSlackFloats) return false;
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
-    // a tile (64 x 128 for up to 64 channels, else 128 x 256) may straddle two images, not three
+    // a tile (64 x 128 for up to 64 channels, else 128 x 256) may straddle two images, not three.  (Images of
+    // fewer than 256 positions with more channels would run on 64 x 64 tiles, where the column path is as fast:
+    // 0.315 ms against 0.306 ms for the three contractions of 32 x 256 -> 256 x 14 x 14.)
     return n_img >= (xch <= 64 ? 128 : 256) && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
 }
 
 static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const FusedGeom &g,
-                                 int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad)
+                                 int B, int ych, int yh, int yw, int xch, int kh, int kw, int pad, int dil = 1)
 {
     const long long quads = (long long)B * ych * g.Hp * g.Wp / 4;
     // the implicit filter gradient may read a few elements past the last plane and expects zeros
     const PrepareExtras ex = {scratch, 0, scratch + quads * 4, (int)(g.gyp_floats - quads * 4), w, scratch + g.gyp_floats,
                               ych, xch, kh * kw, 0};
-    if (!launch_pad_border_with(st, gy, scratch, B, ych, yh, yw, g.Hp, g.Wp, kh - 1 - pad, kw - 1 - pad, &ex)) {
+    if (!launch_pad_border_with(st, gy, scratch, B, ych, yh, yw, g.Hp, g.Wp, dil * (kh - 1) - pad, dil * (kw - 1) - pad, &ex)) {
         hipLaunchKernelGGL(zero_slack_kernel, dim3(4), dim3(256), 0, st, ex.lead, ex.n_lead, ex.tail, ex.n_tail);
         hipLaunchKernelGGL(filter_taps_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w,
                            scratch + g.gyp_floats, ych, xch, kh * kw);
@@ -480,12 +484,13 @@ static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w
 // row and column before the first plane.
 constexpr long long kFwdLeadFloats = kSlackFloats;
 
-static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, FusedGeom *g)
+static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, int pad, FusedGeom *g, int dil = 1)
 {
-    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
-    if (OH < 1 || OW < 1 || pad > kh - 1 || pad > kw - 1) return false;
-    // seen as an input gradient: "gy" = x [C, H, W], "gx" = y [K, OH, OW], border kh-1-pad' = pad
-    return kh == kw && fused_geom(B, C, H, W, K, kh, kw, kh - 1 - pad, OH, OW, g);
+    const int ekh = dil * (kh - 1) + 1, ekw = dil * (kw - 1) + 1;
+    const int OH = H + 2 * pad - ekh + 1, OW = W + 2 * pad - ekw + 1;
+    if (dil < 1 || OH < 1 || OW < 1 || pad > ekh - 1 || pad > ekw - 1) return false;
+    // seen as an input gradient: "gy" = x [C, H, W], "gx" = y [K, OH, OW], border ekh-1-pad' = pad
+    return kh == kw && fused_geom(B, C, H, W, K, kh, kw, ekh - 1 - pad, OH, OW, g, dil);
 }
 
 // Positions of the flattened padded plane that the implicit filter gradient contracts over: all
@@ -504,11 +509,11 @@ static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
 // ---- column-free convolution: forward and filter gradient ---------------------------------------
 // No counterpart of these in the reference, which always materialises the columns
 // (conv2d.rs:25-112, 631-734); they compute the same y and gw from a rearranged copy of x: the
-// zero-bordered input for stride 1, its four phase planes for stride 2 (conv_s2.hip).  dilation must
-// be 1.  `xpad`: ag_conv2d_nocols_scratch_floats() floats, written by the forward and read by the
+// zero-bordered input for stride 1 (any dilation), its four phase planes for stride 2 (conv_s2.hip; dilation
+// 1 only).  `xpad`: ag_conv2d_nocols_scratch_floats() floats, written by the forward and read by the
 // filter gradient.  0 floats = geometry not supported (use ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32).
 namespace ag {
-static bool nocols_mode(int stride, int dilation) { return dilation == 1 && (stride == 1 || stride == 2); }
+static bool nocols_mode(int stride, int dilation) { return (stride == 1 && dilation >= 1) || (stride == 2 && dilation == 1); }
 }  // namespace ag
 
 extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh, int kw, int pad, int stride,
@@ -520,7 +525,7 @@ extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, in
         return s2_geom(B, C, H, W, K, kh, kw, pad, &g2) ? (size_t)(g2.xph_floats + g2.wf_floats) : 0;
     }
     FusedGeom g;
-    if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g)) return 0;
+    if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation)) return 0;
     return (size_t)(kFwdLeadFloats + g.gyp_floats + g.wr_floats);
 }
 
@@ -539,7 +544,7 @@ extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const fl
         return s2_fwd_prepare(st, x, w, xpad, g2, B, C, H, W, K, kh, kw, pad);
     }
     FusedGeom g;
-    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad), AG_ERR_INVALID_DIMS,
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) && aligned16(xpad), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
     float *xp = xpad + kFwdLeadFloats, *wf = xp + g.gyp_floats;
     const long long quads = (long long)B * C * g.Hp * g.Wp / 4;
@@ -565,11 +570,11 @@ extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float
         return s2_fwd_gemm(as_stream(stream), xpad, xpad + g2.xph_floats, y, g2, B, C, K, kh, kw);
     }
     FusedGeom g;
-    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
     const float *xp = xpad + kFwdLeadFloats;
-    return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1,
-                                kh, kw, g.Hp, g.Wp);
+    return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - dilation * (kh - 1),
+                                W + 2 * pad - dilation * (kw - 1), kh, kw, g.Hp, g.Wp, dilation);
 }
 
 extern "C" ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y, float *xpad,
@@ -598,13 +603,13 @@ extern "C" ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, cons
         return s2_fwd_gemm(st, xpad, wf, y, g2, B, C, K, kh, kw);
     }
     FusedGeom g;
-    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && aligned16(xpad) && aligned16(y) && aligned16(wf),
+    AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) && aligned16(xpad) && aligned16(y) && aligned16(wf),
                AG_ERR_INVALID_DIMS, "conv2d (column-free): geometry not supported");
     hipLaunchKernelGGL(filter_taps_fwd_kernel, dim3((unsigned)((g.wr_floats + 255) / 256)), dim3(256), 0, st, w, wf, K, C,
                        kh * kw);
     if (ag_status_t s = check_launch("conv2d")) return s;
-    return gemm_conv_input_grad(st, wf, xpad + kFwdLeadFloats, y, B, K, C, H + 2 * pad - kh + 1, W + 2 * pad - kw + 1, kh, kw,
-                                g.Hp, g.Wp);
+    return gemm_conv_input_grad(st, wf, xpad + kFwdLeadFloats, y, B, K, C, H + 2 * pad - dilation * (kh - 1),
+                                W + 2 * pad - dilation * (kw - 1), kh, kw, g.Hp, g.Wp, dilation);
 }
 
 // gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the start
@@ -619,9 +624,10 @@ extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H
         return s2_geom(B, C, H, W, K, kh, kw, pad, &g2) ? s2_filter_grad_workspace(g2, B, C, K, kh, kw) : 0;
     }
     FusedGeom g, gg;
-    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
-    if (2 * pad != kh - 1 || 2 * pad != kw - 1 || K % 4 != 0 || !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) ||
-        !fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg) || g.Hp != gg.Hp || g.Wp != gg.Wp ||
+    const int OH = H + 2 * pad - dilation * (kh - 1), OW = W + 2 * pad - dilation * (kw - 1);
+    if (2 * pad != dilation * (kh - 1) || 2 * pad != dilation * (kw - 1) || K % 4 != 0 ||
+        !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) ||
+        !fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) || g.Hp != gg.Hp || g.Wp != gg.Wp ||
         (long long)C * g.Hp * g.Wp >= (1LL << 30))
         return 0;
     const int kq = filter_grad_positions(g, OH, pad);
@@ -642,16 +648,17 @@ extern "C" ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, cons
         return s2_filter_grad(as_stream(stream), xpad, gypad, gw, g2, B, C, K, kh, kw, ws, ws_bytes);
     }
     FusedGeom g, gg;
-    const int OH = H + 2 * pad - kh + 1, OW = W + 2 * pad - kw + 1;
-    AG_REQUIRE(2 * pad == kh - 1 && 2 * pad == kw - 1 && K % 4 == 0 && C >= 1 &&
-                   fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g) && fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg) &&
+    const int OH = H + 2 * pad - dilation * (kh - 1), OW = W + 2 * pad - dilation * (kw - 1);
+    AG_REQUIRE(2 * pad == dilation * (kh - 1) && 2 * pad == dilation * (kw - 1) && K % 4 == 0 && C >= 1 &&
+                   fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) &&
+                   fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) &&
                    g.Hp == gg.Hp && g.Wp == gg.Wp && aligned16(xpad) && aligned16(gypad),
                AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): geometry not supported");
     const int kq = filter_grad_positions(g, OH, pad);
     AG_REQUIRE(kq > 0 && (long long)C * g.Hp * g.Wp < (1LL << 30), AG_ERR_INVALID_DIMS,
                "conv2d_filter_grad (column-free): plane too small or too many channels");
     return gemm_conv_filter_grad(as_stream(stream), gypad, xpad + kFwdLeadFloats, gw, ws, ws_bytes, B, K, C, kh, kw, pad, g.Hp,
-                                 g.Wp, kq);
+                                 g.Wp, kq, dilation);
 }
 
 extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const float *w,
@@ -671,16 +678,16 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
                AG_ERR_INCOMPATIBLE_SHAPE,
                "conv2d_transpose: output %dx%d too small for input %dx%d (k=%dx%d stride=%d pad=%d dilation=%d)", xh,
                xw, yh, yw, kh, kw, stride, pad, dilation);
-    // Stride 1, dilation 1: the gradient is accumulated over filter taps inside one GEMM that
+    // Stride 1: the gradient is accumulated over filter taps inside one GEMM that
     // reads a zero-bordered copy of gy; the columns (conv2d_transpose.rs:148-151) are never
     // written.  The sum runs over (tap, filter) instead of filters then taps, within tolerance.
     FusedGeom fg;
-    if (stride == 1 && dilation == 1 && g_fused_input_grad &&
-        fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
+    if (stride == 1 && g_fused_input_grad &&
+        fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg, dilation) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
         aligned16(gcols) && aligned16(gx)) {
-        if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad)) return s;
+        if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad, dilation)) return s;
         return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
-                                    fg.Wp);
+                                    fg.Wp, dilation);
     }
     // Stride 2: parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
     // is large enough to serve as their scratch.  Only from 2^24 column elements on: below that the
@@ -746,7 +753,7 @@ extern "C" size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int 
         return (size_t)(g2.gyp_floats + g2.wf_floats + g2.gxp_floats);
     }
     FusedGeom g;
-    return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) ? (size_t)(g.gyp_floats + g.wr_floats) : 0;
+    return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) ? (size_t)(g.gyp_floats + g.wr_floats) : 0;
 }
 
 extern "C" ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w, float *scratch,
@@ -763,9 +770,9 @@ extern "C" ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const 
         return s2_igrad_prepare(as_stream(stream), gy, w, scratch, g2, B, xch, ych, kh, kw, pad);
     }
     FusedGeom g;
-    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch), AG_ERR_INVALID_DIMS,
+    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) && aligned16(scratch), AG_ERR_INVALID_DIMS,
                "conv_input_grad_prepare: geometry not supported by the column-free path");
-    return fused_prepare(as_stream(stream), gy, w, scratch, g, B, ych, yh, yw, xch, kh, kw, pad);
+    return fused_prepare(as_stream(stream), gy, w, scratch, g, B, ych, yh, yw, xch, kh, kw, pad, dilation);
 }
 
 extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, float *gx, int B, int ych,
@@ -782,8 +789,8 @@ extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *sc
         return s2_igrad_gemm(as_stream(stream), scratch, gx, g2, B, xch, ych, xh, xw);
     }
     FusedGeom g;
-    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g) && aligned16(scratch) && aligned16(gx),
+    AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) && aligned16(scratch) && aligned16(gx),
                AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: geometry not supported by the column-free path");
     return gemm_conv_input_grad(as_stream(stream), scratch + g.gyp_floats, scratch, gx, B, xch, ych, xh, xw, kh, kw, g.Hp,
-                                g.Wp);
+                                g.Wp, dilation);
 }

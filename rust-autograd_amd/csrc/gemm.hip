@@ -804,6 +804,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.conv_wp = p.conv_w = p.conv_kw = 0;
     p.conv_pair_w = p.conv_pair_a = 0;
     p.conv_phase = 0;
+    p.conv_dil = 1;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
     p.tiles_m = (int)cdiv(c.M, kCfgs[cfg].bm);
@@ -883,7 +884,7 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
 // pair_h x pair_w and receive row parity pair_a).
 static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
                                       int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase, int pair_w = 0,
-                                      int pair_a = 0, int pair_h = 0)
+                                      int pair_a = 0, int pair_h = 0, int dil = 1)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
@@ -899,6 +900,7 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.n_off = 0;
     p.conv_wp = Wp; p.conv_w = W; p.conv_kw = kw;
     p.conv_phase = phase;
+    p.conv_dil = dil;
     p.conv_pair_w = pair_w; p.conv_pair_a = pair_a;
     if (pair_w != 0) {
         p.ldc = (long long)pair_h * pair_w;
@@ -908,9 +910,11 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.rows_plane = p.rows_phase = 0;
     // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
     // CU); else 128 x 256, or 128 x 128 when an image has fewer than 256 columns
-    const int cfg = C <= 32   ? kDirectCfg32
-                    : C <= 64 ? (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64 ? kDirectCfg64Narrow : kDirectCfg64)
-                              : (p.n_img >= 256 ? 14 : 13);
+    int cfg = C <= 32   ? kDirectCfg32
+              : C <= 64 ? (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64 ? kDirectCfg64Narrow : kDirectCfg64)
+                        : (p.n_img >= 256 ? 14 : 13);
+    if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && kCfgs[g_force_cfg].bn <= p.n_img)
+        cfg = g_force_cfg;  // test hook
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n;
@@ -958,9 +962,9 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
 }
 
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
-                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp)
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil)
 {
-    return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0);
+    return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0, 0, 0, 0, dil);
 }
 
 ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,
@@ -998,7 +1002,7 @@ size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq)
 // split into four phase planes per channel (stride 2).
 static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const float *xp, float *gw, void *ws, size_t ws_bytes,
                                          int B, int Kf, int C, int kh, int kw, int Wp, int kq, long long a_plane,
-                                         long long b_plane, unsigned phase)
+                                         long long b_plane, unsigned phase, int dil = 1)
 {
     const int taps = kh * kw;
     GemmParams p;
@@ -1018,6 +1022,7 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     p.conv_wp = p.conv_w = p.conv_kw = 0;
     p.conv_pair_w = p.conv_pair_a = 0;
     p.conv_phase = 0;
+    p.conv_dil = dil;
     p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)b_plane; p.rows_phase = phase;
     p.C = gw;
     if (p.splits > 1) {
@@ -1040,12 +1045,12 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
 }
 
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
-                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq)
+                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq, int dil)
 {
     const long long plane = (long long)Hp * Wp;
     // positions are counted from the first gradient value
     return conv_filter_grad_gemm(st, gyp + ((long long)pad * Wp + pad), xp, gw, ws, ws_bytes, B, Kf, C, kh, kw, Wp, kq, plane,
-                                 plane, 0);
+                                 plane, 0, dil);
 }
 
 size_t gemm_conv_filter_grad_stride2_workspace(int B, int Kf, int C, int taps)

@@ -83,11 +83,11 @@ struct DirectTile {
         }
     }
     // k-contiguous rows that are (channel, tap) pairs of a zero-bordered input (implicit filter
-    // gradient): row n starts (n / taps) * plane + ky * wp + kx elements after the origin.
+    // gradient): row n starts (n / taps) * plane + (ky * wp + kx) * dil elements after the origin.
     // `phase` != 0 (stride 2): the input is split into four phase planes of `phase` elements each and
     // tap (ky, kx) reads phase (ky&1, kx&1) shifted by (ky>>1) rows and (kx>>1) elements.
     __device__ inline void init_conv_rows(int row0, int rows, int taps, int kw, int wp, unsigned plane, unsigned phase,
-                                          int wave, int lane)
+                                          int dil, int wave, int lane)
     {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
@@ -97,7 +97,7 @@ struct DirectTile {
             const int ch = row / taps, tap = row - ch * taps;
             const int ky = tap / kw, kx = tap - ky * kw;
             const unsigned shift = phase != 0 ? (unsigned)((ky & 1) * 2 + (kx & 1)) * phase + (unsigned)((ky >> 1) * wp + (kx >> 1))
-                                              : (unsigned)(ky * wp + kx);
+                                              : (unsigned)((ky * wp + kx) * dil);
             off[i] = ((unsigned)ch * plane + shift + (unsigned)(c * 4)) * 4u;
         }
     }
@@ -256,7 +256,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     const float *pb_group = nullptr;           // stride-2 forward: B origin of the current group of 32 channels
     int fkt = 0, f_left = 0, f_kx = 0, f_ky = 0;
     const int conv_first_shift =
-        p.conv_wp != 0 && p.conv_phase == 0 ? (p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1) : 0;
+        p.conv_wp != 0 && p.conv_phase == 0 ? ((p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1)) * p.conv_dil : 0;
     Cursor fcur = first;
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
@@ -265,7 +265,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
             ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
         } else if (KB && p.rows_taps != 0) {
-            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, wave, lane);
+            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, p.conv_dil, wave, lane);
         } else {
             ldr_b.init(ldb, it.n0, p.N, wave, lane);
         }
@@ -315,9 +315,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 pa += p.sAk;
                 if (++f_kx == p.conv_kw) {  // next tap: one column to the left, or up a row
                     f_kx = 0;
-                    pb += p.conv_kw - 1 - p.conv_wp;
+                    pb += (p.conv_kw - 1 - p.conv_wp) * p.conv_dil;
                 } else {
-                    pb -= 1;
+                    pb -= p.conv_dil;
                 }
             }
         } else if (++fkt == kt_per) {

@@ -35,6 +35,9 @@ struct GemmParams {
     // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
     // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
     int conv_wp, conv_w, conv_kw;
+    // Dilation of the stride-1 forms (input gradient and filter gradient): every tap shift above and
+    // below is multiplied by it.  1 for the stride-2 forms.
+    int conv_dil;
     // Stride-2 input gradient, both column parities of row parity conv_pair_a in one product
     // (conv_pair_w != 0): row m of the result is (channel m / 2, column parity m % 2), column (i, j)
     // is pixel (2i + conv_pair_a, 2j + m % 2) of an output plane conv_pair_w wide, so the two parities
@@ -72,9 +75,9 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
 // split over images.
 size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq);
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
-                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq);
+                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq, int dil = 1);
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
-                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp);
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil = 1);
 // Stride-2 forward over phase planes (see GemmParams::conv_phase): wf [K][kh*kw][C] in natural tap
 // order, xph [B][C][4][Hpp][Wpp], y [B][K][OH][OW].
 // The pair form of the implicit input gradient (see GemmParams::conv_pair_w): wr [2C][kh*kw*Kf], gyp bordered

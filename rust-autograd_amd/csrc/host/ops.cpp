@@ -162,7 +162,7 @@ struct Conv2DFilterGrad : Op, ConvHyper {  // conv2d.rs:736-776
         const int B = (int)gy.shape()[0], K = (int)gy.shape()[1], P = (int)(gy.shape()[2] * gy.shape()[3]);
         const int CK = (int)(w.shape()[1] * w.shape()[2] * w.shape()[3]);
         NdArray gw = NdArray::empty(w.shape());
-        if (cols.ndim() == 1) {  // the rearranged input of a column-free Conv2D (stride 1 or 2, dilation 1)
+        if (cols.ndim() == 1) {  // the rearranged input of a column-free Conv2D (stride 1, or stride 2 with dilation 1)
             const int C = (int)w.shape()[1], kh = (int)w.shape()[2], kw = (int)w.shape()[3];
             const int OH = (int)gy.shape()[2], OW = (int)gy.shape()[3];
             // extents of x: from the optional fourth input (only its shape is read), else what a unit

@@ -838,6 +838,31 @@ def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, p
     assert_close(gxv, orc.conv2d_transpose(gyv, wv, pad, 1, 1, out_hw=(H, H)), "gx", scale=np.abs(gxv).max())
 
 
+@pytest.mark.parametrize("B,Cin,Cout,H,k,pad,d", [(64, 32, 64, 32, 3, 2, 2), (40, 64, 32, 30, 3, 3, 3)])
+def test_dilated_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, pad, d):
+    # a dilated "same" stride-1 convolution large enough for Conv2D to go column-free: the kept second output is
+    # the bordered input (rank 1) and the three operators read their taps `d` apart; `columns=True` keeps the
+    # reference's columns, and both agree with the oracle
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    wv = glorot(rng, (Cout, Cin, k, k))
+    oy, ocols = orc.conv2d_fwd(xv, wv, pad, 1, d)
+    gyv = (2 * oy).astype(np.float32)
+    ogw = orc.conv2d_filter_grad(ocols, gyv, wv.shape)
+    ogx = orc.conv2d_transpose(gyv, wv, pad, 1, d, out_hw=(H, H))
+    for columns in (False, True):
+        env = G.VariableEnvironment()
+        c = env.context()
+        x, w = c.placeholder("x", list(xv.shape)), c.placeholder("w", list(wv.shape))
+        y = c.dilated_conv2d(x, w, pad, 1, d, columns=columns)
+        gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+        say(f"dilated conv through the graph B={B} C={Cin} K={Cout} H={H} d={d} columns={columns}")
+        yv, gxv, gwv, kept = c.eval([y, gx, gw, c.nth_tensor(y, 1)], {"x": xv, "w": wv})
+        assert (kept.ndim == 1) == (not columns)
+        assert_close(yv, oy, "y", scale=1.0)
+        assert_close(gwv, ogw, "gw", scale=np.abs(ogw).max())
+        assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max())
+
+
 @pytest.mark.parametrize("H", [32, 33])
 def test_conv2d_stride2_column_free_through_the_graph_and_the_column_switch(G, orc, rng, H):
     # stride 2 at a size where Conv2D goes column-free: the kept second output is the phase-split input

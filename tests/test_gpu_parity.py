@@ -627,6 +627,95 @@ def test_conv2d_column_free_random_geometries_exact(K):
     assert ran_fwd >= 20 and ran_bwd >= 5, (ran_fwd, ran_bwd)
 
 
+DILATED_NOCOLS_CASES = [  # B, C, K, H, W, k, pad, dilation
+    (2, 64, 64, 28, 28, 3, 2, 2),    # the dilated configuration, 2 of its images: a "same" convolution
+    (3, 32, 64, 20, 22, 3, 2, 2),    # uneven extents
+    (2, 32, 32, 24, 24, 3, 3, 3),    # dilation 3, "same"
+    (2, 64, 160, 19, 19, 5, 4, 2),   # 5x5 taps two apart, two row tiles of filters
+    (2, 32, 64, 24, 24, 3, 0, 2),    # no padding: forward and input gradient only
+    (2, 32, 32, 26, 26, 3, 1, 2),    # pad below the "same" value
+    (2, 32, 64, 20, 20, 3, 4, 2),    # pad equal to the filter's reach
+]
+
+
+@pytest.mark.parametrize("case", DILATED_NOCOLS_CASES)
+def test_conv2d_column_free_dilated(K, orc, rng, case):
+    """Dilated stride-1 convolution without columns: the taps of the implicit GEMMs are `dilation`
+    elements and rows apart in the zero-bordered planes.  Forward, input gradient and (for "same"
+    geometries) filter gradient against the f64 oracle, and bit for bit against the columns path on
+    integer-valued data (a tap read one element off cannot hide in a tolerance)."""
+    B, C, Kc, H, W, k, p, d = case
+    L = K.capi.lib()
+    OH, OW = H + 2 * p - d * (k - 1), W + 2 * p - d * (k - 1)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, OH, OW)).astype(np.float32)
+    say("dilated column-free forward", case)
+    res = K.conv2d_nocols(dev(x), dev(w), p, 1, d)
+    assert res is not None, "geometry expected to be supported"
+    y, xpad = res
+    y64, cols64 = orc.conv2d_fwd(x.astype(np.float64), w.astype(np.float64), p, 1, d)
+    yabs, colsabs = orc.conv2d_fwd(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), p, 1, d)
+    y32, cols32 = orc.conv2d_fwd(x, w, p, 1, d)
+    assert tuple(y.shape) == y64.shape == (B, Kc, OH, OW)
+    assert_close_conditioned(host(y), y64, yabs, "dilated column-free forward", ref32=y32)
+    say("dilated staged input gradient", case)
+    staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 1, d)
+    assert staged is not None
+    gx, gypad = staged
+    gx64 = orc.conv2d_transpose(gy.astype(np.float64), w.astype(np.float64), p, 1, d, out_hw=(H, W))
+    gxabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, d, out_hw=(H, W))
+    assert_close_conditioned(host(gx), gx64, gxabs, "dilated staged input gradient",
+                             ref32=orc.conv2d_transpose(gy, w, p, 1, d, out_hw=(H, W)))
+    same = 2 * p == d * (k - 1)
+    assert (L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, d) > 0) == same
+    if same:
+        say("dilated column-free filter gradient", case)
+        gw = host(K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p, 1, d))
+        gw64 = orc.conv2d_filter_grad(cols64, gy.astype(np.float64), w.shape)
+        gwabs = orc.conv2d_filter_grad(colsabs, np.abs(gy).astype(np.float64), w.shape)
+        assert_close_conditioned(gw, gw64, gwabs, "dilated column-free filter gradient",
+                                 ref32=orc.conv2d_filter_grad(cols32, gy, w.shape))
+    # integer-valued data: bit for bit equal to the columns path
+    xi = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    wi = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gyi = rng.integers(-2, 3, (B, Kc, OH, OW)).astype(np.float32)
+    say("dilated column-free exact", case)
+    yi, xpadi = K.conv2d_nocols(dev(xi), dev(wi), p, 1, d)
+    yi_cols, colsi = K.conv2d(dev(xi), dev(wi), p, 1, d)
+    assert np.array_equal(host(yi), host(yi_cols))
+    gxi, gypadi = K.conv_input_grad_staged(dev(gyi), dev(wi), p, (H, W), 1, d)
+    gxi_cols, _ = K.conv2d_transpose(dev(gyi), dev(wi), p, 1, d, out_hw=(H, W), return_cols=True)
+    assert np.array_equal(host(gxi), host(gxi_cols))
+    if same:
+        gwi = K.conv2d_filter_grad_nocols(xpadi, gypadi, xi.shape, wi.shape, p, 1, d)
+        assert np.array_equal(host(gwi), host(K.conv2d_filter_grad(colsi, dev(gyi), wi.shape)))
+
+
+@pytest.mark.parametrize("cfg", [13, 14, 18, 19, 21])
+@pytest.mark.parametrize("d", [1, 2])
+def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d):
+    # the implicit forward and input gradient on each tile shape of the direct-to-LDS kernel that they can run
+    # on (the library picks one by channel count and size): integer-valued data, bit for bit the columns path
+    B, C, Kc, H, W, k = 3, 64, 96, 22, 26, 3
+    p = d
+    L = K.capi.lib()
+    x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
+    y_cols, _ = K.conv2d(dev(x), dev(w), p, 1, d)
+    gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, d, out_hw=(H, W), return_cols=True)
+    say("column-free with a forced tile shape", (cfg, d))
+    L.ag_test_gemm_force_config(cfg)
+    try:
+        y, _ = K.conv2d_nocols(dev(x), dev(w), p, 1, d)
+        gx, _ = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 1, d)
+    finally:
+        L.ag_test_gemm_force_config(-1)
+    assert np.array_equal(host(y), host(y_cols))
+    assert np.array_equal(host(gx), host(gx_cols))
+
+
 def test_conv2d_column_free_headline_size_matches_columns_path(K):
     # the benchmark's own shape (B=256, 64 -> 128 channels, 56x56, 3x3): the three column-free results
     # against the library's column path, which the smaller cases pin to the oracle
