@@ -910,10 +910,24 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
     // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
-    // CU); else 128 x 256, or 128 x 128 when an image has fewer than 256 columns
-    int cfg = C <= 32   ? kDirectCfg32
-              : C <= 64 ? (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64 ? kDirectCfg64Narrow : kDirectCfg64)
-                        : (p.n_img >= 256 ? 14 : 13);
+    // CU); else 128 x 256 (128 x 128 when an image has fewer than 256 columns) or 64 x 128, whichever needs less
+    // time by rounds of the persistent grid times the cost of a tile: padding rows and the idle part of a last
+    // round cost as much as real work (B = 128, 64 -> 192 channels, 28 x 28: 0.30 ms on 128 x 256 tiles -- 256
+    // rows in 3.2 rounds -- against 0.21 ms on 64 x 128 ones)
+    int cfg = C <= 32 ? kDirectCfg32 : kDirectCfg64;
+    if (C > 32 && C <= 64) {
+        if (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64) cfg = kDirectCfg64Narrow;
+    } else if (C > 64) {
+        const long long G = direct_grid(num_cus());
+        const int wide = p.n_img >= 256 ? 14 : 13;
+        const long long wide_tiles = cdiv(C, 128) * cdiv(p.N, kCfgs[wide].bn);
+        double wide_rounds = (double)cdiv(wide_tiles, G);
+        if (wide == 14 && C <= 128 && wide_tiles > G && wide_tiles % G != 0)  // the narrow-tile tail launch below
+            wide_rounds = (double)(wide_tiles / G) + 0.3;
+        const double wide_cost = wide_rounds * 128.0 * kCfgs[wide].bn / (wide == 14 ? 1.0 : 0.9);
+        const double small_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 128), 2 * G) * 2.0 * 64.0 * 128.0 / 0.95;
+        cfg = wide_cost <= small_cost ? wide : kDirectCfg64;
+    }
     if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && kCfgs[g_force_cfg].bn <= p.n_img)
         cfg = g_force_cfg;  // test hook
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
@@ -988,7 +1002,10 @@ static int conv_filter_grad_cfg(int Kf, long long cols)
     if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs) return g_force_cfg;  // test hook
     if (Kf <= 32) return kDirectCfg32;
     if (Kf <= 64) return cols >= 512 ? kDirectCfg64 : kDirectCfg64Narrow;
-    return 17;
+    // 192 x 128 where that pads less (160 or 192 filters: 0.90 against 1.21 ms at B = 64, 160 -> 160, 56 x 56)
+    const double tall = (double)(cdiv(Kf, 192) * 192) * (double)(cdiv(cols, 128) * 128) / 0.95;
+    const double wide = (double)(cdiv(Kf, 128) * 128) * (double)(cdiv(cols, 192) * 192);
+    return tall < wide ? 16 : 17;
 }
 
 static int conv_filter_grad_splits(int B, int Kf, int C, int taps, int kq)
