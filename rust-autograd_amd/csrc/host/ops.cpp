@@ -84,6 +84,68 @@ struct ZerosLike : Op {
     void grad(GradientContext &ctx) const override { ctx.append_input_grad(std::nullopt); }
 };
 
+// A constant spread over the extents of input 0: what broadcasting a constant gradient back through a
+// reduction gives (ReduceSumToScalarGrad, ReduceGradCommon: reduction_ops.rs:139-159, 459-512) when that
+// gradient is itself a constant -- the seed scalar(1) of a back-propagation and everything between it and the
+// first tensor that depends on data.  One fill instead of a fill, a broadcast per reduction and a division per
+// mean: the nodes it stands for are never evaluated.  `mean_axes[j]`: the value is divided by the product of
+// those extents of input 1 + j, as f32, for the j-th mean reduction the constant passed back through -- the
+// arithmetic of the nodes it replaces, in their order.
+struct FilledLike : Op {
+    float value;
+    std::vector<std::vector<int>> mean_axes;
+    FilledLike(float v, std::vector<std::vector<int>> m) : value(v), mean_axes(std::move(m)) {}
+    const char *name() const override { return "FilledLike"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        float v = value;
+        for (size_t j = 0; j < mean_axes.size(); ++j) {
+            const NdArray x = ctx.input(1 + j);
+            const int rank = x.ndim();
+            float len = 1.f;
+            for (int a : mean_axes[j]) {
+                const int ax = a < 0 ? a + rank : a;
+                if (ax < 0 || ax >= rank) return OpError::make(ErrorKind::OutOfBounds, "reduce: axis out of range");
+                len *= (float)x.shape()[(size_t)ax];
+            }
+            v = v / len;
+        }
+        ctx.append_output(NdArray::filled(ctx.input(0).shape(), v));
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        for (size_t i = 0; i < ctx.num_inputs(); ++i) ctx.append_input_grad(std::nullopt);
+    }
+};
+
+// The broadcast of `gy` over the extents of `x` as a FilledLike node when gy is a constant (a Scalar or a
+// FilledLike node); `mean_axes` != null: followed by the division by those extents of x.
+std::optional<Tensor> constant_broadcast(Graph *g, Tensor gy, Tensor x, const std::vector<int> *mean_axes)
+{
+    const TensorInternal &n = g->node(gy.id);
+    float value;
+    std::vector<std::vector<int>> divisions;
+    std::vector<Tensor> refs;
+    if (const auto *s = dynamic_cast<const ScalarOp *>(n.op.get())) {
+        value = s->value;
+    } else if (const auto *f = dynamic_cast<const FilledLike *>(n.op.get())) {
+        value = f->value;
+        divisions = f->mean_axes;
+        for (size_t i = 1; i < n.incoming_nodes.size(); ++i) refs.push_back(g->tensor(n.incoming_nodes[i].id));
+    } else {
+        return std::nullopt;
+    }
+    if (mean_axes) {
+        divisions.push_back(*mean_axes);
+        refs.push_back(x);
+    }
+    TensorBuilder b = g->builder();
+    b.append_input(x, false);
+    for (const Tensor &r : refs) b.append_input(r, false);
+    return b.build(std::make_unique<FilledLike>(value, std::move(divisions)));
+}
+
 // ------------------------------------------------------------------------------------------
 // convolution                                   conv_ops/conv2d.rs, conv_ops/conv2d_transpose.rs
 // ------------------------------------------------------------------------------------------
@@ -679,6 +741,10 @@ struct ReduceSum : Op {
     }
     void grad(GradientContext &ctx) const override
     {
+        if (const auto c = constant_broadcast(ctx.graph(), ctx.output_grad(), ctx.input(0), mean ? &axes : nullptr)) {
+            ctx.append_input_grad(*c);
+            return;
+        }
         const Tensor gx = build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceGradCommon>(axes, mean, !keep_dims));
         ctx.append_input_grad(gx);
     }
@@ -724,6 +790,10 @@ struct ReduceSumToScalarGrad : Op {  // :139-159; input 1 is x (for its extents)
 
 void ReduceSumToScalar::grad(GradientContext &ctx) const
 {
+    if (const auto c = constant_broadcast(ctx.graph(), ctx.output_grad(), ctx.input(0), nullptr)) {
+        ctx.append_input_grad(*c);
+        return;
+    }
     ctx.append_input_grad(build(ctx.graph(), {ctx.output_grad(), ctx.input(0)}, std::make_unique<ReduceSumToScalarGrad>()));
 }
 
@@ -950,6 +1020,13 @@ struct AddN : Op {  // array_ops.rs:503-535
         for (size_t i = 0; i < n; ++i) xs.push_back(ctx.input(i));
         if (n == 1) {
             ctx.append_output_view(xs[0]);
+            return OpError::none();
+        }
+        // the empty outputs of in-place updates (one zero scalar shared by all of them) add up to that zero
+        bool all_empty = true;
+        for (const NdArray &x : xs) all_empty = all_empty && x.allocation() == NdArray::shared_zero().allocation();
+        if (all_empty) {
+            ctx.append_empty_output();
             return OpError::none();
         }
         for (size_t i = 1; i < n; ++i)

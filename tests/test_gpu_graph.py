@@ -508,6 +508,37 @@ def test_relu_of_a_sum_is_one_node_with_the_values_and_gradients_of_two(G, orc, 
     assert gfb.shape == (1, 5, 1, 1) and np.array_equal(gfb.view(np.uint32), gpb.view(np.uint32))
 
 
+def test_constant_gradients_through_reductions_are_one_fill_with_the_bits_of_the_chain(G, rng):
+    """The seed of a back-propagation is a constant, and so is what the reductions at the end of a loss broadcast it
+    to: those nodes are built as one FilledLike node (a single fill at evaluation) whose value goes through the
+    divisions of the mean reductions in their order.  Against the unfolded chain, which a seed fed at run time
+    forces (same bits), and against the arithmetic done by hand."""
+    B, D = 3, 7
+    xv = rng.standard_normal((B, D)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x = c.placeholder("x", [B, D])
+    seed = c.placeholder("seed", [1])
+    loss = c.reduce_mean(c.reduce_mean(x, [1], True), [0], False)        # [1]
+    (g_folded,) = c.grad([loss], [x])
+    (g_chain,) = c.grad_with_default([loss], [x], [seed])
+    assert g_folded.op_name == "FilledLike" and g_chain.op_name == "ReduceGradCommon"
+    sq = c.reduce_mean(c.mul(x, x), [0, 1], True)                         # data-dependent below the reduction
+    (h_folded,) = c.grad([sq], [x])
+    (h_chain,) = c.grad_with_default([sq], [x], [c.placeholder("seed0", [1, 1])])
+    say("constant gradients folded into one fill")
+    a, b, hf, hc, total = c.eval([g_folded, g_chain, h_folded, h_chain, c.sum_all(x)],
+                                 {"x": xv, "seed": np.ones(1, np.float32), "seed0": np.ones((1, 1), np.float32)})
+    want = np.float32(np.float32(np.float32(1) / np.float32(B)) / np.float32(D))
+    assert a.shape == (B, D) and np.array_equal(a, np.full((B, D), want, np.float32))
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(hf.view(np.uint32), hc.view(np.uint32))
+    assert_close(hf, 2 * xv.astype(np.float64) / (B * D), "gradient of mean(x*x)", scale=1.0)
+    # the gradient of a plain sum: ones, with no reduction evaluated at all
+    (ones,) = c.grad([c.sum_all(x)], [x])
+    assert ones.op_name == "FilledLike" and np.array_equal(ones.eval({"x": xv}), np.ones((B, D), np.float32))
+
+
 def test_updates_that_do_not_wait_for_the_device_equal_waiting_ones(G, rng):
     """Optimizer::update returns once its work is enqueued.  Forty steps in a row, each fed from one host buffer
     that is overwritten as soon as update() returns, must leave the variables with exactly the bits of the same
