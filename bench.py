@@ -423,6 +423,15 @@ def micro_pool(torch, Kn, capi, dev, g, iters=10, only=False):
         ms = time_events(torch, bwd, iters)
         res["maxpool_bwd" + suffix] = {"ms": round(ms, 4), "GB/s": round(by / ms / 1e6, 1), "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
                                        **(traffic_fields("maxpool_bwd", ms) if step else {}), "note": place}
+        if not only and step:
+            # the same backward with the gradient of the ReLU in front of the pooling applied as it stores: one more
+            # operand (the ReLU's input) is read
+            bwd_relu = lambda: cp(Lp.ag_maxpool2d_bwd_relu_f32(sp(), pp(gy), pp(am), pp(il), pp(x), pp(gx), 256, 128, 56, 56, 3, 0, 2))
+            ms = time_events(torch, bwd_relu, iters)
+            byr = by + 4.0 * x.numel()
+            res["maxpool_bwd_relu_grad"] = {"ms": round(ms, 4), "GB/s": round(byr / ms / 1e6, 1), "frac_hbm": round(byr / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                            "note": "MaxPool2DGrad and ReLUGrad in one pass (two passes: the backward above plus a "
+                                                    "read-read-write pass over [256,128,56,56]); " + place}
         del yb, ab, gb, tb, y, am, gy, il
     return res
 

@@ -245,6 +245,15 @@ ag_status_t ag_maxpool2d_bwd_f32(ag_stream_t stream, const float *gy, const floa
                                  const uint8_t *taps, float *gx, int B, int C, int H, int W,
                                  int size, int pad, int stride);
 
+/* MaxPool2DGrad::compute followed by the gradient of the ReLU in front of the pooling
+ * (activation_ops.rs:161-166: greater(x, 0) * gy), in one pass over gx:
+ * gx = greater(relu_x, 0) * max_pool2d_grad(gy), with the bits of the two operators run one after the
+ * other.  relu_x [B,C,H,W] is the ReLU's input, or its output (same sign pattern).  The other
+ * arguments are those of ag_maxpool2d_bwd_f32. */
+ag_status_t ag_maxpool2d_bwd_relu_f32(ag_stream_t stream, const float *gy, const float *argmax,
+                                      const uint8_t *taps, const float *relu_x, float *gx, int B,
+                                      int C, int H, int W, int size, int pad, int stride);
+
 /* Replaces MaxPool2DGradGrad::compute -> max_pool_grad_grad_f32 (max_pool2d.rs:297-331, 137-159):
  * ggy[i] = ggx[argmax[i]].  Same taps / argmax rule as the backward. */
 ag_status_t ag_maxpool2d_gradgrad_f32(ag_stream_t stream, const float *ggx, const float *argmax,

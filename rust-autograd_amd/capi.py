@@ -73,6 +73,7 @@ PROTOTYPES = {
     "ag_conv2d_transpose_filter_grad_f32": (c_i, [c_p] * 5 + [c_i] * 12 + [c_p, c_sz]),
     "ag_maxpool2d_fwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
     "ag_maxpool2d_bwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
+    "ag_maxpool2d_bwd_relu_f32": (c_i, [c_p] * 6 + [c_i] * 7),
     "ag_maxpool2d_gradgrad_f32": (c_i, [c_p] * 5 + [c_i] * 7),
     "ag_sum_all_f32_workspace": (c_sz, [c_sz]),
     "ag_sum_all_f32": (c_i, [c_p, c_p, c_sz, c_p, c_p, c_sz]),

@@ -510,13 +510,18 @@ struct MaxPool2DGrad : Op, PoolHyper {  // max_pool2d.rs:245-295
     // is reconstructed like the reference (max_pool2d.rs:263-264); MaxPool2D::grad passes x so
     // that the gradient has x's size (the reference's reconstruction is too small whenever
     // (H - size) is not a multiple of the stride, and it then writes out of bounds).
-    explicit MaxPool2DGrad(PoolHyper h) : PoolHyper(h) {}
-    const char *name() const override { return "MaxPool2DGrad"; }
+    // relu_masked: one more input at the end, the input (or output) x of a ReLU; the result is multiplied by
+    // greater(x, 0) as it is stored -- this node then stands for ReLUGrad(x, MaxPool2DGrad(...)), the pair that
+    // every conv -> relu -> pool block back-propagates through (relu_grad_node builds it).
+    bool relu_masked;
+    explicit MaxPool2DGrad(PoolHyper h, bool masked = false) : PoolHyper(h), relu_masked(masked) {}
+    const char *name() const override { return relu_masked ? "MaxPool2DGradReLU" : "MaxPool2DGrad"; }
     OpError compute(ComputeContext &ctx) const override
     {
         const NdArray gy = ctx.input(0), argmax = ctx.input(1), idx = ctx.input(2);
         int in_h = -1, in_w = -1;
-        if (ctx.num_inputs() > 3) {
+        const size_t plain_inputs = ctx.num_inputs() - (relu_masked ? 1 : 0);
+        if (plain_inputs > 3) {
             const NdArray like = ctx.input(3);
             if (like.ndim() == 4) {
                 in_h = (int)like.shape()[2];
@@ -527,22 +532,21 @@ struct MaxPool2DGrad : Op, PoolHyper {  // max_pool2d.rs:245-295
         const int xh = in_h >= 0 ? in_h : ag_pool_grad_in_size(yh, size, pad, stride);
         const int xw = in_w >= 0 ? in_w : ag_pool_grad_in_size(yw, size, pad, stride);
         NdArray gx = NdArray::empty({B, C, xh, xw});
-        const OpError e = from_status(ag_maxpool2d_bwd_f32(ctx.stream(), gy.ptr(), argmax.ptr(),
-                                                           reinterpret_cast<const uint8_t *>(idx.ptr()), gx.ptr(), B, C, xh, xw,
-                                                           size, pad, stride));
+        OpError e;
+        if (relu_masked) {
+            const NdArray mask = ctx.input(ctx.num_inputs() - 1);
+            if (mask.shape() != gx.shape()) return OpError::make(ErrorKind::IncompatibleShape, "relu grad: shapes differ");
+            e = from_status(ag_maxpool2d_bwd_relu_f32(ctx.stream(), gy.ptr(), argmax.ptr(), reinterpret_cast<const uint8_t *>(idx.ptr()),
+                                                      mask.ptr(), gx.ptr(), B, C, xh, xw, size, pad, stride));
+        } else {
+            e = from_status(ag_maxpool2d_bwd_f32(ctx.stream(), gy.ptr(), argmax.ptr(), reinterpret_cast<const uint8_t *>(idx.ptr()),
+                                                 gx.ptr(), B, C, xh, xw, size, pad, stride));
+        }
         if (!e.ok()) return e;
         ctx.append_output(gx);
         return OpError::none();
     }
-    void grad(GradientContext &ctx) const override
-    {
-        const Tensor ggx = ctx.output_grad(), argmax = ctx.input(1), idx = ctx.input(2);
-        const Tensor ggy = build(ctx.graph(), {ggx, argmax, idx}, std::make_unique<MaxPool2DGradGrad>(PoolHyper{pad, stride, size}));
-        ctx.append_input_grad(ggy);
-        ctx.append_input_grad(std::nullopt);
-        ctx.append_input_grad(std::nullopt);
-        if (ctx.num_inputs() > 3) ctx.append_input_grad(std::nullopt);
-    }
+    void grad(GradientContext &ctx) const override;
 };
 
 struct MaxPool2D : Op, PoolHyper {  // max_pool2d.rs:166-243
@@ -820,6 +824,33 @@ struct ReLUGrad : Op {  // greater(x, 0) * gy as one kernel (activation_ops.rs:1
     }
 };
 
+// ReLUGrad(x, gy) as a node; when gy is the gradient of a max pooling, as one node with it (the MaxPool2DGrad node
+// that gy names is then evaluated only if something else asks for it).
+Tensor relu_grad_node(Graph *g, Tensor x, Tensor gy)
+{
+    const TensorInternal &n = g->node(gy.id);
+    const auto *pool = dynamic_cast<const MaxPool2DGrad *>(n.op.get());
+    if (pool && !pool->relu_masked && n.incoming_nodes.size() >= 3) {
+        TensorBuilder b = g->builder();
+        for (const IncomingTensor &in : n.incoming_nodes) b.append_input_with_selector(g->tensor(in.id), false, in.array_selector);
+        b.append_input(x, false);
+        return b.build(std::make_unique<MaxPool2DGrad>(PoolHyper{pool->pad, pool->stride, pool->size}, true));
+    }
+    return build(g, {x, gy}, std::make_unique<ReLUGrad>());
+}
+
+void MaxPool2DGrad::grad(GradientContext &ctx) const
+{
+    // second order: gx is linear in gy; the mask of the fused form multiplies the incoming gradient first
+    Tensor ggx = ctx.output_grad();
+    const size_t n = ctx.num_inputs();
+    if (relu_masked) ggx = build(ctx.graph(), {ctx.input(n - 1), ggx}, std::make_unique<ReLUGrad>());
+    const Tensor argmax = ctx.input(1), idx = ctx.input(2);
+    const Tensor ggy = build(ctx.graph(), {ggx, argmax, idx}, std::make_unique<MaxPool2DGradGrad>(PoolHyper{pad, stride, size}));
+    ctx.append_input_grad(ggy);
+    for (size_t i = 1; i < n; ++i) ctx.append_input_grad(std::nullopt);
+}
+
 struct ReLU : Op {  // activation_ops.rs:154-167
     const char *name() const override { return "ReLU"; }
     OpError compute(ComputeContext &ctx) const override
@@ -833,7 +864,7 @@ struct ReLU : Op {  // activation_ops.rs:154-167
     }
     void grad(GradientContext &ctx) const override
     {
-        ctx.append_input_grad(build(ctx.graph(), {ctx.input(0), ctx.output_grad()}, std::make_unique<ReLUGrad>()));
+        ctx.append_input_grad(relu_grad_node(ctx.graph(), ctx.input(0), ctx.output_grad()));
     }
 };
 
@@ -983,7 +1014,7 @@ struct AddReLU : Op {
     }
     void grad(GradientContext &ctx) const override
     {
-        const Tensor g = build(ctx.graph(), {ctx.output(), ctx.output_grad()}, std::make_unique<ReLUGrad>());
+        const Tensor g = relu_grad_node(ctx.graph(), ctx.output(), ctx.output_grad());
         ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(0)}, std::make_unique<MaybeReduceSum>()));
         ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(1)}, std::make_unique<MaybeReduceSum>()));
     }

@@ -288,6 +288,17 @@ def max_pool2d_grad(gy, argmax, taps, x_shape, pool_size, pad, stride):
     return gx
 
 
+def max_pool2d_grad_relu(gy, argmax, taps, relu_x, pool_size, pad, stride):
+    """MaxPool2DGrad and the gradient of the ReLU in front of the pooling in one pass:
+    greater(relu_x, 0) * max_pool2d_grad(gy)."""
+    gy, relu_x = _f32(gy, "max_pool2d_grad"), _f32(relu_x, "max_pool2d_grad")
+    B, Cc, H, W = relu_x.shape
+    gx = _empty(tuple(relu_x.shape), gy)
+    check(capi.lib().ag_maxpool2d_bwd_relu_f32(_stream(), _ptr(gy), _ptr(argmax), _ptr(taps), _ptr(relu_x), _ptr(gx),
+                                               B, Cc, H, W, pool_size, pad, stride))
+    return gx
+
+
 def max_pool2d_grad_grad(ggx, argmax, taps, pool_size, pad, stride):
     ggx = _f32(ggx, "max_pool2d_grad_grad")
     B, Cc, H, W = ggx.shape

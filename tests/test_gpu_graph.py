@@ -508,6 +508,36 @@ def test_relu_of_a_sum_is_one_node_with_the_values_and_gradients_of_two(G, orc, 
     assert gfb.shape == (1, 5, 1, 1) and np.array_equal(gfb.view(np.uint32), gpb.view(np.uint32))
 
 
+@pytest.mark.parametrize("H,size,stride", [(14, 2, 2), (28, 2, 2), (13, 3, 2), (9, 2, 1)])
+def test_relu_gradient_behind_a_pooling_is_one_node_with_the_pooling_gradient(G, rng, H, size, stride):
+    """max_pool2d(relu(x)): the gradient that reaches x is built as one node (the pooling's backward with the ReLU's
+    mask applied as it stores) instead of MaxPool2DGrad followed by ReLUGrad.  Values and second-order gradients
+    must have the bits of the two-node form, which a reshape between the ReLU and the pooling forces."""
+    B, C = 3, 5
+    xv = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    x = c.placeholder("x", [B, C, H, H])
+    OH = (H - size) // stride + 1
+    wts = c.placeholder("wts", [B, C, OH, OH])
+    fused_y = c.max_pool2d(c.relu(x), size, 0, stride)
+    plain_y = c.max_pool2d(c.reshape(c.relu(x), [B, C, H, H]), size, 0, stride)
+    (gf,) = c.grad([c.sum_all(c.mul(fused_y, wts))], [x])
+    (gp,) = c.grad([c.sum_all(c.mul(plain_y, wts))], [x])
+    assert gf.op_name == "MaxPool2DGradReLU" and gp.op_name == "ReLUGrad"
+    # second order: the gradient of <gx, v> with respect to the weights of the first-order loss
+    v = c.placeholder("v", [B, C, H, H])
+    (hf,) = c.grad([c.sum_all(c.mul(gf, v))], [wts])
+    (hp,) = c.grad([c.sum_all(c.mul(gp, v))], [wts])
+    wv = rng.standard_normal((B, C, OH, OH)).astype(np.float32)
+    vv = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    say(f"relu gradient fused into the pooling backward H={H} size={size} stride={stride}")
+    a, b, ha, hb = c.eval([gf, gp, hf, hp], {"x": xv, "wts": wv, "v": vv})
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(ha.view(np.uint32), hb.view(np.uint32))
+    assert np.count_nonzero(a) > 0 and np.all(a[xv <= 0] == 0)
+
+
 def test_constant_gradients_through_reductions_are_one_fill_with_the_bits_of_the_chain(G, rng):
     """The seed of a back-propagation is a constant, and so is what the reductions at the end of a loss broadcast it
     to: those nodes are built as one FilledLike node (a single fill at evaluation) whose value goes through the

@@ -1057,6 +1057,20 @@ def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
     gx_i = host(K.max_pool2d_grad(dev(gy), am, il, x.shape, size, 0, stride))
     assert np.array_equal(gx_f.view(np.uint32), ogx.view(np.uint32))
     assert np.array_equal(gx_i.view(np.uint32), ogx.view(np.uint32))
+    # the backward with the gradient of a ReLU in front of the pooling folded into its stores: the bits of
+    # greater(r, 0) * gx (activation_ops.rs:161-166), including 0 * NaN = NaN where a masked pixel receives a NaN
+    say("max_pool bwd + relu grad", case)
+    r = rng.standard_normal(x.shape).astype(np.float32)
+    r.reshape(-1)[::7] = 0.0                                    # zeros are not positive
+    gyn = gy.copy()
+    gyn.reshape(-1)[0] = np.nan
+    for g_in, idx in ((gy, None), (gy, il), (gyn, il)):
+        plain = host(K.max_pool2d_grad(dev(g_in), am, idx, x.shape, size, 0, stride))
+        with np.errstate(invalid="ignore"):
+            want = (r > 0).astype(np.float32) * plain
+        fused = host(K.max_pool2d_grad_relu(dev(g_in), am, idx, dev(r), size, 0, stride))
+        assert np.array_equal(fused.view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(fused.view(np.uint32), host(K.relu_grad(dev(r), dev(plain))).view(np.uint32))
     ggx = rng.standard_normal(x.shape).astype(np.float32)
     say("max_pool gradgrad", case)
     for idx in (None, il):
