@@ -47,7 +47,7 @@ CALIBRATION_KERNEL = "ag::ew_vec_kernel<ag::ScaleF<false> >"
 CALIBRATION_KIB = float(1 << 20)
 _STEP, _POOL, _COLS = ("profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt", "profiles/maxpool_c4_hbm_traffic.txt",
                        "profiles/conv2d_columns_c4_hbm_traffic.txt")
-_DL = "ag::gemm_dl_kernel<%s>"
+_DL = "ag::gemm_dl_kernel<%s, false>"   # the last argument: no dilation
 PROFILE_TRAFFIC = {
     # the step (column-free)
     "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false", "avg")]),
@@ -57,7 +57,7 @@ PROFILE_TRAFFIC = {
     "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max")]),
     # per-kernel section: pooling, and the column-materialising operators
     "maxpool_fwd": (_POOL, [("ag::maxpool_fwd_lds_kernel<3, 2>", "avg")]),
-    "maxpool_bwd": (_POOL, [("ag::maxpool_bwd_s2_kernel<true, 3, 16>", "avg")]),
+    "maxpool_bwd": (_POOL, [("ag::maxpool_bwd_s2_kernel<true, 3, 16, false>", "avg")]),
     "im2col": (_COLS, [("ag::im2col_same_kernel<3, 3, 1, 16>", "avg")]),
     "col2im": (_COLS, [("ag::col2im_same_kernel<3, 3, 1, 16>", "avg")]),
     "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false", "avg")]),

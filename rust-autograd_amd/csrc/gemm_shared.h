@@ -35,9 +35,6 @@ struct GemmParams {
     // elements; column n of a batch is pixel (n / conv_wp, n % conv_wp), stored to the dense
     // [.., H, conv_w] output only when n % conv_wp < conv_w.  0 = ordinary GEMM.
     int conv_wp, conv_w, conv_kw;
-    // Dilation of the stride-1 forms (input gradient and filter gradient): every tap shift above and
-    // below is multiplied by it.  1 for the stride-2 forms.
-    int conv_dil;
     // Stride-2 input gradient, both column parities of row parity conv_pair_a in one product
     // (conv_pair_w != 0): row m of the result is (channel m / 2, column parity m % 2), column (i, j)
     // is pixel (2i + conv_pair_a, 2j + m % 2) of an output plane conv_pair_w wide, so the two parities
@@ -56,6 +53,9 @@ struct GemmParams {
     unsigned rows_plane;
     unsigned rows_phase;  // != 0: stride-2 filter gradient, row (channel, ky, kx) starts at
                           // channel*rows_plane + ((ky&1)*2 + (kx&1))*rows_phase + (ky>>1)*rows_wp + (kx>>1)
+    // Dilation of the stride-1 forms (input gradient and filter gradient): every tap shift above is multiplied by
+    // it.  1 for the stride-2 forms.
+    int conv_dil;
 };
 
 // Elements of the contraction that one accumulation chain of the MFMA kernels covers before its sum
