@@ -47,12 +47,12 @@ CALIBRATION_KERNEL = "ag::ew_vec_kernel<ag::ScaleF<false> >"
 CALIBRATION_KIB = float(1 << 20)
 _STEP, _POOL, _COLS = ("profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt", "profiles/maxpool_c4_hbm_traffic.txt",
                        "profiles/conv2d_columns_c4_hbm_traffic.txt")
-_DL = "ag::gemm_dl_kernel<%s, false>"   # the last argument: no dilation
+_DL = "ag::gemm_dl_kernel<%s>"   # the last template argument: 1 = implicit convolution over filter taps, 3 = ordinary product
 PROFILE_TRAFFIC = {
     # the step (column-free)
-    "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false", "avg")]),
-    "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
-    "gemm_input_grad": (_STEP, [(_DL % "64, 128, 32, 32, 64, 3, true, false", "avg")]),
+    "gemm_fwd": (_STEP, [(_DL % "128, 256, 32, 64, 64, 3, true, false, 1", "avg"), (_DL % "128, 128, 32, 64, 64, 3, true, false, 1", "avg")]),
+    "gemm_filter_grad": (_STEP, [(_DL % "128, 192, 32, 32, 96, 3, true, true, 3", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
+    "gemm_input_grad": (_STEP, [(_DL % "64, 128, 32, 32, 64, 3, true, false, 1", "avg")]),
     "fwd_prepare": (_STEP, [("ag::pad_border_fast_kernel", "min")]),
     "input_grad_prepare": (_STEP, [("ag::pad_border_fast_kernel", "max")]),
     # per-kernel section: pooling, and the column-materialising operators
@@ -60,9 +60,9 @@ PROFILE_TRAFFIC = {
     "maxpool_bwd": (_POOL, [("ag::maxpool_bwd_s2_kernel<true, 3, 16, false>", "avg")]),
     "im2col": (_COLS, [("ag::im2col_same_kernel<3, 3, 1, 16>", "avg")]),
     "col2im": (_COLS, [("ag::col2im_same_kernel<3, 3, 1, 16>", "avg")]),
-    "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false", "avg")]),
-    "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
-    "gemm_input_grad_columns": (_COLS, [(_DL % "192, 128, 32, 96, 32, 3, false, false", "avg")]),
+    "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false, 3", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false, 3", "avg")]),
+    "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true, 3", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
+    "gemm_input_grad_columns": (_COLS, [(_DL % "192, 128, 32, 96, 32, 3, false, false, 3", "avg")]),
 }
 _profile_cache = {}
 _profile_strict = True   # False under --only: the passes that produce the summaries cannot depend on them

@@ -1,5 +1,4 @@
 // fp32 GEMM on the matrix cores with operand tiles loaded from global memory straight into LDS.
-#include <type_traits>
 
 #include "gemm_shared.h"
 
@@ -155,13 +154,20 @@ struct DirectTile {
     }
 };
 
-// DIL: the taps of the implicit convolution forms are p.conv_dil apart.  A template parameter because the kernels
-// without dilation lose 1.5 % when the tap steps of their k loop are variables instead of the constant 1 (0.930
-// against 0.916 ms for the forward product of the headline step).
-template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, bool DIL = false>
+// CONV: how the k loop walks its operands, a template parameter because the scalar work between two k tiles sits on
+// the critical path of the loads.  With the dilation as a kernel argument (a variable tap step instead of the
+// constant 1) the undilated forward product of the headline step took 0.930 instead of 0.916 ms; with the tests
+// "is this a convolution / a phase walk" decided at compile time it takes 0.905 ms, the input gradient 0.937
+// instead of 0.964, the filter gradient 0.868 instead of 0.906 and the 4096^3 NT / TN products 0.965 / 0.971
+// instead of 0.994 / 0.996 ms.
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV = 0>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
 {
-    const int conv_dil = DIL ? p.conv_dil : 1;
+    // CONV 1 / 2: the tap walk of the implicit convolution (conv_wp != 0, no phase planes) known at compile time,
+    // without / with dilation; 3: an ordinary product, known at compile time; 0: told apart at run time (what is
+    // left: the stride-2 forward over phase planes)
+    const int conv_dil = CONV == 2 ? p.conv_dil : 1;
+    const bool taps = CONV == 3 ? false : CONV != 0 || p.conv_wp != 0;
     static_assert(STAGES >= 3 && STAGES <= 8, "ring of three to eight tiles");
     static_assert(BK == 16 || BK == 32, "k tile");
     constexpr int KK = BK / 8;  // groups of four MFMA k steps per tile
@@ -260,7 +266,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     const float *pb_group = nullptr;           // stride-2 forward: B origin of the current group of 32 channels
     int fkt = 0, f_left = 0, f_kx = 0, f_ky = 0;
     const int conv_first_shift =
-        p.conv_wp != 0 && p.conv_phase == 0 ? ((p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1)) * conv_dil : 0;
+        CONV == 3 ? 0 : CONV != 0 || (p.conv_wp != 0 && p.conv_phase == 0) ? ((p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1)) * conv_dil : 0;
     Cursor fcur = first;
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
@@ -269,13 +275,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
             ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
         } else if (KB && p.rows_taps != 0) {
-            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, conv_dil, wave, lane);
+            ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, p.conv_dil, wave, lane);
         } else {
             ldr_b.init(ldb, it.n0, p.N, wave, lane);
         }
         pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
         pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
-        if (p.conv_wp != 0) {  // first tap (0, 0): the largest shift (input gradient), or phase (0, 0) unshifted
+        if (taps) {  // first tap (0, 0): the largest shift (input gradient), or phase (0, 0) unshifted
             pb_group = pb;
             pb += conv_first_shift;
             f_kx = f_ky = 0;
@@ -291,7 +297,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 cursor_next(fcur);
                 f_begin();
             }
-        } else if (p.conv_phase != 0) {
+        } else if (CONV == 0 && p.conv_phase != 0) {
             // Stride-2 forward: all taps of one group of 32 channels in natural order, then the next group.
             if (++fkt == p.kbatch) {
                 fkt = 0;
@@ -307,7 +313,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 }
                 pb = pb_group + (long long)((f_ky & 1) * 2 + (f_kx & 1)) * p.conv_phase + (f_ky >> 1) * p.conv_wp + (f_kx >> 1);
             }
-        } else if (p.conv_wp != 0) {
+        } else if (taps) {
             // Implicit input gradient: for one group of 32 filters all taps are visited in turn
             // (they read nearly the same rows of B, which stay in the cache), then the next group.
             if (++fkt == p.kbatch) {  // fkt counts taps here
@@ -657,9 +663,12 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
     constexpr int NT = (BM / WM) * (BN / WN) * 64;
 #define AG_GEMM_DL_CASE(KA_, KB_)                                                                     \
     if constexpr ((KA_ || BM % 64 == 0) && (KB_ || BN % 64 == 0)) if (ka == KA_ && kb == KB_) {      \
-        auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_>;                                 \
-        if constexpr (KA_) /* the convolution forms have a k-contiguous A */                          \
-            if (p.conv_dil != 1) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, true>;      \
+        auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 3>;                              \
+        if constexpr (KA_ && !KB_) /* the implicit convolution over filter taps */                    \
+            if (p.conv_phase != 0) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 0>;       \
+            else if (p.conv_wp != 0)                                                                  \
+                kern = p.conv_dil != 1 ? gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 2>         \
+                                       : gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 1>;        \
         long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \
         if (g >= p.total_blocks) g = p.total_blocks;        /* one item per block */                 \
         else g = g >= kXcds ? g - g % kXcds : kXcds;         /* the kernel steps items by grid / 8 */ \
