@@ -523,7 +523,7 @@ def micro_rest(torch, Kn, capi, dev, g, iters=10):
     A = torch.randn(4096, 4096, device=dev, generator=g)
     Bm = torch.randn(4096, 4096, device=dev, generator=g)
     for name, ta, tb in (("matmul_4096_NN", False, False), ("matmul_4096_NT", False, True), ("matmul_4096_TN", True, False)):
-        ms = time_events(torch, lambda: Kn.matmul(A, Bm, ta, tb), 10)
+        ms = time_events(torch, lambda: Kn.matmul(A, Bm, ta, tb), 10, warm=10)
         tf = 2.0 * 4096 ** 3 / ms / 1e9
         res[name] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
     del A, Bm
