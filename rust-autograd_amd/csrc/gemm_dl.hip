@@ -289,7 +289,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         fkt = 0;
         f_left = it.nt;
     };
+    // Past the end of the block's stream the origins stay where they are: the loads that the k loop keeps issuing
+    // read the last tile again (into ring slots that nothing reads any more), so that the loop has no "is there a
+    // tile left" test in front of every load and one steady wait count.
     auto fetch_advance = [&]() {
+        if (!f_valid) return;
         if (--f_left == 0) {
             fw += gridDim.x;
             f_valid = fw < total;
@@ -549,7 +553,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 
     Frag af[2][MI], bf[2][NI];
     unsigned fill_addr = lds_wave;  // LDS byte address (this wave's share) of the slot being filled
-    auto second_half = [&](const bool fetching, const float *cur, const float *nxt, bool last) {
+    auto second_half = [&](const float *cur, const float *nxt, bool last) {
         constexpr int NM = (KK - KK / 2) * 4 * MI * NI;  // MFMAs in this half
 #ifdef AG_DL_SPACING
         constexpr int SPACING = AG_DL_SPACING;
@@ -572,7 +576,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                                                                          acc[i][j], 0, 0, 0);
                         const int m = (((kk - KK / 2) * 4 + s4) * MI + i) * NI + j;
                         const int load = m / SPACING;
-                        if (m % SPACING == SPACING - 1 && load < L && fetching) {
+                        if (m % SPACING == SPACING - 1 && load < L) {
                             __builtin_amdgcn_sched_barrier(0);
                             if (load < LoadA::PER_WAVE) ldr_a.issue_one(load, pa, fill_addr);
                             else ldr_b.issue_one(load - LoadA::PER_WAVE, pb, fill_addr + BM * BK * 4u);
@@ -586,19 +590,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 
     // Prologue: tiles 0 .. STAGES-2 of the stream.
     f_begin();
-    bool all_issued = true;  // did the last attempt to issue a tile find one?
 #pragma unroll
     for (int st = 0; st < STAGES - 1; ++st) {
-        all_issued = f_valid;
-        if (f_valid) {
-            ldr_a.template issue<0, 8>(pa, fill_addr);
-            ldr_b.template issue<0, 8>(pb, fill_addr + BM * BK * 4u);
-            fetch_advance();
-        }
+        ldr_a.template issue<0, 8>(pa, fill_addr);
+        ldr_b.template issue<0, 8>(pb, fill_addr + BM * BK * 4u);
+        fetch_advance();
         fill_addr += TILE * 4u;
     }
-    if (all_issued) wait_loads_then_barrier<(STAGES - 2) * L>();
-    else wait_loads_then_barrier<0>();
+    wait_loads_then_barrier<(STAGES - 2) * L>();
 
     unsigned cw = blockIdx.x;
     Cursor ccur = first;
@@ -628,16 +627,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             // The next tile must have landed; tiles further ahead may still be in flight.
-            if (!all_issued) wait_loads_then_barrier<0>();
-            else if (after_epilogue) wait_loads_then_barrier<AFTER_EPILOGUE>();
+            if (after_epilogue) wait_loads_then_barrier<AFTER_EPILOGUE>();
             else wait_loads_then_barrier<STEADY>();
             after_epilogue = false;
-            all_issued = f_valid;
             // Every wave has left the previous tile's slot.  Its loads are issued one at a time
             // between the MFMAs of the rest of this tile: a clump of loads would leave the matrix
             // pipe idle while the wave issues them, and all waves of the block would queue at the
             // address unit right after the barrier.
-            second_half(all_issued, cur, nxt, last);
+            second_half(cur, nxt, last);
             fill_addr = fill_addr + TILE * 4u == lds_wave + STAGES * TILE * 4u ? lds_wave : fill_addr + TILE * 4u;
             cur = nxt;
             if (--chain_left == 0 && c_left - 1 > CHAIN / 4) {
@@ -649,7 +646,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         } while (--c_left != 0);
         if (chained) take_back();
         const bool counted = write_out(ci);
-        if (last_item) break;
+        if (last_item) {
+            // the loads issued past the end of the stream must land before the block gives up its LDS
+            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+            break;
+        }
         after_epilogue = counted;
         cw += gridDim.x;
         cursor_next(ccur);
