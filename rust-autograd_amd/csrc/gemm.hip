@@ -1021,10 +1021,30 @@ static int conv_filter_grad_splits(int B, int Kf, int C, int taps, int kq)
     return (int)cdiv(B, per);
 }
 
+// A block that sums one whole image is as fine as the splits get, and it takes a fixed time (0.28 ms for a 56 x 56
+// plane on a 128 x 192 tile) however few of them there are: below about a hundred images the chip would be part
+// empty for that long.  Small batches therefore also cut the flattened plane into equal chunks of positions, which
+// the kernel sees as a batch of independent products (origins a chunk apart), each with partial sums of its own;
+// the fold adds them all in a fixed order.  Returns the number of chunks (a divisor of the plane's k tiles).
+static int conv_filter_grad_chunks(int B, int Kf, int C, int taps, int kq)
+{
+    if (kq < 512 || kq % 32 != 0) return 1;
+    const int cfg = conv_filter_grad_cfg(Kf, (long long)C * taps);
+    const long long tiles = cdiv(Kf, kCfgs[cfg].bm) * cdiv((long long)C * taps, kCfgs[cfg].bn);
+    const long long blocks = tiles * conv_filter_grad_splits(B, Kf, C, taps, kq);
+    if (blocks >= 768) return 1;
+    long long want = cdiv(1024, blocks);
+    const int kt = kq / 32;
+    if (want > kt / 8) want = kt / 8;  // at least eight k tiles per chunk
+    for (long long c = want; c >= 2; --c)
+        if (kt % c == 0) return (int)c;
+    return 1;
+}
+
 size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq)
 {
-    const int splits = conv_filter_grad_splits(B, Kf, C, taps, kq);
-    return splits > 1 ? sizeof(float) * (size_t)splits * Kf * C * taps : 16;
+    const long long partials = (long long)conv_filter_grad_splits(B, Kf, C, taps, kq) * conv_filter_grad_chunks(B, Kf, C, taps, kq);
+    return partials > 1 ? sizeof(float) * (size_t)partials * Kf * C * taps : 16;
 }
 
 // a_plane / b_plane: elements per row of A (one filter's gradient plane) and per channel of B; phase != 0: B is
@@ -1054,20 +1074,28 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     p.conv_dil = dil;
     p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)b_plane; p.rows_phase = phase;
     p.C = gw;
-    if (p.splits > 1) {
-        const size_t need = sizeof(float) * (size_t)p.splits * p.M * p.N;
+    // (the stride-2 form keeps whole planes: its workspace is sized without knowing kq)
+    const int chunks = phase == 0 ? conv_filter_grad_chunks(B, Kf, C, taps, kq) : 1;
+    const long long partials = (long long)p.splits * chunks;
+    // chunk z of every plane is "batch" z of the product: origins kq / chunks positions apart, partial sums in the
+    // slots z * splits .. z * splits + splits - 1
+    p.K = kq / chunks;
+    p.sA = p.sB = p.K;
+    p.sC = (long long)p.splits * p.sCsplit;
+    if (partials > 1) {
+        const size_t need = sizeof(float) * (size_t)partials * p.M * p.N;
         AG_REQUIRE(ws && ws_bytes >= need, AG_ERR_INVALID_DIMS, "conv2d_filter_grad: workspace of %zu bytes needed, %zu given",
                    need, ws_bytes);
-        p.C = static_cast<float *>(ws);
     }
     const int cfg = conv_filter_grad_cfg(Kf, (long long)C * taps);
     p.tiles_m = (int)cdiv(p.M, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
-    p.total_blocks = (unsigned)((long long)p.tiles_m * p.tiles_n * p.splits);
+    p.total_blocks = (unsigned)((long long)p.tiles_m * p.tiles_n * partials);
+    if (partials > 1) p.C = static_cast<float *>(ws);
     launch_direct(st, cfg, true, true, p, num_cus(), g_grid_scale);
-    if (ag_status_t s = check_launch("conv2d_filter_grad")) return s;
-    if (p.splits > 1) {
-        launch_fold(st, static_cast<const float *>(ws), p.splits, p.sCsplit, gw, p.M, p.N, (long long)p.N, 1.f, 0.f);
+    if (ag_status_t e = check_launch("conv2d_filter_grad")) return e;
+    if (partials > 1) {
+        launch_fold(st, static_cast<const float *>(ws), (int)partials, p.sCsplit, gw, p.M, p.N, (long long)p.N, 1.f, 0.f);
         return check_launch("conv2d_filter_grad");
     }
     return AG_OK;

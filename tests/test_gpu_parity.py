@@ -716,6 +716,25 @@ def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d):
     assert np.array_equal(host(gx), host(gx_cols))
 
 
+@pytest.mark.parametrize("B,C,Kc,H,W,k,p", [(1, 32, 64, 44, 44, 3, 1), (3, 64, 128, 56, 56, 3, 1), (2, 32, 32, 60, 36, 5, 2)])
+def test_conv2d_column_free_filter_grad_of_a_small_batch_is_cut_into_position_chunks(K, rng, B, C, Kc, H, W, k, p):
+    # with few images the filter gradient also splits every plane into chunks of positions (more partial sums,
+    # one launch): integer-valued data, so the result must equal the columns path bit for bit, and the workspace
+    # the library asks for must be the one it then accepts
+    L = K.capi.lib()
+    x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
+    one_image = Kc * C * k * k * 4
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, 1) > B * one_image, "expected more partial sums than images"
+    say("column-free filter gradient in position chunks", (B, C, Kc, H, W, k, p))
+    y, xpad = K.conv2d_nocols(dev(x), dev(w), p)
+    _, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
+    _, gypad = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+    gw = K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p)
+    assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape)))
+
+
 def test_conv2d_column_free_headline_size_matches_columns_path(K):
     # the benchmark's own shape (B=256, 64 -> 128 channels, 56x56, 3x3): the three column-free results
     # against the library's column path, which the smaller cases pin to the oracle
