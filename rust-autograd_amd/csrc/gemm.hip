@@ -601,9 +601,11 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
 {
     if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) return g_force_cfg == kDirectCfg32 && !a_kcontig ? kDirectCfg64 : g_force_cfg;
     if (direct) {
-        // 128x256, 256x128, 192x128, 128x192, 128x128, and 64x128 (two blocks per CU) for outputs of up to 64 rows
-        static const int dl[] = {14, 15, 16, 17, 13, kDirectCfg64};
-        static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.92, 0.8};
+        // 128x256, 256x128, 192x128, 128x192, 128x128, and 64x128 / 64x64 (two blocks per CU); the efficiencies are
+        // what each tile reaches on 6144^3, where every one of them has whole rounds (144 TFLOP/s = 1)
+        static const int dl[] = {14, 15, 16, 17, 13, kDirectCfg64, kDirectCfg64Narrow};
+        static const double eff[] = {1.0, 1.0, 0.98, 0.98, 0.93, 0.95, 0.89};
+        constexpr int kCandidates = 7;
         // The cheapest tile among those that give the chip at least half a round of blocks: padded
         // area over efficiency, counted in whole rounds of the persistent grid while there are few
         // of them (264 blocks on 256 CUs take two rounds, 200 take one).
@@ -621,11 +623,11 @@ static int choose_cfg(int M, int N, int K, long long zcount, bool accumulate, bo
         if (!accumulate && K <= 512 && M >= 64 && cdiv(M, 128) * cdiv(N, 128) * zcount < 8 * cus2) return kDirectCfg64;
         int best = -1;
         double best_cost = 1e300;
-        for (int c = 0; c < 6; ++c) {
+        for (int c = 0; c < kCandidates; ++c) {
             const TileCfg &t = kCfgs[dl[c]];
             const long long tm = cdiv(M, t.bm), tn = cdiv(N, t.bn);
             const long long blocks = tm * tn * zcount;
-            const long long grid = direct_grid(num_cus()) * (dl[c] == kDirectCfg64 ? 2 : 1);
+            const long long grid = direct_grid(num_cus()) * (t.bm == 64 ? 2 : 1);
             if (blocks < direct_grid(num_cus()) / 2) continue;
             const bool whole_rounds = blocks < 8 * grid && !(tail_split && t.bm == 128 && tm == 1);
             const long long counted = whole_rounds ? cdiv(blocks, grid) * grid : blocks;
