@@ -735,8 +735,11 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     AG_REQUIRE(c.A && c.B, AG_ERR_INVALID_DIMS, "%s: null operand", who);
     // A long contraction that misses the direct-to-LDS kernel only because K is not a multiple of
     // its k tile: the whole tiles go there, the remaining K % 32 are accumulated on top by the
-    // register-staged kernel (2-3 % of the work).
-    if (c.K % 32 != 0 && c.K >= 256 && (c.kbatch > 1 || c.K >= 1024) && g_force_cfg < 0 && !direct_ok(c)) {
+    // register-staged kernel (2-3 % of the work).  A single product shorter than 1024 does so only while its
+    // output is small: the second pass reads and writes C once more (1000^3: 55 -> 40 us; 4096 x 4096 x 520 would
+    // go from 170 to 223 us).
+    const bool worth_two_passes = c.kbatch > 1 || c.K >= 1024 || (c.K >= 512 && (long long)c.M * c.N <= 2500000);
+    if (c.K % 32 != 0 && c.K >= 256 && worth_two_passes && g_force_cfg < 0 && !direct_ok(c)) {
         GemmCall body = c;
         body.K = c.K - c.K % 32;
         // only when the body really lands on the direct-to-LDS kernel (enough tiles for it)

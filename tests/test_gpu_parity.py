@@ -390,7 +390,8 @@ def test_matmul_with_a_handful_of_columns(K, rng, m, n, k, ta):
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_long_k_with_a_tail(K, rng, ta, tb):
     """K = 32 q + r: whole k tiles on the direct-to-LDS kernel, the remaining r accumulated on top."""
-    for (m, n, k, batch, beta) in ((256, 384, 1040, 3, 0.0), (128, 512, 2060, 2, 0.5)):
+    # (the last case: a single product shorter than 1024 with a small output, which also takes the two passes)
+    for (m, n, k, batch, beta) in ((256, 384, 1040, 3, 0.0), (128, 512, 2060, 2, 0.5), (1000, 1000, 520, 1, 0.0)):
         a = rng.standard_normal((batch, k, m) if ta else (batch, m, k)).astype(np.float32)
         b = rng.standard_normal((batch, n, k) if tb else (batch, k, n)).astype(np.float32)
         c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
