@@ -349,6 +349,14 @@ ag_status_t ag_sparse_softmax_xent_f32(ag_stream_t stream, const float *logits, 
 ag_status_t ag_sparse_softmax_xent_grad_f32(ag_stream_t stream, const float *log_softmax,
                                             const float *labels, const float *gy, float *gx,
                                             size_t rows, size_t classes);
+/* The same gradient computed from the logits (xent_ops.rs:63-115 and 139-153 in one kernel, the bits
+ * of the two functions above run one after the other), for a training step that never reads the loss
+ * and so need not run the forward.  gy [rows] may be NULL: every row's upstream gradient is then
+ * gy_const (a mean over the batch: 1 / rows). */
+ag_status_t ag_sparse_softmax_xent_grad_logits_f32(ag_stream_t stream, const float *logits,
+                                                   const float *labels, const float *gy,
+                                                   float gy_const, float *gx, size_t rows,
+                                                   size_t classes);
 
 /* ---- entry point that allocates nothing ----------------------------------------------------- */
 

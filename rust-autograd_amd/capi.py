@@ -96,6 +96,7 @@ PROTOTYPES = {
     "ag_fill_f32": (c_i, [c_p, c_p, c_f, c_sz]),
     "ag_sparse_softmax_xent_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
     "ag_sparse_softmax_xent_grad_f32": (c_i, [c_p] * 5 + [c_sz, c_sz]),
+    "ag_sparse_softmax_xent_grad_logits_f32": (c_i, [c_p] * 4 + [c_f, c_p, c_sz, c_sz]),
     "ag_conv_input_grad_scratch_floats": (C.c_size_t, [c_i] * 12),
     "ag_conv_input_grad_prepare_f32": (c_i, [c_p, c_p, c_p, c_p] + [c_i] * 12),
     "ag_conv_input_grad_gemm_f32": (c_i, [c_p, c_p, c_p] + [c_i] * 12),

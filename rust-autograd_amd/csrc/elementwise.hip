@@ -311,6 +311,33 @@ __global__ __launch_bounds__(256) void sparse_xent_grad_kernel(const float *__re
     }
 }
 
+// The gradient straight from the logits: the log-softmax of sparse_xent_kernel and the arithmetic of
+// sparse_xent_grad_kernel in one pass, one thread per row, so that a training step that never reads the loss does not
+// run the forward kernel at all.  gy == null: every row's upstream gradient is gy_const.
+__global__ __launch_bounds__(256) void sparse_xent_grad_logits_kernel(const float *__restrict__ logits,
+                                                                      const float *__restrict__ labels,
+                                                                      const float *__restrict__ gy, float gy_const,
+                                                                      float *__restrict__ gx, size_t rows, size_t classes)
+{
+    AG_EW_LOOP(r, rows)
+    {
+        const float *row = logits + r * classes;
+        float mx = -FLT_MAX;
+        for (size_t c = 0; c < classes; ++c) mx = fmaxf(mx, row[c]);
+        float s = 0.f;
+        for (size_t c = 0; c < classes; ++c) s += expf(row[c] - mx);
+        const float lse = logf(s) + mx;
+        size_t label;
+        const bool ok = label_of(labels[r], classes, &label);
+        const float g = gy ? gy[r] : gy_const;
+        for (size_t c = 0; c < classes; ++c) {
+            float e = expf(row[c] - lse);
+            if (c == label) e -= 1.f;
+            gx[r * classes + c] = ok ? e * g : __builtin_nanf("");
+        }
+    }
+}
+
 }  // namespace ag
 
 using namespace ag;
@@ -528,4 +555,20 @@ extern "C" ag_status_t ag_sparse_softmax_xent_grad_f32(ag_stream_t stream, const
                "SparseSoftmaxCrossEntropyGrad: null pointer");
     AG_EW_ENTRY("SparseSoftmaxCrossEntropyGrad", sparse_xent_grad_kernel, rows * classes, log_softmax,
                 labels, gy, gx, rows, classes);
+}
+
+// SparseSoftmaxCrossEntropy's gradient without its forward (xent_ops.rs:63-115 and 139-153 in one kernel): the bits of
+// ag_sparse_softmax_xent_f32 followed by ag_sparse_softmax_xent_grad_f32.  gy [rows] may be NULL: then every row's
+// upstream gradient is gy_const (the mean of a batch loss: 1 / rows).
+extern "C" ag_status_t ag_sparse_softmax_xent_grad_logits_f32(ag_stream_t stream, const float *logits, const float *labels,
+                                                              const float *gy, float gy_const, float *gx, size_t rows,
+                                                              size_t classes)
+{
+    AG_REQUIRE(classes >= 1 || rows == 0, AG_ERR_INCOMPATIBLE_SHAPE,
+               "SparseSoftmaxCrossEntropyGrad: logits need at least one class");
+    AG_REQUIRE(rows == 0 || (logits && labels && gx), AG_ERR_INVALID_DIMS, "SparseSoftmaxCrossEntropyGrad: null pointer");
+    if (rows == 0) return AG_OK;
+    hipLaunchKernelGGL(sparse_xent_grad_logits_kernel, dim3(ew_grid(rows, 1)), dim3(256), 0, as_stream(stream), logits, labels,
+                       gy, gy_const, gx, rows, classes);
+    return check_launch("SparseSoftmaxCrossEntropyGrad");
 }

@@ -96,11 +96,12 @@ struct FilledLike : Op {
     std::vector<std::vector<int>> mean_axes;
     FilledLike(float v, std::vector<std::vector<int>> m) : value(v), mean_axes(std::move(m)) {}
     const char *name() const override { return "FilledLike"; }
-    OpError compute(ComputeContext &ctx) const override
+    // The constant after its divisions; division j reads the extents of input `first_ref + j`.
+    OpError resolve(ComputeContext &ctx, size_t first_ref, float *out) const
     {
         float v = value;
         for (size_t j = 0; j < mean_axes.size(); ++j) {
-            const NdArray x = ctx.input(1 + j);
+            const NdArray x = ctx.input(first_ref + j);
             const int rank = x.ndim();
             float len = 1.f;
             for (int a : mean_axes[j]) {
@@ -110,6 +111,14 @@ struct FilledLike : Op {
             }
             v = v / len;
         }
+        *out = v;
+        return OpError::none();
+    }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        float v;
+        const OpError e = resolve(ctx, 1, &v);
+        if (!e.ok()) return e;
         ctx.append_output(NdArray::filled(ctx.input(0).shape(), v));
         return OpError::none();
     }
@@ -1156,6 +1165,45 @@ struct SparseSoftmaxCrossEntropyGrad : Op {  // xent_ops.rs:139-158
     }
 };
 
+// The same gradient computed from the logits, so that an evaluation that never asks for the loss does not run the
+// forward at all.  Inputs (logits, labels, gy); or, when the upstream gradient is a constant (a FilledLike node: the
+// mean of a batch loss), (logits, labels, the inputs of that node), with the constant resolved on the host and handed
+// to the kernel as an argument -- no array is filled for it.
+struct SparseSoftmaxCrossEntropyGradLogits : Op {
+    std::optional<FilledLike> constant;
+    explicit SparseSoftmaxCrossEntropyGradLogits(std::optional<FilledLike> c) : constant(std::move(c)) {}
+    const char *name() const override { return "SparseSoftmaxCrossEntropyGradLogits"; }
+    OpError compute(ComputeContext &ctx) const override
+    {
+        const NdArray x = ctx.input(0), t = ctx.input(1);
+        if (x.ndim() != 2)
+            return OpError::make(ErrorKind::IncompatibleShape,
+                                 "SparseSoftmaxCrossEntropy: given first argument's ndim is not 2: shape=" + shape_str(x.shape()));
+        if (t.len() != (size_t)x.shape()[0]) throw Panic("Batch size mismatch: inputs vs labels");
+        float value = 0.f;
+        const float *gy = nullptr;
+        NdArray gy_array;
+        if (constant) {
+            const OpError e = constant->resolve(ctx, 3, &value);  // input 2 is the constant's shape source
+            if (!e.ok()) return e;
+        } else {
+            gy_array = ctx.input(2);
+            if (gy_array.len() != (size_t)x.shape()[0]) return OpError::make(ErrorKind::IncompatibleShape, "SparseSoftmaxCrossEntropyGrad: one upstream gradient per row expected");
+            gy = gy_array.ptr();
+        }
+        NdArray gx = NdArray::empty(x.shape());
+        const OpError e = from_status(ag_sparse_softmax_xent_grad_logits_f32(ctx.stream(), x.ptr(), t.ptr(), gy, value, gx.ptr(),
+                                                                             (size_t)x.shape()[0], (size_t)x.shape()[1]));
+        if (!e.ok()) return e;
+        ctx.append_output(gx);
+        return OpError::none();
+    }
+    void grad(GradientContext &ctx) const override
+    {
+        for (size_t i = 0; i < ctx.num_inputs(); ++i) ctx.append_input_grad(std::nullopt);
+    }
+};
+
 struct SparseSoftmaxCrossEntropy : Op {  // xent_ops.rs:63-137
     const char *name() const override { return "SparseSoftmaxCrossEntropy"; }
     OpError compute(ComputeContext &ctx) const override
@@ -1179,9 +1227,33 @@ struct SparseSoftmaxCrossEntropy : Op {  // xent_ops.rs:63-137
     }
     void grad(GradientContext &ctx) const override
     {
-        const Tensor t = ctx.input(1), gy = ctx.output_grad();
-        const Tensor log_x = tensor_ops::nth_tensor(ctx.output(), 1);
-        ctx.append_input_grad(build(ctx.graph(), {log_x, t, gy}, std::make_unique<SparseSoftmaxCrossEntropyGrad>()));
+        // from the logits rather than from this node's log-softmax (same bits): the forward then runs only when
+        // something asks for the loss
+        const Tensor x = ctx.input(0), t = ctx.input(1), gy = ctx.output_grad();
+        Graph *g = ctx.graph();
+        const TensorInternal &gn = g->node(gy.id);
+        TensorBuilder b = g->builder();
+        b.append_input(x, false);
+        b.append_input(t, false);
+        std::optional<FilledLike> constant;
+        if (const auto *f = dynamic_cast<const FilledLike *>(gn.op.get())) {
+            constant.emplace(f->value, f->mean_axes);
+            // The constant usually takes its extents from this node's own loss [rows, 1] (the mean over the batch of
+            // the loss): the logits [rows, classes] stand in wherever only the row count is read, so that the
+            // gradient does not depend on the forward.
+            const TensorID self = ctx.output().id;
+            for (size_t i = 0; i < gn.incoming_nodes.size(); ++i) {
+                const IncomingTensor &in = gn.incoming_nodes[i];
+                bool rows_only = true;  // input 0 gives the fill's shape, which nothing reads here
+                if (i >= 1)
+                    for (int a : f->mean_axes[i - 1]) rows_only = rows_only && (a == 0 || a == -2);
+                if (in.id == self && in.array_selector == 0 && rows_only) b.append_input(x, false);
+                else b.append_input_with_selector(g->tensor(in.id), false, in.array_selector);
+            }
+        } else {
+            b.append_input(gy, false);
+        }
+        ctx.append_input_grad(b.build(std::make_unique<SparseSoftmaxCrossEntropyGradLogits>(std::move(constant))));
         ctx.append_input_grad(std::nullopt);  // the reference builds a label gradient "that won't be used in most cases"
     }
 };

@@ -480,3 +480,13 @@ def sparse_softmax_cross_entropy_grad(log_softmax, labels, gy):
     check(capi.lib().ag_sparse_softmax_xent_grad_f32(_stream(), _ptr(lsm), _ptr(labels), _ptr(gy), _ptr(gx),
                                                      lsm.shape[0], lsm.shape[1]))
     return gx
+
+
+def sparse_softmax_cross_entropy_grad_from_logits(logits, labels, gy):
+    """The gradient without the forward's log-softmax; `gy`: a tensor of one value per row, or a float."""
+    logits, labels = _f32(logits, "SparseSoftmaxCrossEntropyGrad"), _f32(labels, "SparseSoftmaxCrossEntropyGrad")
+    gx = torch.empty_like(logits)
+    const = isinstance(gy, (int, float))
+    check(capi.lib().ag_sparse_softmax_xent_grad_logits_f32(_stream(), _ptr(logits), _ptr(labels), None if const else _ptr(gy),
+                                                            float(gy) if const else 0.0, _ptr(gx), logits.shape[0], logits.shape[1]))
+    return gx

@@ -64,6 +64,7 @@ extern "C" {
     pub fn ag_fill_f32(stream: AgStream, out: *mut f32, value: f32, n: usize) -> AgStatus;
     pub fn ag_sparse_softmax_xent_f32(stream: AgStream, logits: *const f32, labels: *const f32, loss: *mut f32, log_softmax: *mut f32, rows: usize, classes: usize) -> AgStatus;
     pub fn ag_sparse_softmax_xent_grad_f32(stream: AgStream, log_softmax: *const f32, labels: *const f32, gy: *const f32, gx: *mut f32, rows: usize, classes: usize) -> AgStatus;
+    pub fn ag_sparse_softmax_xent_grad_logits_f32(stream: AgStream, logits: *const f32, labels: *const f32, gy: *const f32, gy_const: f32, gx: *mut f32, rows: usize, classes: usize) -> AgStatus;
     pub fn ag_matmul_f32_static_scratch_bytes() -> usize;
     pub fn ag_matmul_f32_noalloc(stream: AgStream, transA: c_int, transB: c_int, M: c_int, N: c_int, K: c_int, A: *const f32, lda: c_int, B: *const f32, ldb: c_int, C: *mut f32, ldc: c_int) -> AgStatus;
 }

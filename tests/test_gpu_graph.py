@@ -569,6 +569,31 @@ def test_constant_gradients_through_reductions_are_one_fill_with_the_bits_of_the
     assert ones.op_name == "FilledLike" and np.array_equal(ones.eval({"x": xv}), np.ones((B, D), np.float32))
 
 
+def test_cross_entropy_gradient_is_built_on_the_logits(G, orc, rng):
+    """The gradient of sparse_softmax_cross_entropy is one node over the logits (not over the forward's log-softmax
+    output), with the constant of a batch mean handed to its kernel as an argument; a data-dependent upstream gradient
+    goes in as an array.  Values against the oracle's two-step form."""
+    rows, classes = 37, 11
+    lv = (rng.standard_normal((rows, classes)) * 2).astype(np.float32)
+    tv = rng.integers(0, classes, (rows, 1)).astype(np.float32)
+    wv = rng.standard_normal((rows, 1)).astype(np.float32)
+    env = G.VariableEnvironment()
+    c = env.context()
+    logits, t, w = c.placeholder("l", [rows, classes]), c.placeholder("t", [rows, 1]), c.placeholder("w", [rows, 1])
+    loss = c.sparse_softmax_cross_entropy(logits, t)
+    (g_mean,) = c.grad([c.reduce_mean(loss, [0], False)], [logits])
+    (g_weighted,) = c.grad([c.sum_all(c.mul(loss, w))], [logits])
+    assert g_mean.op_name == "SparseSoftmaxCrossEntropyGradLogits" and g_weighted.op_name == "SparseSoftmaxCrossEntropyGradLogits"
+    assert g_mean.num_inputs == 4          # logits, labels, and the constant's two extent sources (both the logits)
+    assert g_weighted.num_inputs == 3      # logits, labels, the upstream gradient
+    say("cross-entropy gradient from the logits")
+    a, b, lossv = c.eval([g_mean, g_weighted, loss], {"l": lv, "t": tv, "w": wv})
+    _, olsm = orc.sparse_softmax_xent(lv, tv)
+    assert_close(a, orc.sparse_softmax_xent_grad(olsm, tv, np.full((rows, 1), np.float32(1) / np.float32(rows), np.float32)), "mean")
+    assert_close(b, orc.sparse_softmax_xent_grad(olsm, tv, wv), "weighted")
+    assert lossv.shape == (rows, 1)
+
+
 def test_updates_that_do_not_wait_for_the_device_equal_waiting_ones(G, rng):
     """Optimizer::update returns once its work is enqueued.  Forty steps in a row, each fed from one host buffer
     that is overwritten as soon as update() returns, must leave the variables with exactly the bits of the same

@@ -1477,6 +1477,30 @@ def test_sparse_softmax_cross_entropy_flags_bad_labels(K, orc, rng):
         assert_close(host(lsm), olsm, "log_softmax does not depend on the labels")
 
 
+def test_sparse_softmax_cross_entropy_gradient_straight_from_the_logits(K, orc, rng):
+    """One kernel from the logits (no forward): the bits of the forward's log-softmax followed by the gradient kernel,
+    with a per-row upstream gradient and with a constant one; bad labels give NaN rows as they do there."""
+    for rows, classes in ((128, 10), (1000, 10), (257, 7), (200, 64), (130, 100), (1, 1)):
+        logits = (rng.standard_normal((rows, classes)) * 3).astype(np.float32)
+        labels = rng.integers(0, classes, size=(rows, 1)).astype(np.float32)
+        gy = rng.standard_normal((rows, 1)).astype(np.float32)
+        say("xent gradient from logits", rows, classes)
+        _, lsm = K.sparse_softmax_cross_entropy(dev(logits), dev(labels))
+        two_step = host(K.sparse_softmax_cross_entropy_grad(lsm, dev(labels), dev(gy)))
+        fused = host(K.sparse_softmax_cross_entropy_grad_from_logits(dev(logits), dev(labels), dev(gy)))
+        assert np.array_equal(fused.view(np.uint32), two_step.view(np.uint32))
+        c = 1.0 / rows
+        two_step = host(K.sparse_softmax_cross_entropy_grad(lsm, dev(labels), dev(np.full((rows, 1), c, np.float32))))
+        fused = host(K.sparse_softmax_cross_entropy_grad_from_logits(dev(logits), dev(labels), c))
+        assert np.array_equal(fused.view(np.uint32), two_step.view(np.uint32))
+        _, olsm = orc.sparse_softmax_xent(logits, labels)
+        assert_close(fused, orc.sparse_softmax_xent_grad(olsm, labels, np.full((rows, 1), c, np.float32)), "gradient against the oracle")
+    logits = rng.standard_normal((6, 5)).astype(np.float32)
+    labels = np.array([0, -1, 4, 5, np.nan, 2], np.float32)
+    gx = host(K.sparse_softmax_cross_entropy_grad_from_logits(dev(logits), dev(labels), 0.5))
+    assert np.isnan(gx[[1, 3, 4]]).all() and np.isfinite(gx[[0, 2, 5]]).all()
+
+
 def test_sparse_softmax_cross_entropy(K, orc, rng):
     logits = (rng.standard_normal((128, 10)) * 3).astype(np.float32)
     labels = rng.integers(0, 10, size=(128, 1)).astype(np.float32)
