@@ -179,9 +179,9 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, floa
  * planes x'[2i+a][2j+b] for stride 2 -- and runs one implicit GEMM over the filter taps.  The filter
  * gradient contracts that copy with the zero-bordered upstream gradient that
  * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images
- * in splits that need the workspace; for stride 1 "same" convolutions only
- * (2*pad == dilation*(kh-1) == dilation*(kw-1),
- * K a multiple of 32), so that both copies share one padded plane shape.  The contraction runs a
+ * in splits that need the workspace; for stride 1 with any padding up to the filter's reach
+ * dilation*(k-1) (K a multiple of 32; the two copies always share one row pitch, their plane
+ * heights differ unless the convolution keeps the size).  The contraction runs a
  * few elements past a plane, but only over zeros of both operands (the planes are sized for that),
  * so a NaN or infinity in one channel of x reaches the gradients of that channel only; within the
  * channel it can reach filter taps that the reference's columns would not pair it with (0 * NaN at

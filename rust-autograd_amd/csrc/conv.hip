@@ -441,15 +441,21 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     // (32) and reads the other operand up to kh-1 rows and kw-1 elements further: rows are added until
     // everything it reads past a plane's own data is zero -- the rows below the data, then the top
     // border of the next plane up to the first data element of its first data row -- so that no value
-    // of a neighbouring plane (which could be a NaN) ever meets one of those zeros.
+    // of a neighbouring plane (which could be a NaN) ever meets one of those zeros.  A plane plays one of two
+    // parts there: as the gradient it is read from its first data element on (border `top`), as the input it is
+    // read from its origin on but up to a filter's reach further, which comes to the same bound with the border
+    // of the other part (`pad`): the larger of the two sizes the plane.
     const int top = ekh - 1 - pad, left = ekw - 1 - pad;
+    const int guard_t = top > pad ? top : pad, guard_l = left > pad ? left : pad;
     g->Wp = yw + left;
     for (;; ++g->Wp) {
         if (g->Wp > xw + ekw + 6) return false;
-        if (((long long)xh * g->Wp) % 4 != 0) continue;
+        // (the rows of this tensor and of the one it is contracted into: the bordered copies of x and of gy then
+        // come out with one row pitch, which the implicit filter gradient needs)
+        if (((long long)xh * g->Wp) % 4 != 0 || ((long long)yh * g->Wp) % 4 != 0) continue;
         g->Hp = xh + ekh - 1;
         const long long kq = (((long long)xh * g->Wp + 31) / 32) * 32;
-        while (((long long)g->Hp * g->Wp) % 4 != 0 || (long long)(g->Hp - top) * g->Wp - left < kq) ++g->Hp;
+        while (((long long)g->Hp * g->Wp) % 4 != 0 || (long long)(g->Hp - guard_t) * g->Wp - guard_l < kq) ++g->Hp;
         break;
     }
     // past the last plane the reads run into kSlackFloats zeroed floats
@@ -496,12 +502,18 @@ static bool fused_fwd_geom(int B, int C, int H, int W, int K, int kh, int kw, in
 // Positions of the flattened padded plane that the implicit filter gradient contracts over: all
 // rows that hold gradient values, rounded up to the GEMM's k tile.  0 = the rounding would reach
 // past zeros.
-static int filter_grad_positions(const FusedGeom &g, int OH, int pad)
+// `gx`: the bordered input (border pad), `gg`: the bordered gradient (border reach - pad, reach = dil * (k - 1)).
+static int filter_grad_positions(const FusedGeom &gx, const FusedGeom &gg, int OH, int pad, int reach)
 {
-    // past the end of a plane the next plane's top border (pad rows and pad elements of zeros) or the
-    // zeroed slack follows; fused_geom has sized the plane so that nothing else is reached
-    const long long kq = (((long long)OH * g.Wp + 31) / 32) * 32;
-    return kq <= (long long)(g.Hp - pad) * g.Wp - pad ? (int)kq : 0;
+    // The gradient is read from its first value on: what follows its OH rows must be zeros up to position kq (its
+    // bottom rows, then the next plane's top border or the zeroed slack).  The input is read from its origin on,
+    // up to `reach` rows and elements past position kq: that may run into the next plane's top border (pad rows and
+    // elements of zeros) but not into its data.  Both come to the same bound; fused_geom sizes the planes for it.
+    const long long kq = (((long long)OH * gx.Wp + 31) / 32) * 32;
+    const int b = reach - pad;
+    if (gx.Wp != gg.Wp || b < 0) return 0;
+    const bool ok = kq <= (long long)(gx.Hp - b) * gx.Wp - b && kq <= (long long)(gg.Hp - b) * gg.Wp - b;
+    return ok ? (int)kq : 0;
 }
 
 }  // namespace ag
@@ -613,8 +625,9 @@ extern "C" ag_status_t ag_conv2d_nocols_with_filter_f32(ag_stream_t stream, cons
 }
 
 // gypad: the zero-bordered upstream gradient written by ag_conv_input_grad_prepare_f32 (the start
-// of its scratch).  Stride 1: the geometry must be a "same" convolution (2*pad == k-1) so that x
-// and gy share one padded plane shape.
+// of its scratch).  Stride 1: x' carries a border of pad, gy' one of reach - pad (reach = dilation * (k - 1)); both
+// have the row pitch W + pad (rounded alike), so a position of the flattened gy' plane and the same position of the
+// x' plane shifted by a tap are the two factors of one product.  Their plane heights differ unless 2 * pad == reach.
 extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H, int W, int K, int kh, int kw, int pad,
                                                              int stride, int dilation)
 {
@@ -625,12 +638,11 @@ extern "C" size_t ag_conv2d_filter_grad_nocols_f32_workspace(int B, int C, int H
     }
     FusedGeom g, gg;
     const int OH = H + 2 * pad - dilation * (kh - 1), OW = W + 2 * pad - dilation * (kw - 1);
-    if (2 * pad != dilation * (kh - 1) || 2 * pad != dilation * (kw - 1) || K % 4 != 0 ||
-        !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) ||
-        !fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) || g.Hp != gg.Hp || g.Wp != gg.Wp ||
-        (long long)C * g.Hp * g.Wp >= (1LL << 30))
+    if (K % 4 != 0 || !fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) ||
+        !fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) || (long long)C * g.Hp * g.Wp >= (1LL << 30) ||
+        (long long)K * gg.Hp * gg.Wp >= (1LL << 30))
         return 0;
-    const int kq = filter_grad_positions(g, OH, pad);
+    const int kq = filter_grad_positions(g, gg, OH, pad, dilation * (kh - 1));
     return kq ? gemm_conv_filter_grad_workspace(B, K, C, kh * kw, kq) : 0;
 }
 
@@ -649,16 +661,15 @@ extern "C" ag_status_t ag_conv2d_filter_grad_nocols_f32(ag_stream_t stream, cons
     }
     FusedGeom g, gg;
     const int OH = H + 2 * pad - dilation * (kh - 1), OW = W + 2 * pad - dilation * (kw - 1);
-    AG_REQUIRE(2 * pad == dilation * (kh - 1) && 2 * pad == dilation * (kw - 1) && K % 4 == 0 && C >= 1 &&
-                   fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) &&
-                   fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) &&
-                   g.Hp == gg.Hp && g.Wp == gg.Wp && aligned16(xpad) && aligned16(gypad),
+    AG_REQUIRE(K % 4 == 0 && C >= 1 && fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) &&
+                   fused_geom(B, K, OH, OW, C, kh, kw, pad, H, W, &gg, dilation) && aligned16(xpad) && aligned16(gypad),
                AG_ERR_INVALID_DIMS, "conv2d_filter_grad (column-free): geometry not supported");
-    const int kq = filter_grad_positions(g, OH, pad);
-    AG_REQUIRE(kq > 0 && (long long)C * g.Hp * g.Wp < (1LL << 30), AG_ERR_INVALID_DIMS,
-               "conv2d_filter_grad (column-free): plane too small or too many channels");
-    return gemm_conv_filter_grad(as_stream(stream), gypad, xpad + kFwdLeadFloats, gw, ws, ws_bytes, B, K, C, kh, kw, pad, g.Hp,
-                                 g.Wp, kq, dilation);
+    const int reach = dilation * (kh - 1);
+    const int kq = filter_grad_positions(g, gg, OH, pad, reach);
+    AG_REQUIRE(kq > 0 && (long long)C * g.Hp * g.Wp < (1LL << 30) && (long long)K * gg.Hp * gg.Wp < (1LL << 30), AG_ERR_INVALID_DIMS,
+               "conv2d_filter_grad (column-free): the bordered planes of x and gy do not line up, or too many channels");
+    return gemm_conv_filter_grad(as_stream(stream), gypad, xpad + kFwdLeadFloats, gw, ws, ws_bytes, B, K, C, kh, kw, reach - pad,
+                                 gg.Hp, g.Hp, g.Wp, kq, dilation);
 }
 
 extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *gy, const float *w,

@@ -1107,12 +1107,11 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
 }
 
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
-                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq, int dil)
+                                  int B, int Kf, int C, int kh, int kw, int border, int Hp_gy, int Hp_x, int Wp, int kq, int dil)
 {
-    const long long plane = (long long)Hp * Wp;
-    // positions are counted from the first gradient value
-    return conv_filter_grad_gemm(st, gyp + ((long long)pad * Wp + pad), xp, gw, ws, ws_bytes, B, Kf, C, kh, kw, Wp, kq, plane,
-                                 plane, 0, dil);
+    // positions are counted from the first gradient value, `border` rows and elements into a plane of gyp
+    return conv_filter_grad_gemm(st, gyp + ((long long)border * Wp + border), xp, gw, ws, ws_bytes, B, Kf, C, kh, kw, Wp, kq,
+                                 (long long)Hp_gy * Wp, (long long)Hp_x * Wp, 0, dil);
 }
 
 size_t gemm_conv_filter_grad_stride2_workspace(int B, int Kf, int C, int taps)

@@ -75,7 +75,8 @@ void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &
 // split over images.
 size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq);
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
-                                  int B, int Kf, int C, int kh, int kw, int pad, int Hp, int Wp, int kq, int dil = 1);
+                                  int B, int Kf, int C, int kh, int kw, int border, int Hp_gy, int Hp_x, int Wp, int kq,
+                                  int dil = 1);
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
                                  int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil = 1);
 // Stride-2 forward over phase planes (see GemmParams::conv_phase): wf [K][kh*kw][C] in natural tap

@@ -902,7 +902,8 @@ def test_add_broadcast_and_the_reduced_gradient(G, rng, shape, bshape):
 
 
 # ------------------------------------------------------------------------------- column-free convolution in the graph
-@pytest.mark.parametrize("B,Cin,Cout,H,k,pad", [(64, 32, 64, 32, 3, 1), (24, 64, 128, 36, 3, 1), (32, 32, 32, 28, 5, 2)])
+@pytest.mark.parametrize("B,Cin,Cout,H,k,pad", [(64, 32, 64, 32, 3, 1), (24, 64, 128, 36, 3, 1), (32, 32, 32, 28, 5, 2),
+                                               (64, 32, 64, 36, 3, 0), (56, 32, 32, 32, 3, 2)])   # and without / with more than "same" padding
 def test_conv2d_column_free_through_the_graph(G, orc, rng, B, Cin, Cout, H, k, pad):
     # channel counts that are multiples of 32, "same" stride-1 convolution: Conv2D keeps a zero-bordered
     # input instead of the columns and all three operators run column-free; values against the oracle

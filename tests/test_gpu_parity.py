@@ -523,8 +523,9 @@ NOCOLS_CASES = [  # B, C (a multiple of 32), K (filters), H, W, k, pad
     (3, 32, 64, 18, 18, 5, 2),    # 5x5 "same"
     (2, 64, 160, 17, 17, 3, 1),   # odd width; more than 128 filters: two row tiles
     (4, 32, 64, 14, 14, 3, 1),    # config 2's second convolution
-    (2, 32, 32, 20, 20, 3, 0),    # no padding: forward only (the filter gradient needs a "same" convolution)
-    (2, 32, 64, 24, 24, 3, 2),    # pad equal to k - 1: forward only
+    (2, 32, 32, 20, 20, 3, 0),    # no padding: x is its own bordered copy, gy gets k - 1 rows and columns
+    (2, 32, 64, 24, 24, 3, 2),    # pad equal to k - 1: gy is its own bordered copy
+    (3, 64, 64, 30, 26, 5, 1),    # 5x5 with less than "same" padding
 ]
 
 
@@ -549,7 +550,8 @@ def test_conv2d_column_free_forward_and_filter_grad(K, orc, rng, case):
     assert_close_conditioned(host(y), y64, yabs, "column-free forward", ref32=y32)
     y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
     assert_close_conditioned(host(y_cols), y64, yabs, "columns forward", ref32=y32)
-    if 2 * p != k - 1:
+    if K.capi.lib().ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, 1) == 0:
+        assert 2 * p != k - 1, "a same-size convolution is always supported"
         return
     say("column-free filter gradient", case)
     staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
@@ -668,8 +670,9 @@ def test_conv2d_column_free_dilated(K, orc, rng, case):
     gxabs = orc.conv2d_transpose(np.abs(gy).astype(np.float64), np.abs(w).astype(np.float64), p, 1, d, out_hw=(H, W))
     assert_close_conditioned(host(gx), gx64, gxabs, "dilated staged input gradient",
                              ref32=orc.conv2d_transpose(gy, w, p, 1, d, out_hw=(H, W)))
-    same = 2 * p == d * (k - 1)
-    assert (L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, d) > 0) == same
+    # (any padding, as long as the bordered planes of x and gy come out with one row pitch; always for "same")
+    same = L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, d) > 0
+    assert same or 2 * p != d * (k - 1)
     if same:
         say("dilated column-free filter gradient", case)
         gw = host(K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p, 1, d))
@@ -783,7 +786,9 @@ def test_conv2d_with_cols_matches_oracle(K, orc, rng):
         assert np.array_equal(host(K.conv2d_with_cols(cols, dev(w), OH, OW)), host(y))
 
 
-@pytest.mark.parametrize("case", [(3, 64, 64, 14, 14, 3, 1), (2, 64, 128, 56, 56, 3, 1), (2, 32, 32, 16, 16, 5, 2)])
+@pytest.mark.parametrize("case", [(3, 64, 64, 14, 14, 3, 1), (2, 64, 128, 56, 56, 3, 1), (2, 32, 32, 16, 16, 5, 2),
+                                  # other paddings: the planes of x and gy have different heights
+                                  (3, 32, 64, 20, 20, 3, 0), (2, 64, 32, 24, 28, 3, 2), (3, 32, 32, 22, 18, 5, 1), (2, 32, 64, 20, 24, 5, 4)])
 def test_conv2d_column_free_filter_grad_keeps_a_nan_inside_its_channel(K, orc, rng, case):
     """The implicit filter gradient contracts a few positions past each plane.  What it reads there
     must be zeros of both operands: a NaN anywhere in one channel of x -- corners and edges included,
@@ -792,7 +797,8 @@ def test_conv2d_column_free_filter_grad_keeps_a_nan_inside_its_channel(K, orc, r
     B, C, Kc, H, W, k, p = case
     x = rng.standard_normal((B, C, H, W)).astype(np.float32)
     w = rng.uniform(-0.1, 0.1, (Kc, C, k, k)).astype(np.float32)
-    gy = rng.standard_normal((B, Kc, H, W)).astype(np.float32)
+    gy = rng.standard_normal((B, Kc, H + 2 * p - k + 1, W + 2 * p - k + 1)).astype(np.float32)
+    assert K.capi.lib().ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, 1) > 0
     bad = C // 2
     for b in (0, B - 1):
         x[b, bad, 0, :] = np.nan
@@ -912,10 +918,14 @@ def test_conv2d_column_free_refuses_other_geometries(K, rng):
     assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1, 1, 1) == 0      # C not a multiple of 32
     assert L.ag_conv2d_nocols_scratch_floats(2, 32, 4, 4, 32, 3, 3, 1, 1, 1) == 0       # plane too small
     assert K.conv2d_nocols(dev(np.zeros((2, 3, 28, 28), np.float32)), dev(np.zeros((32, 3, 3, 3), np.float32)), 1) is None
-    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 32, 3, 3, 0, 1, 1) >= 0
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 30, 3, 3, 1, 1, 1) == 0   # 30 filters
     x = dev(np.zeros(4096, np.float32))
-    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 32, 3, 3, 0, 1, 1, None, 0)
+    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 30, 3, 3, 1, 1, 1, None, 0)
     assert rc == 4 and b"geometry not supported" in L.ag_last_error()
+    # a supported geometry without the workspace it needs is refused before anything is launched
+    assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 32, 3, 3, 0, 1, 1) > 16
+    rc = L.ag_conv2d_filter_grad_nocols_f32(None, K._ptr(x), K._ptr(x), K._ptr(x), 2, 32, 20, 20, 32, 3, 3, 0, 1, 1, None, 0)
+    assert rc == 4 and b"workspace" in L.ag_last_error()
 
 
 FUSED_CASES = [  # B, C (input channels of the conv), K (filters), H, W, k, pad
