@@ -463,10 +463,8 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
-    // a tile (64 x 128 for up to 64 channels, else 128 x 256) may straddle two images, not three.  (Images of
-    // fewer than 256 positions with more channels would run on 64 x 64 tiles, where the column path is as fast:
-    // 0.315 ms against 0.306 ms for the three contractions of 32 x 256 -> 256 x 14 x 14.)
-    return n_img >= (xch <= 64 ? 128 : 256) && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
+    // a tile (at most 128 columns wide while an image has fewer than 256 positions) may straddle two images, not three
+    return n_img >= 128 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
 }
 
 static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const FusedGeom &g,
@@ -693,9 +691,12 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
     // reads a zero-bordered copy of gy; the columns (conv2d_transpose.rs:148-151) are never
     // written.  The sum runs over (tap, filter) instead of filters then taps, within tolerance.
     FusedGeom fg;
+    // (images of fewer than 256 padded positions with more than 64 channels run on 64-row tiles, and while their
+    // columns stay in the cache the column path is ahead: 32 x 256 -> 256 channels, 14 x 14: 0.084 against 0.108 ms;
+    // at eight times the batch 0.71 against 0.54 ms)
     if (stride == 1 && g_fused_input_grad &&
         fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg, dilation) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
-        aligned16(gcols) && aligned16(gx)) {
+        ((long long)xh * fg.Wp >= 256 || xch <= 64 || (long long)B * M * P >= (1LL << 24)) && aligned16(gcols) && aligned16(gx)) {
         if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad, dilation)) return s;
         return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
                                     fg.Wp, dilation);

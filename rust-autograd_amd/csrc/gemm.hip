@@ -932,6 +932,10 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
         const double wide_cost = wide_rounds * 128.0 * kCfgs[wide].bn / (wide == 14 ? 1.0 : 0.9);
         const double small_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 128), 2 * G) * 2.0 * 64.0 * 128.0 / 0.95;
         cfg = wide_cost <= small_cost ? wide : kDirectCfg64;
+        // a problem of less than a round of those: 64 x 64 tiles (32 x 256 -> 256 channels, 14 x 14: 0.100 against
+        // 0.108 ms)
+        const double narrow_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 64), 2 * G) * 2.0 * 64.0 * 64.0 / 0.78;
+        if (narrow_cost < 0.9 * (wide_cost <= small_cost ? wide_cost : small_cost)) cfg = kDirectCfg64Narrow;
     }
     if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && kCfgs[g_force_cfg].bn <= p.n_img)
         cfg = g_force_cfg;  // test hook
