@@ -463,8 +463,8 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
-    // a tile (at most 128 columns wide while an image has fewer than 256 positions) may straddle two images, not three
-    return n_img >= 128 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
+    // (a tile may cover any number of images)
+    return n_img >= 16 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
 }
 
 static ag_status_t fused_prepare(hipStream_t st, const float *gy, const float *w, float *scratch, const FusedGeom &g,

@@ -921,7 +921,8 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     // rows in 3.2 rounds -- against 0.21 ms on 64 x 128 ones)
     int cfg = C <= 32 ? kDirectCfg32 : kDirectCfg64;
     if (C > 32 && C <= 64) {
-        if (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && p.n_img >= 64) cfg = kDirectCfg64Narrow;
+        // (the stride-2 forms keep to tiles that cover at most two images)
+        if (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && (p.n_img >= 64 || (phase == 0 && pair_w == 0))) cfg = kDirectCfg64Narrow;
     } else if (C > 64) {
         const long long G = direct_grid(num_cus());
         const int wide = p.n_img >= 256 ? 14 : 13;
@@ -937,7 +938,7 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
         const double narrow_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 64), 2 * G) * 2.0 * 64.0 * 64.0 / 0.78;
         if (narrow_cost < 0.9 * (wide_cost <= small_cost ? wide_cost : small_cost)) cfg = kDirectCfg64Narrow;
     }
-    if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && kCfgs[g_force_cfg].bn <= p.n_img)
+    if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && (pair_w == 0 && phase == 0 || kCfgs[g_force_cfg].bn <= p.n_img))
         cfg = g_force_cfg;  // test hook
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);

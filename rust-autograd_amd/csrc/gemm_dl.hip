@@ -122,6 +122,24 @@ struct DirectTile {
             off[i] = ((unsigned)(k * ld + n) + extra) * 4u;
         }
     }
+    // The same for batches narrower than a tile (the 7 x 7 planes of a late convolution layer): a tile may run over
+    // any number of them, `left` batches remain from the one it starts in (that one included).
+    __device__ inline void init_folded_many(int ld, int r0, int n_img, int left, unsigned next, int wave, int lane)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int pos = (i * NW + wave) * 64 + lane;
+            const int k = pos / CPR, cn = (pos % CPR) ^ (((k >> 2) & 1) * 8);
+            int n = r0 + cn * 4;
+            int q = n / n_img;
+            n -= q * n_img;
+            if (q >= left) {  // beyond the operand: clamped
+                q = left - 1;
+                n = n_img - 4;
+            }
+            off[i] = ((unsigned)(k * ld + n) + (unsigned)q * next) * 4u;
+        }
+    }
     __device__ static inline long long k_step(int ld) { return KC ? BK : (long long)BK * ld; }
 
     // Load number `i` (a constant after unrolling) of this wave.
@@ -272,8 +290,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         const Item it = item_of(fcur);
         ldr_a.init(lda, it.m0, p.M, wave, lane);
         if (!KB && p.n_img != 0) {
-            const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
-            ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
+            if (CONV != 0 && p.n_img < BN) {
+                // (implicit convolution over small planes)
+                ldr_b.init_folded_many(ldb, it.r0, p.n_img, (p.N - (it.n0 - it.r0)) / p.n_img, (unsigned)p.sB, wave, lane);
+            } else {
+                const bool has_next = it.n0 - it.r0 + p.n_img < p.N;  // p.N = batches * n_img here
+                ldr_b.init_folded(ldb, it.r0, p.n_img, has_next ? (unsigned)p.sB : 0u, wave, lane);
+            }
         } else if (KB && p.rows_taps != 0) {
             ldr_b.init_conv_rows(it.n0, p.N, p.rows_taps, p.rows_kw, p.rows_wp, p.rows_plane, p.rows_phase, p.conv_dil, wave, lane);
         } else {
@@ -454,7 +477,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             alpha = p.alpha;
             beta = p.beta;
         }
-        if (p.conv_wp != 0) {
+        if (CONV != 3 && p.conv_wp != 0) {
             // implicit input gradient: column -> pixel of the (possibly next) image; the columns
             // of the zero border are dropped
             const int row_base = it.m0 + wm * WM + 4 * half;
@@ -465,7 +488,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 int col = it.r0 + wn * WN + l31 + j * 32;
                 const bool in_range = it.n0 + wn * WN + l31 + j * 32 < p.N;
                 long long img = 0;
-                if (col >= p.n_img) {
+                if (p.n_img < BN) {  // small planes: the tile covers several images
+                    const int q = col / p.n_img;
+                    col -= q * p.n_img;
+                    img = q * p.sC;
+                } else if (col >= p.n_img) {
                     col -= p.n_img;
                     img = p.sC;
                 }

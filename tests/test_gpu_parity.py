@@ -739,6 +739,28 @@ def test_conv2d_column_free_filter_grad_of_a_small_batch_is_cut_into_position_ch
     assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape)))
 
 
+@pytest.mark.parametrize("B,C,Kc,H,W,k,p", [(9, 64, 96, 7, 7, 3, 1), (37, 32, 32, 8, 8, 3, 1), (20, 160, 64, 7, 9, 3, 1), (130, 32, 64, 5, 5, 3, 1),
+                                           (6, 64, 192, 10, 10, 5, 2), (11, 32, 64, 7, 7, 3, 0)])
+def test_conv2d_column_free_on_planes_smaller_than_a_tile(K, rng, B, C, Kc, H, W, k, p):
+    # the 7 x 7 planes of a late layer: a tile of the implicit GEMMs covers several images (and the end of the batch);
+    # integer-valued data, so all three results must equal the columns path bit for bit
+    OH, OW = H + 2 * p - k + 1, W + 2 * p - k + 1
+    x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+    w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gy = rng.integers(-2, 3, (B, Kc, OH, OW)).astype(np.float32)
+    say("column-free on small planes", (B, C, Kc, H, W, k, p))
+    res = K.conv2d_nocols(dev(x), dev(w), p)
+    assert res is not None
+    y, xpad = res
+    y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, 1)
+    assert np.array_equal(host(y), host(y_cols))
+    gx, gypad = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W))
+    gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, 1, out_hw=(H, W), return_cols=True)
+    assert np.array_equal(host(gx), host(gx_cols))
+    gw = K.conv2d_filter_grad_nocols(xpad, gypad, x.shape, w.shape, p)
+    assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape)))
+
+
 def test_conv2d_column_free_headline_size_matches_columns_path(K):
     # the benchmark's own shape (B=256, 64 -> 128 channels, 56x56, 3x3): the three column-free results
     # against the library's column path, which the smaller cases pin to the oracle
@@ -916,7 +938,7 @@ def test_conv2d_stride2_filter_grad_keeps_a_nan_inside_its_channel(K, rng):
 def test_conv2d_column_free_refuses_other_geometries(K, rng):
     L = K.capi.lib()
     assert L.ag_conv2d_nocols_scratch_floats(2, 3, 28, 28, 32, 3, 3, 1, 1, 1) == 0      # C not a multiple of 32
-    assert L.ag_conv2d_nocols_scratch_floats(2, 32, 4, 4, 32, 3, 3, 1, 1, 1) == 0       # plane too small
+    assert L.ag_conv2d_nocols_scratch_floats(2, 32, 2, 2, 32, 3, 3, 1, 1, 1) == 0       # plane too small
     assert K.conv2d_nocols(dev(np.zeros((2, 3, 28, 28), np.float32)), dev(np.zeros((32, 3, 3, 3), np.float32)), 1) is None
     assert L.ag_conv2d_filter_grad_nocols_f32_workspace(2, 32, 20, 20, 30, 3, 3, 1, 1, 1) == 0   # 30 filters
     x = dev(np.zeros(4096, np.float32))
@@ -981,8 +1003,9 @@ def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
     assert_close_conditioned(host(gx), o64, oabs, "staged input grad")
     # geometries the column-free path does not take report 0 and are refused
     assert L.ag_conv_input_grad_scratch_floats(B, 48, H, W, C, k, k, p, 1, 1, H, W) == 0          # filters not a multiple of 32
-    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 1, 1, 8, 8) == 0           # fewer than 128 columns per image
-    assert L.ag_conv_input_grad_scratch_floats(B, Kc, H, W, C, k, k, p, 1, 2, H, W) == 0          # dilation
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 8, 8, C, k, k, p, 1, 1, 8, 8) > 0            # planes smaller than a tile are fine
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, 2, 2, C, k, k, p, 1, 1, 2, 2) == 0           # fewer than 16 columns per image
+    assert L.ag_conv_input_grad_scratch_floats(B, Kc, H, W, C, k, k, p, 1, 2, H, W) == 0          # extents that do not fit the dilation
     assert L.ag_conv_input_grad_scratch_floats(B, Kc, H, W, C, k, k, p, 3, 1, H, W) == 0          # stride 3
     with pytest.raises(K.capi.InvalidDims, match="not supported"):
         K.check(L.ag_conv_input_grad_prepare_f32(K._stream(), K._ptr(gyd), K._ptr(wd), K._ptr(scratch), B, 48, H, W,
