@@ -174,8 +174,9 @@ ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *scratch, floa
  * -> fast_im2col_gemm_fused_kernel, conv2d.rs:25-112; conv2d_filter_grad_impl, conv2d.rs:631-734);
  * the results are those of ag_conv2d_fwd_f32 / ag_conv2d_filter_grad_f32 within the floating-point
  * tolerance (other summation order).  The forward writes a rearranged copy of x into `xpad`
- * (ag_conv2d_nocols_scratch_floats() floats; 0 = geometry not supported: C a multiple of 32, planes
- * of at least 128 padded elements, ...) -- the zero-bordered input for stride 1, its four phase
+ * (ag_conv2d_nocols_scratch_floats() floats; 0 = geometry not supported: C a multiple of 32, square
+ * filters, for stride 2 planes of at least 128 padded elements, ...) -- the zero-bordered input for
+ * stride 1, its four phase
  * planes x'[2i+a][2j+b] for stride 2 -- and runs one implicit GEMM over the filter taps.  The filter
  * gradient contracts that copy with the zero-bordered upstream gradient that
  * ag_conv_input_grad_prepare_f32 leaves at the start of its scratch (`gypad`), summed over images
