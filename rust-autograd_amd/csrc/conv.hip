@@ -463,7 +463,10 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
-    // (a tile may cover any number of images)
+    // a tile may cover any number of images; the loader's 32-bit byte offsets reach over a k tile's 32 planes and as many
+    // images further as a tile of up to 256 columns can run into
+    const long long more_imgs = n_img >= 256 ? 1 : 256 / n_img + 1;
+    if (32 * plane + more_imgs * ych * plane >= (1LL << 30)) return false;
     return n_img >= 16 && B * n_img < 0x7fffffffLL && ych * plane < (1LL << 30);
 }
 
