@@ -36,9 +36,15 @@ typedef __attribute__((address_space(3))) float lds_float_t;
 template <int LDS_IMM>
 __device__ inline void dma16(const float *base, unsigned byte_off, unsigned lds_wave_base)
 {
+    // (the base is wave-uniform; naming its halves as first-lane values keeps it in scalar registers for the
+    // assembly below whatever the compiler did with the pointer arithmetic before -- free when it is there already)
+    const unsigned long long bits = reinterpret_cast<unsigned long long>(base);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)bits);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(bits >> 32));
+    const float *sbase = reinterpret_cast<const float *>(((unsigned long long)hi << 32) | lo);
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(lds_wave_base), "v"(byte_off), "s"(base), "n"(LDS_IMM)
+                 : "s"(lds_wave_base), "v"(byte_off), "s"(sbase), "n"(LDS_IMM)
                  : "m0", "scc");
 }
 
