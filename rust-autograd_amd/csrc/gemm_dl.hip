@@ -183,15 +183,17 @@ struct DirectTile {
 // constant 1) the undilated forward product of the headline step took 0.930 instead of 0.916 ms; with the tests
 // "is this a convolution / a phase walk" decided at compile time it takes 0.905 ms, the input gradient 0.937
 // instead of 0.964, the filter gradient 0.868 instead of 0.906 and the 4096^3 NT / TN products 0.965 / 0.971
-// instead of 0.994 / 0.996 ms.
-template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV = 0>
+// instead of 0.994 / 0.996 ms; the stride-2 forward over phase planes 0.291 instead of 0.300 ms.
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
 {
-    // CONV 1 / 2: the tap walk of the implicit convolution (conv_wp != 0, no phase planes) known at compile time,
-    // without / with dilation; 3: an ordinary product, known at compile time; 0: told apart at run time (what is
-    // left: the stride-2 forward over phase planes)
+    // CONV 1 / 2: the tap walk of the implicit convolution (conv_wp != 0, no phase planes), without / with
+    // dilation; 3: an ordinary product; 4: the stride-2 forward, whose taps walk the four phase planes
+    static_assert(CONV >= 1 && CONV <= 4, "walk of the k loop");
+    constexpr bool shifts = CONV == 1 || CONV == 2;  // taps as shifts within one plane
+    constexpr bool phases = CONV == 4;
+    constexpr bool taps = shifts || phases;
     const int conv_dil = CONV == 2 ? p.conv_dil : 1;
-    const bool taps = CONV == 3 ? false : CONV != 0 || p.conv_wp != 0;
     static_assert(STAGES >= 3 && STAGES <= 8, "ring of three to eight tiles");
     static_assert(BK == 16 || BK == 32, "k tile");
     constexpr int KK = BK / 8;  // groups of four MFMA k steps per tile
@@ -290,13 +292,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     const float *pb_group = nullptr;           // stride-2 forward: B origin of the current group of 32 channels
     int fkt = 0, f_left = 0, f_kx = 0, f_ky = 0;
     const int conv_first_shift =
-        CONV == 3 ? 0 : CONV != 0 || (p.conv_wp != 0 && p.conv_phase == 0) ? ((p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1)) * conv_dil : 0;
+        shifts ? ((p.kbatch / p.conv_kw - 1) * p.conv_wp + (p.conv_kw - 1)) * conv_dil : 0;
     Cursor fcur = first;
     auto f_begin = [&]() {
         const Item it = item_of(fcur);
         ldr_a.init(lda, it.m0, p.M, wave, lane);
         if (!KB && p.n_img != 0) {
-            if (CONV != 0 && p.n_img < BN) {
+            if (shifts && p.n_img < BN) {
                 // (implicit convolution over small planes)
                 ldr_b.init_folded_many(ldb, it.r0, p.n_img, (p.N - (it.n0 - it.r0)) / p.n_img, (unsigned)p.sB, wave, lane);
             } else {
@@ -330,7 +332,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 cursor_next(fcur);
                 f_begin();
             }
-        } else if (CONV == 0 && p.conv_phase != 0) {
+        } else if (phases) {
             // Stride-2 forward: all taps of one group of 32 channels in natural order, then the next group.
             if (++fkt == p.kbatch) {
                 fkt = 0;
@@ -483,7 +485,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             alpha = p.alpha;
             beta = p.beta;
         }
-        if (CONV != 3 && p.conv_wp != 0) {
+        if (taps) {
             // implicit input gradient: column -> pixel of the (possibly next) image; the columns
             // of the zero border are dropped
             const int row_base = it.m0 + wm * WM + 4 * half;
@@ -494,7 +496,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 int col = it.r0 + wn * WN + l31 + j * 32;
                 const bool in_range = it.n0 + wn * WN + l31 + j * 32 < p.N;
                 long long img = 0;
-                if (p.n_img < BN) {  // small planes: the tile covers several images
+                if (shifts && p.n_img < BN) {  // small planes: the tile covers several images
                     const int q = col / p.n_img;
                     col -= q * p.n_img;
                     img = q * p.sC;
@@ -699,7 +701,7 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
     if constexpr ((KA_ || BM % 64 == 0) && (KB_ || BN % 64 == 0)) if (ka == KA_ && kb == KB_) {      \
         auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 3>;                              \
         if constexpr (KA_ && !KB_) /* the implicit convolution over filter taps */                    \
-            if (p.conv_phase != 0) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 0>;       \
+            if (p.conv_phase != 0) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 4>;       \
             else if (p.conv_wp != 0)                                                                  \
                 kern = p.conv_dil != 1 ? gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 2>         \
                                        : gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 1>;        \
