@@ -630,6 +630,49 @@ def test_conv2d_column_free_random_geometries_exact(K):
     assert ran_fwd >= 20 and ran_bwd >= 5, (ran_fwd, ran_bwd)
 
 
+def test_conv2d_column_free_random_dilations_paddings_and_batches_exact(K):
+    # a second fixed sample, over what the first leaves out: dilations 1 to 3, every padding from 0 to the filter's
+    # reach, 2 x 2 filters, planes from 4 x 4 up, batches from 1 to 40 (small planes put several images into one
+    # tile, small batches cut the filter gradient's planes into chunks).  Integer-valued data: equal to the columns
+    # path bit for bit wherever the library accepts the geometry.
+    r = np.random.default_rng(20240923)
+    L = K.capi.lib()
+    ran = [0, 0, 0]
+    for _ in range(60):
+        k = int(r.choice([2, 3, 3, 5]))
+        d = int(r.choice([1, 1, 2, 3]))
+        reach = d * (k - 1)
+        p = int(r.integers(0, reach + 1))
+        B = int(r.choice([1, 2, 3, 5, 8, 17, 40]))
+        C = int(r.choice([32, 64, 96, 128]))
+        Kc = int(r.choice([32, 64, 96, 160]))
+        lo = max(reach + 1 - 2 * p, 4)
+        H, W = int(r.integers(lo, 45)), int(r.integers(lo, 45))
+        if B >= 17:
+            H, W = min(H, 24), min(W, 24)
+        OH, OW = H + 2 * p - reach, W + 2 * p - reach
+        geo = (B, C, Kc, H, W, k, p, d)
+        x = r.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+        gy = r.integers(-2, 3, (B, Kc, OH, OW)).astype(np.float32)
+        say("column-free random geometry with dilation", geo)
+        y_cols, cols = K.conv2d(dev(x), dev(w), p, 1, d)
+        res = K.conv2d_nocols(dev(x), dev(w), p, 1, d)
+        if res is not None:
+            ran[0] += 1
+            assert np.array_equal(host(res[0]), host(y_cols)), geo
+        gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, d, out_hw=(H, W), return_cols=True)
+        staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 1, d)
+        if staged is not None:
+            ran[1] += 1
+            assert np.array_equal(host(staged[0]), host(gx_cols)), geo
+        if res is not None and staged is not None and L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 1, d) > 0:
+            ran[2] += 1
+            gw = K.conv2d_filter_grad_nocols(res[1], staged[1], x.shape, w.shape, p, 1, d)
+            assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape))), geo
+    assert min(ran) >= 40, ran
+
+
 DILATED_NOCOLS_CASES = [  # B, C, K, H, W, k, pad, dilation
     (2, 64, 64, 28, 28, 3, 2, 2),    # the dilated configuration, 2 of its images: a "same" convolution
     (3, 32, 64, 20, 22, 3, 2, 2),    # uneven extents
