@@ -960,6 +960,46 @@ def test_conv2d_stride2_column_free(K, orc, rng, case):
                           host(K.conv2d_filter_grad(colsi, dev(gi), w.shape)))
 
 
+def test_conv2d_stride2_column_free_random_geometries_exact(K):
+    # a fixed sample of stride-2 geometries (filters of 2 to 5 taps a side, every padding below the filter size, odd
+    # and even extents, 1 to 17 images): integer-valued data, so the phase-plane forward, the pair-form or four-parity
+    # input gradient and the filter gradient must equal the columns path bit for bit wherever the library accepts
+    # the geometry
+    r = np.random.default_rng(20241005)
+    L = K.capi.lib()
+    ran = [0, 0, 0]
+    for _ in range(40):
+        k = int(r.choice([2, 3, 3, 4, 5]))
+        p = int(r.integers(0, k))
+        B = int(r.choice([1, 2, 3, 5, 8, 17]))
+        C = int(r.choice([32, 64, 96, 128]))
+        Kc = int(r.choice([32, 64, 96, 160]))
+        H, W = int(r.integers(20, 70)), int(r.integers(20, 70))
+        if B >= 8:
+            H, W = min(H, 40), min(W, 40)
+        OH, OW = (H + 2 * p - k) // 2 + 1, (W + 2 * p - k) // 2 + 1
+        geo = (B, C, Kc, H, W, k, p)
+        x = r.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+        gy = r.integers(-2, 3, (B, Kc, OH, OW)).astype(np.float32)
+        say("stride-2 column-free random geometry", geo)
+        y_cols, cols = K.conv2d(dev(x), dev(w), p, 2, 1)
+        res = K.conv2d_nocols(dev(x), dev(w), p, 2, 1)
+        if res is not None:
+            ran[0] += 1
+            assert np.array_equal(host(res[0]), host(y_cols)), geo
+        gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 2, 1, out_hw=(H, W), return_cols=True)
+        staged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 2, 1)
+        if staged is not None:
+            ran[1] += 1
+            assert np.array_equal(host(staged[0]), host(gx_cols)), geo
+        if res is not None and staged is not None and L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, 2, 1) > 0:
+            ran[2] += 1
+            gw = K.conv2d_filter_grad_nocols(res[1], staged[1], x.shape, w.shape, p, 2, 1)
+            assert np.array_equal(host(gw), host(K.conv2d_filter_grad(cols, dev(gy), w.shape))), geo
+    assert min(ran) >= 30, ran
+
+
 def test_conv2d_stride2_filter_grad_keeps_a_nan_inside_its_channel(K, rng):
     B, C, Kc, H, W, k, p = 2, 64, 64, 28, 28, 3, 1
     x = rng.standard_normal((B, C, H, W)).astype(np.float32)
