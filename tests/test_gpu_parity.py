@@ -447,6 +447,35 @@ def test_conv2d_filter_grad_of_a_thin_first_layer(K, orc, rng, B, C, Kc, H, W, k
     assert np.array_equal(gwi, exact.astype(np.float32))
 
 
+def test_matmul_and_batch_matmul_random_shapes_exact_on_small_integers(K):
+    # a fixed sample of shapes around the tile edges (1, 31..33, 63..65, 127..129, 255..257, K tails, the 3136-long
+    # contraction of the dense layer), both transpositions, with and without a batch: small integers, so every sum is
+    # exact in f32 and the result must equal numpy's f64 product bit for bit whichever tile, split or tail pass ran
+    r = np.random.default_rng(20241017)
+    dims = [1, 2, 3, 7, 10, 31, 32, 33, 63, 64, 65, 96, 100, 127, 128, 129, 192, 200, 255, 256, 257, 384, 500, 512,
+            520, 777, 1000, 1024, 1500, 2048, 3136]
+    for _ in range(80):
+        m, n, k = (int(r.choice(dims)) for _ in range(3))
+        ta, tb = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        batch = int(r.choice([0, 0, 1, 2, 5, 16]))
+        if m * n * k > 1.2e9:
+            k = 64
+        if batch and m * n * k * batch > 6e8:
+            batch = 1
+        sa = (k, m) if ta else (m, k)
+        sb = (n, k) if tb else (k, n)
+        if batch:
+            sa, sb = (batch,) + sa, (batch,) + sb
+        a = r.integers(-2, 3, sa).astype(np.float32)
+        b = r.integers(-2, 3, sb).astype(np.float32)
+        say("matmul random shape", (m, n, k, ta, tb, batch))
+        got = host((K.batch_matmul if batch else K.matmul)(dev(a), dev(b), ta, tb))
+        a2 = np.swapaxes(a, -1, -2) if ta else a
+        b2 = np.swapaxes(b, -1, -2) if tb else b
+        want = np.matmul(a2.astype(np.float64), b2.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(got, want), (m, n, k, ta, tb, batch)
+
+
 def test_gemm_degenerate_k_and_beta(K, rng):
     c0 = rng.random((5, 6), dtype=np.float32)
     c = dev(c0)
