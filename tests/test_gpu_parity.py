@@ -1243,6 +1243,43 @@ def test_max_pool_forward_backward_bit_exact(K, orc, rng, case):
         assert np.array_equal(ggy, orc.maxpool2d_gradgrad(ggx, oam, oy.shape))
 
 
+def test_max_pool_random_geometries_with_ties_bit_exact(K, orc):
+    # a fixed sample of windows (2 to 7), steps (1 to 4) and planes (down to one window, up to rows of 3000), on data
+    # with 2, 3, 8 or many distinct values, so that most windows hold ties: values, argmax, tap bytes, both backward
+    # forms, the backward with the ReLU gradient folded in and the second-order op against the CPU restatement
+    r = np.random.default_rng(20241101)
+    for _ in range(50):
+        size = int(r.choice([2, 2, 3, 3, 4, 5, 7]))
+        stride = int(r.choice([1, 2, 2, 2, 3, 4]))
+        B, C = int(r.integers(1, 6)), int(r.choice([1, 2, 3, 5, 16, 33]))
+        H, W = int(r.integers(size, 70)), int(r.integers(size, 140))
+        if r.integers(0, 8) == 0:
+            W, H = int(r.integers(200, 3000)), int(r.integers(size, 12))
+        case = (B, C, H, W, size, stride)
+        levels = int(r.choice([2, 3, 8, 1000000]))
+        x = (r.integers(0, levels, (B, C, H, W)) / np.float32(7)).astype(np.float32) - np.float32(0.3)
+        say("max_pool random geometry", case, levels)
+        y, am, il = K.max_pool2d(dev(x), size, 0, stride)
+        oy, oam, oil = orc.maxpool2d_fwd(x, size, 0, stride)
+        assert np.array_equal(host(y), oy), case
+        assert np.array_equal(host(am).view(np.uint32), oam.view(np.uint32)), case
+        assert np.array_equal(host(il), orc.maxpool2d_taps(oil, W, size, stride)), case
+        gy = r.standard_normal(oy.shape).astype(np.float32)
+        ogx, skipped = orc.maxpool2d_bwd(gy, oam, x.shape)
+        assert skipped == 0
+        relu_x = r.standard_normal(x.shape).astype(np.float32)
+        relu_x.reshape(-1)[::5] = 0.0
+        masked = (relu_x > 0).astype(np.float32) * ogx
+        ggx = r.standard_normal(x.shape).astype(np.float32)
+        oggy = orc.maxpool2d_gradgrad(ggx, oam, oy.shape)
+        for idx in (None, il):
+            gx = host(K.max_pool2d_grad(dev(gy), am, idx, x.shape, size, 0, stride))
+            assert np.array_equal(gx.view(np.uint32), ogx.view(np.uint32)), case
+            fused = host(K.max_pool2d_grad_relu(dev(gy), am, idx, dev(relu_x), size, 0, stride))
+            assert np.array_equal(fused.view(np.uint32), masked.view(np.uint32)), case
+            assert np.array_equal(host(K.max_pool2d_grad_grad(dev(ggx), am, idx, size, 0, stride)), oggy), case
+
+
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 1000])
 def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows):
     """The stride-2 backward walks chunks of output rows; whatever their length (one row, odd
