@@ -1124,6 +1124,38 @@ def test_conv2d_input_grad_staged_entry_points(K, orc, rng):
                                                  C, k, k, p, 1, 1, H, W))
 
 
+def test_conv2d_operators_random_geometries_exact_on_small_integers(K, orc):
+    # the general (column) path over a fixed random sample of what the reference accepts: filters of 1 to 5 taps,
+    # strides and dilations 1 to 3, paddings 0 to 3 (also beyond the filter's reach), channel counts that are not
+    # multiples of anything.  Small integers: forward, filter gradient and the transposed convolution at the
+    # reference's reconstructed output size must equal the CPU restatement bit for bit.
+    r = np.random.default_rng(20241113)
+    ran = 0
+    for _ in range(60):
+        k = int(r.choice([1, 2, 3, 4, 5]))
+        s_, d = int(r.choice([1, 1, 2, 3])), int(r.choice([1, 1, 2, 3]))
+        p = int(r.integers(0, 4))
+        B, C, Kc = int(r.integers(1, 5)), int(r.choice([1, 3, 8, 17, 32, 48])), int(r.choice([1, 5, 16, 32, 40, 64]))
+        H, W = int(r.integers(3, 40)), int(r.integers(3, 40))
+        if H + 2 * p < d * (k - 1) + 1 or W + 2 * p < d * (k - 1) + 1:
+            continue
+        geo = (B, C, Kc, H, W, k, p, s_, d)
+        x = r.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+        say("conv2d random geometry", geo)
+        oy, ocols = orc.conv2d_fwd(x, w, p, s_, d)
+        y, cols = K.conv2d(dev(x), dev(w), p, s_, d)
+        assert np.array_equal(host(y), oy), geo
+        gy = r.integers(-2, 3, oy.shape).astype(np.float32)
+        assert np.array_equal(host(K.conv2d_filter_grad(cols, dev(gy), w.shape)),
+                              orc.conv2d_filter_grad(ocols, gy, w.shape)), geo
+        ogx = orc.conv2d_transpose(gy, w, p, s_, d)
+        gx = host(K.conv2d_transpose(dev(gy), dev(w), p, s_, d))
+        assert gx.shape == ogx.shape and np.array_equal(gx, ogx), geo
+        ran += 1
+    assert ran >= 45, ran
+
+
 def test_conv2d_all_ones_closed_form(K):
     """Ones input and ones filter: y = C * (number of in-bounds taps); exact integers in f32."""
     B, C, Kc, H = 2, 64, 128, 56
@@ -1400,6 +1432,30 @@ def test_reduce_sum_and_mean(K, orc, rng, axes, keep):
         assert_close_conditioned(got, truth, cond, "reduce")
         # short axes are folded sequentially, in the reference's order => same bits as the f32 oracle
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_reduce_random_shapes_and_axes_exact_on_small_integers(K):
+    # a fixed random sample of ranks 1 to 4, extents on both sides of the vector and wave widths, any subset of axes
+    # (none included), keep_dims either way: integer data, so sums are exact and must equal numpy's; means are that
+    # sum times one rounding of the division
+    r = np.random.default_rng(20241119)
+    for _ in range(80):
+        rank = int(r.integers(1, 5))
+        shape = tuple(int(r.choice([1, 2, 3, 5, 8, 17, 32, 33, 64, 100, 257])) for _ in range(rank))
+        if np.prod(shape) > 2e7:
+            continue
+        axes = sorted(r.choice(rank, int(r.integers(0, rank + 1)), replace=False).tolist())
+        keep, mean = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        x = r.integers(-4, 5, shape).astype(np.float32)
+        say("reduce random shape", shape, axes, keep, mean)
+        got = host(K.reduce_sum(dev(x), axes, keep, mean))
+        want = x.astype(np.float64).sum(axis=tuple(axes), keepdims=keep) if axes else x.astype(np.float64)
+        assert got.shape == want.shape, (shape, axes, keep)
+        if mean:
+            count = np.float32(np.prod([shape[a] for a in axes])) if axes else np.float32(1)
+            np.testing.assert_allclose(got, want.astype(np.float32) / count, rtol=2e-7, atol=0)
+        else:
+            assert np.array_equal(got, want.astype(np.float32)), (shape, axes, keep)
 
 
 def test_reduce_mean_config2_loss_shape(K, orc, rng):
