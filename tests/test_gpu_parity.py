@@ -1755,6 +1755,35 @@ def test_sparse_softmax_cross_entropy(K, orc, rng):
         K.sparse_softmax_cross_entropy(dev(logits.reshape(-1)), dev(labels))
 
 
+def test_empty_operands_give_empty_or_zero_results(K):
+    # extents of zero anywhere (no images, no filters, no rows, an empty contraction or reduction): every operator
+    # returns the empty result, or the zeros that an empty sum is (ndarray's behaviour for the reference), and
+    # launches nothing that could read or write
+    z = lambda *s: torch.zeros(*s, device="cuda")
+    o = lambda *s: torch.ones(*s, device="cuda")
+    say("empty operands")
+    assert tuple(K.matmul(z(0, 5), o(5, 3)).shape) == (0, 3)
+    assert tuple(K.matmul(o(4, 5), z(5, 0)).shape) == (4, 0)
+    assert np.array_equal(host(K.matmul(z(4, 0), z(0, 3))), np.zeros((4, 3), np.float32))
+    assert tuple(K.batch_matmul(z(0, 4, 5), z(0, 5, 3)).shape) == (0, 4, 3)
+    assert tuple(K.conv2d(z(0, 3, 8, 8), o(4, 3, 3, 3), 1, 1, 1)[0].shape) == (0, 4, 8, 8)
+    assert tuple(K.conv2d(o(2, 3, 8, 8), z(0, 3, 3, 3), 1, 1, 1)[0].shape) == (2, 0, 8, 8)
+    assert K.conv2d_nocols(z(0, 32, 8, 8), o(32, 32, 3, 3), 1, 1, 1) is None
+    assert tuple(K.conv2d_transpose(z(0, 4, 8, 8), o(4, 3, 3, 3), 1, 1, 1).shape) == (0, 3, 8, 8)
+    assert tuple(K.max_pool2d(z(0, 3, 8, 8), 2, 0, 2)[0].shape) == (0, 3, 4, 4)
+    assert tuple(K.max_pool2d(z(2, 0, 8, 8), 2, 0, 2)[0].shape) == (2, 0, 4, 4)
+    assert np.array_equal(host(K.reduce_sum(z(3, 0, 4), [1])), np.zeros((3, 4), np.float32))
+    assert tuple(K.reduce_sum(z(3, 0, 4), [0]).shape) == (0, 4)
+    assert float(K.sum_all(z(0))) == 0.0
+    assert tuple(K.relu(z(0)).shape) == (0,)
+    assert tuple(K.add_n([z(0), z(0)]).shape) == (0,)
+    assert tuple(K.sparse_softmax_cross_entropy(z(0, 10), z(0))[0].shape) == (0, 1)
+    t = o(1)
+    K.adam_update(z(0), z(0), z(0), z(0), t)
+    torch.cuda.synchronize()
+    assert float(t) == 2.0
+
+
 # =============================================================================== end-to-end config 1
 def test_config1_conv_block_forward_backward(K, orc, rng):
     """conv(1->32, 3x3, pad 1) -> ReLU -> max_pool 2x2/2 -> sum; grads w.r.t. x and w."""
