@@ -247,3 +247,27 @@ def test_conv_batch_whose_columns_exceed_2_pow_31_elements(K):
     assert torch.equal(staged[0], gx_cols)
     del staged, gx_cols, gy, x
     torch.cuda.empty_cache()
+
+
+def test_max_pool_over_more_than_2_pow_31_elements(K):
+    # [1500, 128, 112, 112] = 2.4e9 elements, 2 x 2 windows that do not overlap (every input element receives at most
+    # one gradient, so no summation order is involved): values and backward bit for bit against torch's own pooling
+    # with its int64 indices, which shares nothing with the kernels here
+    import torch.nn.functional as F
+    B, C, H, W = 1500, 128, 112, 112
+    assert B * C * H * W > 2**31
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    x = torch.randn(B, C, H, W, device="cuda", generator=gen)
+    say("max_pool over 2.4e9 elements: forward")
+    y, am, taps = K.max_pool2d(x, 2, 0, 2)
+    ty, tidx = F.max_pool2d(x, 2, 2, return_indices=True)
+    assert torch.equal(y, ty)
+    del ty
+    gy = torch.randn(tuple(y.shape), device="cuda", generator=gen)
+    say("max_pool over 2.4e9 elements: backward")
+    gx = K.max_pool2d_grad(gy, am, taps, tuple(x.shape), 2, 0, 2)
+    want = torch.zeros_like(x).view(B, C, -1).scatter_add_(2, tidx.view(B, C, -1), gy.view(B, C, -1)).view_as(x)
+    assert torch.equal(gx, want)
+    del x, y, am, taps, tidx, gy, gx, want
+    torch.cuda.empty_cache()
