@@ -271,3 +271,26 @@ def test_max_pool_over_more_than_2_pow_31_elements(K):
     assert torch.equal(gx, want)
     del x, y, am, taps, tidx, gy, gx, want
     torch.cuda.empty_cache()
+
+
+def test_reductions_and_elementwise_over_more_than_2_pow_31_elements(K):
+    # [1500, 128, 112, 112] = 2.4e9 small integers: every partial sum stays below 2^24 in magnitude, so the sums are
+    # exact in any order and must equal torch's (f64 where torch's own f32 order could round); the elementwise
+    # kernels must reach the last element
+    B, C, H, W = 1500, 128, 112, 112
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    x = torch.randint(-3, 4, (B, C, H, W), device="cuda", generator=gen).float()
+    say("reductions over 2.4e9 elements")
+    assert torch.equal(K.reduce_sum(x, [2, 3]), x.sum(dim=(2, 3)))
+    assert torch.equal(K.reduce_sum(x, [0]), x.sum(dim=0))
+    assert torch.equal(K.reduce_sum(x, [0, 2, 3]), x.double().sum(dim=(0, 2, 3)).float())
+    assert torch.equal(K.reduce_mean(x, [1], True), x.mean(dim=1, keepdim=True))
+    assert float(K.sum_all(x)) == float(x.double().sum())
+    say("elementwise over 2.4e9 elements")
+    b = torch.randint(-3, 4, (1, C, 1, 1), device="cuda", generator=gen).float()
+    assert torch.equal(K.relu(x), torch.relu(x))
+    assert torch.equal(K.add_broadcast_relu(x, b), torch.relu(x + b))
+    assert torch.equal(K.broadcast_grad(b, tuple(x.shape), [0, 2, 3]), b.expand_as(x))
+    del x
+    torch.cuda.empty_cache()
