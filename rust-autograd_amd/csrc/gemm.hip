@@ -733,6 +733,42 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         return check_launch(who);
     }
     AG_REQUIRE(c.A && c.B, AG_ERR_INVALID_DIMS, "%s: null operand", who);
+    // Tile offsets inside one operand slice are 32-bit.  A single product with an operand of 2^31 elements or more
+    // is cut in two until the pieces fit: along that operand's own rows where they are rows or columns of the
+    // output (two independent products), else along k (the second piece accumulates on top of the first).
+    if (c.kbatch == 1 && partials_only < 0) {
+        const long long lim = 0x7fffffffLL;
+        const long long a_all = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
+        const long long b_all = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
+        if (a_all >= lim || b_all >= lim) {
+            auto half = [](int n) { return n >= 512 ? n / 2 - (n / 2) % 256 : n / 2; };  // keeps tiles and alignment whole
+            GemmCall lo = c, hi = c;
+            bool cut = true;
+            if (a_all >= lim && !c.transA && c.M > 1) {
+                lo.M = half(c.M);
+                hi.M = c.M - lo.M;
+                hi.A = c.A + (long long)lo.M * c.lda;
+                hi.C = c.C + (long long)lo.M * c.ldc;
+            } else if (b_all >= lim && c.transB && c.N > 1) {
+                lo.N = half(c.N);
+                hi.N = c.N - lo.N;
+                hi.B = c.B + (long long)lo.N * c.ldb;
+                hi.C = c.C + lo.N;
+            } else if (c.K > 1) {
+                lo.K = half(c.K);
+                hi.K = c.K - lo.K;
+                hi.beta = 1.f;
+                hi.A = c.A + (c.transA ? (long long)lo.K * c.lda : (long long)lo.K);
+                hi.B = c.B + (c.transB ? (long long)lo.K : (long long)lo.K * c.ldb);
+            } else {
+                cut = false;  // one row or column longer than 2^31: refused below
+            }
+            if (cut) {
+                if (ag_status_t s = run_gemm(st, who, lo, ws, ws_bytes, splits)) return s;
+                return run_gemm(st, who, hi, ws, ws_bytes, splits);
+            }
+        }
+    }
     // A long contraction that misses the direct-to-LDS kernel only because K is not a multiple of
     // its k tile: the whole tiles go there, the remaining K % 32 are accumulated on top by the
     // register-staged kernel (2-3 % of the work).  A single product shorter than 1024 does so only while its

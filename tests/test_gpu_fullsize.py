@@ -294,3 +294,28 @@ def test_reductions_and_elementwise_over_more_than_2_pow_31_elements(K):
     assert torch.equal(K.broadcast_grad(b, tuple(x.shape), [0, 2, 3]), b.expand_as(x))
     del x
     torch.cuda.empty_cache()
+
+
+def test_matmul_with_an_operand_of_more_than_2_pow_31_elements(K):
+    # a [70000, 32768] operand (2.29e9 elements, past the kernels' 32-bit tile offsets) on either side and in either
+    # storage order: the library cuts such a product along the big operand's rows where those are output rows or
+    # columns, else along k.  Small integers, so every result is exact whatever the order of the sums.
+    big, kk, small = 70000, 32768, 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4)
+    X = torch.randint(-2, 3, (big, kk), device="cuda", generator=gen).float()
+    S = torch.randint(-2, 3, (kk, small), device="cuda", generator=gen).float()
+    St = S.t().contiguous()
+    assert X.numel() > 2**31
+    say("matmul, 2.29e9-element A [M,K]: rows cut")
+    assert torch.equal(K.matmul(X, S), X @ S)
+    say("matmul, 2.29e9-element B [N,K] transposed: columns cut")
+    assert torch.equal(K.matmul(St, X, False, True), St @ X.t())
+    Xt = X.t().contiguous()
+    del X
+    say("matmul, 2.29e9-element A [K,M] transposed: k cut")
+    assert torch.equal(K.matmul(Xt, S, True, False), Xt.t() @ S)
+    say("matmul, 2.29e9-element B [K,N]: k cut")
+    assert torch.equal(K.matmul(St, Xt), St @ Xt)
+    del Xt
+    torch.cuda.empty_cache()
