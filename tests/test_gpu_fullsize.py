@@ -319,3 +319,22 @@ def test_matmul_with_an_operand_of_more_than_2_pow_31_elements(K):
     assert torch.equal(K.matmul(St, Xt), St @ Xt)
     del Xt
     torch.cuda.empty_cache()
+
+
+def test_matmul_with_an_output_of_more_than_2_pow_31_elements(K):
+    # [70000, 64] x [64, 32768]: 2.29e9 output elements through the direct-to-LDS kernel (k = 64) and, with k = 40,
+    # through the register-staged one; small integers, exact
+    M, N, kk = 70000, 32768, 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    A = torch.randint(-2, 3, (M, kk), device="cuda", generator=gen).float()
+    B = torch.randint(-2, 3, (kk, N), device="cuda", generator=gen).float()
+    ref = A @ B
+    say("matmul with 2.29e9 output elements")
+    assert torch.equal(K.matmul(A, B), ref)
+    assert torch.equal(K.matmul(A.t().contiguous(), B, True, False), ref)
+    del ref
+    say("matmul with 2.29e9 output elements, k = 40")
+    assert torch.equal(K.matmul(A[:, :40].contiguous(), B[:40].contiguous()), A[:, :40] @ B[:40])
+    del A, B
+    torch.cuda.empty_cache()
