@@ -218,31 +218,33 @@ def test_config5_transposed_conv_32_images(K, orc):
                        ref32=orc.conv2d_transpose_filter_grad(x, gy, w.shape, pad, stride, 1))
 
 
-def test_conv_batch_whose_columns_exceed_2_pow_31_elements(K):
-    # B = 1200 images of the headline shape: 2.17e9 column elements (8.7 GB), past what a 32-bit element index
-    # reaches.  Small integers, generated on the device: the column path and the column-free path, which share no
-    # indexing code, must agree bit for bit on y, gw and gx; the magnitudes say the sums are not trivially zero.
-    B, C, Kf, H, k, p = 1200, 64, 128, 56, 3, 1
-    assert B * C * k * k * H * H > 2**31
+@pytest.mark.parametrize("stride,B", [(1, 1200), (2, 4800)])
+def test_conv_batch_whose_columns_exceed_2_pow_31_elements(K, stride, B):
+    # 1200 images of the headline shape (4800 at stride 2): 2.17e9 column elements (8.7 GB), past what a 32-bit
+    # element index reaches.  Small integers, generated on the device: the column path and the column-free path,
+    # which share no indexing code, must agree bit for bit on y, gw and gx; the magnitudes say the sums are not
+    # trivially zero.
+    C, Kf, H, k, p = 64, 128, 56, 3, 1
+    assert B * C * k * k * (H // stride) ** 2 > 2**31
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
     x = torch.randint(-3, 4, (B, C, H, H), device="cuda", generator=gen).float()
     w = torch.randint(-2, 3, (Kf, C, k, k), device="cuda", generator=gen).float()
     say("conv2d with 2.17e9 column elements: column-free forward")
-    res = K.conv2d_nocols(x, w, p, 1, 1)
+    res = K.conv2d_nocols(x, w, p, stride, 1)
     assert res is not None
     say("conv2d with 2.17e9 column elements: column forward")
-    y, cols = K.conv2d(x, w, p, 1, 1)
+    y, cols = K.conv2d(x, w, p, stride, 1)
     assert torch.equal(y, res[0]) and float(y.abs().max()) > 50
     gy = torch.randint(-2, 3, tuple(y.shape), device="cuda", generator=gen).float()
     del y
     say("conv2d with 2.17e9 column elements: filter gradients")
-    staged = K.conv_input_grad_staged(gy, w, p, (H, H), 1, 1)
-    gw = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), p, 1, 1)
+    staged = K.conv_input_grad_staged(gy, w, p, (H, H), stride, 1)
+    gw = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), p, stride, 1)
     assert torch.equal(gw, K.conv2d_filter_grad(cols, gy, tuple(w.shape))) and float(gw.abs().max()) > 1000
     del cols, res
     say("conv2d with 2.17e9 column elements: input gradients")
-    gx_cols, gcols = K.conv2d_transpose(gy, w, p, 1, 1, out_hw=(H, H), return_cols=True)
+    gx_cols, gcols = K.conv2d_transpose(gy, w, p, stride, 1, out_hw=(H, H), return_cols=True)
     del gcols
     assert torch.equal(staged[0], gx_cols)
     del staged, gx_cols, gy, x
