@@ -681,13 +681,20 @@ struct GemmCall {
     int batch, kbatch;
 };
 
-static bool direct_ok(const GemmCall &c)
+// What the direct-to-LDS kernel asks of the operands' layout (their size apart).
+static bool direct_layout_ok(const GemmCall &c)
 {
     auto mult4 = [](long long v) { return v % 4 == 0; };
     if (c.K % 32 != 0 || !aligned16(c.A) || !aligned16(c.B)) return false;
     if (!mult4(c.lda) || !mult4(c.ldb) || !mult4(c.sA) || !mult4(c.sB) || !mult4(c.sAk) || !mult4(c.sBk)) return false;
     if (c.transA && (c.M % 4 != 0 || c.M < 4)) return false;   // A is m-contiguous
     if (!c.transB && (c.N % 4 != 0 || c.N < 4)) return false;  // B is n-contiguous
+    return true;
+}
+
+static bool direct_ok(const GemmCall &c)
+{
+    if (!direct_layout_ok(c)) return false;
     // byte offsets inside one operand slice are unsigned 32-bit
     const long long a_span = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
     const long long b_span = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
@@ -733,11 +740,14 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
         return check_launch(who);
     }
     AG_REQUIRE(c.A && c.B, AG_ERR_INVALID_DIMS, "%s: null operand", who);
-    // Tile offsets inside one operand slice are 32-bit.  A single product with an operand of 2^31 elements or more
-    // is cut in two until the pieces fit: along that operand's own rows where they are rows or columns of the
-    // output (two independent products), else along k (the second piece accumulates on top of the first).
+    // Tile offsets inside one operand slice are 32-bit: element offsets in the register-staged kernel, byte
+    // offsets in the direct-to-LDS kernel.  A single product with an operand of 2^31 elements or more (2^30 where
+    // the layout suits the direct-to-LDS kernel, so that large products stay on it: 32768^3 is four launches of
+    // 16384 x 32768 x 16384) is cut in two until the pieces fit: along that operand's own rows where they are rows
+    // or columns of the output (two independent products), else along k (the second piece accumulates on top of
+    // the first).
     if (c.kbatch == 1 && partials_only < 0) {
-        const long long lim = 0x7fffffffLL;
+        const long long lim = direct_layout_ok(c) && c.K >= 64 ? (1LL << 30) : 0x7fffffffLL;
         const long long a_all = c.transA ? (long long)(c.K - 1) * c.lda + c.M : (long long)(c.M - 1) * c.lda + c.K;
         const long long b_all = c.transB ? (long long)(c.N - 1) * c.ldb + c.K : (long long)(c.K - 1) * c.ldb + c.N;
         if (a_all >= lim || b_all >= lim) {
