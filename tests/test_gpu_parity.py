@@ -1784,6 +1784,47 @@ def test_empty_operands_give_empty_or_zero_results(K):
     assert float(t) == 2.0
 
 
+def test_calls_from_several_host_threads_on_their_own_streams(K):
+    # the library keeps no state between calls beyond what it reads once about the device: four host threads, each
+    # on a HIP stream of its own, run products, both convolution paths, pooling and reductions at the same time;
+    # small integers, so every result must be exactly torch's (or the other path's)
+    import threading
+    errors = []
+
+    def work(seed):
+        try:
+            stream = torch.cuda.Stream()
+            gen = torch.Generator(device="cuda")
+            gen.manual_seed(seed)
+            with torch.cuda.stream(stream):
+                for it in range(20):
+                    a = torch.randint(-2, 3, (300 + 37 * (it % 5), 520), device="cuda", generator=gen).float()
+                    b = torch.randint(-2, 3, (520, 200 + 64 * (it % 3)), device="cuda", generator=gen).float()
+                    if not torch.equal(K.matmul(a, b), a @ b):
+                        errors.append(("matmul", seed, it))
+                    x = torch.randint(-3, 4, (4, 32, 20, 20), device="cuda", generator=gen).float()
+                    w = torch.randint(-2, 3, (64, 32, 3, 3), device="cuda", generator=gen).float()
+                    y, _ = K.conv2d(x, w, 1, 1, 1)
+                    r = K.conv2d_nocols(x, w, 1, 1, 1)
+                    if r is None or not torch.equal(y, r[0]):
+                        errors.append(("conv2d", seed, it))
+                    if not torch.equal(K.max_pool2d(y, 2, 0, 2)[0], torch.nn.functional.max_pool2d(y, 2, 2)):
+                        errors.append(("max_pool", seed, it))
+                    if not torch.equal(K.reduce_sum(y, [0, 2, 3]), y.sum(dim=(0, 2, 3))):
+                        errors.append(("reduce_sum", seed, it))
+                stream.synchronize()
+        except Exception as e:                       # a failure in a thread must fail the test, not vanish
+            errors.append(("exception", seed, repr(e)[:200]))
+
+    say("four host threads on four streams")
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:5]
+
+
 # =============================================================================== end-to-end config 1
 def test_config1_conv_block_forward_backward(K, orc, rng):
     """conv(1->32, 3x3, pad 1) -> ReLU -> max_pool 2x2/2 -> sum; grads w.r.t. x and w."""
