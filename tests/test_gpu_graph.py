@@ -1004,3 +1004,51 @@ def test_conv2d_column_free_second_order(G, orc, rng):
     want = orc.conv2d_transpose(gyv, rv, 1, 1, 1, out_hw=(H, H)).astype(np.float64) + \
         orc.conv2d_transpose((2 * oyr).astype(np.float32), wv, 1, 1, 1, out_hw=(H, H)).astype(np.float64)
     assert_close(ggxv, want, "ggx", scale=np.abs(want).max())
+
+
+def test_many_steps_with_changing_batch_sizes_do_not_grow_memory(G, rng):
+    # the evaluator's arena and the staging ring are reused from step to step: after a warm-up that has seen every
+    # batch size, hundreds of further training steps of the small CNN (graph rebuilt and fed every step, Adam
+    # update, batch size changing from step to step) leave the device's used memory and the process's peak host
+    # memory where they were
+    import resource
+
+    import torch
+    env = G.VariableEnvironment()
+    params = {"w1": glorot(rng, (32, 1, 3, 3)), "w2": glorot(rng, (64, 32, 3, 3)),
+              "w3": rng.uniform(-0.04, 0.04, (3136, 10)).astype(np.float32),
+              "b1": np.zeros((1, 32, 28, 28), np.float32), "b2": np.zeros((1, 64, 14, 14), np.float32),
+              "b3": np.zeros((1, 10), np.float32)}
+    ids = {k: env.set(k, a) for k, a in params.items()}
+    names = list(params)
+    adam = G.Adam(env, [ids[k] for k in names], alpha=1e-3)
+    sizes = [128, 64, 100, 128, 32]
+
+    def step(bs):
+        c = env.context()
+        v = {k: c.variable(ids[k]) for k in names}
+        x, t = c.placeholder("x", [-1, 1, 28, 28]), c.placeholder("y", [-1, 1])
+        z = c.max_pool2d(c.relu(c.conv2d(x, v["w1"], 1, 1) + v["b1"]), 2, 0, 2)
+        z = c.max_pool2d(c.relu(c.conv2d(z, v["w2"], 1, 1) + v["b2"]), 2, 0, 2)
+        logits = c.matmul(c.reshape(z, [-1, 3136]), v["w3"]) + v["b3"]
+        loss = c.reduce_mean(c.sparse_softmax_cross_entropy(logits, t), [0], False)
+        grads = c.grad([loss], [v[k] for k in names])
+        adam.update([v[k] for k in names], grads, c,
+                    {"x": rng.random((bs, 1, 28, 28), dtype=np.float32),
+                     "y": rng.integers(0, 10, (bs, 1)).astype(np.float32)})
+
+    def used():
+        G.synchronize()
+        free, total = torch.cuda.mem_get_info()
+        return total - free, resource.getrusage(resource.RUSAGE_SELF).ru_maxrss
+
+    say("memory over many steps: warm-up")
+    for i in range(40):
+        step(sizes[i % 5])
+    dev0, host0 = used()
+    say("memory over many steps: 400 steps")
+    for i in range(400):
+        step(sizes[i % 5])
+    dev1, host1 = used()
+    assert dev1 - dev0 <= 8 << 20, (dev0, dev1)          # bytes; other tests' torch tensors may be freed meanwhile
+    assert host1 - host0 <= 16 << 10, (host0, host1)     # KiB
