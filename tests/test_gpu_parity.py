@@ -476,6 +476,35 @@ def test_matmul_and_batch_matmul_random_shapes_exact_on_small_integers(K):
         assert np.array_equal(got, want), (m, n, k, ta, tb, batch)
 
 
+def test_matmul_keeps_a_nan_or_an_infinity_in_its_row_or_column(K):
+    # one NaN or one infinity in one operand (positive data otherwise, so that no inf - inf arises): the result has
+    # NaN / inf in exactly the row or column that numpy's product has, whichever tiles, splits of the contraction
+    # or tail passes ran and whatever the loads past the end of a block's stream re-read
+    r = np.random.default_rng(20241123)
+    dims = [1, 3, 31, 32, 64, 65, 100, 128, 200, 256, 257, 512, 520, 1000, 1024, 3136]
+    for _ in range(50):
+        m, n, k = (int(r.choice(dims)) for _ in range(3))
+        ta, tb = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        batch = int(r.choice([0, 0, 3]))
+        sa = (k, m) if ta else (m, k)
+        sb = (n, k) if tb else (k, n)
+        if batch:
+            sa, sb = (batch,) + sa, (batch,) + sb
+        a = r.integers(1, 3, sa).astype(np.float32)
+        b = r.integers(1, 3, sb).astype(np.float32)
+        which = int(r.integers(0, 4))
+        target = a if which < 2 else b
+        idx = tuple(int(r.integers(0, s_)) for s_ in target.shape)
+        target[idx] = np.nan if which % 2 == 0 else np.inf
+        say("matmul with a NaN / inf", (m, n, k, ta, tb, batch, which, idx))
+        got = host((K.batch_matmul if batch else K.matmul)(dev(a), dev(b), ta, tb))
+        a2 = np.swapaxes(a, -1, -2) if ta else a
+        b2 = np.swapaxes(b, -1, -2) if tb else b
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = np.matmul(a2.astype(np.float64), b2.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(got, want, equal_nan=True), (m, n, k, ta, tb, batch, which, idx)
+
+
 def test_gemm_degenerate_k_and_beta(K, rng):
     c0 = rng.random((5, 6), dtype=np.float32)
     c = dev(c0)
