@@ -1229,6 +1229,35 @@ def test_conv2d_transpose_and_filter_grad(K, orc, rng, case):
     assert_close_conditioned(host(gw), g64, gabs, "conv2d_transpose filter grad")
 
 
+def test_conv2d_transpose_and_its_filter_grad_random_geometries_exact(K, orc):
+    # the transposed convolution with an explicit output extent (the reconstructed one, or one of the up to
+    # stride - 1 larger extents that map back onto the same input) and its filter gradient over a fixed random
+    # sample of filters, strides, dilations, paddings and channel counts: small integers, bit for bit the CPU
+    # restatement
+    r = np.random.default_rng(20241124)
+    ran = 0
+    for _ in range(70):
+        k, s_, d = int(r.choice([1, 2, 3, 4, 5])), int(r.choice([1, 1, 2, 3])), int(r.choice([1, 1, 2]))
+        p = int(r.integers(0, 3))
+        B, ych, xch = int(r.integers(1, 5)), int(r.choice([1, 3, 8, 32, 64])), int(r.choice([1, 5, 16, 32, 64]))
+        yh, yw = int(r.integers(2, 24)), int(r.integers(2, 24))
+        xh = orc.conv_transpose_out_size(yh, k, p, s_, d) + int(r.integers(0, s_))
+        xw = orc.conv_transpose_out_size(yw, k, p, s_, d) + int(r.integers(0, s_))
+        if xh < 1 or xw < 1 or orc.conv_out_size(xh, k, p, s_, d) != yh or orc.conv_out_size(xw, k, p, s_, d) != yw:
+            continue
+        geo = (B, ych, xch, yh, yw, xh, xw, k, p, s_, d)
+        t_in = r.integers(-2, 3, (B, ych, yh, yw)).astype(np.float32)      # input of the transposed convolution
+        w = r.integers(-2, 3, (ych, xch, k, k)).astype(np.float32)
+        g_out = r.integers(-3, 4, (B, xch, xh, xw)).astype(np.float32)     # gradient of its output
+        say("conv2d_transpose random geometry", geo)
+        assert np.array_equal(host(K.conv2d_transpose(dev(t_in), dev(w), p, s_, d, out_hw=(xh, xw))),
+                              orc.conv2d_transpose(t_in, w, p, s_, d, out_hw=(xh, xw))), geo
+        assert np.array_equal(host(K.conv2d_transpose_filter_grad(dev(t_in), dev(g_out), w.shape, p, s_, d)),
+                              orc.conv2d_transpose_filter_grad(t_in, g_out, w.shape, p, s_, d)), geo
+        ran += 1
+    assert ran >= 40, ran
+
+
 def test_conv2d_errors_follow_reference(K):
     x = torch.zeros(1, 3, 8, 8, device="cuda")
     with pytest.raises(K.capi.IncompatibleShape, match=r"conv2d: filter must be 4D"):
