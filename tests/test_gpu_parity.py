@@ -1699,6 +1699,23 @@ def test_add_and_relu_in_one_pass_has_the_bits_of_the_two_operations(K, rng, sha
     assert np.array_equal(fused, want)
 
 
+def test_add_broadcast_and_its_gradient_random_shapes_exact(K):
+    # ranks 1 to 4, any subset of axes of the second operand of extent 1: the sum, the sum with the ReLU folded in and
+    # the broadcast that is the gradient's other half, on small integers against numpy's broadcasting
+    r = np.random.default_rng(20241125)
+    for _ in range(80):
+        rank = int(r.integers(1, 5))
+        shape = tuple(int(r.choice([1, 2, 3, 4, 7, 16, 33, 64, 100])) for _ in range(rank))
+        bshape = tuple(1 if r.integers(0, 2) else s_ for s_ in shape)
+        x = r.integers(-4, 5, shape).astype(np.float32)
+        b = r.integers(-4, 5, bshape).astype(np.float32)
+        say("add with broadcast, random shape", shape, bshape)
+        assert np.array_equal(host(K.add_broadcast(dev(x), dev(b))), x + b), (shape, bshape)
+        assert np.array_equal(host(K.add_broadcast_relu(dev(x), dev(b))), np.maximum(x + b, 0)), (shape, bshape)
+        unit = [i for i, t in enumerate(bshape) if t == 1]
+        assert np.array_equal(host(K.broadcast_grad(dev(b), shape, unit)), np.broadcast_to(b, shape)), (shape, bshape)
+
+
 def test_add_broadcast_rejects_other_extents(K, rng):
     from rust_autograd_amd import capi
     x, b = dev(np.zeros((4, 3), np.float32)), dev(np.zeros((2, 3), np.float32))
