@@ -731,6 +731,53 @@ def test_conv2d_column_free_random_dilations_paddings_and_batches_exact(K):
     assert min(ran) >= 40, ran
 
 
+def test_conv2d_column_free_random_geometries_gaussian_data_within_the_contraction_bar(K):
+    # Gaussian data over a fixed random sample of column-free geometries (stride 1 with dilation, stride 2, batches up
+    # to 200, so that tiles, splits and position chunks of every kind run): y, gx and gw against torch's f64
+    # convolutions, every element within 2e-6 of the contraction of the absolute values (about 32 f32 roundoffs of
+    # the quantity that rounding errors scale with; the worst seen is 5e-7)
+    import torch.nn.functional as F
+    r = np.random.default_rng(20241126)
+    L = K.capi.lib()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    ran = 0
+    for _ in range(40):
+        s_, k = int(r.choice([1, 1, 2])), int(r.choice([3, 3, 5]))
+        d = 1 if s_ == 2 else int(r.choice([1, 1, 2]))
+        reach = d * (k - 1)
+        p = int(r.integers(0, (k if s_ == 2 else reach + 1)))
+        B, C, Kc = int(r.choice([1, 4, 16, 64, 200])), int(r.choice([32, 64, 128])), int(r.choice([32, 64, 128, 192]))
+        lo = max(reach + 1, 20 if s_ == 2 else 7)
+        H, W = int(r.integers(lo, 60)), int(r.integers(lo, 60))
+        while B * max(C, Kc) * H * W > 2e7:
+            B = max(B // 2, 1)
+        geo = (B, C, Kc, H, W, k, p, s_, d)
+        x = torch.randn(B, C, H, W, device="cuda", generator=gen)
+        w = torch.randn(Kc, C, k, k, device="cuda", generator=gen) * 0.1
+        say("column-free random geometry, gaussian data", geo)
+        res = K.conv2d_nocols(x, w, p, s_, d)
+        if res is None:
+            continue
+        gy = torch.randn(tuple(res[0].shape), device="cuda", generator=gen)
+        staged = K.conv_input_grad_staged(gy, w, p, (H, W), s_, d)
+        if staged is None:
+            continue
+        ran += 1
+        xd, wd, gd = x.double(), w.double(), gy.double()
+
+        def worst(got, truth, scale):
+            return float(((got.double() - truth).abs() / scale.clamp_min(1e-30)).max())
+        assert worst(res[0], F.conv2d(xd, wd, None, s_, p, d), F.conv2d(xd.abs(), wd.abs(), None, s_, p, d)) <= 2e-6, geo
+        assert worst(staged[0], torch.nn.grad.conv2d_input(x.shape, wd, gd, s_, p, d),
+                     torch.nn.grad.conv2d_input(x.shape, wd.abs(), gd.abs(), s_, p, d)) <= 2e-6, geo
+        if L.ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, Kc, k, k, p, s_, d) > 0:
+            gw = K.conv2d_filter_grad_nocols(res[1], staged[1], tuple(x.shape), tuple(w.shape), p, s_, d)
+            assert worst(gw, torch.nn.grad.conv2d_weight(xd, w.shape, gd, s_, p, d),
+                         torch.nn.grad.conv2d_weight(xd.abs(), w.shape, gd.abs(), s_, p, d)) <= 2e-6, geo
+    assert ran >= 30, ran
+
+
 DILATED_NOCOLS_CASES = [  # B, C, K, H, W, k, pad, dilation
     (2, 64, 64, 28, 28, 3, 2, 2),    # the dilated configuration, 2 of its images: a "same" convolution
     (3, 32, 64, 20, 22, 3, 2, 2),    # uneven extents
