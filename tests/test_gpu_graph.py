@@ -1052,3 +1052,35 @@ def test_many_steps_with_changing_batch_sizes_do_not_grow_memory(G, rng):
     dev1, host1 = used()
     assert dev1 - dev0 <= 8 << 20, (dev0, dev1)          # bytes; other tests' torch tensors may be freed meanwhile
     assert host1 - host0 <= 16 << 10, (host0, host1)     # KiB
+
+
+def test_conv2d_and_gradients_through_the_graph_random_geometries_exact(G, orc):
+    # Conv2D with any stride, dilation and padding, channel counts on both sides of what the column-free paths take
+    # and batches on both sides of the operator's size switch: y, gx and gw through the graph (whichever path the
+    # operator picks) against the CPU restatement, small integers, bit for bit
+    r = np.random.default_rng(20241127)
+    for _ in range(40):
+        s_, k, d = int(r.choice([1, 1, 2])), int(r.choice([2, 3, 3, 5])), int(r.choice([1, 1, 2]))
+        reach = d * (k - 1)
+        p = int(r.integers(0, reach + 1))
+        B, C, Kc = int(r.choice([1, 3, 8, 40, 150])), int(r.choice([3, 32, 64, 96])), int(r.choice([8, 32, 64, 160]))
+        H, W = int(r.integers(max(reach + 1, 6), 50)), int(r.integers(max(reach + 1, 6), 50))
+        while B * max(C, Kc) * H * W > 8e6:
+            B = max(B // 2, 1)
+        geo = (B, C, Kc, H, W, k, p, s_, d)
+        x = r.integers(-3, 4, (B, C, H, W)).astype(np.float32)
+        w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+        oy, ocols = orc.conv2d_fwd(x, w, p, s_, d)
+        m = r.integers(-2, 3, oy.shape).astype(np.float32)
+        say(f"conv2d through the graph, random geometry {geo}")
+        env = G.VariableEnvironment()
+        wid = env.set("w", w)
+        c = env.context()
+        xt, wt = c.placeholder("x", [-1, C, H, W]), c.variable(wid)
+        mt = c.placeholder("m", [-1] + list(oy.shape[1:]))
+        y = c.dilated_conv2d(xt, wt, p, s_, d)
+        gx, gw = c.grad([c.sum_all(c.mul(y, mt))], [xt, wt])
+        vy, vgx, vgw = c.eval([y, gx, gw], {"x": x, "m": m})
+        assert np.array_equal(vy, oy), geo
+        assert np.array_equal(vgx, orc.conv2d_transpose(m, w, p, s_, d, out_hw=(H, W))), geo
+        assert np.array_equal(vgw, orc.conv2d_filter_grad(ocols, m, w.shape)), geo
