@@ -150,6 +150,37 @@ __global__ __launch_bounds__(256) void maxpool_bwd_tile2_kernel(const float *__r
     *reinterpret_cast<float2 *>(row + g.W) = bottom;
 }
 
+// Forward of 2 x 2 windows at stride 2 over a plane with even extents, one thread per window: two 8-byte loads (a
+// wave's loads cover two whole input rows of contiguous memory), the scan in the reference's order (first maximum
+// wins, strict comparison starting from -FLT_MAX), three coalesced stores.  No staging and no barrier: on the small
+// planes of a launch-bound network ([128,32,28,28]: 8.2 -> about 5 us) that is what the time went to.
+__global__ __launch_bounds__(256) void maxpool_fwd_tile2_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                float *__restrict__ argmax, uint8_t *__restrict__ taps,
+                                                                PoolGeom g, long long outputs)
+{
+    const long long o = blockIdx.x * 256ll + threadIdx.x;
+    if (o >= outputs) return;
+    const int per_plane = g.OH * g.OW;
+    const long long plane = o / per_plane;
+    const int e = (int)(o - plane * per_plane);
+    const int oy = e / g.OW, ox = e - oy * g.OW;
+    const long long at = plane * (long long)g.H * g.W + (long long)(2 * oy) * g.W + 2 * ox;  // whole-tensor offset of tap 0
+    const float2 top = *reinterpret_cast<const float2 *>(x + at), bottom = *reinterpret_cast<const float2 *>(x + at + g.W);
+    const float v[4] = {top.x, top.y, bottom.x, bottom.y};
+    float best = -FLT_MAX;
+    int best_tap = kNoTap;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const bool gt = v[t] > best;
+        best = gt ? v[t] : best;
+        best_tap = gt ? t : best_tap;
+    }
+    const long long flat = at + (best_tap >> 1) * g.W + (best_tap & 1);
+    y[o] = best;
+    argmax[o] = best_tap != kNoTap ? (float)(unsigned long long)flat : 0.f;  // the offset by value, rounded to nearest even
+    if (taps) taps[o] = (uint8_t)best_tap;
+}
+
 constexpr int kPoolLdsBytes = 32 * 1024;
 // A plane that does not fit half of that is cut into bands of at most this many staged bytes:
 // eight resident blocks per CU measured better than fewer, larger ones (112x112 planes: 0.242 ms
@@ -568,7 +599,12 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
                "max_pool2d: a tap byte addresses windows of up to %d x %d (got %d)", kMaxTapSize, kMaxTapSize, size);
     if (g.OH <= 0 || g.OW <= 0) return AG_OK;
     const long long row_bytes = (long long)W * 4;
-    if (row_bytes * size <= kPoolLdsBytes) {
+    if (size == 2 && stride == 2 && H % 2 == 0 && W % 2 == 0 && ((uintptr_t)x & 7u) == 0) {
+        const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
+        AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
+        hipLaunchKernelGGL(maxpool_fwd_tile2_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), x, y, argmax,
+                           taps, g, outputs);
+    } else if (row_bytes * size <= kPoolLdsBytes) {
         // rows of output per band so that the staged input rows fit the LDS budget
         const long long budget = (long long)H * row_bytes <= kPoolLdsBytes / 2 || row_bytes * size > kPoolBandBytes
                                      ? kPoolLdsBytes : kPoolBandBytes;
@@ -612,7 +648,10 @@ static ag_status_t maxpool2d_bwd(ag_stream_t stream, const float *gy, const floa
     AG_REQUIRE(taps || (long long)B * C * H * W <= kExactFloatIndexLimit, AG_ERR_INVALID_DIMS,
                "max_pool2d_grad: an f32 cannot hold offsets into %lld elements exactly (> 2^24); pass the tap bytes",
                (long long)B * C * H * W);
-    if (size == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && W % 4 != 0 && (reinterpret_cast<uintptr_t>(gx) & 7) == 0 &&
+    // (rows of whole quads go to the register kernel below, whose 16-byte stores are worth more on large tensors;
+    // up to 2^23 elements its set-up is what counts: [128,32,28,28] 10.0 us there, 5 us here)
+    const bool small_tensor = (long long)B * C * H * W <= (1LL << 23);
+    if (size == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && (W % 4 != 0 || small_tensor) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0 &&
         (reinterpret_cast<uintptr_t>(relu_x) & 7) == 0 && g.OH > 0 && g.OW > 0) {
         const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);
