@@ -19,7 +19,8 @@ void ag_test_gemm_force_splits(int splits);
 void ag_test_gemm_force_grid(int blocks_per_cu);
 /* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): it may take the implicit GEMM. */
 void ag_test_conv_fused_input_grad(int on);
-/* Output rows per chunk of the stride-2 pooling kernels (0 = automatic). */
+/* Output rows per chunk of the stride-2 pooling kernels (0 = automatic); a negative value instead keeps 2 x 2
+   windows off the one-thread-per-window kernels, so that the staged and register kernels see those geometries too. */
 void ag_test_pool_chunk_rows(int rows);
 
 #if defined(__GNUC__)

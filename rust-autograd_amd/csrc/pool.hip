@@ -153,7 +153,8 @@ __global__ __launch_bounds__(256) void maxpool_bwd_tile2_kernel(const float *__r
 // Forward of 2 x 2 windows at stride 2 over a plane with even extents, one thread per window: two 8-byte loads (a
 // wave's loads cover two whole input rows of contiguous memory), the scan in the reference's order (first maximum
 // wins, strict comparison starting from -FLT_MAX), three coalesced stores.  No staging and no barrier: on the small
-// planes of a launch-bound network ([128,32,28,28]: 8.2 -> about 5 us) that is what the time went to.
+// planes of a launch-bound network ([128,32,28,28]: 8.2 -> about 5 us) that is what the time went to.  Large tensors
+// with rows of whole quads stay on the staged kernel.
 __global__ __launch_bounds__(256) void maxpool_fwd_tile2_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                                 float *__restrict__ argmax, uint8_t *__restrict__ taps,
                                                                 PoolGeom g, long long outputs)
@@ -584,7 +585,8 @@ constexpr long long kExactFloatIndexLimit = 1LL << 24;
 using namespace ag;
 
 // Test hook (ag_test_hooks.h; not part of the operator surface): output rows per chunk of the
-// stride-2 pooling kernels for later calls of this thread (0 = automatic).
+// stride-2 pooling kernels for later calls of this thread (0 = automatic; negative: automatic, and 2 x 2 windows
+// stay off the one-thread-per-window kernels where another kernel can take them).
 extern "C" void ag_test_pool_chunk_rows(int rows) { ag::g_chunk_rows = rows; }
 
 extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, float *y,
@@ -599,7 +601,10 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
                "max_pool2d: a tap byte addresses windows of up to %d x %d (got %d)", kMaxTapSize, kMaxTapSize, size);
     if (g.OH <= 0 || g.OW <= 0) return AG_OK;
     const long long row_bytes = (long long)W * 4;
-    if (size == 2 && stride == 2 && H % 2 == 0 && W % 2 == 0 && ((uintptr_t)x & 7u) == 0) {
+    // (up to 2^23 elements, where a launch's set-up counts, and for rows that are no whole quads; beyond that the
+    // staged kernel's 16-byte loads win: [256,128,112,112] 0.41 against 0.44 ms)
+    const bool tile2 = W % 4 != 0 || ((long long)B * C * H * W <= (1LL << 23) && g_chunk_rows >= 0);
+    if (size == 2 && stride == 2 && H % 2 == 0 && W % 2 == 0 && ((uintptr_t)x & 7u) == 0 && tile2) {
         const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d: too many tiles (%lld)", blocks);
         hipLaunchKernelGGL(maxpool_fwd_tile2_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), x, y, argmax,
@@ -651,7 +656,7 @@ static ag_status_t maxpool2d_bwd(ag_stream_t stream, const float *gy, const floa
     // (rows of whole quads go to the register kernel below, whose 16-byte stores are worth more on large tensors;
     // up to 2^23 elements its set-up is what counts: [128,32,28,28] 10.0 us there, 5 us here)
     const bool small_tensor = (long long)B * C * H * W <= (1LL << 23);
-    if (size == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && (W % 4 != 0 || small_tensor) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0 &&
+    if (size == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && (W % 4 != 0 || (small_tensor && g_chunk_rows >= 0)) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0 &&
         (reinterpret_cast<uintptr_t>(relu_x) & 7) == 0 && g.OH > 0 && g.OW > 0) {
         const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
         AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "max_pool2d_grad: too many tiles (%lld)", blocks);

@@ -1417,6 +1417,33 @@ def test_max_pool_random_geometries_with_ties_bit_exact(K, orc):
             assert np.array_equal(host(K.max_pool2d_grad_grad(dev(ggx), am, idx, size, 0, stride)), oggy), case
 
 
+@pytest.mark.parametrize("shape", [(3, 5, 28, 28), (2, 4, 14, 16), (1, 3, 8, 4), (2, 2, 56, 64), (1, 2, 2, 2)])
+def test_max_pool_2x2_tiling_kernels_have_the_bits_of_the_staged_and_register_kernels(K, rng, shape):
+    # 2 x 2 windows at stride 2 over even planes of a small tensor run one thread per window; the test hook keeps
+    # them off those kernels, so the same geometry also goes through the staged forward and the register / staged
+    # backward: values, argmax, tap bytes, both backward forms and the backward with the ReLU gradient must not
+    # differ in a bit (ties included)
+    L = K.capi.lib()
+    x = (rng.integers(0, 5, shape) / np.float32(3)).astype(np.float32)
+    relu_x = rng.standard_normal(shape).astype(np.float32)
+    gy = rng.standard_normal((shape[0], shape[1], shape[2] // 2, shape[3] // 2)).astype(np.float32)
+    results = []
+    for hook in (0, -1):
+        L.ag_test_pool_chunk_rows(hook)
+        try:
+            say("max_pool 2x2 tiling, hook", hook, shape)
+            y, am, tp = K.max_pool2d(dev(x), 2, 0, 2)
+            outs = [host(y), host(am), host(tp)]
+            for idx in (None, tp):
+                outs.append(host(K.max_pool2d_grad(dev(gy), am, idx, shape, 2, 0, 2)))
+                outs.append(host(K.max_pool2d_grad_relu(dev(gy), am, idx, dev(relu_x), 2, 0, 2)))
+        finally:
+            L.ag_test_pool_chunk_rows(0)
+        results.append(outs)
+    for a, b in zip(*results):
+        assert a.shape == b.shape and a.tobytes() == b.tobytes()
+
+
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 1000])
 def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows):
     """The stride-2 backward walks chunks of output rows; whatever their length (one row, odd
