@@ -127,10 +127,12 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
     ap.add_argument("--cpu-images", type=int, default=B, help="images per step of the CPU baseline (default: the whole batch)")
-    ap.add_argument("--only", choices=("pool", "columns", "config1", "config2"),
+    ap.add_argument("--only", choices=("pool", "columns", "config1", "config2", "stride2", "config5", "config3", "reduce", "adam",
+                                       "elementwise"),
                     help="run only one part of the per-kernel section (for profiler passes): the two pooling kernels, "
-                         "the column-materialising convolution kernels, or the steps of configuration 1 / 2 "
-                         "through the host operator layer")
+                         "the column-materialising convolution kernels, the steps of configuration 1 / 2 through the host "
+                         "operator layer, the stride-2 variant of the headline, the dilated and transposed convolutions of "
+                         "configuration 5, the dense products of configuration 3, the reductions, Adam, or the elementwise glue")
     ap.add_argument("--no-traffic", action="store_true",
                     help="leave the HBM-traffic fields out (for the profiler passes that produce the summaries those "
                          "fields are read from)")
@@ -267,6 +269,16 @@ def main():
             res = micro_pool(torch, Kn, capi, dev, g, iters=3, only=True)
         elif args.only == "columns":
             res = micro_columns(torch, Kn, capi, dev, g, iters=3)
+        elif args.only in ("stride2", "config5"):
+            res = other_conv_configs(torch, Kn, dev, g, which=args.only)
+        elif args.only == "config3":
+            res = micro_matmul(torch, Kn, dev, g)
+        elif args.only == "reduce":
+            res = micro_reduce(torch, Kn, dev, g, iters=3)
+        elif args.only == "adam":
+            res = micro_adam(torch, Kn, dev, g, iters=3)
+        elif args.only == "elementwise":
+            res = micro_elementwise(torch, Kn, dev, g, iters=3)
         else:
             res = graph_steps(which=args.only)
         if args.pmc_calibration:
@@ -480,7 +492,6 @@ def micro_columns(torch, Kn, capi, dev, g, iters=10):
 
 def micro_rest(torch, Kn, capi, dev, g, iters=10):
     res = {}
-    Bn, Kf, Hh = 256, 128, 56
     # a plain copy (ag_scale_f32 by 1.0) of 2^28 floats: what a streaming kernel with one read and one write stream reaches
     src = torch.ones(1 << 28, device=dev)
     dst = torch.empty_like(src)
@@ -488,38 +499,88 @@ def micro_rest(torch, Kn, capi, dev, g, iters=10):
     res["copy_2^28"] = {"ms": round(ms, 4), "GB/s": round(8.0 * src.numel() / ms / 1e6, 1),
                         "frac_hbm": round(8.0 * src.numel() / ms / 1e6 / HBM_PEAK_GBS, 4)}
     del src, dst
-    # reduce_sum (to scalar) and Adam on 2^26 elements
+    res.update(micro_reduce(torch, Kn, dev, g, iters))
+    res.update(micro_adam(torch, Kn, dev, g, iters))
+    res.update(micro_elementwise(torch, Kn, dev, g, iters))
+    res.update(micro_matmul(torch, Kn, dev, g))
+    res.update(other_conv_configs(torch, Kn, dev, g))
+    res.update(graph_steps())
+    return res
+
+
+def hbm_entry(key, ms, nbytes, note=None):
+    """One bandwidth-bound entry: algorithmic bytes over the measured time, plus the counter-derived traffic of the
+    tracked summary where PROFILE_TRAFFIC names the entry."""
+    e = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    if key in PROFILE_TRAFFIC:
+        e.update(traffic_fields(key, ms))
+    if note:
+        e["note"] = note
+    return e
+
+
+def micro_reduce(torch, Kn, dev, g, iters=10):
+    """reduce_sum to a scalar on 2^26 elements and the axis reductions over the pool input's shape [256,128,56,56]:
+    the per-channel (conv bias) gradient, one axis, the rows.  Algorithmic bytes: 4 per input element."""
+    res = {}
     n = 1 << 26
     a = torch.randn(n, device=dev, generator=g)
-    ms = time_events(torch, lambda: Kn.sum_all(a), 10)
-    res["sum_all_2^26"] = {"ms": round(ms, 4), "GB/s": round(4.0 * n / ms / 1e6, 1), "frac_hbm": round(4.0 * n / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    # axis reductions over the pool input's shape: the per-channel (conv bias) gradient, one axis, the rows
-    a4 = torch.randn(Bn, Kf, Hh, Hh, device=dev, generator=g)
+    ms = time_events(torch, lambda: Kn.sum_all(a), iters)
+    res["sum_all_2^26"] = hbm_entry("sum_all_2^26", ms, 4.0 * n)
+    del a
+    a4 = torch.randn(256, 128, 56, 56, device=dev, generator=g)
     for name, axes in (("reduce_sum_[256,128,56,56]_axes_0_2_3", [0, 2, 3]), ("reduce_sum_[256,128,56,56]_axis_0", [0]),
                        ("reduce_mean_[256,128,56,56]_axes_2_3", [2, 3])):
         fn = Kn.reduce_mean if "mean" in name else Kn.reduce_sum
-        ms = time_events(torch, lambda: fn(a4, axes), 10)
-        res[name] = {"ms": round(ms, 4), "GB/s": round(4.0 * a4.numel() / ms / 1e6, 1),
-                     "frac_hbm": round(4.0 * a4.numel() / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    del a4
-    # Adam streams four arrays of one size in lockstep.  hipMalloc (and torch's allocator) hand out addresses with the
-    # same low 21 bits, which sends all four streams to the same DRAM banks at the same time; the host operator
-    # layer's arena therefore staggers its large blocks by multiples of 4 KiB.  Both placements are timed.
+        ms = time_events(torch, lambda: fn(a4, axes), iters)
+        res[name] = hbm_entry(name, ms, 4.0 * a4.numel())
+    return res
+
+
+def micro_adam(torch, Kn, dev, g, iters=10):
+    """The fused Adam update on 2^26 elements (28 bytes per element: p, g, m, v read; p, m, v written), with the four
+    arrays 4 KiB apart modulo 2 MiB (what the host operator layer's arena hands out) and with all four on 2 MiB
+    boundaries (what hipMalloc and torch's allocator hand out)."""
+    res = {}
+    n = 1 << 26
+    a = torch.randn(n, device=dev, generator=g)
     t = torch.ones(1, device=dev)
     for name, step in (("adam_2^26", 1024), ("adam_2^26_operands_2MiB_aligned", 0)):
         bufs = [torch.zeros(n + 3 * step, device=dev) for _ in range(4)]
         ga, p, m, v = (b[i * step:i * step + n] for i, b in enumerate(bufs))
         ga.copy_(a)
         p.normal_(generator=g)
-        ms = time_events(torch, lambda: Kn.adam_update(p, ga, m, v, t), 10)
-        res[name] = {"ms": round(ms, 4), "GB/s": round(28.0 * n / ms / 1e6, 1), "frac_hbm": round(28.0 * n / ms / 1e6 / HBM_PEAK_GBS, 4),
-                     "note": ("param, grad, m, v start 0, 4, 8, 12 KiB past a 2 MiB boundary (the host layer's arena placement)" if step
-                              else "param, grad, m, v all start on a 2 MiB boundary")}
+        ms = time_events(torch, lambda: Kn.adam_update(p, ga, m, v, t), iters)
+        res[name] = hbm_entry(name, ms, 28.0 * n,
+                              "param, grad, m, v start 0, 4, 8, 12 KiB past a 2 MiB boundary (the host layer's arena placement)"
+                              if step else "param, grad, m, v all start on a 2 MiB boundary")
         del bufs, ga, p, m, v
-    p = m = v = None
-    del a, p, m, v
+    return res
 
-    # dense contractions of config 3
+
+def micro_elementwise(torch, Kn, dev, g, iters=10):
+    """The elementwise glue at the headline activation shape [256,128,56,56] (411 MB per operand)."""
+    res = {}
+    x = torch.randn(256, 128, 56, 56, device=dev, generator=g)
+    gy = torch.randn_like(x)
+    bias = torch.randn(1, 128, 1, 1, device=dev, generator=g)
+    nb = 4.0 * x.numel()
+    ms = time_events(torch, lambda: Kn.relu(x), iters)
+    res["relu_[256,128,56,56]"] = hbm_entry("relu_[256,128,56,56]", ms, 2 * nb)
+    ms = time_events(torch, lambda: Kn.relu_grad(x, gy), iters)
+    res["relu_grad_[256,128,56,56]"] = hbm_entry("relu_grad_[256,128,56,56]", ms, 3 * nb)
+    ms = time_events(torch, lambda: Kn.add_broadcast_relu(x, bias), iters)
+    res["add_bias_relu_[256,128,56,56]"] = hbm_entry("add_bias_relu_[256,128,56,56]", ms, 2 * nb,
+                                                     "relu(x + b) with b [1,128,1,1] in one pass")
+    ms = time_events(torch, lambda: Kn.bias_grad(gy), iters)
+    res["bias_grad_[256,128,56,56]"] = hbm_entry("bias_grad_[256,128,56,56]", ms, nb,
+                                                 "MaybeReduceSum of the gradient of a [1,128,1,1] bias: sum over axes 0, 2, 3")
+    return res
+
+
+def micro_matmul(torch, Kn, dev, g):
+    """The dense contractions of configuration 3: 4096^3 in the three layouts of forward and gradients, 64 x 512^3."""
+    res = {}
     A = torch.randn(4096, 4096, device=dev, generator=g)
     Bm = torch.randn(4096, 4096, device=dev, generator=g)
     for name, ta, tb in (("matmul_4096_NN", False, False), ("matmul_4096_NT", False, True), ("matmul_4096_TN", True, False)):
@@ -529,19 +590,30 @@ def micro_rest(torch, Kn, capi, dev, g, iters=10):
     del A, Bm
     A = torch.randn(64, 512, 512, device=dev, generator=g)
     Bm = torch.randn(64, 512, 512, device=dev, generator=g)
-    ms = time_events(torch, lambda: Kn.batch_matmul(A, Bm), 10)
-    tf = 2.0 * 64 * 512 ** 3 / ms / 1e9
-    res["batch_matmul_64x512"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
-    res.update(other_conv_configs(torch, Kn, dev, g))
-    res.update(graph_steps())
+    for name, ta, tb in (("batch_matmul_64x512", False, False), ("batch_matmul_64x512_NT", False, True),
+                         ("batch_matmul_64x512_TN", True, False)):
+        ms = time_events(torch, lambda: Kn.batch_matmul(A, Bm, ta, tb), 10)
+        tf = 2.0 * 64 * 512 ** 3 / ms / 1e9
+        res[name] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
     return res
 
 
-def other_conv_configs(torch, Kn, dev, g):
+def other_conv_configs(torch, Kn, dev, g, which=None):
     """Operator-level conv2d forward + both gradients at the remaining convolution configurations
-    (stride-2 variant of the headline; dilated and transposed convolutions of configuration 5)."""
+    (stride-2 variant of the headline; dilated and transposed convolutions of configuration 5).  Each entry holds
+    the time of the three operators launched back to back and of each operator on its own."""
     out = {}
     L = Kn.capi.lib()
+
+    def entry(Bn, flop, ms_all, parts, path=None):
+        e = {"ms": round(ms_all, 4), "images/s": round(Bn / ms_all * 1e3, 1), "TFLOP/s": round(flop / ms_all / 1e9, 2),
+             "frac_mfma": round(flop / ms_all / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4)}
+        for k, ms in parts.items():
+            e[k + "_ms"] = round(ms, 4)
+            e[k + "_frac_mfma"] = round(flop / 3 / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4)
+        if path:
+            e["path"] = path
+        return e
 
     def conv_case(name, Bn, Cc, Kf, Hh, k, pad, stride, dil):
         """Forward, filter gradient and input gradient the way the host Conv2D operator runs them:
@@ -550,43 +622,55 @@ def other_conv_configs(torch, Kn, dev, g):
         w = torch.randn(Kf, Cc, k, k, device=dev, generator=g) * 0.05
         y, cols = Kn.conv2d(x, w, pad, stride, dil)
         gy = torch.randn_like(y)
-        del cols
         free = Kn.conv2d_nocols(x, w, pad, stride, dil) is not None and \
             Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil) is not None and \
             L.ag_conv2d_filter_grad_nocols_f32_workspace(Bn, Cc, Hh, Hh, Kf, k, k, pad, stride, dil) > 0
+        if free:
+            del cols
+            yy, xp = Kn.conv2d_nocols(x, w, pad, stride, dil)
+            gx, scratch = Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil)
+            fwd = lambda: Kn.conv2d_nocols(x, w, pad, stride, dil)
+            igrad = lambda: Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil)
+            fgrad = lambda: Kn.conv2d_filter_grad_nocols(xp, scratch, tuple(x.shape), tuple(w.shape), pad, stride, dil)
+        else:
+            fwd = lambda: Kn.conv2d(x, w, pad, stride, dil)
+            igrad = lambda: Kn.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(Hh, Hh))
+            fgrad = lambda: Kn.conv2d_filter_grad(cols, gy, tuple(w.shape))
 
         def step():
-            if free:
-                yy, xp = Kn.conv2d_nocols(x, w, pad, stride, dil)
-                gx, scratch = Kn.conv_input_grad_staged(gy, w, pad, (Hh, Hh), stride, dil)
-                Kn.conv2d_filter_grad_nocols(xp, scratch, tuple(x.shape), tuple(w.shape), pad, stride, dil)
-            else:
-                yy, cc = Kn.conv2d(x, w, pad, stride, dil)
-                Kn.conv2d_filter_grad(cc, gy, tuple(w.shape))
-                Kn.conv2d_transpose(gy, w, pad, stride, dil, out_hw=(Hh, Hh))
+            fwd()
+            igrad()     # (its bordered copy of gy is what the column-free filter gradient reads)
+            fgrad()
 
         ms = time_events(torch, step, 8)
+        parts = {"fwd": time_events(torch, fwd, 8), "input_grad": time_events(torch, igrad, 8),
+                 "filter_grad": time_events(torch, fgrad, 8)}
         flop = 3 * 2.0 * Bn * Kf * y.shape[2] * y.shape[3] * Cc * k * k
-        out[name] = {"ms": round(ms, 4), "images/s": round(Bn / ms * 1e3, 1), "TFLOP/s": round(flop / ms / 1e9, 2),
-                     "frac_mfma": round(flop / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4), "path": "column-free" if free else "columns"}
+        out[name] = entry(Bn, flop, ms, parts, "column-free" if free else "columns")
 
-    conv_case("conv2d_fwd_bwd_stride2_B256_64to128_56x56", 256, 64, 128, 56, 3, 1, 2, 1)
-    conv_case("conv2d_fwd_bwd_dilated_B32_256to256_14x14", 32, 256, 256, 14, 3, 2, 1, 2)
-    # transposed convolution 128 -> 64, 4x4, stride 2, pad 1: [32,128,14,14] -> [32,64,28,28], forward and both gradients
-    x = torch.randn(32, 128, 14, 14, device=dev, generator=g)
-    w = (torch.rand(128, 64, 4, 4, device=dev, generator=g) - 0.5) * 0.2
-    yt = Kn.conv2d_transpose(x, w, 1, 2)
-    go = torch.randn_like(yt)
+    if which in (None, "stride2"):
+        conv_case("conv2d_fwd_bwd_stride2_B256_64to128_56x56", 256, 64, 128, 56, 3, 1, 2, 1)
+    if which in (None, "config5"):
+        conv_case("conv2d_fwd_bwd_dilated_B32_256to256_14x14", 32, 256, 256, 14, 3, 2, 1, 2)
+        # transposed convolution 128 -> 64, 4x4, stride 2, pad 1: [32,128,14,14] -> [32,64,28,28], forward and both gradients
+        x = torch.randn(32, 128, 14, 14, device=dev, generator=g)
+        w = (torch.rand(128, 64, 4, 4, device=dev, generator=g) - 0.5) * 0.2
+        yt = Kn.conv2d_transpose(x, w, 1, 2)
+        go = torch.randn_like(yt)
+        fwd = lambda: Kn.conv2d_transpose(x, w, 1, 2)
+        igrad = lambda: Kn.conv2d(go, w, 1, 2)                  # gradient w.r.t. the input of the transposed conv
+        fgrad = lambda: Kn.conv2d_transpose_filter_grad(x, go, tuple(w.shape), 1, 2)
 
-    def tstep():
-        Kn.conv2d_transpose(x, w, 1, 2)
-        Kn.conv2d(go, w, 1, 2)                                  # gradient w.r.t. the input of the transposed conv
-        Kn.conv2d_transpose_filter_grad(x, go, tuple(w.shape), 1, 2)
+        def tstep():
+            fwd()
+            igrad()
+            fgrad()
 
-    ms = time_events(torch, tstep, 8)
-    tflop = 3 * 2.0 * 32 * 128 * 14 * 14 * 64 * 16
-    out["conv2d_transpose_fwd_bwd_B32_128to64_14to28"] = {"ms": round(ms, 4), "images/s": round(32 / ms * 1e3, 1),
-                                                          "TFLOP/s": round(tflop / ms / 1e9, 2)}
+        ms = time_events(torch, tstep, 8)
+        parts = {"fwd": time_events(torch, fwd, 8), "input_grad": time_events(torch, igrad, 8),
+                 "filter_grad": time_events(torch, fgrad, 8)}
+        tflop = 3 * 2.0 * 32 * 128 * 14 * 14 * 64 * 16
+        out["conv2d_transpose_fwd_bwd_B32_128to64_14to28"] = entry(32, tflop, ms, parts)
     return out
 
 

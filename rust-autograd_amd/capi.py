@@ -9,6 +9,8 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libag_hip.so")
+# The same sources built with -DAG_TEST_HOOKS: the tuning hooks of csrc/ag_test_hooks.h exist only there.
+TEST_LIB_PATH = os.path.join(_HERE, "libag_hip_test.so")
 
 c_f = C.c_float
 c_i = C.c_int
@@ -111,33 +113,64 @@ PROTOTYPES = {
     "ag_matmul_f32_noalloc": (c_i, [c_p, c_i, c_i, c_i, c_i, c_i, c_p, c_i, c_p, c_i, c_p, c_i]),
 }
 
-# Test hooks (csrc/ag_test_hooks.h): thread-local overrides used by the test-suite, not part of the boundary.
+# Test hooks (csrc/ag_test_hooks.h): thread-local overrides used by the test-suite, not part of the boundary and
+# exported by libag_hip_test.so only.
 TEST_HOOKS = {
     "ag_test_gemm_force_config": (None, [c_i]),
     "ag_test_gemm_force_splits": (None, [c_i]),
     "ag_test_gemm_force_grid": (None, [c_i]),
-    "ag_test_conv_fused_input_grad": (None, [c_i]),
     "ag_test_pool_chunk_rows": (None, [c_i]),
 }
 
-_lib = None
+_lib = None        # what lib() returns: the shipped library, or the test flavour inside use_test_library()
+_product = None
+_test = None
+
+
+def _load(path, tables):
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with rust-autograd_amd/csrc/build.sh (there is no CPU fallback)")
+    handle = C.CDLL(path)
+    for table in tables:
+        for name, (res, args) in table.items():
+            fn = getattr(handle, name)  # AttributeError names the missing symbol
+            fn.restype = res
+            fn.argtypes = args
+    return handle
 
 
 def lib():
     """The loaded library.  Raises if it has not been built (run __graft_entry__.build())."""
-    global _lib
+    global _lib, _product
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError(
-                f"{LIB_PATH} is missing: build it with rust-autograd_amd/csrc/build.sh "
-                "(there is no CPU fallback)")
-        handle = C.CDLL(LIB_PATH)
-        for name, (res, args) in list(PROTOTYPES.items()) + list(TEST_HOOKS.items()):
-            fn = getattr(handle, name)  # AttributeError names the missing symbol
-            fn.restype = res
-            fn.argtypes = args
-        _lib = handle
+        if _product is None:
+            _product = _load(LIB_PATH, [PROTOTYPES])
+        _lib = _product
     return _lib
+
+
+def test_lib():
+    """libag_hip_test.so: the operator boundary plus the hooks of csrc/ag_test_hooks.h."""
+    global _test
+    if _test is None:
+        _test = _load(TEST_LIB_PATH, [PROTOTYPES, TEST_HOOKS])
+    return _test
+
+
+class use_test_library:
+    """Context manager: inside it lib() -- and with it every launcher of kernels.py -- is the test flavour of the
+    library, so that a test can force tile configurations, split counts and chunk sizes (single-threaded use)."""
+
+    def __enter__(self):
+        global _lib
+        self.saved = lib()
+        _lib = test_lib()
+        return _lib
+
+    def __exit__(self, *exc):
+        global _lib
+        _lib = self.saved
+        return False
 
 
 def last_error():

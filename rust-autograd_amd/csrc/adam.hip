@@ -160,6 +160,12 @@ extern "C" ag_status_t ag_adam_update_multi_f32(ag_stream_t stream, int count, f
         for (int j = 0; j < i; ++j)
             AG_REQUIRE(ts[j] != ts[i] && (ns[i] == 0 || ns[j] == 0 || (params[j] != params[i] && ms[j] != ms[i] && vs[j] != vs[i])),
                        AG_ERR_INVALID_DIMS, "adam: parameters %d and %d share an array; update them in separate calls", j, i);
+        // a gradient that another entry of the same launch writes (its param, m or v) would be read while it changes
+        for (int j = 0; j < count; ++j)
+            AG_REQUIRE(j == i || ns[i] == 0 || ns[j] == 0 ||
+                           (grads[i] != params[j] && grads[i] != ms[j] && grads[i] != vs[j]),
+                       AG_ERR_INVALID_DIMS,
+                       "adam: the gradient of parameter %d is an array that parameter %d updates; update them in separate calls", i, j);
         const int vec = aligned16(params[i]) && aligned16(grads[i]) && aligned16(ms[i]) && aligned16(vs[i]);
         const size_t items = ns[i] == 0 ? 0 : (vec ? ns[i] / 4 + 1 : ns[i]);
         tab.p[i] = params[i];

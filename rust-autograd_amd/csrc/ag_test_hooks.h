@@ -1,6 +1,7 @@
-/* Test hooks of libag_hip.so: exported for the library's own test-suite and tuning runs, NOT part of
- * the operator boundary (include/ag_hip.h).  Every hook sets an override that is local to the
- * calling thread, so other threads' calls are never affected. */
+/* Test hooks: exported only by libag_hip_test.so, the flavour of the kernel library that build.sh compiles with
+ * -DAG_TEST_HOOKS for the test-suite and tuning runs.  The shipped libag_hip.so is built without them and exports
+ * exactly the operator boundary (include/ag_hip.h).  Every hook sets an override that is local to the calling
+ * thread, so other threads' calls are never affected. */
 #ifndef AG_TEST_HOOKS_H
 #define AG_TEST_HOOKS_H
 
@@ -17,8 +18,6 @@ void ag_test_gemm_force_config(int cfg);
 void ag_test_gemm_force_splits(int splits);
 /* Blocks per CU of the persistent GEMM grid (0 = as many as stay resident). */
 void ag_test_gemm_force_grid(int blocks_per_cu);
-/* 0: ag_conv2d_transpose_f32 always runs GEMM + col2im; 1 (default): it may take the implicit GEMM. */
-void ag_test_conv_fused_input_grad(int on);
 /* Output rows per chunk of the stride-2 pooling kernels (0 = automatic); a negative value instead keeps 2 x 2
    windows off the one-thread-per-window kernels, so that the staged and register kernels see those geometries too. */
 void ag_test_pool_chunk_rows(int rows);

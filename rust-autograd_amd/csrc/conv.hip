@@ -3,7 +3,6 @@
 // batched: one im2col launch and one strided-batched GEMM launch per operator instead of one
 // task per image, and one split-accumulation GEMM instead of an image-sequential beta=1 loop.
 #include "ag_internal.h"
-#include "ag_test_hooks.h"
 #include "conv_shared.h"
 #include "gemm_shared.h"
 
@@ -250,7 +249,6 @@ extern "C" ag_status_t ag_conv2d_filter_grad_f32(ag_stream_t stream, const float
 
 namespace ag {
 
-static thread_local bool g_fused_input_grad = true;  // test hook (ag_test_hooks.h), per calling thread
 
 // gyp[plane][r][s] = gy[plane][r - top][s - left] inside the image, 0 in the border; four
 // consecutive elements of the flattened padded plane per thread (its extent is a multiple of 4).
@@ -697,7 +695,7 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
     // (images of fewer than 256 padded positions with more than 64 channels run on 64-row tiles, and while their
     // columns stay in the cache the column path is ahead: 32 x 256 -> 256 channels, 14 x 14: 0.084 against 0.108 ms;
     // at eight times the batch 0.71 against 0.54 ms)
-    if (stride == 1 && g_fused_input_grad &&
+    if (stride == 1 &&
         fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg, dilation) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
         ((long long)xh * fg.Wp >= 256 || xch <= 64 || (long long)B * M * P >= (1LL << 24)) && aligned16(gcols) && aligned16(gx)) {
         if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad, dilation)) return s;
@@ -710,7 +708,7 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
     // convolution [32,128,14,14] -> [32,64,28,28] with both gradients takes 0.21 ms this way against
     // 0.13 ms over columns).
     S2Geom g2;
-    if (stride == 2 && dilation == 1 && g_fused_input_grad && (long long)B * M * P >= (1LL << 24) &&
+    if (stride == 2 && dilation == 1 && (long long)B * M * P >= (1LL << 24) &&
         s2_geom(B, xch, xh, xw, ych, kh, kw, pad, &g2) && g2.OH == yh &&
         g2.OW == yw && g2.gyp_floats + g2.wf_floats + g2.gxp_floats <= (long long)B * M * P && aligned16(gcols) && aligned16(gx)) {
         if (ag_status_t s = s2_igrad_prepare(as_stream(stream), gy, w, gcols, g2, B, xch, ych, kh, kw, pad)) return s;
@@ -750,10 +748,6 @@ extern "C" ag_status_t ag_conv2d_transpose_filter_grad_f32(ag_stream_t stream, c
     return ag_gemm_batchsum_f32(stream, 0, 1, ych, (int)N, (int)P, 1.f, x, (int)P, (long long)ych * P, gycols,
                                 (int)P, N * P, 0.f, gw, (int)N, B, ws, ws_bytes);
 }
-
-// Test hook (ag_test_hooks.h; not part of the operator surface): 0 makes ag_conv2d_transpose_f32 calls of
-// this thread always take the GEMM + col2im path, 1 (default) lets them use the implicit GEMM.
-extern "C" void ag_test_conv_fused_input_grad(int on) { ag::g_fused_input_grad = on != 0; }
 
 // The two stages of the column-free stride-1 input gradient, for callers that time or schedule
 // them separately.  `scratch` holds ag_conv_input_grad_scratch_floats() floats (0 = this

@@ -25,7 +25,9 @@
 #include <mutex>
 #include <type_traits>
 
+#ifdef AG_TEST_HOOKS
 #include "ag_test_hooks.h"
+#endif
 #include "gemm_shared.h"
 
 namespace ag {
@@ -524,8 +526,16 @@ static int resident_blocks(Kern kern, int threads, int fallback)
     return n;
 }
 
-// Test hook (ag_test_hooks.h), per calling thread: blocks per CU of the persistent grid (0 = resident count).
+// Test hooks (ag_test_hooks.h; built only into the test flavour of the library, -DAG_TEST_HOOKS), per calling
+// thread: blocks per CU of the persistent grid (0 = resident count), a forced tile configuration (-1 = automatic
+// choice) and a forced split count of accumulated-batch products (0 = automatic).
+#ifdef AG_TEST_HOOKS
 static thread_local int g_grid_scale = 0;
+static thread_local int g_force_cfg = -1;
+static thread_local int g_force_splits = 0;
+#else
+constexpr int g_grid_scale = 0, g_force_cfg = -1, g_force_splits = 0;
+#endif
 
 template <int BM, int BN, int BK, int WM, int WN, int OCC, int STAGES>
 static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
@@ -553,9 +563,6 @@ static void launch_cfg(hipStream_t st, int la, int lb, const GemmParams &p)
     AG_GEMM_CASE(LMN, LMN)
 #undef AG_GEMM_CASE
 }
-
-static thread_local int g_force_cfg = -1;  // test hook (ag_test_hooks.h), per calling thread
-static thread_local int g_force_splits = 0;  // test hook (ag_test_hooks.h), per calling thread
 
 // Tile configurations {BM, BN}; see launch() for BK, the wave tile and the occupancy target.
 static const TileCfg kCfgs[] = {{128, 128}, {128, 64}, {64, 128}, {64, 64},
@@ -1211,11 +1218,13 @@ static int matmul_slices(int M, int N, int K)
 
 using namespace ag;
 
-// Test hooks (ag_test_hooks.h; not part of the operator surface).  Each sets a thread-local
-// override that later calls made by the same thread observe.
+#ifdef AG_TEST_HOOKS
+// Test hooks (ag_test_hooks.h; not part of the operator surface and not in the shipped library).  Each sets a
+// thread-local override that later calls made by the same thread observe.
 extern "C" void ag_test_gemm_force_config(int cfg) { g_force_cfg = cfg; }
 extern "C" void ag_test_gemm_force_splits(int splits) { g_force_splits = splits; }
 extern "C" void ag_test_gemm_force_grid(int blocks_per_cu) { g_grid_scale = blocks_per_cu; }
+#endif
 
 extern "C" ag_status_t ag_gemm_f32(ag_stream_t stream, int transA, int transB, int M, int N, int K,
                                    float alpha, const float *A, int lda, long long strideA, const float *B,

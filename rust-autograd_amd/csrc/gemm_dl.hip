@@ -590,11 +590,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     unsigned fill_addr = lds_wave;  // LDS byte address (this wave's share) of the slot being filled
     auto second_half = [&](const float *cur, const float *nxt, bool last) {
         constexpr int NM = (KK - KK / 2) * 4 * MI * NI;  // MFMAs in this half
-#ifdef AG_DL_SPACING
-        constexpr int SPACING = AG_DL_SPACING;
-#else
         constexpr int SPACING = NM / L;                   // MFMAs between two loads
-#endif
         static_assert(SPACING >= 1, "more loads than MFMAs");
 #pragma unroll
         for (int kk = KK / 2; kk < KK; ++kk) {

@@ -994,8 +994,11 @@ struct AddOp : Op {  // binary_ops.rs:147-166, 304-346
 
 // AddOp followed by ReLU as one node: what tensor_ops::relu builds when its argument is an AddOp node, with
 // that node's two operands as inputs.  The value is relu(a + b) bit for bit; the AddOp node stays in the graph and
-// is evaluated only if something else asks for it.  The gradient is the mask taken from this node's own OUTPUT
-// (y > 0 exactly where a + b > 0), handed to both operands the way AddOp::grad does.
+// is evaluated only if something else asks for it.  For back-propagation the node's only input is the AddOp
+// node itself (`backprop_inputs`): the gradient it hands on is the mask taken from this node's own OUTPUT
+// (y > 0 exactly where a + b > 0) -- what ReLU::grad hands to its argument (activation_ops.rs:154-167) -- and
+// AddOp::grad carries it on to the operands, so that the sum stays differentiable like any other node
+// (grad(loss, [a + b]) and everything else that names the sum see the graph of the two operations).
 struct AddReLU : Op {
     const char *name() const override { return "AddReLU"; }
     OpError compute(ComputeContext &ctx) const override
@@ -1011,9 +1014,18 @@ struct AddReLU : Op {
             return OpError::make(ErrorKind::IncompatibleShape,
                                  "AddOp: unsupported broadcast " + shape_str(a.shape()) + " + " + shape_str(b.shape()));
         }
-        if (a.shape().empty() || a.shape().size() > 8)
-            return OpError::make(ErrorKind::IncompatibleShape, "AddOp: rank " + std::to_string(a.shape().size()) + " not in 1..8");
+        if (a.shape().size() > 8)
+            return OpError::make(ErrorKind::IncompatibleShape, "AddOp: rank " + std::to_string(a.shape().size()) + " not in 0..8");
         NdArray y = NdArray::empty(a.shape());
+        if (a.shape().empty()) {
+            // 0-dimensional operands whose rank was not known when the graph was built: the two operations in turn
+            const float *xs[2] = {a.ptr(), b.ptr()};
+            OpError e0 = from_status(ag_add_n_f32(ctx.stream(), xs, 2, y.ptr(), a.len()));
+            if (e0.ok()) e0 = from_status(ag_relu_f32(ctx.stream(), y.ptr(), y.ptr(), y.len()));
+            if (!e0.ok()) return e0;
+            ctx.append_output(y);
+            return OpError::none();
+        }
         const std::vector<int> shape(a.shape().begin(), a.shape().end());
         const OpError e = from_status(ag_add_broadcast_relu_f32(ctx.stream(), a.ptr(), b.ptr(), y.ptr(), shape.data(),
                                                                 bshape.data(), (int)shape.size()));
@@ -1023,9 +1035,8 @@ struct AddReLU : Op {
     }
     void grad(GradientContext &ctx) const override
     {
-        const Tensor g = relu_grad_node(ctx.graph(), ctx.output(), ctx.output_grad());
-        ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(0)}, std::make_unique<MaybeReduceSum>()));
-        ctx.append_input_grad(build(ctx.graph(), {g, ctx.input(1)}, std::make_unique<MaybeReduceSum>()));
+        // one back-prop input: the AddOp node
+        ctx.append_input_grad(relu_grad_node(ctx.graph(), ctx.output(), ctx.output_grad()));
     }
 };
 
@@ -1333,10 +1344,19 @@ Tensor relu(Tensor x)
 {
     // relu(a + b): one fused node over a and b (the bias-activation step after a convolution)
     const TensorInternal &n = x.graph->node(x.id);
+    // (the sum itself is the node's back-prop input; operands known to be 0-dimensional keep the two nodes: the fused
+    // kernel takes ranks 1..8)
     if (dynamic_cast<const AddOp *>(n.op.get()) && n.incoming_nodes.size() == 2 && n.incoming_nodes[0].array_selector == 0 &&
-        n.incoming_nodes[1].array_selector == 0 && !n.incoming_nodes[0].allow_mut && !n.incoming_nodes[1].allow_mut)
-        return build(x.graph, {x.graph->tensor(n.incoming_nodes[0].id), x.graph->tensor(n.incoming_nodes[1].id)},
-                     std::make_unique<AddReLU>());
+        n.incoming_nodes[1].array_selector == 0 && !n.incoming_nodes[0].allow_mut && !n.incoming_nodes[1].allow_mut) {
+        const TensorInternal &lhs = x.graph->node(n.incoming_nodes[0].id);
+        const bool rank0 = lhs.known_shape && lhs.known_shape->empty();
+        if (!rank0)
+            return x.graph->builder()
+                .append_input(x.graph->tensor(n.incoming_nodes[0].id), false)
+                .append_input(x.graph->tensor(n.incoming_nodes[1].id), false)
+                .append_backprop_input(x)
+                .build(std::make_unique<AddReLU>());
+    }
     return build(x.graph, {x}, std::make_unique<ReLU>());
 }
 Tensor add(Tensor a, Tensor b) { return build(a.graph, {a, b}, std::make_unique<AddOp>()); }
@@ -1358,7 +1378,7 @@ Tensor sparse_softmax_cross_entropy(Tensor logits, Tensor labels)
     return build(logits.graph, {logits, labels}, std::make_unique<SparseSoftmaxCrossEntropy>());
 }
 
-Tensor scalar(float v, Graph *g) { return g->builder().build(std::make_unique<ScalarOp>(v)); }
+Tensor scalar(float v, Graph *g) { return g->builder().set_known_shape(Shape{}).build(std::make_unique<ScalarOp>(v)); }
 
 Tensor zeros_like(Tensor x)
 {

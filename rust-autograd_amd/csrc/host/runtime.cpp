@@ -405,6 +405,10 @@ Tensor TensorBuilder::build(std::unique_ptr<Op> op)
 {
     int rank = 0;
     for (const IncomingTensor &in : in_nodes_) rank = std::max(rank, graph_->node(in.id).topo_rank + 1);
+    // (a back-prop input that is not an input -- the sum behind a fused AddReLU -- must also rank below this node,
+    // or the gradient builder's heap could reach it before this node has handed it its gradient)
+    if (backprop_inputs_)
+        for (const IncomingTensor &in : *backprop_inputs_) rank = std::max(rank, graph_->node(in.id).topo_rank + 1);
     auto n = std::make_unique<TensorInternal>();
     n->op = std::move(op);
     n->incoming_nodes = std::move(in_nodes_);
@@ -517,6 +521,20 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
 {
     std::unordered_map<TensorID, StorageEntry> storage;  // every output lives until eval returns
     DeferredUpdates deferred;                            // in-place optimizer updates, batched
+    // A node that panics ends the evaluation; the updates queued by the nodes before it have already happened
+    // as far as the reference is concerned (each AdamOp runs at its own node), so they are applied on the way out.
+    struct FlushOnUnwind {
+        DeferredUpdates &d;
+        bool armed = true;
+        ~FlushOnUnwind()
+        {
+            if (!armed) return;
+            try {
+                d.flush();
+            } catch (...) {
+            }
+        }
+    } flush_on_unwind{deferred};
     auto would_not_visit = [&](const TensorInternal &n) {
         return n.is_placeholder || n.is_variable() || storage.count(n.id) != 0;
     };
@@ -576,6 +594,7 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
                 if (!would_not_visit(node(in.id))) dfs.emplace_back(in.id, false);
         }
     }
+    flush_on_unwind.armed = false;
     deferred.flush();
     std::vector<EvalResult> ret;
     for (const Tensor &t : tensors) {

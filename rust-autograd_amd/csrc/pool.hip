@@ -8,7 +8,9 @@
 #include <cfloat>
 
 #include "ag_internal.h"
+#ifdef AG_TEST_HOOKS
 #include "ag_test_hooks.h"
+#endif
 
 namespace ag {
 
@@ -131,7 +133,9 @@ __global__ __launch_bounds__(256) void maxpool_bwd_tile2_kernel(const float *__r
         const long long a = (long long)argmax[o] - xbase - (long long)(2 * oy) * g.W - 2 * ox;
         tap = a == 0 ? 0 : a == 1 ? 1 : a == g.W ? 2 : a == g.W + 1 ? 3 : kNoTap;
     }
-    const float v = gy[o];
+    // 0 + gy as in the reference's scatter onto a zeroed plane (max_pool2d.rs:123-131) and in the gather kernels:
+    // a gradient of -0.0 (what an upstream 0 * negative leaves) arrives as +0.0
+    const float v = 0.f + gy[o];
     float2 top, bottom;
     top.x = tap == 0 ? v : 0.f;
     top.y = tap == 1 ? v : 0.f;
@@ -567,7 +571,11 @@ static int lanes_per_row(int W)
     return W4 <= 4 ? 4 : W4 <= 8 ? 8 : W4 <= 16 ? 16 : W4 <= 32 ? 32 : 64;
 }
 
-static thread_local int g_chunk_rows = 0;  // test hook (ag_test_hooks.h), per calling thread
+#ifdef AG_TEST_HOOKS
+static thread_local int g_chunk_rows = 0;  // test hook (ag_test_hooks.h; test flavour of the library only), per calling thread
+#else
+constexpr int g_chunk_rows = 0;
+#endif
 // Output rows per chunk of the stride-2 backward.  Short chunks win by a wide margin although each
 // re-reads the window row above it (one byte and one float per output): 256 x 128 planes of
 // 56 x 56 take 0.120 ms as whole planes, 0.113 with 9 rows, 0.103 with 3 and 0.082-0.091 with 2
@@ -584,10 +592,12 @@ constexpr long long kExactFloatIndexLimit = 1LL << 24;
 
 using namespace ag;
 
-// Test hook (ag_test_hooks.h; not part of the operator surface): output rows per chunk of the
-// stride-2 pooling kernels for later calls of this thread (0 = automatic; negative: automatic, and 2 x 2 windows
-// stay off the one-thread-per-window kernels where another kernel can take them).
+#ifdef AG_TEST_HOOKS
+// Test hook (ag_test_hooks.h; not part of the operator surface and not in the shipped library): output rows per
+// chunk of the stride-2 pooling kernels for later calls of this thread (0 = automatic; negative: automatic, and
+// 2 x 2 windows stay off the one-thread-per-window kernels where another kernel can take them).
 extern "C" void ag_test_pool_chunk_rows(int rows) { ag::g_chunk_rows = rows; }
+#endif
 
 extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, float *y,
                                             float *argmax, uint8_t *taps, int B, int C, int H,

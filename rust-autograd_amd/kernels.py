@@ -185,15 +185,22 @@ def conv2d_transpose(gy, w, pad, stride, dilation=1, out_hw=None, return_cols=Fa
     gx = _empty((B, xch, xh, xw), gy)
     gcols = _empty((B, xch * kh * kw, yh * yw), gy)
     L = capi.lib()
-    if return_cols:  # the caller wants the columns: keep to the GEMM + col2im path
-        L.ag_test_conv_fused_input_grad(0)
-    try:
-        check(L.ag_conv2d_transpose_f32(_stream(), _ptr(gy), _ptr(w), _ptr(gx), _ptr(gcols), B, ych, yh, yw,
+    if return_cols:
+        # the caller wants the columns: the reference's two steps through their own entry points, the GEMM
+        # gcols_b = w^T . gy_b (conv2d_transpose.rs:114-116, 167-182) and col2im (conv_ops/mod.rs:178-223), with the
+        # operator's argument checks done by a call on an empty batch
+        check(L.ag_conv2d_transpose_f32(_stream(), _ptr(gy), _ptr(w), _ptr(gx), _ptr(gcols), 0, ych, yh, yw,
                                         xch, kh, kw, pad, stride, dilation, xh, xw))
-    finally:
-        if return_cols:
-            L.ag_test_conv_fused_input_grad(1)
-    return (gx, gcols) if return_cols else gx
+        M, P = xch * kh * kw, yh * yw
+        if B and M and P:
+            check(L.ag_gemm_f32(_stream(), 1, 0, M, P, ych, 1.0, _ptr(w), M, 0, _ptr(gy), P, ych * P, 0.0, _ptr(gcols), P,
+                                M * P, B))
+        check(L.ag_col2im_f32(_stream(), _ptr(gcols), _ptr(gx), B, xch, xh, xw, kh, kw, pad, pad, stride, stride,
+                              dilation, dilation, yh, yw))
+        return gx, gcols
+    check(L.ag_conv2d_transpose_f32(_stream(), _ptr(gy), _ptr(w), _ptr(gx), _ptr(gcols), B, ych, yh, yw,
+                                    xch, kh, kw, pad, stride, dilation, xh, xw))
+    return gx
 
 
 def conv2d_nocols(x, w, pad, stride=1, dilation=1):

@@ -31,3 +31,17 @@ def orc():
 @pytest.fixture()
 def rng():
     return np.random.default_rng(20240611)
+
+
+@pytest.fixture()
+def hooked():
+    """The test flavour of the kernel library (libag_hip_test.so: the same sources built with the tuning hooks of
+    csrc/ag_test_hooks.h) for the duration of one test: every launcher of kernels.py goes through it, and the test
+    can force tile configurations, split counts and chunk sizes.  The shipped library has no such hooks."""
+    from __graft_entry__ import load_package
+
+    load_package()
+    from rust_autograd_amd import capi
+
+    with capi.use_test_library() as lib:
+        yield lib

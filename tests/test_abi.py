@@ -46,17 +46,26 @@ def test_ctypes_prototypes_cover_the_header(capi):
     capi.lib()
 
 
-def test_exports_are_the_header_plus_the_test_hooks(capi):
-    """Nothing is exported beyond include/ag_hip.h and the thread-local test hooks of
-    csrc/ag_test_hooks.h, and the hooks are not declared in the public header."""
-    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True).stdout
-    exported = sorted(l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("ag_"))
+def _exported(path):
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True).stdout
+    return sorted(l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("ag_"))
+
+
+def test_shipped_library_exports_exactly_the_header(capi):
+    """libag_hip.so exports the functions of include/ag_hip.h and nothing else: no test or tuning hook."""
+    assert _exported(capi.LIB_PATH) == sorted(_declared_functions())
+    assert not [n for n in _declared_functions() if n.startswith("ag_test_")]
+
+
+def test_test_flavour_exports_the_header_plus_the_hooks(capi):
+    """libag_hip_test.so (the same sources with -DAG_TEST_HOOKS) adds the thread-local hooks of
+    csrc/ag_test_hooks.h, which the public header does not declare."""
     hooks_h = open(os.path.join(ROOT, "rust-autograd_amd", "csrc", "ag_test_hooks.h")).read()
     hooks_h = re.sub(r"/\*.*?\*/", "", hooks_h, flags=re.S)
     hooks = sorted(set(re.findall(r"\b(ag_test_[a-z0-9_]+)\s*\(", hooks_h)))
     assert hooks == sorted(capi.TEST_HOOKS)
-    assert not [n for n in _declared_functions() if n.startswith("ag_test_")]
-    assert exported == sorted(_declared_functions() + hooks)
+    assert _exported(capi.TEST_LIB_PATH) == sorted(_declared_functions() + hooks)
+    capi.test_lib()  # loads, and every prototype and hook resolves
 
 
 def test_library_has_gfx950_code_object(capi):

@@ -115,7 +115,7 @@ def _conv_paths(K, x, w, gy, pad, stride, dil):
 
 
 @pytest.mark.parametrize("stride", [1, 2])
-def test_config4_conv_b256_against_direct_definition(K, stride):
+def test_config4_conv_b256_against_direct_definition(K, orc, stride):
     B, C, Kf, H, k, pad = 256, 64, 128, 56, 3, 1
     OH = (H + 2 * pad - k) // stride + 1
     rng = np.random.default_rng(256 + stride)
@@ -135,12 +135,22 @@ def test_config4_conv_b256_against_direct_definition(K, stride):
     y_t, y_a = direct_y(x, w, yi, pad, stride, 1), direct_y(np.abs(x), np.abs(w), yi, pad, stride, 1)
     gx_t, gx_a = direct_gx(gy, w, xi, pad, stride, 1), direct_gx(np.abs(gy), np.abs(w), xi, pad, stride, 1)
     gw_t, gw_a = direct_gw(x, gy, chans, k, k, pad, stride, 1), direct_gw(np.abs(x), np.abs(gy), chans, k, k, pad, stride, 1)
+    # the reference's own arithmetic on the whole batch: the f32 oracle (im2col, SGEMM through OpenBLAS where it is
+    # loaded, image-sequential filter gradient, col2im), sampled at the same elements -- bars 2 and 3 at the shape
+    # the headline metric is quoted on
+    say("config 4 B=256 stride", stride, "f32 oracle on the whole batch")
+    o_y, o_cols = orc.conv2d_fwd(x, w, pad, stride, 1, threads=16)
+    o_gw = orc.conv2d_filter_grad(o_cols, gy, w.shape)
+    del o_cols
+    o_gx = orc.conv2d_transpose(gy, w, pad, stride, 1, out_hw=(H, H), threads=16)
+    y_32, gx_32, gw_32 = o_y[tuple(yi.T)], o_gx[tuple(xi.T)], o_gw[:, chans]
+    del o_y, o_gx
     for name, (y, gw, gx) in _conv_paths(K, dev(x), dev(w), dev(gy), pad, stride, 1).items():
         say("config 4 B=256 stride", stride, name)
         yv, gwv, gxv = host(y), host(gw), host(gx)
-        assert_contraction(yv[tuple(yi.T)], y_t, y_a, f"{name} y")
-        assert_contraction(gxv[tuple(xi.T)], gx_t, gx_a, f"{name} gx")
-        assert_contraction(gwv[:, chans], gw_t, gw_a, f"{name} gw")
+        assert_contraction(yv[tuple(yi.T)], y_t, y_a, f"stride {stride} {name} y", ref32=y_32)
+        assert_contraction(gxv[tuple(xi.T)], gx_t, gx_a, f"stride {stride} {name} gx", ref32=gx_32)
+        assert_contraction(gwv[:, chans], gw_t, gw_a, f"stride {stride} {name} gw", ref32=gw_32)
     # integer-valued data: every partial sum is an integer below 2^24, so f32 is exact in any order
     x = rng.integers(-3, 4, x.shape).astype(np.float32)
     w = rng.integers(-2, 3, w.shape).astype(np.float32)

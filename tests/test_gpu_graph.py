@@ -227,6 +227,46 @@ def test_config2_training_steps_with_adam(G, orc, rng):
         assert env.find(f"{ids[k]}m", "adam") is not None and env.find(f"{ids[k]}v", "adam") is not None
 
 
+def test_config2_free_running_loss_trajectory(G, orc, rng):
+    """Four training steps on one batch with nothing re-synchronised in between: the device runs its own graph with
+    its own Adam state, the oracle its own stages (its own ReLU masks and pooling indices) with the oracle's Adam.
+    Single elements may part ways (an activation within rounding of zero, a gradient that is rounding noise moving
+    its parameter by alpha the other way); the loss, a mean over the batch, must follow the oracle's trajectory to
+    1e-3 relative, and must fall."""
+    B = 128
+    params = cnn_params(rng)
+    env = G.VariableEnvironment()
+    ids = {k: env.set(k, a) for k, a in params.items()}
+    names = ["w1", "w2", "w3", "b1", "b2", "b3"]
+    adam = G.Adam(env, [ids[k] for k in names], alpha=1e-3)
+    ref = OracleCNN(orc, params)
+    m = {k: np.zeros_like(a) for k, a in params.items()}
+    vv = {k: np.zeros_like(a) for k, a in params.items()}
+    tt = {k: np.ones(1, np.float32) for k in params}
+    xv = rng.random((B, 1, 28, 28), dtype=np.float32)
+    lab = rng.integers(0, 10, (B, 1)).astype(np.float32)
+    got, want = [], []
+    for step in range(4):
+        c = env.context()
+        v, logits, loss, _ = build_cnn(G, env, c)
+        mean_loss = c.reduce_mean(loss, [0], False)
+        grads = c.grad([mean_loss], [v[k] for k in names])
+        say(f"config 2 free-running step {step}")
+        update = adam.get_update_op([v[k] for k in names], grads, c)
+        # the loss is requested last, so it is visited first: it is the loss before this step's update
+        got.append(float(np.asarray(c.eval([update, mean_loss], {"x": xv, "y": lab})[1]).reshape(-1)[0]))
+        oloss, _, og = ref.step_grads(xv, lab)
+        want.append(float(np.asarray(oloss).reshape(-1)[0]))
+        for k in names:
+            orc.adam(ref.p[k], og[k], m[k], vv[k], tt[k], alpha=1e-3)
+    say(f"losses {got} oracle {want}")
+    for step, (a, b) in enumerate(zip(got, want)):
+        assert abs(a - b) <= 1e-3 * abs(b), f"step {step}: loss {a} against the oracle's {b}"
+    assert got[-1] < got[0] and want[-1] < want[0]
+    for k in names:   # the parameters themselves stay within a few steps' worth of alpha of the oracle's
+        assert np.abs(env.array(ids[k]) - ref.p[k]).max() <= 4 * 2.1e-3
+
+
 def test_grad_helper_returns_every_variable_of_the_namespace(G, rng):
     env = G.VariableEnvironment()
     env.set("a", rng.random((4, 3), dtype=np.float32))
@@ -508,6 +548,48 @@ def test_relu_of_a_sum_is_one_node_with_the_values_and_gradients_of_two(G, orc, 
     assert gfb.shape == (1, 5, 1, 1) and np.array_equal(gfb.view(np.uint32), gpb.view(np.uint32))
 
 
+def test_the_sum_inside_a_fused_relu_stays_differentiable(G, rng):
+    """relu(z) with z = a + b is one fused node over a and b, but z itself must stay on the back-propagation path:
+    the gradient with respect to z is greater(z, 0) * gy (activation_ops.rs:154-167), also when z feeds a second
+    consumer, and with respect to a and b it is the bits of the unfused graph."""
+    env = G.VariableEnvironment()
+    av = rng.standard_normal((6, 5, 4, 4)).astype(np.float32)
+    bv = rng.standard_normal((1, 5, 1, 1)).astype(np.float32)
+    wv = rng.standard_normal((6, 5, 4, 4)).astype(np.float32)
+    aid, bid = env.set("a", av), env.set("b", bv)
+    c = env.context()
+    a, b = c.variable(aid), c.variable(bid)
+    wts = c.placeholder("wts", [6, 5, 4, 4])
+    z = a + b
+    fused = c.relu(z)
+    assert fused.op_name == "AddReLU"
+    zp = a + b
+    plain = c.relu(c.reshape(zp, [6, 5, 4, 4]))
+    assert plain.op_name == "ReLU"
+    (gz,) = c.grad([c.sum_all(c.mul(fused, wts))], [z])
+    (gzp,) = c.grad([c.sum_all(c.mul(plain, wts))], [zp])
+    (gzd,) = c.grad_with_default([fused], [z], [wts])
+    # z with a second consumer: both contributions must meet in its gradient, and reach a and b
+    both = c.sum_all(c.mul(fused, wts)) + c.sum_all(c.mul(z, wts))
+    gz2, ga2, gb2 = c.grad([both], [z, a, b])
+    bothp = c.sum_all(c.mul(plain, wts)) + c.sum_all(c.mul(zp, wts))
+    gzp2, gap2, gbp2 = c.grad([bothp], [zp, a, b])
+    say("gradient with respect to the sum inside relu(a + b)")
+    r = c.eval([gz, gzp, gzd, gz2, ga2, gb2, gzp2, gap2, gbp2], {"wts": wv})
+    mask = (av + bv > 0)
+    assert np.array_equal(r[0], wv * mask) and np.array_equal(r[0].view(np.uint32), r[1].view(np.uint32))
+    assert np.array_equal(r[2], wv * mask)
+    assert np.array_equal(r[3], wv * mask + wv)
+    for got, want in zip(r[3:6], r[6:9]):
+        assert got.shape == want.shape and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # operands of rank 0 keep the two nodes (the fused kernel takes ranks 1..8), with the same value
+    s = c.relu(c.scalar(-2.0) + c.scalar(0.5))
+    t = c.relu(c.scalar(2.0) + c.scalar(0.5))
+    assert s.op_name == "ReLU"
+    sv, tv = c.eval([s, t], {})
+    assert sv.shape == () and float(sv) == 0.0 and float(tv) == 2.5
+
+
 @pytest.mark.parametrize("H,size,stride", [(14, 2, 2), (28, 2, 2), (13, 3, 2), (9, 2, 1)])
 def test_relu_gradient_behind_a_pooling_is_one_node_with_the_pooling_gradient(G, rng, H, size, stride):
     """max_pool2d(relu(x)): the gradient that reaches x is built as one node (the pooling's backward with the ReLU's
@@ -655,6 +737,28 @@ def test_batched_adam_updates_keep_the_evaluation_order(G, orc, rng):
         pb, mb, vb = bv.copy(), np.zeros_like(bv), np.zeros_like(bv)
         orc.adam(pb, (bv + bv).astype(np.float32), mb, vb, np.ones(1, np.float32), alpha=0.25)
         assert_close(env.array(bid), pb, "b after the step")
+
+
+def test_updates_queued_before_a_panicking_node_are_still_applied(G, orc, rng):
+    """The AdamOp nodes of an evaluation are queued and launched together.  When a later node of the same evaluation
+    panics (a placeholder that was fed an array of another shape), the updates queued before it have happened as far
+    as the reference is concerned -- each AdamOp runs at its own node, src/evaluation.rs:310-329 -- so the
+    evaluation applies them on its way out."""
+    env = G.VariableEnvironment()
+    wv = rng.random((6, 5), dtype=np.float32) + 1.0
+    wid = env.set("w", wv)
+    adam = G.Adam(env, [wid], alpha=0.25)
+    c = env.context()
+    w = c.variable(wid)
+    (gw,) = c.grad([c.sum_all(c.mul(w, w))], [w])
+    update = adam.get_update_op([w], [gw], c)
+    bad = c.relu(c.placeholder("q", [3, 3]))
+    say("an evaluation that panics after its update node")
+    with pytest.raises(G.Panic):
+        c.eval([bad, update], {"q": np.zeros((2, 2), np.float32)})   # the last tensor is visited first
+    p, m, v, t = wv.copy(), np.zeros_like(wv), np.zeros_like(wv), np.ones(1, np.float32)
+    orc.adam(p, (wv + wv).astype(np.float32), m, v, t, alpha=0.25)
+    assert_close(env.array(wid), p, "w after the interrupted evaluation")
 
 
 # ------------------------------------------------------------------------------- the reference's own gradient tests

@@ -177,8 +177,8 @@ def test_gemm_all_layouts(K, orc, rng, shape, ta, tb):
 
 
 @pytest.mark.parametrize("cfg", list(range(13)))
-def test_gemm_every_tile_configuration(K, rng, cfg):
-    L = K.capi.lib()
+def test_gemm_every_tile_configuration(K, rng, cfg, hooked):
+    L = hooked
     m, n, k = 200, 333, 130
     a = rng.random((m, k), dtype=np.float32)
     b = rng.random((k, n), dtype=np.float32)
@@ -199,10 +199,10 @@ DIRECT_CFGS = list(range(13, 22))  # operand tiles loaded from global memory str
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("cfg", DIRECT_CFGS)
-def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb):
+def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb, hooked):
     """K a multiple of 32, aligned operands: ragged M / N edges, a K of one and of several tiles,
     and a batch large enough that every persistent block walks more than one output tile."""
-    L = K.capi.lib()
+    L = hooked
     for (m, n, k, batch) in ((200, 332, 32, 1), (200, 332, 160, 3), (256, 384, 64, 80), (64, 64, 96, 5)):
         a = rng.random((batch, k, m) if ta else (batch, m, k), dtype=np.float32)
         b = rng.random((batch, n, k) if tb else (batch, k, n), dtype=np.float32)
@@ -223,11 +223,11 @@ def test_gemm_direct_to_lds_configurations(K, rng, cfg, ta, tb):
 @pytest.mark.parametrize("tb", [0, 1])
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("cfg", DIRECT_CFGS + [-1])
-def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
+def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb, hooked):
     """A shared by all batches (stride 0, the conv filter matrix): with B and C n-contiguous the
     batches are tiled side by side along n, so tiles straddle two batches and the last tile runs
     past the last batch; with B transposed the batches stay separate.  alpha / beta included."""
-    L = K.capi.lib()
+    L = hooked
     shapes = [(128, 300, 64, 7, 0.0), (200, 260, 32, 3, 0.0), (192, 512, 96, 4, 0.0), (64, 296, 64, 5, -0.5)]
     if cfg == -1:
         # more tiles than the persistent grid has blocks: whole rounds, then a narrow-tile launch
@@ -254,10 +254,10 @@ def test_gemm_direct_to_lds_shared_a_folds_the_batch(K, rng, cfg, ta, tb):
 
 
 @pytest.mark.parametrize("cfg", DIRECT_CFGS)
-def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg):
+def test_gemm_direct_to_lds_accumulated_batch_and_beta(K, rng, cfg, hooked):
     """The filter-gradient form (sum over images, split into a workspace and folded) and the
     alpha / beta epilogue."""
-    L = K.capi.lib()
+    L = hooked
     kf, ck, pp, imgs = 128, 288, 192, 37
     gy = rng.random((imgs, kf, pp), dtype=np.float32)
     cols = rng.random((imgs, ck, pp), dtype=np.float32)
@@ -846,12 +846,12 @@ def test_conv2d_column_free_dilated(K, orc, rng, case):
 
 @pytest.mark.parametrize("cfg", [13, 14, 18, 19, 21])
 @pytest.mark.parametrize("d", [1, 2])
-def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d):
+def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d, hooked):
     # the implicit forward and input gradient on each tile shape of the direct-to-LDS kernel that they can run
     # on (the library picks one by channel count and size): integer-valued data, bit for bit the columns path
     B, C, Kc, H, W, k = 3, 64, 96, 22, 26, 3
     p = d
-    L = K.capi.lib()
+    L = hooked
     x = rng.integers(-3, 4, (B, C, H, W)).astype(np.float32)
     w = rng.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
     gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
@@ -1418,15 +1418,18 @@ def test_max_pool_random_geometries_with_ties_bit_exact(K, orc):
 
 
 @pytest.mark.parametrize("shape", [(3, 5, 28, 28), (2, 4, 14, 16), (1, 3, 8, 4), (2, 2, 56, 64), (1, 2, 2, 2)])
-def test_max_pool_2x2_tiling_kernels_have_the_bits_of_the_staged_and_register_kernels(K, rng, shape):
+def test_max_pool_2x2_tiling_kernels_have_the_bits_of_the_staged_and_register_kernels(K, rng, shape, hooked):
     # 2 x 2 windows at stride 2 over even planes of a small tensor run one thread per window; the test hook keeps
     # them off those kernels, so the same geometry also goes through the staged forward and the register / staged
     # backward: values, argmax, tap bytes, both backward forms and the backward with the ReLU gradient must not
     # differ in a bit (ties included)
-    L = K.capi.lib()
+    L = hooked
     x = (rng.integers(0, 5, shape) / np.float32(3)).astype(np.float32)
     relu_x = rng.standard_normal(shape).astype(np.float32)
     gy = rng.standard_normal((shape[0], shape[1], shape[2] // 2, shape[3] // 2)).astype(np.float32)
+    # signed zeros among the gradients (what an upstream 0 * negative leaves): every kernel stores 0 + gy
+    gy.reshape(-1)[::3] = -0.0
+    gy.reshape(-1)[1::7] = 0.0
     results = []
     for hook in (0, -1):
         L.ag_test_pool_chunk_rows(hook)
@@ -1445,10 +1448,10 @@ def test_max_pool_2x2_tiling_kernels_have_the_bits_of_the_staged_and_register_ke
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 1000])
-def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows):
+def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows, hooked):
     """The stride-2 backward walks chunks of output rows; whatever their length (one row, odd
     lengths, the whole plane) the result is the reference's, bit for bit."""
-    L = K.capi.lib()
+    L = hooked
     for (B, C, H, W, size) in [(2, 3, 56, 56, 3), (1, 2, 28, 28, 2), (1, 2, 11, 8, 3), (3, 1, 9, 12, 2)]:
         x = rng.integers(0, 4, (B, C, H, W)).astype(np.float32)   # many ties
         y, am, taps = K.max_pool2d(dev(x), size, 0, 2)

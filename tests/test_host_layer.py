@@ -99,6 +99,21 @@ def test_topo_rank_is_one_more_than_the_deepest_input(G):
     assert (a.topo_rank, b.topo_rank, s.topo_rank) == (1, 2, 3)
 
 
+def test_the_sum_behind_a_fused_relu_is_on_the_backprop_path(G):
+    # relu(a + b) is one AddReLU node over a and b whose back-prop input is the AddOp node: the sum must rank
+    # below it and receive greater(z, 0) * gy (activation_ops.rs:154-167), not zeros
+    env, c, x, w = small_graph(G)
+    y = c.placeholder("y", [-1, 1, 8, 8])
+    z = c.add(x, y)
+    r = c.relu(z)
+    assert r.op_name == "AddReLU" and r.num_inputs == 2 and r.topo_rank == z.topo_rank + 1
+    gz, gx = c.grad([c.sum_all(r)], [z, x])
+    assert gz.op_name == "ReLUGrad"
+    assert gx.op_name == "MaybeReduceSum"
+    # 0-dimensional operands keep the two nodes
+    assert c.relu(c.add(c.scalar(1.0), c.scalar(2.0))).op_name == "ReLU"
+
+
 def test_bad_handles_panic_with_a_message(G):
     env, c, x, w = small_graph(G)
     with pytest.raises(G.Panic, match="out of range"):

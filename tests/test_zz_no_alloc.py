@@ -28,11 +28,23 @@ def _both(torch, capi, K, a, b, ta, tb):
     ref = K.matmul(a, b, ta, tb)
     out = torch.full((m, n), float("nan"), dtype=torch.float32, device=a.device)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    before = torch.cuda.memory_allocated()
-    capi.check(L.ag_matmul_f32_noalloc(stream, int(ta), int(tb), m, n, k, C.c_void_p(a.data_ptr()), a.shape[1],
-                                       C.c_void_p(b.data_ptr()), b.shape[1], C.c_void_p(out.data_ptr()), n))
-    assert torch.cuda.memory_allocated() == before
+    def call():
+        capi.check(L.ag_matmul_f32_noalloc(stream, int(ta), int(tb), m, n, k, C.c_void_p(a.data_ptr()), a.shape[1],
+                                           C.c_void_p(b.data_ptr()), b.shape[1], C.c_void_p(out.data_ptr()), n))
+
+    # A first call may load the kernel's code object and look the array's address up; from then on nothing may
+    # change the device's free memory: torch's counter only sees torch's own allocator, hipMemGetInfo (what
+    # mem_get_info reads) sees a hipMalloc or hipFree from anywhere in the process.
+    call()
     torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    out.fill_(float("nan"))
+    call()
+    torch.cuda.synchronize()
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory moved during a call that must not allocate"
     return ref, out
 
 
