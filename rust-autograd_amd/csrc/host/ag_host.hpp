@@ -79,13 +79,17 @@ class NdArray {
     NdArray deep_copy() const;
     std::vector<float> to_host() const;  // synchronises the stream
     void copy_from_host(const float *data);  // overwrites the elements in place; synchronises
+    // Called before the calling thread enqueues work that reads / overwrites the elements: if another thread's
+    // stream used the array last, the caller's stream is ordered after it (a no-op for a thread's own arrays).
+    void will_read() const;
+    void will_write() const;
 
   private:
     Shape shape_;
     std::shared_ptr<DeviceBlock> block_;
 };
 
-void *current_stream();  // hipStream_t used by every op (the null stream)
+void *current_stream();  // hipStream_t of the calling thread: every op it evaluates is ordered on it
 void synchronize();
 
 // ---------------------------------------------------------------------------------------------

@@ -15,22 +15,98 @@ namespace ag {
 namespace host {
 
 // ---------------------------------------------------------------------------------------------
+// Streams.  The reference evaluates a graph on the thread that owns it (Graph is neither Send nor Sync,
+// src/graph.rs:17-47); here every host thread that evaluates graphs has a stream of its own (non-blocking, default
+// priority), created at its first use and handed to a later thread when this one ends.  Everything a thread enqueues
+// -- kernels, feeds, read-backs -- is ordered on its stream, so evaluations on different threads overlap on the
+// device and none of them waits for the null stream.
+// ---------------------------------------------------------------------------------------------
+namespace {
+void check(hipError_t e, const char *what)
+{
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+struct StreamPool {  // streams of threads that have ended (never destroyed: the runtime may outlive or precede us at exit)
+    std::mutex mu;
+    std::vector<hipStream_t> idle;
+};
+StreamPool &stream_pool()
+{
+    static StreamPool *p = new StreamPool;  // leaked on purpose: thread-local destructors may run after statics elsewhere
+    return *p;
+}
+struct ThreadStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t handoff = nullptr;  // marks "everything enqueued so far" on another thread's stream
+    hipStream_t get()
+    {
+        if (!stream) {
+            StreamPool &pool = stream_pool();
+            {
+                std::lock_guard<std::mutex> lk(pool.mu);
+                if (!pool.idle.empty()) {
+                    stream = pool.idle.back();
+                    pool.idle.pop_back();
+                }
+            }
+            if (!stream) check(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+        }
+        return stream;
+    }
+    ~ThreadStream()
+    {
+        if (!stream) return;
+        StreamPool &pool = stream_pool();
+        std::lock_guard<std::mutex> lk(pool.mu);
+        pool.idle.push_back(stream);  // its arena blocks stay with it
+    }
+};
+thread_local ThreadStream t_stream;
+
+// Orders the calling thread's stream after everything enqueued so far on `other`.
+void wait_for_stream(hipStream_t other)
+{
+    hipStream_t mine = t_stream.get();
+    if (other == mine) return;
+    if (!t_stream.handoff) check(hipEventCreateWithFlags(&t_stream.handoff, hipEventDisableTiming), "hipEventCreate");
+    check(hipEventRecord(t_stream.handoff, other), "hipEventRecord");
+    check(hipStreamWaitEvent(mine, t_stream.handoff, 0), "hipStreamWaitEvent");
+}
+}  // namespace
+
+void *current_stream() { return t_stream.get(); }
+
+void synchronize() { check(hipStreamSynchronize(t_stream.get()), "hipStreamSynchronize"); }
+
+// ---------------------------------------------------------------------------------------------
 // caching device arena: freed blocks are kept in per-size free lists, so a training loop that
 // rebuilds its graph every step (as the reference does, src/variable.rs:670-683) stops calling
-// hipMalloc after the first step.
+// hipMalloc after the first step.  The lists are per stream: a block goes back to the list of the stream it
+// was allocated for and is handed out again only to work on that stream, which is ordered after whatever used
+// the block before.
 // ---------------------------------------------------------------------------------------------
 struct DeviceBlock {
     void *ptr = nullptr;   // what the array uses
     void *base = nullptr;  // what hipMalloc returned
     size_t bytes = 0;
+    hipStream_t owner = nullptr;  // the stream whose free list the block returns to
+    // Hand-offs between threads: the stream that last wrote the block and the streams that have read it since.
+    // A thread that touches a block last used on another thread's stream first orders its own stream after that
+    // one (NdArray::will_read / will_write); the callers serialise their accesses, as the reference's borrow rules
+    // make them.  `constant`: written once, synchronously, before anyone else sees it (the shared zero).
+    std::mutex mu;
+    hipStream_t writer = nullptr;
+    std::vector<hipStream_t> readers;
+    bool constant = false;
     ~DeviceBlock();
 };
 
 namespace {
 // Large blocks start a rotating multiple of 4 KiB into their allocation.  hipMalloc hands out addresses with the
-// same low 21 bits, and an elementwise kernel that streams several such arrays in lockstep (Adam: param, grad, m, v)
-// then sends all of its streams to the same DRAM banks at the same time: 0.354 ms against 0.313 ms for the Adam
-// update of 2^26 elements with the arrays 4 KiB apart modulo 2 MiB.
+// same low 21 bits, and an elementwise kernel that streams several such arrays in lockstep then sends all of its
+// streams to the same DRAM banks at the same time (the pooling backward over gy, the tap bytes and gx moves
+// between 0.83 and 0.91 of its best with the placement).
 constexpr size_t kStaggerFrom = (size_t)1 << 20, kStaggerStep = 4096, kStaggerSlots = 16;
 
 struct Arena {
@@ -38,24 +114,26 @@ struct Arena {
         void *base, *ptr;
     };
     std::mutex mu;
-    std::multimap<size_t, Free> free_blocks;
+    std::map<hipStream_t, std::multimap<size_t, Free>> free_blocks;
     size_t next_slot = 0;
     ~Arena()
     {
-        for (auto &kv : free_blocks) (void)hipFree(kv.second.base);
+        for (auto &per_stream : free_blocks)
+            for (auto &kv : per_stream.second) (void)hipFree(kv.second.base);
     }
     static size_t round_up(size_t bytes)
     {
         const size_t q = bytes < (1u << 20) ? 256 : (1u << 16);
         return (bytes + q - 1) / q * q;
     }
-    bool take(size_t bytes, Free *out)
+    bool take(hipStream_t st, size_t bytes, Free *out)
     {
         std::lock_guard<std::mutex> lk(mu);
-        auto it = free_blocks.lower_bound(bytes);
-        if (it != free_blocks.end() && it->first <= bytes + bytes / 8) {
+        auto &list = free_blocks[st];
+        auto it = list.lower_bound(bytes);
+        if (it != list.end() && it->first <= bytes + bytes / 8) {
             *out = it->second;
-            free_blocks.erase(it);
+            list.erase(it);
             return true;
         }
         return false;
@@ -65,10 +143,10 @@ struct Arena {
         std::lock_guard<std::mutex> lk(mu);
         return (next_slot++ % kStaggerSlots) * kStaggerStep;
     }
-    void give(size_t bytes, Free f)
+    void give(hipStream_t st, size_t bytes, Free f)
     {
         std::lock_guard<std::mutex> lk(mu);
-        free_blocks.emplace(bytes, f);
+        free_blocks[st].emplace(bytes, f);
     }
 };
 Arena &arena()
@@ -76,16 +154,13 @@ Arena &arena()
     static Arena a;
     return a;
 }
-void check(hipError_t e, const char *what)
-{
-    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
-}
 std::shared_ptr<DeviceBlock> allocate(size_t bytes)
 {
     auto blk = std::make_shared<DeviceBlock>();
     blk->bytes = Arena::round_up(bytes ? bytes : 4);
+    blk->owner = blk->writer = t_stream.get();
     Arena::Free f;
-    if (arena().take(blk->bytes, &f)) {
+    if (arena().take(blk->owner, blk->bytes, &f)) {
         blk->base = f.base;
         blk->ptr = f.ptr;
         return blk;
@@ -105,12 +180,53 @@ size_t product(const Shape &s)
 
 DeviceBlock::~DeviceBlock()
 {
-    if (base) arena().give(bytes, Arena::Free{base, ptr});
+    if (!base) return;
+    // The block returns to its owner's list.  If other streams used it last, the owner must not reuse it before
+    // they are done: the thread that drops the last reference orders the owner after them here.
+    std::vector<hipStream_t> others;
+    if (writer && writer != owner) others.push_back(writer);
+    for (hipStream_t r : readers)
+        if (r != owner) others.push_back(r);
+    for (hipStream_t o : others) {
+        hipEvent_t ev = nullptr;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess) {
+            (void)hipEventRecord(ev, o);
+            (void)hipStreamWaitEvent(owner, ev, 0);
+            (void)hipEventDestroy(ev);
+        }
+    }
+    arena().give(owner, bytes, Arena::Free{base, ptr});
 }
 
-void *current_stream() { return nullptr; }  // the null stream: every op is ordered on it
+void NdArray::will_read() const
+{
+    if (!block_ || block_->constant) return;
+    hipStream_t mine = t_stream.get(), w;
+    {
+        std::lock_guard<std::mutex> lk(block_->mu);
+        w = block_->writer;
+        if (w == mine && block_->readers.empty()) return;  // the usual case: a thread's own array
+        if (std::find(block_->readers.begin(), block_->readers.end(), mine) == block_->readers.end()) block_->readers.push_back(mine);
+    }
+    if (w && w != mine) wait_for_stream(w);
+}
 
-void synchronize() { check(hipStreamSynchronize(nullptr), "hipStreamSynchronize"); }
+void NdArray::will_write() const
+{
+    if (!block_ || block_->constant) return;
+    hipStream_t mine = t_stream.get();
+    std::vector<hipStream_t> before;
+    {
+        std::lock_guard<std::mutex> lk(block_->mu);
+        if (block_->writer == mine && block_->readers.empty()) return;
+        if (block_->writer && block_->writer != mine) before.push_back(block_->writer);
+        for (hipStream_t r : block_->readers)
+            if (r != mine) before.push_back(r);
+        block_->writer = mine;
+        block_->readers.clear();
+    }
+    for (hipStream_t o : before) wait_for_stream(o);
+}
 
 size_t NdArray::len() const { return product(shape_); }
 
@@ -137,7 +253,13 @@ NdArray NdArray::zeros(const Shape &shape) { return filled(shape, 0.f); }
 
 NdArray NdArray::shared_zero()
 {
-    static const NdArray zero = zeros({});
+    // written once and complete before anyone else sees it: threads read it without ordering their streams
+    static const NdArray zero = [] {
+        NdArray z = zeros({});
+        synchronize();
+        z.block_->constant = true;
+        return z;
+    }();
     return zero;
 }
 
@@ -153,7 +275,10 @@ class StagingRing {
     static constexpr size_t kBytes = 16u << 20;
     ~StagingRing()
     {
-        if (base_) (void)hipHostFree(base_);
+        if (base_) {
+            (void)hipStreamSynchronize(stream_);  // transfers out of the ring may still be in flight when a thread ends
+            (void)hipHostFree(base_);
+        }
         if (drained_) (void)hipEventDestroy(drained_);
     }
     // Device-to-host through the same ring; returns after the data has arrived in `dst`.
@@ -205,8 +330,10 @@ class StagingRing {
         if (base_) return;
         check(hipHostMalloc(&base_, kBytes, hipHostMallocDefault), "hipHostMalloc");
         check(hipEventCreateWithFlags(&drained_, hipEventDisableTiming), "hipEventCreate");
+        stream_ = static_cast<hipStream_t>(current_stream());
     }
     std::mutex mu_;
+    hipStream_t stream_ = nullptr;
     void *base_ = nullptr;
     hipEvent_t drained_ = nullptr;
     size_t used_ = 0;
@@ -214,7 +341,9 @@ class StagingRing {
 };
 StagingRing &staging()
 {
-    static StagingRing r;
+    // one ring per host thread, like the stream its transfers are ordered on: a slot is reused once the
+    // transfers that THIS thread enqueued have left it
+    thread_local StagingRing r;
     return r;
 }
 }  // namespace
@@ -228,6 +357,7 @@ NdArray NdArray::from_host(const Shape &shape, const float *data)
 
 void NdArray::copy_from_host(const float *data)
 {
+    will_write();
     if (len()) staging().upload(ptr(), data, len() * sizeof(float));
 }
 
@@ -242,6 +372,7 @@ NdArray NdArray::reshaped(const Shape &shape) const
 NdArray NdArray::deep_copy() const
 {
     NdArray a = empty(shape_);
+    will_read();
     if (len())
         check(hipMemcpyAsync(a.ptr(), ptr(), len() * sizeof(float), hipMemcpyDeviceToDevice,
                              static_cast<hipStream_t>(current_stream())),
@@ -252,6 +383,7 @@ NdArray NdArray::deep_copy() const
 std::vector<float> NdArray::to_host() const
 {
     std::vector<float> out(len());
+    will_read();
     if (len()) staging().download(out.data(), ptr(), len() * sizeof(float));
     else synchronize();
     return out;
@@ -271,6 +403,7 @@ NdArray ComputeContext::input(size_t i)
         throw Panic("Bad op impl: input(" + std::to_string(i) + ")/input_mut(" + std::to_string(i) +
                     ") cannot be called twice");
     x.taken = true;
+    x.array.will_read();
     return x.array;
 }
 
@@ -284,6 +417,7 @@ NdArray ComputeContext::input_mut(size_t i)
         throw Panic("Bad op impl: input(" + std::to_string(i) + ")/input_mut(" + std::to_string(i) +
                     ") cannot be called twice");
     x.taken = true;
+    x.array.will_write();
     return x.array;
 }
 

@@ -708,6 +708,88 @@ def test_updates_that_do_not_wait_for_the_device_equal_waiting_ones(G, rng):
     assert np.array_equal(b1.view(np.uint32), b2.view(np.uint32))
 
 
+def _small_training(G, seed, steps=25):
+    r = np.random.default_rng(seed)
+    env = G.VariableEnvironment()
+    wid = env.set("w", r.standard_normal((8, 1, 3, 3)).astype(np.float32) * 0.3)
+    bid = env.set("b", np.zeros((1, 8, 1, 1), np.float32))
+    adam = G.Adam(env, [wid, bid], alpha=0.01)
+    for step in range(steps):
+        xv = r.standard_normal((16, 1, 12, 12)).astype(np.float32)
+        c = env.context()
+        w, b = c.variable(wid), c.variable(bid)
+        x = c.placeholder("x", [-1, 1, 12, 12])
+        loss = c.sum_all(c.max_pool2d(c.relu(c.conv2d(x, w, 1, 1) + b), 2, 0, 2))
+        gw, gb = c.grad([loss], [w, b])
+        adam.update([w, b], [gw, gb], c, {"x": xv})
+    return env.array(wid), env.array(bid)
+
+
+def test_four_host_threads_train_at_once_each_on_its_own_stream(G):
+    """Every host thread that evaluates graphs has a stream, a staging ring and arena lists of its own (the
+    reference's graphs live on one thread each, src/graph.rs:17-47).  Four threads train four small models at the
+    same time; each must end with exactly the bits of the same training run alone."""
+    import threading
+    want = {seed: _small_training(G, seed) for seed in range(4)}
+    got, errors = {}, []
+
+    def work(seed):
+        try:
+            got[seed] = _small_training(G, seed)
+        except Exception as e:                       # a failure in a thread must fail the test, not vanish
+            errors.append((seed, repr(e)[:300]))
+
+    say("four host threads, four trainings through the host layer")
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for seed in range(4):
+        for a, b in zip(got[seed], want[seed]):
+            assert np.isfinite(a).all() and np.array_equal(a.view(np.uint32), b.view(np.uint32)), f"thread {seed}"
+
+
+def test_arrays_handed_from_one_thread_to_another_are_ordered(G, orc):
+    """An environment created on one thread, trained on a second and read on the first: each thread's work is ordered
+    on its own stream, and an array that another thread's stream used last makes the next user wait for that stream
+    (no host synchronisation is needed between the hand-offs beyond joining the thread)."""
+    import threading
+    r = np.random.default_rng(3)
+    env = G.VariableEnvironment()
+    wv = r.standard_normal((64, 512)).astype(np.float32)
+    wv = (np.sign(wv) * (4.0 + np.abs(wv))).astype(np.float32)   # far from zero: three steps of 0.5 keep the sign
+    wid = env.set("w", wv)                      # uploaded on the main thread's stream, not waited for
+    adam = G.Adam(env, [wid], alpha=0.5)
+    errors = []
+
+    def work():
+        try:
+            for _ in range(3):
+                c = env.context()
+                w = c.variable(wid)
+                (gw,) = c.grad([c.sum_all(c.mul(w, w))], [w])
+                adam.update([w], [gw], c)       # returns once enqueued on the worker's stream
+        except Exception as e:
+            errors.append(repr(e)[:300])
+
+    say("environment handed between two threads")
+    t = threading.Thread(target=work)
+    t.start()
+    t.join()
+    assert not errors, errors
+    c = env.context()                           # back on the main thread: reads what the worker's stream wrote
+    w = c.variable(wid)
+    (sq,) = c.eval([c.mul(w, w)])
+    final = env.array(wid)
+    p, m, v, t = wv.copy(), np.zeros_like(wv), np.zeros_like(wv), np.ones(1, np.float32)
+    for _ in range(3):
+        orc.adam(p, (p + p).astype(np.float32), m, v, t, alpha=0.5)
+    assert_close(final, p, "w after three steps on another thread")
+    assert np.abs(final - wv).min() > 0.1 and np.array_equal(sq, final * final)
+
+
 def test_batched_adam_updates_keep_the_evaluation_order(G, orc, rng):
     """The AdamOp nodes of one evaluation go out as one launch, but a node that reads a variable after its
     AdamOp ran must see the updated array, exactly as if every update had run at its own node.  The evaluator
