@@ -572,9 +572,10 @@ def micro_elementwise(torch, Kn, dev, g, iters=10):
     ms = time_events(torch, lambda: Kn.add_broadcast_relu(x, bias), iters)
     res["add_bias_relu_[256,128,56,56]"] = hbm_entry("add_bias_relu_[256,128,56,56]", ms, 2 * nb,
                                                      "relu(x + b) with b [1,128,1,1] in one pass")
-    ms = time_events(torch, lambda: Kn.bias_grad(gy), iters)
-    res["bias_grad_[256,128,56,56]"] = hbm_entry("bias_grad_[256,128,56,56]", ms, nb,
-                                                 "MaybeReduceSum of the gradient of a [1,128,1,1] bias: sum over axes 0, 2, 3")
+    ms = time_events(torch, lambda: Kn.add_n([x, gy]), iters)
+    res["add_n_2x[256,128,56,56]"] = hbm_entry("add_n_2x[256,128,56,56]", ms, 3 * nb,
+                                               "AddN of two gradients (also AddOp of equal shapes); the gradient of a [1,128,1,1] "
+                                               "bias is the entry reduce_sum_[256,128,56,56]_axes_0_2_3")
     return res
 
 

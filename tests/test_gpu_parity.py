@@ -1663,7 +1663,10 @@ def test_broadcast_grad(K, orc, rng):
 
 
 # =============================================================================== Adam
-@pytest.mark.parametrize("n", [1, 10, 288, 18432, 31360, 100003])
+# (from 2^20 elements on whole runs of 16384 elements go through the form whose streams are skewed in time: exactly
+# 2^20, runs plus a tail of whole quads, runs plus a partial quad, and a tail of one element)
+@pytest.mark.parametrize("n", [1, 10, 288, 18432, 31360, 100003, 1 << 20, (1 << 20) + 3 * 16384 + 4096, (1 << 21) + 16384 + 1027,
+                               (1 << 20) + 1])
 def test_adam_matches_oracle_over_steps(K, orc, rng, n):
     p = rng.standard_normal(n).astype(np.float32)
     m, v, t = np.zeros(n, np.float32), np.zeros(n, np.float32), np.array([1.0], np.float32)
@@ -1683,7 +1686,7 @@ def test_adam_matches_oracle_over_steps(K, orc, rng, n):
 def test_adam_several_parameters_in_one_launch(K, rng):
     """ag_adam_update_multi_f32 against one ag_adam_update_f32 per parameter: bit-identical param, m, v and t
     over three steps; sizes with partial quads, one element, an empty parameter and a misaligned one."""
-    sizes = [25088, 1, 0, 4099, 288, 31360, 10, 7]
+    sizes = [25088, 1, 0, 4099, 288, 31360, 10, 7, (1 << 20) + 16384 + 777]   # the last one takes the run form
     def fresh():
         r = np.random.default_rng(3)
         ps = [dev(r.standard_normal(n + 1).astype(np.float32)) for n in sizes]
