@@ -309,26 +309,29 @@ struct PrepareExtras {
 // The same copy with the divisions replaced by multiplications: grid.y walks the images, so the
 // element counter stays small enough for n / d == umulhi(n, floor(2^32 / d) + 1) to be exact (the
 // host checks the range).  gyp [B][planes][Hp][Wp]; quads_img = planes * Hp * Wp / 4.
-// The last row of the grid (blockIdx.y == gridDim.y - 1) copies nothing: it does the two small jobs that go with
-// every bordered copy -- zeroing the slack around the planes and writing the filter in the tap order of the
-// implicit GEMM -- so that preparing an operand is one launch.
+// The same launch does the two small jobs that go with every bordered copy -- zeroing the slack around the planes
+// and writing the filter in the tap order of the implicit GEMM -- so that preparing an operand is one launch.  They
+// are dealt out over the threads of the whole grid, one element (or a few) each: the filter is gathered at a
+// stride of a whole filter row, a load per element that waits out the memory latency, and 590 k elements (256 ->
+// 256 channels, 3 x 3) in the hands of one grid row of 72 blocks took 15 us where the copy itself takes 5.
 __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__restrict__ gy, float *__restrict__ gyp,
                                                               unsigned quads_img, unsigned planes, int OH, int OW, int Wp,
                                                               int top, int left, unsigned plane_quads, unsigned m_plane,
                                                               unsigned m_row, int B, PrepareExtras ex)
 {
-    const unsigned ny = gridDim.y - 1;
-    if (blockIdx.y == ny) {
-        const int tid = (int)(blockIdx.x * 256u + threadIdx.x), nth = (int)(gridDim.x * 256u);
-        for (int i = tid; i < ex.n_lead + ex.n_tail; i += nth) {
-            if (i < ex.n_lead) ex.lead[i] = 0.f;
-            else ex.tail[i - ex.n_lead] = 0.f;
+    const unsigned ny = gridDim.y;
+    {
+        const long long gt = ((long long)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        const int slack = ex.n_lead + ex.n_tail, total = slack + (ex.wt ? ex.Kf * ex.C * ex.taps : 0);
+        if (gt < total) {
+            const long long nth = (long long)gridDim.x * gridDim.y * 256;
+            for (long long i = gt; i < total; i += nth) {
+                if (i < ex.n_lead) ex.lead[i] = 0.f;
+                else if (i < slack) ex.tail[i - ex.n_lead] = 0.f;
+                else ex.wt[i - slack] = ex.fwd ? filter_tap_fwd(ex.w, (int)(i - slack), ex.C, ex.taps)
+                                               : filter_tap(ex.w, (int)(i - slack), ex.Kf, ex.C, ex.taps);
+            }
         }
-        if (ex.wt) {
-            const int total = ex.Kf * ex.C * ex.taps;
-            for (int e = tid; e < total; e += nth) ex.wt[e] = ex.fwd ? filter_tap_fwd(ex.w, e, ex.C, ex.taps) : filter_tap(ex.w, e, ex.Kf, ex.C, ex.taps);
-        }
-        return;
     }
     const unsigned qi = blockIdx.x * 256u + threadIdx.x;
     if (qi >= quads_img) return;
@@ -367,9 +370,9 @@ static bool launch_pad_border_with(hipStream_t st, const float *src, float *dst,
     if (fast) {
         const unsigned m_plane = (unsigned)((1ULL << 32) / (unsigned long long)plane_quads) + 1u;
         const unsigned m_row = (unsigned)((1ULL << 32) / (unsigned long long)Wp) + 1u;
-        // one grid row per image (at most 65534) plus the row of the small jobs
-        const dim3 grid((unsigned)((quads_img + 255) / 256), (unsigned)(B < 65534 ? B : 65534) + 1u);
-        const bool fits = extras && (!extras->wt || (long long)extras->Kf * extras->C * extras->taps < 0x7fffffffLL);
+        // one grid row per image (at most 65534)
+        const dim3 grid((unsigned)((quads_img + 255) / 256), (unsigned)(B < 65534 ? B : 65534));
+        const bool fits = extras && (!extras->wt || (long long)extras->Kf * extras->C * extras->taps < 0x7ffff000LL);
         PrepareExtras ex = {};
         if (fits) ex = *extras;
         hipLaunchKernelGGL(pad_border_fast_kernel, grid, dim3(256), 0, st, src, dst, (unsigned)quads_img, (unsigned)planes, OH, OW,
@@ -421,7 +424,8 @@ constexpr long long kSlackFloats = 1024;
 // Geometry of the implicit (column-free) stride-1 input gradient.
 struct FusedGeom {
     int Hp, Wp;
-    long long gyp_floats, wr_floats;  // scratch layout: zero-bordered gy, then the tap-major filter
+    long long gyp_floats, wr_floats;  // scratch layout: zero-bordered gy, then the tap-major filter,
+    long long ws_floats;              // then the partial results of a split contraction (0: none)
 };
 
 // False when the geometry does not allow the implicit path.
@@ -461,6 +465,7 @@ static bool fused_geom(int B, int ych, int yh, int yw, int xch, int kh, int kw, 
     const long long plane = (long long)g->Hp * g->Wp, n_img = (long long)xh * g->Wp;
     g->gyp_floats = (long long)B * ych * plane + kSlackFloats;  // slack: the last taps read a little past a plane
     g->wr_floats = (long long)xch * kh * kw * ych;
+    g->ws_floats = (long long)gemm_conv_input_grad_ws_floats(B, xch, ych, xh, xw, g->Wp, kh * kw);
     // a tile may cover any number of images; the loader's 32-bit byte offsets reach over a k tile's 32 planes and as many
     // images further as a tile of up to 256 columns can run into
     const long long more_imgs = n_img >= 256 ? 1 : 256 / n_img + 1;
@@ -537,7 +542,7 @@ extern "C" size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, in
     }
     FusedGeom g;
     if (!fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation)) return 0;
-    return (size_t)(kFwdLeadFloats + g.gyp_floats + g.wr_floats);
+    return (size_t)(kFwdLeadFloats + g.gyp_floats + g.wr_floats + g.ws_floats);
 }
 
 // The two stages of the forward, for callers that time or schedule them separately.
@@ -584,8 +589,10 @@ extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float
     AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
     const float *xp = xpad + kFwdLeadFloats;
+    float *ws = const_cast<float *>(xp) + g.gyp_floats + g.wr_floats;  // (the part of xpad behind the filter: transient)
     return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - dilation * (kh - 1),
-                                W + 2 * pad - dilation * (kw - 1), kh, kw, g.Hp, g.Wp, dilation);
+                                W + 2 * pad - dilation * (kw - 1), kh, kw, g.Hp, g.Wp, dilation, g.ws_floats ? ws : nullptr,
+                                (size_t)g.ws_floats);
 }
 
 extern "C" ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y, float *xpad,
@@ -699,8 +706,11 @@ extern "C" ag_status_t ag_conv2d_transpose_f32(ag_stream_t stream, const float *
         fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &fg, dilation) && fg.gyp_floats + fg.wr_floats <= (long long)B * M * P &&
         ((long long)xh * fg.Wp >= 256 || xch <= 64 || (long long)B * M * P >= (1LL << 24)) && aligned16(gcols) && aligned16(gx)) {
         if (ag_status_t s = fused_prepare(as_stream(stream), gy, w, gcols, fg, B, ych, yh, yw, xch, kh, kw, pad, dilation)) return s;
+        // (what the column buffer has left behind the bordered gradient and the filter serves a split contraction)
+        const bool room = fg.ws_floats > 0 && fg.gyp_floats + fg.wr_floats + fg.ws_floats <= (long long)B * M * P;
         return gemm_conv_input_grad(as_stream(stream), gcols + fg.gyp_floats, gcols, gx, B, xch, ych, xh, xw, kh, kw, fg.Hp,
-                                    fg.Wp, dilation);
+                                    fg.Wp, dilation, room ? gcols + fg.gyp_floats + fg.wr_floats : nullptr,
+                                    room ? (size_t)fg.ws_floats : 0);
     }
     // Stride 2: parity GEMMs over one bordered copy of gy (conv_s2.hip), when the columns' buffer
     // is large enough to serve as their scratch.  Only from 2^24 column elements on: below that the
@@ -762,7 +772,7 @@ extern "C" size_t ag_conv_input_grad_scratch_floats(int B, int ych, int yh, int 
         return (size_t)(g2.gyp_floats + g2.wf_floats + g2.gxp_floats);
     }
     FusedGeom g;
-    return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) ? (size_t)(g.gyp_floats + g.wr_floats) : 0;
+    return fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) ? (size_t)(g.gyp_floats + g.wr_floats + g.ws_floats) : 0;
 }
 
 extern "C" ag_status_t ag_conv_input_grad_prepare_f32(ag_stream_t stream, const float *gy, const float *w, float *scratch,
@@ -801,5 +811,5 @@ extern "C" ag_status_t ag_conv_input_grad_gemm_f32(ag_stream_t stream, float *sc
     AG_REQUIRE(fused_geom(B, ych, yh, yw, xch, kh, kw, pad, xh, xw, &g, dilation) && aligned16(scratch) && aligned16(gx),
                AG_ERR_INVALID_DIMS, "conv_input_grad_gemm: geometry not supported by the column-free path");
     return gemm_conv_input_grad(as_stream(stream), scratch + g.gyp_floats, scratch, gx, B, xch, ych, xh, xw, kh, kw, g.Hp,
-                                g.Wp, dilation);
+                                g.Wp, dilation, g.ws_floats ? scratch + g.gyp_floats + g.wr_floats : nullptr, (size_t)g.ws_floats);
 }

@@ -941,9 +941,18 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
 // `phase` != 0: stride-2 forward over four phase planes of `phase` elements per contracted channel.
 // `pair_w` != 0: the pair form of the stride-2 input gradient (C counts the 2 x channels rows; the output planes are
 // pair_h x pair_w and receive row parity pair_a).
+// Tile and split of one implicit convolution product (M = C output rows, N = B * H * Wp padded columns, contraction
+// over taps x Kf).  `splits` > 1: the walk over the Kf / 32 channel groups is cut into that many ranges whose partial
+// results (each laid out like the output) a fixed-order fold adds up -- for products with fewer tiles than the chip
+// has room for, where a slice of the contraction per block keeps every CU busy.
+struct ImplicitPlan {
+    int cfg, splits;
+};
+static ImplicitPlan implicit_plan(int B, int C, int Kf, int H, int Wp, int taps, unsigned phase, int pair_w, bool may_split);
+
 static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
                                       int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase, int pair_w = 0,
-                                      int pair_a = 0, int pair_h = 0, int dil = 1)
+                                      int pair_a = 0, int pair_h = 0, int dil = 1, float *ws = nullptr, size_t ws_floats = 0)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
@@ -967,42 +976,29 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     }
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
     p.rows_plane = p.rows_phase = 0;
-    // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
-    // CU); else 128 x 256 (128 x 128 when an image has fewer than 256 columns) or 64 x 128, whichever needs less
-    // time by rounds of the persistent grid times the cost of a tile: padding rows and the idle part of a last
-    // round cost as much as real work (B = 128, 64 -> 192 channels, 28 x 28: 0.30 ms on 128 x 256 tiles -- 256
-    // rows in 3.2 rounds -- against 0.21 ms on 64 x 128 ones)
-    int cfg = C <= 32 ? kDirectCfg32 : kDirectCfg64;
-    if (C > 32 && C <= 64) {
-        // (the stride-2 forms keep to tiles that cover at most two images)
-        if (cdiv(p.N, 128) < 2 * direct_grid(num_cus()) && (p.n_img >= 64 || (phase == 0 && pair_w == 0))) cfg = kDirectCfg64Narrow;
-    } else if (C > 64) {
-        const long long G = direct_grid(num_cus());
-        const int wide = p.n_img >= 256 ? 14 : 13;
-        const long long wide_tiles = cdiv(C, 128) * cdiv(p.N, kCfgs[wide].bn);
-        double wide_rounds = (double)cdiv(wide_tiles, G);
-        if (wide == 14 && C <= 128 && wide_tiles > G && wide_tiles % G != 0)  // the narrow-tile tail launch below
-            wide_rounds = (double)(wide_tiles / G) + 0.3;
-        const double wide_cost = wide_rounds * 128.0 * kCfgs[wide].bn / (wide == 14 ? 1.0 : 0.9);
-        const double small_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 128), 2 * G) * 2.0 * 64.0 * 128.0 / 0.95;
-        cfg = wide_cost <= small_cost ? wide : kDirectCfg64;
-        // a problem of less than a round of those: 64 x 64 tiles (32 x 256 -> 256 channels, 14 x 14: 0.100 against
-        // 0.108 ms)
-        const double narrow_cost = (double)cdiv(cdiv(C, 64) * cdiv(p.N, 64), 2 * G) * 2.0 * 64.0 * 64.0 / 0.78;
-        if (narrow_cost < 0.9 * (wide_cost <= small_cost ? wide_cost : small_cost)) cfg = kDirectCfg64Narrow;
+    const long long out_floats = pair_w != 0 ? (long long)B * (C / 2) * pair_h * pair_w : (long long)B * C * H * W;
+    const ImplicitPlan plan = implicit_plan(B, C, Kf, H, Wp, kh * kw, phase, pair_w,
+                                            ws != nullptr && phase == 0 && pair_w == 0 && out_floats < 0x7fffffffLL &&
+                                                ws_floats >= 2 * (size_t)out_floats);
+    const int cfg = plan.cfg;
+    p.kb_per_split = (int)cdiv(Kf / 32, plan.splits);
+    p.splits = (int)cdiv(Kf / 32, p.kb_per_split);
+    if ((size_t)p.splits * (size_t)out_floats > ws_floats) {  // (a forced split count the workspace cannot hold)
+        p.splits = 1;
+        p.kb_per_split = Kf / 32;
     }
-    if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && (pair_w == 0 && phase == 0 || kCfgs[g_force_cfg].bn <= p.n_img))
-        cfg = g_force_cfg;  // test hook
+    p.sCsplit = out_floats;
+    if (p.splits > 1) p.C = ws;
     p.tiles_m = (int)cdiv(C, kCfgs[cfg].bm);
     p.tiles_n = (int)cdiv(p.N, kCfgs[cfg].bn);
     const long long blocks = (long long)p.tiles_m * p.tiles_n;
-    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "conv2d_transpose: too many tiles (%lld)", blocks);
-    p.total_blocks = (unsigned)blocks;
+    AG_REQUIRE(blocks * p.splits <= kMaxGridX, AG_ERR_INVALID_DIMS, "conv2d_transpose: too many tiles (%lld)", blocks);
+    p.total_blocks = (unsigned)(blocks * p.splits);
     // whole rounds of the persistent grid with the wide tile, then the remaining columns with a
     // narrower one (as for the folded GEMM over columns)
     int tail_cfg = -1;
     GemmParams tail = p;
-    if (cfg == 14 && p.tiles_m == 1 && g_grid_scale <= 0) {
+    if (cfg == 14 && p.tiles_m == 1 && g_grid_scale <= 0 && p.splits == 1) {
         const long long G = direct_grid(num_cus());
         const long long rounds = blocks / G, rem = blocks % G;
         if (rounds >= 1 && rem > 0) {
@@ -1036,13 +1032,88 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
         launch_direct(st, tail_cfg, true, false, tail, num_cus(), g_grid_scale);
         return check_launch("conv2d_transpose");
     }
+    if (p.splits > 1) {  // the partial results, slot after slot in ascending order of the channel groups
+        launch_fold(st, ws, p.splits, out_floats, gx, 1, (int)out_floats, out_floats, 1.f, 0.f);
+        return check_launch("conv2d_transpose");
+    }
     return AG_OK;
 }
 
-ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
-                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil)
+static ImplicitPlan implicit_plan(int B, int C, int Kf, int H, int Wp, int taps, unsigned phase, int pair_w, bool may_split)
 {
-    return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0, 0, 0, 0, dil);
+    const int n_img = H * Wp;
+    const long long N = (long long)B * n_img;
+    // 32 x 128 for up to 32 output rows; 64 x 128 for up to 64 (64 x 64 while that gives fewer than two blocks per
+    // CU); else 128 x 256 (128 x 128 when an image has fewer than 256 columns) or 64 x 128, whichever needs less
+    // time by rounds of the persistent grid times the cost of a tile: padding rows and the idle part of a last
+    // round cost as much as real work (B = 128, 64 -> 192 channels, 28 x 28: 0.30 ms on 128 x 256 tiles -- 256
+    // rows in 3.2 rounds -- against 0.21 ms on 64 x 128 ones)
+    int cfg = C <= 32 ? kDirectCfg32 : kDirectCfg64;
+    // Fewer 64-row tiles than fill the chip: each block takes a slice of the contraction instead of all of it (a
+    // range of the Kf / 32 channel groups; partial results folded in a fixed order), as many slices as give about a
+    // block per CU.  256 -> 256 channels, 14 x 14, dilation 2: 4 / 8 / 16 images 54 / 56 / 58 us whole, 23 / 33 / 55 us
+    // sliced by 8 / 4 / 2; 8 images of 512 -> 512 channels at 7 x 7: 101 -> 33 us.  From about a block per CU on
+    // slicing loses to whole contractions (32 images: 85 us whole on 64 x 128 tiles, 90 sliced by 2, 93 on 64 x 64 tiles).
+    const int groups = Kf / 32;
+    if (may_split && g_force_cfg < 0 && g_force_splits <= 0 && C > 32 && groups >= 2) {
+        const long long G = direct_grid(num_cus());
+        const int tile = C <= 64 ? kDirectCfg64Narrow : kDirectCfg64;
+        const long long blocks = cdiv(C, 64) * cdiv(N, kCfgs[tile].bn);
+        if (blocks * 5 < G * 3) {
+            long long want = cdiv(G * 4, blocks * 5);
+            if (want > 8) want = 8;
+            if (want > groups) want = groups;
+            const int per = (int)cdiv(groups, want);
+            return ImplicitPlan{tile, (int)cdiv(groups, per)};
+        }
+    }
+    if (C > 32 && C <= 64) {
+        // (the stride-2 forms keep to tiles that cover at most two images)
+        if (cdiv(N, 128) < 2 * direct_grid(num_cus()) && (n_img >= 64 || (phase == 0 && pair_w == 0))) cfg = kDirectCfg64Narrow;
+    } else if (C > 64) {
+        const long long G = direct_grid(num_cus());
+        const int wide = n_img >= 256 ? 14 : 13;
+        const long long wide_tiles = cdiv(C, 128) * cdiv(N, kCfgs[wide].bn);
+        double wide_rounds = (double)cdiv(wide_tiles, G);
+        if (wide == 14 && C <= 128 && wide_tiles > G && wide_tiles % G != 0)  // the narrow-tile tail launch below
+            wide_rounds = (double)(wide_tiles / G) + 0.3;
+        const double wide_cost = wide_rounds * 128.0 * kCfgs[wide].bn / (wide == 14 ? 1.0 : 0.9);
+        const double small_cost = (double)cdiv(cdiv(C, 64) * cdiv(N, 128), 2 * G) * 2.0 * 64.0 * 128.0 / 0.95;
+        cfg = wide_cost <= small_cost ? wide : kDirectCfg64;
+        // a problem of less than a round of those: 64 x 64 tiles (32 x 256 -> 256 channels, 14 x 14: 0.100 against
+        // 0.108 ms)
+        // (only while the 64 x 128 tiles leave the chip well under a block per CU: with 224 of them on 256 CUs they
+        // take 85 us where 448 tiles of 64 x 64 take 93)
+        const double narrow_cost = (double)cdiv(cdiv(C, 64) * cdiv(N, 64), 2 * G) * 2.0 * 64.0 * 64.0 / 0.78;
+        if (narrow_cost < 0.9 * (wide_cost <= small_cost ? wide_cost : small_cost) && cdiv(C, 64) * cdiv(N, 128) * 5 < G * 3)
+            cfg = kDirectCfg64Narrow;
+    }
+    if (g_force_cfg >= kFirstDirectCfg && g_force_cfg < kNumCfgs && g_force_cfg != kDirectCfg32 && (pair_w == 0 && phase == 0 || kCfgs[g_force_cfg].bn <= n_img))
+        cfg = g_force_cfg;  // test hook
+    int splits = 1;
+    if (g_force_splits > 0 && may_split) splits = g_force_splits < Kf / 32 ? g_force_splits : Kf / 32;  // test hook
+    (void)taps;
+    return ImplicitPlan{cfg, splits};
+}
+
+// Floats of workspace that gemm_conv_input_grad wants for the partial results of a split contraction (0: it
+// will not split).
+size_t gemm_conv_input_grad_ws_floats(int B, int C, int Kf, int H, int W, int Wp, int taps)
+{
+    const long long out = (long long)B * C * H * W;
+    if (Kf < 64 || out >= (1LL << 26)) return 0;
+#ifdef AG_TEST_HOOKS
+    return (size_t)out * 8;  // room for forced split counts
+#else
+    const ImplicitPlan plan = implicit_plan(B, C, Kf, H, Wp, taps, 0, 0, true);
+    return plan.splits > 1 ? (size_t)out * plan.splits : 0;
+#endif
+}
+
+ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil, float *ws, size_t ws_floats)
+{
+    return conv_implicit_gemm(st, wr, gyp, gx, B, C, Kf, H, W, kh, kw, Hp, Wp, 0, 0, 0, 0, dil, ws, ws_floats);
 }
 
 ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,

@@ -269,7 +269,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         if (p.n_img != 0) {
             it.bz = it.n0 / p.n_img;
             it.r0 = it.n0 - it.bz * p.n_img;
-            it.sp = 0;
+            it.sp = c.z;  // (only the tap walks are ever split: groups of 32 contracted channels)
         } else if (p.splits == 1) {
             it.bz = c.z;
             it.sp = 0;
@@ -278,7 +278,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             it.sp = c.z % p.splits;
         }
         it.kb0 = it.sp * p.kb_per_split;
-        it.nt = (min(p.kbatch, it.kb0 + p.kb_per_split) - it.kb0) * kt_per;
+        if (taps) {
+            // A tap walk visits every tap for one group of 32 contracted channels, then the next group: a split owns
+            // kb_per_split consecutive groups (all of them when the walk is not split).
+            it.nt = (min(kt_per, it.kb0 + p.kb_per_split) - it.kb0) * p.kbatch;
+        } else {
+            it.nt = (min(p.kbatch, it.kb0 + p.kb_per_split) - it.kb0) * kt_per;
+        }
         return it;
     };
 
@@ -310,8 +316,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         } else {
             ldr_b.init(ldb, it.n0, p.N, wave, lane);
         }
-        pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
-        pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
+        if (taps) {
+            // (first channel group of this split: 32 elements along A's rows, 32 planes of B)
+            pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * BK;
+            pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * step_b;
+        } else {
+            pa = p.A + (long long)it.bz * p.sA + (long long)it.kb0 * p.sAk;
+            pb = p.B + (long long)it.bz * p.sB + (long long)it.kb0 * p.sBk;
+        }
         if (taps) {  // first tap (0, 0): the largest shift (input gradient), or phase (0, 0) unshifted
             pb_group = pb;
             pb += conv_first_shift;
@@ -475,8 +487,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         long long ldc;
         float alpha, beta;
         if (p.splits > 1) {
+            // partial sums: slot it.sp of the workspace, laid out like the output itself for the tap walks
             Cb = p.C + (long long)it.bz * p.sC + (long long)it.sp * p.sCsplit;
-            ldc = p.N;
+            ldc = taps ? p.ldc : p.N;
             alpha = 1.f;
             beta = 0.f;
         } else {

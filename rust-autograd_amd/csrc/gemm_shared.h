@@ -77,8 +77,12 @@ size_t gemm_conv_filter_grad_workspace(int B, int Kf, int C, int taps, int kq);
 ag_status_t gemm_conv_filter_grad(hipStream_t st, const float *gyp, const float *xp, float *gw, void *ws, size_t ws_bytes,
                                   int B, int Kf, int C, int kh, int kw, int border, int Hp_gy, int Hp_x, int Wp, int kq,
                                   int dil = 1);
+// `ws` / `ws_floats`: room for the partial results of a split contraction (gemm_conv_input_grad_ws_floats; may be
+// null, then the contraction is not split).
 ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C,
-                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil = 1);
+                                 int Kf, int H, int W, int kh, int kw, int Hp, int Wp, int dil = 1, float *ws = nullptr,
+                                 size_t ws_floats = 0);
+size_t gemm_conv_input_grad_ws_floats(int B, int C, int Kf, int H, int W, int Wp, int taps);
 // Stride-2 forward over phase planes (see GemmParams::conv_phase): wf [K][kh*kw][C] in natural tap
 // order, xph [B][C][4][Hpp][Wpp], y [B][K][OH][OW].
 // The pair form of the implicit input gradient (see GemmParams::conv_pair_w): wr [2C][kh*kw*Kf], gyp bordered

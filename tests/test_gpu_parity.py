@@ -844,9 +844,9 @@ def test_conv2d_column_free_dilated(K, orc, rng, case):
         assert np.array_equal(host(gwi), host(K.conv2d_filter_grad(colsi, dev(gyi), wi.shape)))
 
 
-@pytest.mark.parametrize("cfg", [13, 14, 18, 19, 21])
+@pytest.mark.parametrize("cfg,splits", [(13, 0), (14, 0), (18, 0), (19, 0), (21, 0), (13, 2), (15, 3), (19, 2), (21, 3)])
 @pytest.mark.parametrize("d", [1, 2])
-def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d, hooked):
+def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, splits, d, hooked):
     # the implicit forward and input gradient on each tile shape of the direct-to-LDS kernel that they can run
     # on (the library picks one by channel count and size): integer-valued data, bit for bit the columns path
     B, C, Kc, H, W, k = 3, 64, 96, 22, 26, 3
@@ -857,13 +857,17 @@ def test_conv2d_column_free_exact_with_every_tile_shape(K, rng, cfg, d, hooked):
     gy = rng.integers(-2, 3, (B, Kc, H, W)).astype(np.float32)
     y_cols, _ = K.conv2d(dev(x), dev(w), p, 1, d)
     gx_cols, _ = K.conv2d_transpose(dev(gy), dev(w), p, 1, d, out_hw=(H, W), return_cols=True)
-    say("column-free with a forced tile shape", (cfg, d))
+    # (splits > 0: the walk over the groups of 32 contracted channels is cut into that many ranges, whose partial
+    # results a fixed-order fold adds up -- 2 groups for the forward's 64 channels, 3 for the gradient's 96 filters)
+    say("column-free with a forced tile shape", (cfg, splits, d))
     L.ag_test_gemm_force_config(cfg)
+    L.ag_test_gemm_force_splits(splits)
     try:
         y, _ = K.conv2d_nocols(dev(x), dev(w), p, 1, d)
         gx, _ = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, W), 1, d)
     finally:
         L.ag_test_gemm_force_config(-1)
+        L.ag_test_gemm_force_splits(0)
     assert np.array_equal(host(y), host(y_cols))
     assert np.array_equal(host(gx), host(gx_cols))
 
@@ -1663,9 +1667,9 @@ def test_broadcast_grad(K, orc, rng):
 
 
 # =============================================================================== Adam
-# (from 2^20 elements on whole runs of 16384 elements go through the form whose streams are skewed in time: exactly
+# (from 2^20 elements on whole runs of 4096 elements go through the form whose streams are skewed in time: exactly
 # 2^20, runs plus a tail of whole quads, runs plus a partial quad, and a tail of one element)
-@pytest.mark.parametrize("n", [1, 10, 288, 18432, 31360, 100003, 1 << 20, (1 << 20) + 3 * 16384 + 4096, (1 << 21) + 16384 + 1027,
+@pytest.mark.parametrize("n", [1, 10, 288, 18432, 31360, 100003, 1 << 20, (1 << 20) + 3 * 4096 + 1024, (1 << 21) + 4096 + 1027,
                                (1 << 20) + 1])
 def test_adam_matches_oracle_over_steps(K, orc, rng, n):
     p = rng.standard_normal(n).astype(np.float32)
@@ -1686,7 +1690,7 @@ def test_adam_matches_oracle_over_steps(K, orc, rng, n):
 def test_adam_several_parameters_in_one_launch(K, rng):
     """ag_adam_update_multi_f32 against one ag_adam_update_f32 per parameter: bit-identical param, m, v and t
     over three steps; sizes with partial quads, one element, an empty parameter and a misaligned one."""
-    sizes = [25088, 1, 0, 4099, 288, 31360, 10, 7, (1 << 20) + 16384 + 777]   # the last one takes the run form
+    sizes = [25088, 1, 0, 4099, 288, 31360, 10, 7, (1 << 20) + 4096 + 777]   # the last one takes the run form
     def fresh():
         r = np.random.default_rng(3)
         ps = [dev(r.standard_normal(n + 1).astype(np.float32)) for n in sizes]
