@@ -200,12 +200,19 @@ __global__ __launch_bounds__(256) void s2_filter_parity_kernel(const float *__re
 // has no tap at a shift.  The GEMM's epilogue then writes gx[c][2i+a][2j .. 2j+1] as one 8-byte store, so no
 // parity-planar intermediate and no interleaving pass exist; the price is the zero taps (3 x 3, pad 1: 12 instead of
 // 9 tap-products per channel pair) on tiles of 128 rows instead of 64.
+// Where the product of a row parity runs on a tile whose waves hold 64 rows, the rows are grouped by parity instead
+// (of every 64 rows the first 32 are column parity 0 of 32 channels, the next 32 parity 1 of the same channels): one
+// of a wave's two 32-row blocks then belongs to each parity, and the kernel leaves out the matrix instructions of a
+// parity at the shifts where it has no tap -- the zero taps cost loads of zeros but no matrix time (3 x 3, pad 1: the
+// work of 9 tap-products per channel pair again; 4 x 4, pad 1: 8 instead of 12).
 struct S2Pair {
     int smax, kwp;           // largest column shift, number of shifts in the union
     long long floats[2];     // elements of the merged filter of row parity a
+    int grouped[2];          // rows of row parity a's filter grouped by column parity
+    unsigned skip[2][2];     // [a][b]: tap slots (m * kwp + n') of row parity a at which column parity b has no tap
 };
 
-static bool s2_pair(const S2Geom &g, int C, int K, int W, S2Pair *pr)
+static bool s2_pair(const S2Geom &g, int B, int C, int K, int W, S2Pair *pr)
 {
     if (W % 2 != 0 || g.W_b[0] != g.W_b[1] || g.W_b[0] < 1 || g.kw_b[0] < 1 || g.kw_b[1] < 1) return false;
     const int smax = g.d_a[0] > g.d_a[1] ? g.d_a[0] : g.d_a[1];
@@ -214,21 +221,36 @@ static bool s2_pair(const S2Geom &g, int C, int K, int W, S2Pair *pr)
     if (g.L + smin < 0) return false;
     pr->smax = smax;
     pr->kwp = smax - smin + 1;
-    for (int a = 0; a < 2; ++a) pr->floats[a] = 2LL * C * g.kh_a[a] * pr->kwp * K;
+    for (int a = 0; a < 2; ++a) {
+        pr->floats[a] = 2LL * C * g.kh_a[a] * pr->kwp * K;
+        const int slots = g.kh_a[a] * pr->kwp;
+        pr->grouped[a] = g.H_a[a] > 0 && slots <= 32 && gemm_conv_input_grad_pair_grouped(B, C, K, g.H_a[a], g.Wc, slots);
+        for (int b = 0; b < 2; ++b) {
+            pr->skip[a][b] = 0;
+            for (int t = 0; t < slots && t < 32; ++t) {
+                const int n = t % pr->kwp - (smax - g.d_a[b]);
+                if (n < 0 || n >= g.kw_b[b]) pr->skip[a][b] |= 1u << t;
+            }
+        }
+    }
     // the merged filters take the place of the parity filters and of the parity-planar result
     return pr->floats[0] + pr->floats[1] <= g.wf_floats + g.gxp_floats && pr->floats[0] + pr->floats[1] < 0x7fffffffLL;
 }
 
 // wp_a[2c + b][m * kwp + n'][k] = w[k][c][2m + alpha_a][2n + alpha_b] with n = n' - (smax - d_b), or 0 when parity b
 // has no tap n there; the filters of a = 0 and a = 1 back to back.
+// `grouped0` / `grouped1`: the rows of that row parity's filter are grouped by column parity (row = 64 * (c / 32) +
+// 32 * b + c % 32) instead of interleaved (row = 2c + b).
 __global__ __launch_bounds__(256) void s2_filter_pair_kernel(const float *__restrict__ w, float *__restrict__ wp, int K, int C,
-                                                             int kh, int kw, int pad, int smax, int kwp, int size0, int total)
+                                                             int kh, int kw, int pad, int smax, int kwp, int size0, int total,
+                                                             int grouped0, int grouped1)
 {
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int a = e >= size0, rest = a ? e - size0 : e;
         const int alpha_a = (a + pad) & 1, kha = (kh - alpha_a + 1) / 2;
         const int k = rest % K, tap = rest / K % (kha * kwp), row = rest / (K * kha * kwp);
-        const int c = row >> 1, b = row & 1;
+        const bool grouped = a ? grouped1 != 0 : grouped0 != 0;
+        const int c = grouped ? (row >> 6) * 32 + (row & 31) : row >> 1, b = grouped ? (row >> 5) & 1 : row & 1;
         const int alpha_b = (b + pad) & 1, kwb = (kw - alpha_b + 1) / 2, d_b = (b + pad) >> 1;
         const int m = tap / kwp, n = tap - m * kwp - (smax - d_b);
         float v = 0.f;
@@ -313,10 +335,10 @@ ag_status_t s2_igrad_prepare(hipStream_t st, const float *gy, const float *w, fl
     launch_pad_border(st, gy, scratch, B, K, g.OH, g.OW, g.Hp, g.Wc, g.T, g.L);
     hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, scratch + (long long)B * K * g.Hp * g.Wc, (int)kS2Slack);
     S2Pair pr;
-    if (s2_pair(g, C, K, g.W_b[0] + g.W_b[1], &pr)) {
+    if (s2_pair(g, B, C, K, g.W_b[0] + g.W_b[1], &pr)) {
         const int total = (int)(pr.floats[0] + pr.floats[1]);
         hipLaunchKernelGGL(s2_filter_pair_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, scratch + g.gyp_floats,
-                           K, C, kh, kw, pad, pr.smax, pr.kwp, (int)pr.floats[0], total);
+                           K, C, kh, kw, pad, pr.smax, pr.kwp, (int)pr.floats[0], total, pr.grouped[0], pr.grouped[1]);
     } else {
         hipLaunchKernelGGL(s2_filter_parity_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
                            scratch + g.gyp_floats, K, C, kh, kw, pad);
@@ -329,7 +351,7 @@ ag_status_t s2_igrad_gemm(hipStream_t st, float *scratch, float *gx, const S2Geo
     const float *gyp = scratch;
     const float *wr = scratch + g.gyp_floats;
     S2Pair pr;
-    if (s2_pair(g, C, K, W, &pr)) {
+    if (s2_pair(g, B, C, K, W, &pr)) {
         // (the prepare step has written the merged filters, so there is no falling back to the parity form here)
         AG_REQUIRE((reinterpret_cast<uintptr_t>(gx) & 7) == 0, AG_ERR_INVALID_DIMS,
                    "conv2d_transpose (column-free, stride 2): the output must be 8-byte aligned");
@@ -339,7 +361,7 @@ ag_status_t s2_igrad_gemm(hipStream_t st, float *scratch, float *gx, const S2Geo
                 // the first shift the GEMM visits is the largest: origin + (kwp - 1) = L + smax
                 const float *origin = gyp + (long long)(g.T - top) * g.Wc + (g.L + pr.smax - (pr.kwp - 1));
                 if (ag_status_t s = gemm_conv_input_grad_pair(st, wr, origin, gx, B, C, K, g.H_a[a], g.W_b[0], g.kh_a[a], pr.kwp,
-                                                              g.Hp, g.Wc, a, H, W))
+                                                              g.Hp, g.Wc, a, H, W, pr.grouped[a] ? pr.skip[a] : nullptr))
                     return s;
             }
             wr += pr.floats[a];

@@ -862,6 +862,8 @@ static ag_status_t run_gemm(hipStream_t st, const char *who, const GemmCall &c, 
     p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
     p.conv_pair_w = p.conv_pair_a = 0;
+    p.conv_pair_grouped = 0;
+    p.conv_pair_skip[0] = p.conv_pair_skip[1] = 0;
     p.conv_phase = 0;
     p.conv_dil = 1;
     p.rows_taps = p.rows_kw = p.rows_wp = 0;
@@ -952,7 +954,8 @@ static ImplicitPlan implicit_plan(int B, int C, int Kf, int H, int Wp, int taps,
 
 static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
                                       int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase, int pair_w = 0,
-                                      int pair_a = 0, int pair_h = 0, int dil = 1, float *ws = nullptr, size_t ws_floats = 0)
+                                      int pair_a = 0, int pair_h = 0, int dil = 1, float *ws = nullptr, size_t ws_floats = 0,
+                                      const unsigned *pair_skip = nullptr)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
@@ -970,6 +973,9 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
     p.conv_phase = phase;
     p.conv_dil = dil;
     p.conv_pair_w = pair_w; p.conv_pair_a = pair_a;
+    p.conv_pair_grouped = pair_skip != nullptr;
+    p.conv_pair_skip[0] = pair_skip ? pair_skip[0] : 0;
+    p.conv_pair_skip[1] = pair_skip ? pair_skip[1] : 0;
     if (pair_w != 0) {
         p.ldc = (long long)pair_h * pair_w;
         p.sC = (long long)(C / 2) * pair_h * pair_w;
@@ -981,6 +987,8 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
                                             ws != nullptr && phase == 0 && pair_w == 0 && out_floats < 0x7fffffffLL &&
                                                 ws_floats >= 2 * (size_t)out_floats);
     const int cfg = plan.cfg;
+    AG_REQUIRE(!pair_skip || (cfg >= 13 && cfg <= 15) || cfg == 18, AG_ERR_INVALID_DIMS,
+               "conv2d_transpose: rows grouped by parity need a tile whose waves hold 64 rows");
     p.kb_per_split = (int)cdiv(Kf / 32, plan.splits);
     p.splits = (int)cdiv(Kf / 32, p.kb_per_split);
     if ((size_t)p.splits * (size_t)out_floats > ws_floats) {  // (a forced split count the workspace cannot hold)
@@ -1117,9 +1125,17 @@ ag_status_t gemm_conv_input_grad(hipStream_t st, const float *wr, const float *g
 }
 
 ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,
-                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout)
+                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout, const unsigned *skip)
 {
-    return conv_implicit_gemm(st, wr, gyp, gx, B, 2 * C, Kf, Ha, Wb, kh, kw, Hp, Wp, 0, Wout, a, Hout);
+    return conv_implicit_gemm(st, wr, gyp, gx, B, 2 * C, Kf, Ha, Wb, kh, kw, Hp, Wp, 0, Wout, a, Hout, 1, nullptr, 0, skip);
+}
+
+// The tiles whose waves hold 64 rows (two 32-row blocks, one per parity): 128 x 128, 128 x 256, 256 x 128, 128 x 64.
+bool gemm_conv_input_grad_pair_grouped(int B, int C, int Kf, int Ha, int Wp, int taps)
+{
+    if (g_force_cfg >= 0) return false;  // (a forced tile may be one of the others)
+    const int cfg = implicit_plan(B, 2 * C, Kf, Ha, Wp, taps, 0, 1, false).cfg;
+    return (cfg >= 13 && cfg <= 15) || cfg == 18;
 }
 
 ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
@@ -1204,6 +1220,8 @@ static ag_status_t conv_filter_grad_gemm(hipStream_t st, const float *a, const f
     p.n_img = 0; p.n_off = 0;
     p.conv_wp = p.conv_w = p.conv_kw = 0;
     p.conv_pair_w = p.conv_pair_a = 0;
+    p.conv_pair_grouped = 0;
+    p.conv_pair_skip[0] = p.conv_pair_skip[1] = 0;
     p.conv_phase = 0;
     p.conv_dil = dil;
     p.rows_taps = taps; p.rows_kw = kw; p.rows_wp = Wp; p.rows_plane = (unsigned)b_plane; p.rows_phase = phase;

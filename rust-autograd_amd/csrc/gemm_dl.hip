@@ -1,5 +1,7 @@
 // fp32 GEMM on the matrix cores with operand tiles loaded from global memory straight into LDS.
 
+#include <type_traits>
+
 #include "gemm_shared.h"
 
 namespace ag {
@@ -188,9 +190,13 @@ template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, 
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
 {
     // CONV 1 / 2: the tap walk of the implicit convolution (conv_wp != 0, no phase planes), without / with
-    // dilation; 3: an ordinary product; 4: the stride-2 forward, whose taps walk the four phase planes
-    static_assert(CONV >= 1 && CONV <= 4, "walk of the k loop");
-    constexpr bool shifts = CONV == 1 || CONV == 2;  // taps as shifts within one plane
+    // dilation; 3: an ordinary product; 4: the stride-2 forward, whose taps walk the four phase planes; 5: the walk
+    // of 1 for the pair form of the stride-2 input gradient with its rows grouped by parity, which leaves out the
+    // matrix instructions of a parity at the taps it does not have
+    static_assert(CONV >= 1 && CONV <= 5, "walk of the k loop");
+    constexpr bool grouped = CONV == 5;
+    static_assert(!grouped || WM == 64, "one 32-row block per parity and wave");
+    constexpr bool shifts = CONV == 1 || CONV == 2 || CONV == 5;  // taps as shifts within one plane
     constexpr bool phases = CONV == 4;
     constexpr bool taps = shifts || phases;
     const int conv_dil = CONV == 2 ? p.conv_dil : 1;
@@ -472,14 +478,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             }
         }
     };
-    auto mfma_frags = [&](const Frag (&af)[MI], const Frag (&bf)[NI]) {
+    // SKIP (grouped pair form only): 1 leaves out the 32-row block of parity 0, 2 that of parity 1
+    auto mfma_frags = [&](auto skip_c, const Frag (&af)[MI], const Frag (&bf)[NI]) {
+        constexpr int SKIP = decltype(skip_c)::value;
 #pragma unroll
         for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
+            for (int i = 0; i < MI; ++i) {
+                if (SKIP != 0 && i == SKIP - 1) continue;
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].v[s4], bf[j].v[s4], acc[i][j], 0, 0, 0);
+            }
     };
     // Returns true when exactly STORES store instructions were issued (interior tile, overwrite).
     auto write_out = [&](const Item &it) -> bool {
@@ -521,6 +531,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                 ok[j] = in_range && ix < p.conv_w;
                 dst0[j] = p.conv_pair_w != 0 ? Cb + img + (long long)(2 * iy + p.conv_pair_a) * p.conv_pair_w + 2 * ix
                                              : Cb + img + iy * p.conv_w + ix;
+            }
+            if (grouped) {
+                // the wave's first 32-row block is parity 0 of 32 channels, its second block parity 1 of the same
+                // channels: value v of the two blocks are neighbours in memory
+                if constexpr (MI == 2) {
+                    const int ch_base = (it.m0 + wm * WM) / 2 + 4 * half;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int ch = ch_base + 8 * (v / 4) + (v % 4);
+#pragma unroll
+                        for (int j = 0; j < NI; ++j)
+                            if (ok[j] && 2 * ch < p.M) {
+                                float2 *dst = reinterpret_cast<float2 *>(dst0[j] + (long long)ch * ldc);
+                                *dst = make_float2(alpha * acc[0][j][v], alpha * acc[1][j][v]);
+                            }
+                    }
+                }
+                return false;
             }
             if (p.conv_pair_w != 0) {
                 // rows come in (channel, parity) pairs: a lane's values v, v + 1 (v even) are the two column
@@ -601,8 +629,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 
     Frag af[2][MI], bf[2][NI];
     unsigned fill_addr = lds_wave;  // LDS byte address (this wave's share) of the slot being filled
-    auto second_half = [&](const float *cur, const float *nxt, bool last) {
-        constexpr int NM = (KK - KK / 2) * 4 * MI * NI;  // MFMAs in this half
+    auto second_half = [&](auto skip_c, const float *cur, const float *nxt, bool last) {
+        constexpr int SKIP = decltype(skip_c)::value;
+        constexpr int MIA = SKIP != 0 ? MI - 1 : MI;        // 32-row blocks that multiply
+        constexpr int NM = (KK - KK / 2) * 4 * MIA * NI;  // MFMAs in this half
         constexpr int SPACING = NM / L;                   // MFMAs between two loads
         static_assert(SPACING >= 1, "more loads than MFMAs");
 #pragma unroll
@@ -613,12 +643,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
 #pragma unroll
             for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
-                for (int i = 0; i < MI; ++i)
+                for (int i = 0; i < MI; ++i) {
+                    if (SKIP != 0 && i == SKIP - 1) continue;
+                    const int ia = SKIP == 1 ? i - 1 : i;  // index among the blocks that multiply
 #pragma unroll
                     for (int j = 0; j < NI; ++j) {
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kk & 1][i].v[s4], bf[kk & 1][j].v[s4],
                                                                          acc[i][j], 0, 0, 0);
-                        const int m = (((kk - KK / 2) * 4 + s4) * MI + i) * NI + j;
+                        const int m = (((kk - KK / 2) * 4 + s4) * MIA + ia) * NI + j;
                         const int load = m / SPACING;
                         if (m % SPACING == SPACING - 1 && load < L) {
                             __builtin_amdgcn_sched_barrier(0);
@@ -628,6 +660,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
                             __builtin_amdgcn_sched_barrier(0);
                         }
                     }
+                }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -658,18 +691,29 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         if (chained) zero_tot();
         int chain_left = CHAIN;
         const bool last_item = cw + gridDim.x >= total;
+        int c_tap = 0;  // (grouped pair form) tap slot of the k tile being multiplied; an item starts at slot 0
         do {  // k tiles of the item: within a chain the accumulators are touched by MFMAs only
             const bool last = c_left == 1 && last_item;  // nothing follows in the stream
             const float *nxt = cur + TILE == ring_end ? lds : cur + TILE;
-
-            // first half of the tile's k range
-#pragma unroll
-            for (int kk = 0; kk < KK / 2; ++kk) {
-                read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);  // all fragment reads of the next group go out first
-                mfma_frags(af[kk & 1], bf[kk & 1]);
-                __builtin_amdgcn_sched_barrier(0);
+            // which parity, if any, has no filter tap at this slot (wave-uniform)
+            int skip = 0;
+            if (grouped) {
+                skip = (p.conv_pair_skip[0] >> c_tap) & 1u ? 1 : ((p.conv_pair_skip[1] >> c_tap) & 1u ? 2 : 0);
+                if (++c_tap == p.kbatch) c_tap = 0;
             }
+            auto first_half = [&](auto skip_c) {
+#pragma unroll
+                for (int kk = 0; kk < KK / 2; ++kk) {
+                    read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);  // all fragment reads of the next group go out first
+                    mfma_frags(skip_c, af[kk & 1], bf[kk & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            // first half of the tile's k range
+            if (grouped && skip == 1) first_half(std::integral_constant<int, grouped ? 1 : 0>{});
+            else if (grouped && skip == 2) first_half(std::integral_constant<int, grouped ? 2 : 0>{});
+            else first_half(std::integral_constant<int, 0>{});
             // The next tile must have landed; tiles further ahead may still be in flight.
             if (after_epilogue) wait_loads_then_barrier<AFTER_EPILOGUE>();
             else wait_loads_then_barrier<STEADY>();
@@ -678,7 +722,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             // between the MFMAs of the rest of this tile: a clump of loads would leave the matrix
             // pipe idle while the wave issues them, and all waves of the block would queue at the
             // address unit right after the barrier.
-            second_half(cur, nxt, last);
+            if (grouped && skip == 1) second_half(std::integral_constant<int, grouped ? 1 : 0>{}, cur, nxt, last);
+            else if (grouped && skip == 2) second_half(std::integral_constant<int, grouped ? 2 : 0>{}, cur, nxt, last);
+            else second_half(std::integral_constant<int, 0>{}, cur, nxt, last);
             fill_addr = fill_addr + TILE * 4u == lds_wave + STAGES * TILE * 4u ? lds_wave : fill_addr + TILE * 4u;
             cur = nxt;
             if (--chain_left == 0 && c_left - 1 > CHAIN / 4) {
@@ -711,7 +757,9 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
         auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 3>;                              \
         if constexpr (KA_ && !KB_) /* the implicit convolution over filter taps */                    \
             if (p.conv_phase != 0) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 4>;       \
-            else if (p.conv_wp != 0)                                                                  \
+            else if (p.conv_pair_grouped != 0) {                                                      \
+                if constexpr (WM == 64) kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 5>;  \
+            } else if (p.conv_wp != 0)                                                                \
                 kern = p.conv_dil != 1 ? gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 2>         \
                                        : gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 1>;        \
         long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \

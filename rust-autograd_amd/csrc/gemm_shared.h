@@ -40,6 +40,12 @@ struct GemmParams {
     // is pixel (2i + conv_pair_a, 2j + m % 2) of an output plane conv_pair_w wide, so the two parities
     // of a channel leave as one 8-byte store.  ldc / sC are the plane / image strides of that output.
     int conv_pair_w, conv_pair_a;
+    // Pair form with its rows grouped by parity (conv_pair_grouped != 0): within every 64 rows of A the first 32 are
+    // column parity 0 of 32 channels and the next 32 parity 1 of the same channels, so that one of a wave's two
+    // 32-row MFMA blocks belongs to each parity; bit t of conv_pair_skip[b] says that parity b has no filter tap at
+    // tap slot t of the union (its rows of A are zero there), and the kernel leaves those matrix instructions out.
+    int conv_pair_grouped;
+    unsigned conv_pair_skip[2];
     // Stride-2 forward (conv_phase != 0): B holds the four phase planes of the zero-bordered input,
     // [batch][K][2][2][Hpp][conv_wp] with phase (a, b) = elements (2i+a, 2j+b), conv_phase elements
     // each; tap (ky, kx), visited in natural order, reads phase (ky&1, kx&1) shifted by
@@ -87,8 +93,13 @@ size_t gemm_conv_input_grad_ws_floats(int B, int C, int Kf, int H, int W, int Wp
 // order, xph [B][C][4][Hpp][Wpp], y [B][K][OH][OW].
 // The pair form of the implicit input gradient (see GemmParams::conv_pair_w): wr [2C][kh*kw*Kf], gyp bordered
 // upstream gradient, gx [B][C][Hout][Wout] receives rows 2i + a, i < Ha, and columns 2j + b, j < Wb.
+// `skip` != null: the rows of wr are grouped by parity and skip[b] lists the tap slots at which parity b is zero
+// (GemmParams::conv_pair_grouped); gemm_conv_input_grad_pair_grouped says whether the product of these extents
+// runs on a tile that supports it (the filter must be written accordingly).
 ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf, int Ha,
-                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout);
+                                      int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout,
+                                      const unsigned *skip = nullptr);
+bool gemm_conv_input_grad_pair_grouped(int B, int C, int Kf, int Ha, int Wp, int taps);
 ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
                                   int OH, int OW, int kh, int kw, int Hpp, int Wpp);
 // Stride-2 filter gradient: gw[k][c][ky][kx] = sum over images and positions q of
