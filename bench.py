@@ -47,6 +47,8 @@ CALIBRATION_KERNEL = "ag::ew_vec_kernel<ag::ScaleF<false> >"
 CALIBRATION_KIB = float(1 << 20)
 _STEP, _POOL, _COLS = ("profiles/conv2d_fwd_bwd_c4_hbm_traffic.txt", "profiles/maxpool_c4_hbm_traffic.txt",
                        "profiles/conv2d_columns_c4_hbm_traffic.txt")
+_RED, _ADAM, _EW = ("profiles/reductions_hbm_traffic.txt", "profiles/adam_2pow26_hbm_traffic.txt",
+                    "profiles/elementwise_256x128x56x56_hbm_traffic.txt")
 _DL = "ag::gemm_dl_kernel<%s>"   # the last template argument: 1 = implicit convolution over filter taps, 3 = ordinary product
 PROFILE_TRAFFIC = {
     # the step (column-free)
@@ -63,6 +65,21 @@ PROFILE_TRAFFIC = {
     "gemm_fwd_columns": (_COLS, [(_DL % "128, 256, 32, 64, 64, 3, true, false, 3", "avg"), (_DL % "128, 64, 32, 64, 32, 3, true, false, 3", "avg")]),
     "gemm_filter_grad_columns": (_COLS, [(_DL % "128, 192, 32, 32, 96, 3, true, true, 3", "avg"), ("ag::splitk_fold_vec_kernel", "avg")]),
     "gemm_input_grad_columns": (_COLS, [(_DL % "192, 128, 32, 96, 32, 3, false, false, 3", "avg")]),
+    # reductions: fold_rows_kernel<64, true> serves the first stage of axes (0,2,3) and the mean over (2,3) (the same
+    # traffic: the whole tensor once); fold_cols_groups_kernel is the small second stage of axes (0,2,3) (min) and the
+    # whole of axis 0 (max)
+    "sum_all_2^26": (_RED, [("ag::sum_stage1_kernel", "avg"), ("ag::sum_stage2_kernel", "avg")]),
+    "reduce_sum_[256,128,56,56]_axes_0_2_3": (_RED, [("ag::fold_rows_kernel<64, true>", "avg"), ("ag::fold_cols_groups_kernel", "min")]),
+    "reduce_sum_[256,128,56,56]_axis_0": (_RED, [("ag::fold_cols_groups_kernel", "max")]),
+    "reduce_mean_[256,128,56,56]_axes_2_3": (_RED, [("ag::fold_rows_kernel<64, true>", "avg")]),
+    # Adam: the same kernel and traffic whatever the placement of the arrays
+    "adam_2^26": (_ADAM, [("ag::adam_kernel", "avg"), ("ag::adam_tick_kernel", "avg")]),
+    "adam_2^26_operands_2MiB_aligned": (_ADAM, [("ag::adam_kernel", "avg"), ("ag::adam_tick_kernel", "avg")]),
+    # elementwise glue
+    "relu_[256,128,56,56]": (_EW, [("ag::ew_vec_kernel<ag::ReluF>", "avg")]),
+    "relu_grad_[256,128,56,56]": (_EW, [("ag::ew_vec_kernel<ag::ReluGradF>", "avg")]),
+    "add_bias_relu_[256,128,56,56]": (_EW, [("ag::ew_vec_kernel<ag::BroadcastF<2, unsigned int> >", "avg")]),
+    "add_n_2x[256,128,56,56]": (_EW, [("ag::ew_vec_kernel<ag::AddNF>", "avg")]),
 }
 _profile_cache = {}
 _profile_strict = True   # False under --only: the passes that produce the summaries cannot depend on them
