@@ -192,11 +192,15 @@ size_t ag_conv2d_nocols_scratch_floats(int B, int C, int H, int W, int K, int kh
 ag_status_t ag_conv2d_fwd_nocols_f32(ag_stream_t stream, const float *x, const float *w, float *y,
                                      float *xpad, int B, int C, int H, int W, int K, int kh, int kw,
                                      int pad, int stride, int dilation);
-/* The two stages of ag_conv2d_fwd_nocols_f32 (rearranged copy of x and tap-major filter; the GEMM). */
+/* The two stages of ag_conv2d_fwd_nocols_f32 (rearranged copy of x and tap-major filter; the GEMM).  The size that
+ * ag_conv2d_nocols_scratch_floats returns may include, behind the copy and the filter, room for the partial results
+ * of a contraction that the GEMM stage slices over channel groups (products with fewer tiles than the chip has CUs):
+ * that part of `xpad` is written by the GEMM stage and means nothing afterwards; the copy in front of it is what
+ * the filter gradient and ag_conv2d_nocols_with_filter_f32 read.  Likewise the scratch of the input gradient. */
 ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const float *x, const float *w, float *xpad,
                                          int B, int C, int H, int W, int K, int kh, int kw, int pad,
                                          int stride, int dilation);
-ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C,
+ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, float *xpad, float *y, int B, int C,
                                       int H, int W, int K, int kh, int kw, int pad, int stride,
                                       int dilation);
 /* The forward GEMM over an existing rearranged copy with another filter: what Conv2DWithCols

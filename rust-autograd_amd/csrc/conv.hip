@@ -573,7 +573,7 @@ extern "C" ag_status_t ag_conv2d_nocols_prepare_f32(ag_stream_t stream, const fl
     return check_launch("conv2d");
 }
 
-extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float *xpad, float *y, int B, int C, int H, int W,
+extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, float *xpad, float *y, int B, int C, int H, int W,
                                                  int K, int kh, int kw, int pad, int stride, int dilation)
 {
     AG_REQUIRE(nocols_mode(stride, dilation), AG_ERR_INVALID_DIMS, "conv2d (column-free): stride %d / dilation %d not supported",
@@ -588,8 +588,8 @@ extern "C" ag_status_t ag_conv2d_nocols_gemm_f32(ag_stream_t stream, const float
     FusedGeom g;
     AG_REQUIRE(fused_fwd_geom(B, C, H, W, K, kh, kw, pad, &g, dilation) && aligned16(xpad) && aligned16(y), AG_ERR_INVALID_DIMS,
                "conv2d (column-free): geometry not supported");
-    const float *xp = xpad + kFwdLeadFloats;
-    float *ws = const_cast<float *>(xp) + g.gyp_floats + g.wr_floats;  // (the part of xpad behind the filter: transient)
+    float *xp = xpad + kFwdLeadFloats;
+    float *ws = xp + g.gyp_floats + g.wr_floats;  // (the part of xpad behind the filter: partial results, transient)
     return gemm_conv_input_grad(as_stream(stream), xp + g.gyp_floats, xp, y, B, K, C, H + 2 * pad - dilation * (kh - 1),
                                 W + 2 * pad - dilation * (kw - 1), kh, kw, g.Hp, g.Wp, dilation, g.ws_floats ? ws : nullptr,
                                 (size_t)g.ws_floats);

@@ -355,8 +355,10 @@ struct Conv2D : Op, ConvHyper {  // conv2d.rs:531-587
         // Column-free path when all three contractions of this convolution support it: the second
         // output, which only Conv2DFilterGrad and Conv2DWithCols read, is then the zero-bordered
         // input (rank 1) instead of the columns.
-        // (small problems are launch-bound and the column path has fewer launches: from 64 MB of columns on)
-        const bool large = (long long)B * C * kh * kw * OH * OW >= (16LL << 20);
+        // (small problems are launch-bound and the column path has fewer launches: from 32 MB of columns on --
+        // 128 images of 32 -> 64 channels at 14 x 14, 7.2 M column elements, cost the same either way; 32 images of
+        // 256 -> 256 channels at 14 x 14 with dilation 2, 14.5 M, take 0.27 ms without columns and 0.31 ms with them)
+        const bool large = (long long)B * C * kh * kw * OH * OW >= (8LL << 20);
         const size_t n_xpad =
             (large && !materialise_columns) ? ag_conv2d_nocols_scratch_floats(B, C, H, W, K, kh, kw, pad, stride, dilation) : 0;
         if (n_xpad > 0 && ag_conv2d_filter_grad_nocols_f32_workspace(B, C, H, W, K, kh, kw, pad, stride, dilation) > 0 &&

@@ -34,7 +34,7 @@ extern "C" {
     pub fn ag_conv2d_nocols_scratch_floats(B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> usize;
     pub fn ag_conv2d_fwd_nocols_f32(stream: AgStream, x: *const f32, w: *const f32, y: *mut f32, xpad: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> AgStatus;
     pub fn ag_conv2d_nocols_prepare_f32(stream: AgStream, x: *const f32, w: *const f32, xpad: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> AgStatus;
-    pub fn ag_conv2d_nocols_gemm_f32(stream: AgStream, xpad: *const f32, y: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> AgStatus;
+    pub fn ag_conv2d_nocols_gemm_f32(stream: AgStream, xpad: *mut f32, y: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> AgStatus;
     pub fn ag_conv2d_nocols_with_filter_f32(stream: AgStream, xpad: *const f32, w: *const f32, wf: *mut f32, y: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> AgStatus;
     pub fn ag_conv2d_filter_grad_nocols_f32_workspace(B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int) -> usize;
     pub fn ag_conv2d_filter_grad_nocols_f32(stream: AgStream, xpad: *const f32, gypad: *const f32, gw: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int, ws: *mut c_void, ws_bytes: usize) -> AgStatus;
