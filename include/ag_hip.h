@@ -240,6 +240,16 @@ ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, float *y, f
                                  uint8_t *taps, int B, int C, int H, int W, int size, int pad,
                                  int stride);
 
+/* ReLU::compute (activation_ops.rs:154-159), optionally with the AddOp in front of it (b != NULL: r = relu(a + b), b of
+ * a's rank with extents bshape[i] equal to a's or 1, as for ag_add_broadcast_relu_f32), followed by MaxPool2D::compute
+ * with a 2 x 2 window at stride 2 in ONE pass over even planes: the relu -> max_pool2d step of a conv block.  Writes r
+ * [B,C,H,W] (the ReLU's result, which the backward reads) and y, argmax, taps [B,C,H/2,W/2] exactly as ag_relu_f32 /
+ * ag_add_broadcast_relu_f32 followed by ag_maxpool2d_fwd_f32 would (same bits).  An optional fusion with no node of its
+ * own in the reference: an evaluator may use it when it is about to evaluate such a pooling whose input has not been
+ * computed yet.  H and W even; a and r 8-byte aligned. */
+ag_status_t ag_relu_maxpool2d_2x2_f32(ag_stream_t stream, const float *a, const float *b, const int *bshape, float *r,
+                                      float *y, float *argmax, uint8_t *taps, int B, int C, int H, int W);
+
 /* Replaces MaxPool2DGrad::compute -> max_pool_grad_f32 (max_pool2d.rs:245-279, 111-135).
  * gy [B,C,OH,OW] -> gx [B,C,H,W] (zero filled, then gx[argmax[i]] += gy[i] in ascending i; done
  * here as a gather that visits the candidate windows of each pixel in that same order, so sums

@@ -88,6 +88,9 @@ int agh_grad_helper(agh_ctx *ctx, const int *losses, int n, const char *ns, int 
 
 /* ---- introspection -------------------------------------------------------------------------- */
 int agh_num_nodes(agh_ctx *ctx);
+/* Pairs of nodes that the evaluations of this context so far ran as one launch (a ReLU, or the ReLU of a sum, with the
+ * 2 x 2 max pooling behind it); the results are those of the nodes evaluated in turn. */
+int agh_fused_pairs(agh_ctx *ctx);
 const char *agh_op_name(agh_ctx *ctx, int tensor);
 int agh_topo_rank(agh_ctx *ctx, int tensor);
 int agh_num_inputs(agh_ctx *ctx, int tensor);

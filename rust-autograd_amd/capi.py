@@ -74,6 +74,7 @@ PROTOTYPES = {
     "ag_conv2d_transpose_f32": (c_i, [c_p] * 5 + [c_i] * 12),
     "ag_conv2d_transpose_filter_grad_f32": (c_i, [c_p] * 5 + [c_i] * 12 + [c_p, c_sz]),
     "ag_maxpool2d_fwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
+    "ag_relu_maxpool2d_2x2_f32": (c_i, [c_p] * 8 + [c_i] * 4),
     "ag_maxpool2d_bwd_f32": (c_i, [c_p] * 5 + [c_i] * 7),
     "ag_maxpool2d_bwd_relu_f32": (c_i, [c_p] * 6 + [c_i] * 7),
     "ag_maxpool2d_gradgrad_f32": (c_i, [c_p] * 5 + [c_i] * 7),

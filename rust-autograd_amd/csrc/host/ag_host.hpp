@@ -172,6 +172,8 @@ class ComputeContext {
     NdArray input(size_t i);
     NdArray input_mut(size_t i);
     size_t num_inputs() const { return xs_.size(); }
+    // Extents of an input without grabbing it (a fusing op decides by them whether it will run).
+    const Shape &input_shape(size_t i) const { return xs_.at(i).array.shape(); }
 
     void append_output(NdArray y) { ys_.push_back(std::move(y)); }
     // A view of an input: copied first when any input is a variable (src/op.rs:273-287).
@@ -213,6 +215,14 @@ class Op {
     virtual const char *name() const = 0;
     virtual OpError compute(ComputeContext &ctx) const = 0;
     virtual void grad(GradientContext &ctx) const = 0;
+    // Evaluation-time fusion with the op that produces input 0 (no counterpart in the reference, whose evaluator
+    // runs every node on its own, src/evaluation.rs:310-329).  When the evaluator reaches a node whose first input has
+    // not been computed yet and fuses_with_producer(that input's op) holds, it gathers the PRODUCER's inputs instead
+    // and calls compute_with_producer: the op may then write the producer's outputs (`producer_outputs`) and its own
+    // (ctx) in one pass and return true, or touch nothing and return false, upon which both nodes are evaluated the
+    // ordinary way.  The results must have the bits of the two nodes evaluated in turn.
+    virtual bool fuses_with_producer(const Op &) const { return false; }
+    virtual bool compute_with_producer(ComputeContext &, const Op &, std::vector<NdArray> *, OpError *) const { return false; }
 };
 
 class TensorBuilder {  // src/tensor.rs:609-803
@@ -310,8 +320,11 @@ class Context : public Graph {  // src/graph.rs Context: graph + variable enviro
     // Graph::eval (src/evaluation.rs:251-363)
     std::vector<EvalResult> eval(const std::vector<Tensor> &tensors,
                                  const std::vector<std::pair<std::string, NdArray>> &feeds);
+    // Pairs of nodes that the evaluations of this context so far ran in one pass (Op::compute_with_producer).
+    size_t fused_pairs() const { return fused_pairs_; }
 
   private:
+    size_t fused_pairs_ = 0;
     VariableEnvironment *env_;
     std::unordered_map<VariableID, TensorID> var_nodes_;
 };

@@ -252,6 +252,7 @@ int agh_grad_helper(agh_ctx *c, const int *losses, int n, const char *ns, int *v
 }
 
 int agh_num_nodes(agh_ctx *c) { return (int)c->ctx.num_nodes(); }
+int agh_fused_pairs(agh_ctx *c) { return (int)c->ctx.fused_pairs(); }
 
 const char *agh_op_name(agh_ctx *c, int t)
 {

@@ -580,6 +580,11 @@ struct MaxPool2D : Op, PoolHyper {  // max_pool2d.rs:166-243
         ctx.append_output(idx);
         return OpError::none();
     }
+    // relu(x) or relu(a + b) in front of a 2 x 2 pooling at stride 2: one pass writes the activation and pools it
+    // (ag_relu_maxpool2d_2x2_f32); defined behind the ReLU ops below.
+    bool fuses_with_producer(const Op &producer) const override;
+    bool compute_with_producer(ComputeContext &ctx, const Op &producer, std::vector<NdArray> *producer_outputs,
+                               OpError *status) const override;
     void grad(GradientContext &ctx) const override
     {
         // max_pool2d.rs:229-242, with the input extent taken from x instead of being reconstructed
@@ -1041,6 +1046,53 @@ struct AddReLU : Op {
         ctx.append_input_grad(relu_grad_node(ctx.graph(), ctx.output(), ctx.output_grad()));
     }
 };
+
+bool MaxPool2D::fuses_with_producer(const Op &producer) const
+{
+    if (size != 2 || stride != 2 || pad != 0) return false;
+    return dynamic_cast<const ReLU *>(&producer) != nullptr || dynamic_cast<const AddReLU *>(&producer) != nullptr;
+}
+
+bool MaxPool2D::compute_with_producer(ComputeContext &ctx, const Op &producer, std::vector<NdArray> *producer_outputs,
+                                      OpError *status) const
+{
+    const bool with_sum = dynamic_cast<const AddReLU *>(&producer) != nullptr;
+    if (ctx.num_inputs() != (with_sum ? 2u : 1u)) return false;
+    const Shape &as = ctx.input_shape(0);
+    if (as.size() != 4 || as[2] < 2 || as[3] < 2 || as[2] % 2 != 0 || as[3] % 2 != 0 || as[0] * as[1] == 0) return false;
+    std::vector<int> bshape;
+    if (with_sum) {  // the operand patterns of AddReLU::compute, for rank 4
+        const Shape &bs = ctx.input_shape(1);
+        if (as == bs) {
+            bshape.assign(as.begin(), as.end());
+        } else if (broadcasts_over_rows(as, bs)) {
+            bshape.assign(as.begin(), as.end());
+            bshape[0] = 1;
+        } else if (!broadcasts_along_axes(as, bs, &bshape)) {
+            return false;
+        }
+        if (bshape.size() != 4) return false;
+    }
+    const NdArray a = ctx.input(0);
+    const NdArray b = with_sum ? ctx.input(1) : NdArray();
+    if ((reinterpret_cast<uintptr_t>(a.ptr()) & 7u) != 0) {  // (never with arrays of the arena; the kernel asks for it)
+        *status = OpError::make(ErrorKind::NdArrayError, "max_pool2d: misaligned input");
+        return true;
+    }
+    const int B = (int)as[0], C = (int)as[1], H = (int)as[2], W = (int)as[3];
+    const Shape ys{B, C, H / 2, W / 2};
+    NdArray r = NdArray::empty(as), y = NdArray::empty(ys), argmax = NdArray::empty(ys);
+    NdArray idx = NdArray::empty({(int64_t)((y.len() + 3) / 4 + 1)});
+    *status = from_status(ag_relu_maxpool2d_2x2_f32(ctx.stream(), a.ptr(), with_sum ? b.ptr() : nullptr,
+                                                    with_sum ? bshape.data() : nullptr, r.ptr(), y.ptr(), argmax.ptr(),
+                                                    reinterpret_cast<uint8_t *>(idx.ptr()), B, C, H, W));
+    if (!status->ok()) return true;
+    producer_outputs->push_back(r);
+    ctx.append_output(y);
+    ctx.append_output(argmax);
+    ctx.append_output(idx);
+    return true;
+}
 
 struct MulOp : Op {  // binary_ops.rs:209-237 (same-shape operands)
     const char *name() const override { return "MulOp"; }

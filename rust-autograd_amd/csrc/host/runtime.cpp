@@ -677,55 +677,141 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
         if (t.graph != this) throw Panic("Detected tensors belonging to different graphs");
         dfs.emplace_back(t.id, false);
     }
+    // Inputs of a node, from the feeds, the environment and what has been computed; the first error among them
+    // is the node's own (src/evaluation.rs:283-309).
+    auto gather = [&](const TensorInternal &n, std::vector<ComputeContext::Input> *inputs) {
+        OpError status;
+        for (const IncomingTensor &in : n.incoming_nodes) {
+            const TensorInternal &src = node(in.id);
+            if (src.is_placeholder) {
+                inputs->push_back({*find_placeholder(feeds, src), ComputeContext::InputKind::NonVariable});
+            } else if (src.is_variable()) {
+                inputs->push_back({env_->array(src.variable_id), in.allow_mut ? ComputeContext::InputKind::RdWrVariable
+                                                                              : ComputeContext::InputKind::RdOnlyVariable});
+            } else {
+                const StorageEntry &e = storage.at(in.id);
+                if (!e.error.ok()) {
+                    status = e.error;
+                    break;
+                }
+                if ((size_t)in.array_selector >= e.outputs.size())
+                    throw Panic("Bad op impl: output selector out of range");
+                inputs->push_back({e.outputs[(size_t)in.array_selector], ComputeContext::InputKind::NonVariable});
+            }
+        }
+        return status;
+    };
+    auto flush_if_touched = [&](const std::vector<ComputeContext::Input> &inputs) {
+        if (deferred.empty()) return;
+        for (const ComputeContext::Input &x : inputs)
+            if (deferred.writes(x.array) || (x.kind == ComputeContext::InputKind::RdWrVariable && deferred.reads(x.array))) {
+                deferred.flush();
+                return;
+            }
+    };
+    // Runs one node the ordinary way and files its result.
+    auto run_node = [&](const TensorInternal &n) {
+        std::vector<ComputeContext::Input> inputs;
+        OpError status = gather(n, &inputs);
+        StorageEntry entry;
+        if (status.ok()) {
+            flush_if_touched(inputs);
+            ComputeContext cc(std::move(inputs), &deferred);
+            status = n.op->compute(cc);
+            if (status.ok()) {
+                if (cc.outputs().empty()) throw Panic("Bad op implementation: empty return value");
+                entry.outputs = std::move(cc.outputs());
+            }
+            if (trace_enabled()) trace_node(n, entry.outputs, status);
+        }
+        entry.error = status;
+        storage.emplace(n.id, std::move(entry));
+    };
+    // The producer of a node's first input when the two can be evaluated in one pass (Op::fuses_with_producer).
+    auto fusable_producer = [&](const TensorInternal &n) -> const TensorInternal * {
+        if (n.incoming_nodes.empty() || n.incoming_nodes[0].array_selector != 0 || n.incoming_nodes[0].allow_mut) return nullptr;
+        const TensorInternal &p = node(n.incoming_nodes[0].id);
+        if (p.is_placeholder || p.is_variable() || !p.op || !n.op->fuses_with_producer(*p.op)) return nullptr;
+        for (const IncomingTensor &in : p.incoming_nodes)
+            if (in.allow_mut) return nullptr;
+        return &p;
+    };
+    // Which of the nodes this evaluation will reach are such producers, and of which node: whoever asks for the
+    // producer first is sent to that node instead, so the pair runs fused whatever the order of the walk.
+    std::unordered_map<TensorID, TensorID> fused_into;
+    {
+        std::vector<TensorID> stack;
+        std::unordered_map<TensorID, bool> seen;
+        for (const Tensor &t : tensors) stack.push_back(t.id);
+        while (!stack.empty()) {
+            const TensorID id = stack.back();
+            stack.pop_back();
+            if (seen[id]) continue;
+            seen[id] = true;
+            const TensorInternal &n = node(id);
+            if (n.is_placeholder || n.is_variable()) continue;
+            if (const TensorInternal *p = fusable_producer(n)) fused_into.emplace(p->id, id);
+            for (const IncomingTensor &in : n.incoming_nodes) stack.push_back(in.id);
+        }
+    }
     while (!dfs.empty()) {
         const auto [id, should_visit] = dfs.back();
         dfs.pop_back();
         const TensorInternal &n = node(id);
+        if (!should_visit) {
+            if (auto it = fused_into.find(id); it != fused_into.end() && !would_not_visit(n) && storage.count(it->second) == 0) {
+                dfs.emplace_back(it->second, false);  // the node that computes this one along with itself
+                continue;
+            }
+        }
         if (should_visit) {
             if (would_not_visit(n)) continue;
-            std::vector<ComputeContext::Input> inputs;
-            OpError status;
-            for (const IncomingTensor &in : n.incoming_nodes) {
-                const TensorInternal &src = node(in.id);
-                if (src.is_placeholder) {
-                    inputs.push_back({*find_placeholder(feeds, src), ComputeContext::InputKind::NonVariable});
-                } else if (src.is_variable()) {
-                    inputs.push_back({env_->array(src.variable_id), in.allow_mut ? ComputeContext::InputKind::RdWrVariable
-                                                                                 : ComputeContext::InputKind::RdOnlyVariable});
-                } else {
-                    const StorageEntry &e = storage.at(in.id);
-                    if (!e.error.ok()) {
-                        status = e.error;
-                        break;
-                    }
-                    if ((size_t)in.array_selector >= e.outputs.size())
-                        throw Panic("Bad op impl: output selector out of range");
-                    inputs.push_back({e.outputs[(size_t)in.array_selector], ComputeContext::InputKind::NonVariable});
-                }
-            }
-            StorageEntry entry;
-            if (status.ok()) {
-                if (!deferred.empty())
-                    for (const ComputeContext::Input &x : inputs)
-                        if (deferred.writes(x.array) ||
-                            (x.kind == ComputeContext::InputKind::RdWrVariable && deferred.reads(x.array))) {
-                            deferred.flush();
-                            break;
-                        }
-                ComputeContext cc(std::move(inputs), &deferred);
-                status = n.op->compute(cc);
+            if (const TensorInternal *p = fusable_producer(n); p && storage.count(p->id) == 0) {
+                // the producer has not run: both nodes in one pass, from the producer's inputs (which the first visit
+                // below has put in front of this node)
+                std::vector<ComputeContext::Input> inputs;
+                OpError status = gather(*p, &inputs);
+                bool fused = false;
                 if (status.ok()) {
-                    if (cc.outputs().empty()) throw Panic("Bad op implementation: empty return value");
-                    entry.outputs = std::move(cc.outputs());
+                    flush_if_touched(inputs);
+                    ComputeContext cc(std::move(inputs), &deferred);
+                    StorageEntry pe, ne;
+                    fused = n.op->compute_with_producer(cc, *p->op, &pe.outputs, &status);
+                    if (fused) {
+                        ++fused_pairs_;
+                        if (status.ok()) {
+                            if (cc.outputs().empty() || pe.outputs.empty()) throw Panic("Bad op implementation: empty return value");
+                            ne.outputs = std::move(cc.outputs());
+                        } else {
+                            pe.outputs.clear();
+                        }
+                        if (trace_enabled()) {
+                            trace_node(*p, pe.outputs, status);
+                            trace_node(n, ne.outputs, status);
+                        }
+                        pe.error = ne.error = status;
+                        storage.emplace(p->id, std::move(pe));
+                        storage.emplace(id, std::move(ne));
+                    }
                 }
-                if (trace_enabled()) trace_node(n, entry.outputs, status);
+                if (fused) continue;
+                run_node(*p);  // not this time (extents the fused form does not take, or an input in error)
             }
-            entry.error = status;
-            storage.emplace(id, std::move(entry));
+            run_node(n);
         } else {
             dfs.emplace_back(id, true);
-            for (const IncomingTensor &in : n.incoming_nodes)
-                if (!would_not_visit(node(in.id))) dfs.emplace_back(in.id, false);
+            const TensorInternal *p = fusable_producer(n);
+            for (size_t i = 0; i < n.incoming_nodes.size(); ++i) {
+                const TensorInternal &src = node(n.incoming_nodes[i].id);
+                if (would_not_visit(src)) continue;
+                if (i == 0 && p) {
+                    // evaluate what the producer reads, not the producer: it is computed together with this node
+                    for (const IncomingTensor &in : p->incoming_nodes)
+                        if (!would_not_visit(node(in.id))) dfs.emplace_back(in.id, false);
+                } else {
+                    dfs.emplace_back(n.incoming_nodes[i].id, false);
+                }
+            }
         }
     }
     flush_on_unwind.armed = false;

@@ -186,6 +186,54 @@ __global__ __launch_bounds__(256) void maxpool_fwd_tile2_kernel(const float *__r
     if (taps) taps[o] = (uint8_t)best_tap;
 }
 
+// The activation in front of such a pooling in the same pass: r = relu(a + b) (b broadcast along the axes where its
+// extent is 1; null = relu(a)) is written out -- the backward needs it -- and pooled as it is produced.  One
+// thread per window as above; the sum is rounded to f32 before the maximum and the maximum before the comparison,
+// so r, y, argmax and the tap bytes have the bits of the separate kernels.
+struct BiasStrides {
+    long long n, c, h, w;  // element strides of b along the axes of a (0 where b is broadcast)
+};
+__global__ __launch_bounds__(256) void relu_maxpool_tile2_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                                 BiasStrides bs, float *__restrict__ r, float *__restrict__ y,
+                                                                 float *__restrict__ argmax, uint8_t *__restrict__ taps,
+                                                                 PoolGeom g, int C, long long outputs)
+{
+    const long long o = blockIdx.x * 256ll + threadIdx.x;
+    if (o >= outputs) return;
+    const int per_plane = g.OH * g.OW;
+    const long long plane = o / per_plane;
+    const int e = (int)(o - plane * per_plane);
+    const int oy = e / g.OW, ox = e - oy * g.OW;
+    const long long at = plane * (long long)g.H * g.W + (long long)(2 * oy) * g.W + 2 * ox;  // whole-tensor offset of tap 0
+    const float2 top = *reinterpret_cast<const float2 *>(a + at), bottom = *reinterpret_cast<const float2 *>(a + at + g.W);
+    float v[4] = {top.x, top.y, bottom.x, bottom.y};
+    if (b) {
+        const long long n = plane / C;
+        const int c = (int)(plane - n * C);
+        const float *bp = b + n * bs.n + c * bs.c + (long long)(2 * oy) * bs.h + (long long)(2 * ox) * bs.w;
+        v[0] = v[0] + bp[0];
+        v[1] = v[1] + bp[bs.w];
+        v[2] = v[2] + bp[bs.h];
+        v[3] = v[3] + bp[bs.h + bs.w];
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] = v[t] > 0.f ? v[t] : 0.f;  // activation_ops.rs:155-159 (a NaN becomes 0)
+    *reinterpret_cast<float2 *>(r + at) = make_float2(v[0], v[1]);
+    *reinterpret_cast<float2 *>(r + at + g.W) = make_float2(v[2], v[3]);
+    float best = -FLT_MAX;
+    int best_tap = kNoTap;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const bool gt = v[t] > best;
+        best = gt ? v[t] : best;
+        best_tap = gt ? t : best_tap;
+    }
+    const long long flat = at + (best_tap >> 1) * g.W + (best_tap & 1);
+    y[o] = best;
+    argmax[o] = best_tap != kNoTap ? (float)(unsigned long long)flat : 0.f;
+    if (taps) taps[o] = (uint8_t)best_tap;
+}
+
 constexpr int kPoolLdsBytes = 32 * 1024;
 // A plane that does not fit half of that is cut into bands of at most this many staged bytes:
 // eight resident blocks per CU measured better than fewer, larger ones (112x112 planes: 0.242 ms
@@ -646,6 +694,36 @@ extern "C" ag_status_t ag_maxpool2d_fwd_f32(ag_stream_t stream, const float *x, 
                            argmax, taps, g, chunks);
     }
     return check_launch("max_pool2d");
+}
+
+extern "C" ag_status_t ag_relu_maxpool2d_2x2_f32(ag_stream_t stream, const float *a, const float *b, const int *bshape, float *r,
+                                                 float *y, float *argmax, uint8_t *taps, int B, int C, int H, int W)
+{
+    PoolGeom g;
+    if ((long long)B * C == 0) return AG_OK;
+    if (ag_status_t s = pool_geom("relu_max_pool2d", B, C, H, W, 2, 0, 2, &g)) return s;
+    AG_REQUIRE(a && r && y && argmax, AG_ERR_INVALID_DIMS, "relu_max_pool2d: null pointer");
+    AG_REQUIRE(H % 2 == 0 && W % 2 == 0, AG_ERR_INVALID_DIMS, "relu_max_pool2d: the 2 x 2 windows must tile the %d x %d plane", H, W);
+    AG_REQUIRE((reinterpret_cast<uintptr_t>(a) & 7u) == 0 && (reinterpret_cast<uintptr_t>(r) & 7u) == 0, AG_ERR_INVALID_DIMS,
+               "relu_max_pool2d: a and r must be 8-byte aligned");
+    BiasStrides bs = {0, 0, 0, 0};
+    if (b) {
+        AG_REQUIRE(bshape, AG_ERR_INVALID_DIMS, "relu_max_pool2d: the extents of b are missing");
+        const int shape[4] = {B, C, H, W};
+        long long stride = 1, st[4];
+        for (int d = 3; d >= 0; --d) {
+            AG_REQUIRE(bshape[d] == shape[d] || bshape[d] == 1, AG_ERR_INCOMPATIBLE_SHAPE,
+                       "relu_max_pool2d: extent %d of b on axis %d is neither 1 nor %d", bshape[d], d, shape[d]);
+            st[d] = bshape[d] == 1 ? 0 : stride;
+            stride *= bshape[d];
+        }
+        bs = BiasStrides{st[0], st[1], st[2], st[3]};
+    }
+    const long long outputs = (long long)B * C * g.OH * g.OW, blocks = (outputs + 255) / 256;
+    AG_REQUIRE(blocks <= kMaxGridX, AG_ERR_INVALID_DIMS, "relu_max_pool2d: too many tiles (%lld)", blocks);
+    hipLaunchKernelGGL(relu_maxpool_tile2_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), a, b, bs, r, y, argmax,
+                       taps, g, C, outputs);
+    return check_launch("relu_max_pool2d");
 }
 
 // RELU: every stored value is multiplied by greater(relu_x, 0) at its position (a template parameter: as a run-time

@@ -60,6 +60,7 @@ PROTOTYPES = {
     "agh_grad_with_default": (_i, [_p, _ip, _ip, _i, _ip, _i, _ip]),
     "agh_grad_helper": (_i, [_p, _ip, _i, _s, _ip, _ip, _i]),
     "agh_num_nodes": (_i, [_p]),
+    "agh_fused_pairs": (_i, [_p]),
     "agh_op_name": (_s, [_p, _i]),
     "agh_topo_rank": (_i, [_p, _i]),
     "agh_num_inputs": (_i, [_p, _i]),
@@ -342,6 +343,10 @@ class Context:
     @property
     def num_nodes(self):
         return lib().agh_num_nodes(self._h)
+
+    @property
+    def fused_pairs(self):
+        return lib().agh_fused_pairs(self._h)
 
     # -- evaluation ---------------------------------------------------------------------------
     def _evaluate(self, entry, tensors, feeds):

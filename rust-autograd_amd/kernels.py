@@ -286,6 +286,27 @@ def max_pool2d(x, pool_size, pad, stride):
     return y, am, il
 
 
+def relu_max_pool2d(a, b=None):
+    """relu(a) or relu(a + b) followed by max_pool2d(2, pad 0, stride 2) in one launch: (r, y, argmax, taps)."""
+    a = _f32(a, "relu_max_pool2d")
+    if a.dim() != 4:
+        raise capi.IncompatibleShape(f"max_pool2d: input must be 4D (got {list(a.shape)})")
+    B, Cc, H, W = a.shape
+    r = torch.empty_like(a)
+    y = _empty((B, Cc, H // 2, W // 2), a)
+    am = torch.empty_like(y)
+    taps = torch.empty(y.shape, dtype=torch.uint8, device=a.device)
+    bshape = None
+    if b is not None:
+        b = _f32(b, "relu_max_pool2d")
+        if b.dim() != 4:
+            raise capi.IncompatibleShape(f"add: operands of rank 4 and {b.dim()}")
+        bshape = (C.c_int * 4)(*b.shape)
+    check(capi.lib().ag_relu_maxpool2d_2x2_f32(_stream(), _ptr(a), _ptr(b), bshape, _ptr(r), _ptr(y), _ptr(am), _ptr(taps),
+                                               B, Cc, H, W))
+    return r, y, am, taps
+
+
 def max_pool2d_grad(gy, argmax, taps, x_shape, pool_size, pad, stride):
     gy = _f32(gy, "max_pool2d_grad")
     B, Cc, H, W = x_shape

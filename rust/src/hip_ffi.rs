@@ -40,6 +40,7 @@ extern "C" {
     pub fn ag_conv2d_filter_grad_nocols_f32(stream: AgStream, xpad: *const f32, gypad: *const f32, gw: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, K: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int, ws: *mut c_void, ws_bytes: usize) -> AgStatus;
     pub fn ag_conv2d_transpose_filter_grad_f32(stream: AgStream, x: *const f32, gy: *const f32, gw: *mut f32, gycols: *mut f32, B: c_int, ych: c_int, yh: c_int, yw: c_int, xch: c_int, H: c_int, W: c_int, kh: c_int, kw: c_int, pad: c_int, stride: c_int, dilation: c_int, ws: *mut c_void, ws_bytes: usize) -> AgStatus;
     pub fn ag_maxpool2d_fwd_f32(stream: AgStream, x: *const f32, y: *mut f32, argmax: *mut f32, taps: *mut u8, B: c_int, C: c_int, H: c_int, W: c_int, size: c_int, pad: c_int, stride: c_int) -> AgStatus;
+    pub fn ag_relu_maxpool2d_2x2_f32(stream: AgStream, a: *const f32, b: *const f32, bshape: *const c_int, r: *mut f32, y: *mut f32, argmax: *mut f32, taps: *mut u8, B: c_int, C: c_int, H: c_int, W: c_int) -> AgStatus;
     pub fn ag_maxpool2d_bwd_f32(stream: AgStream, gy: *const f32, argmax: *const f32, taps: *const u8, gx: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, size: c_int, pad: c_int, stride: c_int) -> AgStatus;
     pub fn ag_maxpool2d_bwd_relu_f32(stream: AgStream, gy: *const f32, argmax: *const f32, taps: *const u8, relu_x: *const f32, gx: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, size: c_int, pad: c_int, stride: c_int) -> AgStatus;
     pub fn ag_maxpool2d_gradgrad_f32(stream: AgStream, ggx: *const f32, argmax: *const f32, taps: *const u8, ggy: *mut f32, B: c_int, C: c_int, H: c_int, W: c_int, size: c_int, pad: c_int, stride: c_int) -> AgStatus;

@@ -620,6 +620,53 @@ def test_relu_gradient_behind_a_pooling_is_one_node_with_the_pooling_gradient(G,
     assert np.count_nonzero(a) > 0 and np.all(a[xv <= 0] == 0)
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_relu_in_front_of_a_2x2_pooling_is_evaluated_with_it(G, rng, with_bias):
+    """max_pool2d(relu(x), 2, 0, 2) and max_pool2d(relu(x + b), 2, 0, 2): when the evaluator reaches the pooling and its
+    input has not been computed, the two nodes run as one launch (the graph keeps both nodes; src/evaluation.rs runs
+    every node on its own).  Values, the ReLU's own result when it is asked for as well, and the gradients must have
+    the bits of the nodes evaluated in turn, whichever of them the walk reaches first."""
+    B, C, H = 3, 5, 12
+    xv = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    bv = rng.standard_normal((1, C, 1, 1)).astype(np.float32)
+    wv = rng.standard_normal((B, C, H // 2, H // 2)).astype(np.float32)
+    env = G.VariableEnvironment()
+    xid, bid = env.set("x", xv), env.set("b", bv)
+
+    def graph(c, split):
+        x, b = c.variable(xid), c.variable(bid)
+        r = c.relu(x + b) if with_bias else c.relu(x)
+        src = c.reshape(r, [B, C, H, H]) if split else r     # the reshape keeps the pooling away from the ReLU
+        y = c.max_pool2d(src, 2, 0, 2)
+        wts = c.placeholder("wts", [B, C, H // 2, H // 2])
+        grads = c.grad([c.sum_all(c.mul(y, wts))], [x, b] if with_bias else [x])
+        return r, y, grads
+
+    say(f"relu evaluated together with the pooling behind it, bias: {with_bias}")
+    results = {}
+    for split in (False, True):
+        for order in ("y first", "r first", "grads only"):
+            c = env.context()
+            r, y, grads = graph(c, split)
+            wanted = {"y first": [y, r] + grads, "r first": [r, y] + grads, "grads only": grads}[order]
+            out = c.eval(wanted, {"wts": wv})
+            assert c.fused_pairs == (0 if split else 1), (split, order, c.fused_pairs)
+            named = dict(zip(["y", "r"] if order == "y first" else ["r", "y"], out[:2])) if order != "grads only" else {}
+            named.update({f"g{i}": g for i, g in enumerate(out[-len(grads):])})
+            results[(split, order)] = named
+    ref = results[(True, "y first")]
+    want_r = np.maximum(xv + bv, 0) if with_bias else np.maximum(xv, 0)
+    assert np.array_equal(ref["r"], want_r)
+    for key, named in results.items():
+        for name, arr in named.items():
+            assert arr.shape == ref[name].shape and np.array_equal(arr.view(np.uint32), ref[name].view(np.uint32)), (key, name)
+    # odd planes do not fuse and still evaluate
+    c = env.context()
+    x5 = c.placeholder("x5", [2, 3, 5, 7])
+    (y5,) = c.eval([c.max_pool2d(c.relu(x5), 2, 0, 2)], {"x5": rng.standard_normal((2, 3, 5, 7)).astype(np.float32)})
+    assert y5.shape == (2, 3, 2, 3) and c.fused_pairs == 0
+
+
 def test_constant_gradients_through_reductions_are_one_fill_with_the_bits_of_the_chain(G, rng):
     """The seed of a back-propagation is a constant, and so is what the reductions at the end of a loss broadcast it
     to: those nodes are built as one FilledLike node (a single fill at evaluation) whose value goes through the

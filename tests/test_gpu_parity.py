@@ -1451,6 +1451,41 @@ def test_max_pool_2x2_tiling_kernels_have_the_bits_of_the_staged_and_register_ke
         assert a.shape == b.shape and a.tobytes() == b.tobytes()
 
 
+@pytest.mark.parametrize("bshape", [None, "same", (1, 5, 1, 1), (1, 5, 12, 16), (3, 1, 1, 16), (1, 1, 1, 1)])
+def test_relu_and_max_pool_in_one_pass_have_the_bits_of_the_two_kernels(K, orc, rng, bshape):
+    """ag_relu_maxpool2d_2x2_f32: relu(a) or relu(a + b) and the 2 x 2 pooling behind it in one launch.  The activation,
+    the pooled values, the f32 argmax and the tap bytes must equal what the separate kernels write -- and the oracle --
+    bit for bit, with ties (the clamped zeros of a ReLU tie in most windows), NaNs and signed zeros in the input."""
+    shape = (3, 5, 12, 16)
+    a = rng.standard_normal(shape).astype(np.float32)
+    a.reshape(-1)[::17] = np.nan
+    a.reshape(-1)[3::23] = -0.0
+    a[1, 2, 4:6, 6:8] = 0.75             # a window of equal positive values: the first one wins
+    b = None
+    if bshape is not None:
+        b = rng.standard_normal(shape if bshape == "same" else bshape).astype(np.float32)
+    say("relu + max_pool in one pass", bshape)
+    r, y, am, taps = K.relu_max_pool2d(dev(a), None if b is None else dev(b))
+    r2 = K.relu(dev(a)) if b is None else K.add_broadcast_relu(dev(a), dev(b))
+    y2, am2, taps2 = K.max_pool2d(r2, 2, 0, 2)
+    for got, want in ((r, r2), (y, y2), (am, am2), (taps, taps2)):
+        assert got.shape == want.shape and host(got).tobytes() == host(want).tobytes()
+    zr = orc.relu(a if b is None else (a + b).astype(np.float32))
+    oy, oam, oil = orc.maxpool2d_fwd(zr, 2, 0, 2)
+    assert np.array_equal(host(r).view(np.uint32), zr.view(np.uint32))
+    assert np.array_equal(host(y).view(np.uint32), oy.view(np.uint32)) and np.array_equal(host(am), oam)
+    assert np.array_equal(host(taps), orc.maxpool2d_taps(oil, shape[3], 2, 2))
+
+
+def test_relu_and_max_pool_in_one_pass_rejects_what_it_does_not_take(K):
+    a = torch.zeros(2, 3, 5, 6, device="cuda")
+    with pytest.raises(K.capi.InvalidDims, match="tile"):
+        K.relu_max_pool2d(a)
+    a = torch.zeros(2, 3, 4, 6, device="cuda")
+    with pytest.raises(K.capi.IncompatibleShape, match="neither 1 nor"):
+        K.relu_max_pool2d(a, torch.zeros(1, 2, 1, 1, device="cuda"))
+
+
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 1000])
 def test_max_pool_backward_any_chunking_of_the_rows(K, orc, rng, rows, hooked):
     """The stride-2 backward walks chunks of output rows; whatever their length (one row, odd
