@@ -3,12 +3,16 @@
 // at src/tensor_ops/gpu_ops.rs next to hip_ffi.rs and device.rs, with `mod` lines in
 // src/tensor_ops/mod.rs.
 //
+// Inputs and outputs go through `DeviceIo` (device.rs): with the crate's host-resident storage each
+// op stages its arrays through the host; under the cargo feature `device_storage` (device_storage.rs)
+// the same bodies pass device arrays from op to op.
+//
 // Each struct carries the hyper-parameters of the CPU op it stands in for (same field names), keeps
 // that op's shape checks and output list, and replaces the numeric core by C-ABI calls.  `grad`
 // builds the same gradient nodes as the CPU op -- out of the Gpu* ops -- so `grad()`, the evaluator
 // and the optimizers (src/gradient.rs, src/evaluation.rs, src/optimizers/) run unchanged.
 // The reference lines each piece follows are cited where it stands.
-use super::device::{stream, DeviceBuf};
+use super::device::{stream, DeviceBuf, DeviceIo};
 use super::hip_ffi as ffi;
 use crate::op::{ComputeContext, GradientContext, Op, OpError};
 use crate::tensor::Tensor;
@@ -66,7 +70,7 @@ fn dims4(s: &[usize], what: &str) -> Result<[usize; 4], OpError> {
 
 impl Op<f32> for GpuConv2D {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (x, w) = (ctx.input(0), ctx.input(1));
+        let (x, w) = (ctx.dev_in(0), ctx.dev_in(1));
         // conv2d_extract_params, conv2d.rs:349-404
         let [b, c, h, wd] = dims4(x.shape(), "conv2d: lhs input")?;
         let [k, c2, kh, kw] = dims4(w.shape(), "conv2d: filter")?;
@@ -78,15 +82,14 @@ impl Op<f32> for GpuConv2D {
             (ffi::ag_conv_out_size(h as c_int, kh as c_int, pad, stride, dil) as usize,
              ffi::ag_conv_out_size(wd as c_int, kw as c_int, pad, stride, dil) as usize)
         };
-        let (dx, dw) = (DeviceBuf::upload(&x), DeviceBuf::upload(&w));
         let dy = DeviceBuf::<f32>::alloc(b * k * oh * ow);
         let dcols = DeviceBuf::<f32>::alloc(b * c * kh * kw * oh * ow);
         ffi::check(unsafe {
-            ffi::ag_conv2d_fwd_f32(stream(), dx.ptr(), dw.ptr(), dy.ptr_mut(), dcols.ptr_mut(), b as c_int, c as c_int,
+            ffi::ag_conv2d_fwd_f32(stream(), x.ptr(), w.ptr(), dy.ptr_mut(), dcols.ptr_mut(), b as c_int, c as c_int,
                                    h as c_int, wd as c_int, k as c_int, kh as c_int, kw as c_int, pad, stride, dil)
         })?;
-        ctx.append_output(dy.download(&[b, k, oh, ow]));
-        ctx.append_output(dcols.download(&[b, c, kw, kh, oh, ow]));
+        ctx.dev_out(dy, &[b, k, oh, ow]);
+        ctx.dev_out(dcols, &[b, c, kw, kh, oh, ow]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -109,20 +112,19 @@ impl Op<f32> for GpuConv2D {
 
 impl Op<f32> for GpuConv2DWithCols {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (cols, w) = (ctx.input(0), ctx.input(1));
+        let (cols, w) = (ctx.dev_in(0), ctx.dev_in(1));
         let [k, c, kh, kw] = dims4(w.shape(), "conv2d_with_cols: filter")?;
         let cs = cols.shape(); // [B, C, kw, kh, OH, OW] (conv2d.rs:484)
         if cs.len() != 6 {
             return Err(bad_shape(format!("conv2d_with_cols: columns must be 6D (got {cs:?})")));
         }
         let (b, oh, ow) = (cs[0], cs[4], cs[5]);
-        let (dcols, dw) = (DeviceBuf::upload(&cols), DeviceBuf::upload(&w));
         let dy = DeviceBuf::<f32>::alloc(b * k * oh * ow);
         ffi::check(unsafe {
-            ffi::ag_conv2d_with_cols_f32(stream(), dcols.ptr(), dw.ptr(), dy.ptr_mut(), b as c_int, (c * kh * kw) as c_int,
+            ffi::ag_conv2d_with_cols_f32(stream(), cols.ptr(), w.ptr(), dy.ptr_mut(), b as c_int, (c * kh * kw) as c_int,
                                          (oh * ow) as c_int, k as c_int)
         })?;
-        ctx.append_output(dy.download(&[b, k, oh, ow]));
+        ctx.dev_out(dy, &[b, k, oh, ow]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -144,21 +146,20 @@ impl Op<f32> for GpuConv2DWithCols {
 
 impl Op<f32> for GpuConv2DFilterGrad {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (cols, gy, w) = (ctx.input(0), ctx.input(1), ctx.input(2));
+        let (cols, gy, w) = (ctx.dev_in(0), ctx.dev_in(1), ctx.dev_in(2));
         let [b, k, oh, ow] = dims4(gy.shape(), "conv2d_filter_grad: gradient")?;
         let [k2, c, kh, kw] = dims4(w.shape(), "conv2d_filter_grad: filter")?;
         if k != k2 {
             return Err(bad_shape(format!("conv2d_filter_grad: {k} gradient channels for {k2} filters")));
         }
         let (ck, p) = (c * kh * kw, oh * ow);
-        let (dcols, dgy) = (DeviceBuf::upload(&cols), DeviceBuf::upload(&gy));
         let dgw = DeviceBuf::<f32>::alloc(k * ck);
         let ws = DeviceBuf::<u8>::alloc(unsafe { ffi::ag_conv2d_filter_grad_f32_workspace(b as c_int, ck as c_int, p as c_int, k as c_int) });
         ffi::check(unsafe {
-            ffi::ag_conv2d_filter_grad_f32(stream(), dcols.ptr(), dgy.ptr(), dgw.ptr_mut(), b as c_int, ck as c_int, p as c_int,
+            ffi::ag_conv2d_filter_grad_f32(stream(), cols.ptr(), gy.ptr(), dgw.ptr_mut(), b as c_int, ck as c_int, p as c_int,
                                            k as c_int, ws.void(), ws.bytes())
         })?;
-        ctx.append_output(dgw.download(&[k, c, kh, kw]));
+        ctx.dev_out(dgw, &[k, c, kh, kw]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -178,7 +179,7 @@ impl Op<f32> for GpuConv2DFilterGrad {
 
 impl Op<f32> for GpuConv2DTranspose {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (gy, w) = (ctx.input(0), ctx.input(1));
+        let (gy, w) = (ctx.dev_in(0), ctx.dev_in(1));
         // conv2d_transpose_extract_params, conv2d_transpose.rs:29-87
         let [b, ych, yh, yw] = dims4(gy.shape(), "conv2d_transpose: Input")?;
         let [ych2, xch, kh, kw] = dims4(w.shape(), "conv2d_transpose: Filter")?;
@@ -191,15 +192,14 @@ impl Op<f32> for GpuConv2DTranspose {
             (ffi::ag_conv_transpose_out_size(yh as c_int, kh as c_int, pad, stride, dil) as usize,
              ffi::ag_conv_transpose_out_size(yw as c_int, kw as c_int, pad, stride, dil) as usize)
         };
-        let (dgy, dw) = (DeviceBuf::upload(&gy), DeviceBuf::upload(&w));
         let dgx = DeviceBuf::<f32>::alloc(b * xch * xh * xw);
         let dgcols = DeviceBuf::<f32>::alloc(b * xch * kh * kw * yh * yw); // the reference's temporary, :148-151
         ffi::check(unsafe {
-            ffi::ag_conv2d_transpose_f32(stream(), dgy.ptr(), dw.ptr(), dgx.ptr_mut(), dgcols.ptr_mut(), b as c_int, ych as c_int,
+            ffi::ag_conv2d_transpose_f32(stream(), gy.ptr(), w.ptr(), dgx.ptr_mut(), dgcols.ptr_mut(), b as c_int, ych as c_int,
                                          yh as c_int, yw as c_int, xch as c_int, kh as c_int, kw as c_int, pad, stride, dil,
                                          xh as c_int, xw as c_int)
         })?;
-        ctx.append_output(dgx.download(&[b, xch, xh, xw]));
+        ctx.dev_out(dgx, &[b, xch, xh, xw]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -215,23 +215,22 @@ impl Op<f32> for GpuConv2DTranspose {
 impl Op<f32> for GpuConv2DTransposeFilterGrad {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
         // inputs (gy, x, w): conv2d_transpose.rs:435-438
-        let (gy, x, w) = (ctx.input(0), ctx.input(1), ctx.input(2));
+        let (gy, x, w) = (ctx.dev_in(0), ctx.dev_in(1), ctx.dev_in(2));
         let [b, xch, h, wd] = dims4(gy.shape(), "conv2d_transpose_filter_grad: gradient")?;
         let [_, ych, yh, yw] = dims4(x.shape(), "conv2d_transpose_filter_grad: input")?;
         let [_, _, kh, kw] = dims4(w.shape(), "conv2d_transpose_filter_grad: filter")?;
         let (pad, stride, dil) = self.0.ints();
-        let (dx, dgy) = (DeviceBuf::upload(&x), DeviceBuf::upload(&gy));
         let dgw = DeviceBuf::<f32>::alloc(ych * xch * kh * kw);
         let dcols = DeviceBuf::<f32>::alloc(b * xch * kh * kw * yh * yw);
         let ws = DeviceBuf::<u8>::alloc(unsafe {
             ffi::ag_conv2d_filter_grad_f32_workspace(b as c_int, (xch * kh * kw) as c_int, (yh * yw) as c_int, ych as c_int)
         });
         ffi::check(unsafe {
-            ffi::ag_conv2d_transpose_filter_grad_f32(stream(), dx.ptr(), dgy.ptr(), dgw.ptr_mut(), dcols.ptr_mut(), b as c_int,
+            ffi::ag_conv2d_transpose_filter_grad_f32(stream(), x.ptr(), gy.ptr(), dgw.ptr_mut(), dcols.ptr_mut(), b as c_int,
                                                      ych as c_int, yh as c_int, yw as c_int, xch as c_int, h as c_int, wd as c_int,
                                                      kh as c_int, kw as c_int, pad, stride, dil, ws.void(), ws.bytes())
         })?;
-        ctx.append_output(dgw.download(&[ych, xch, kh, kw]));
+        ctx.dev_out(dgw, &[ych, xch, kh, kw]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -263,21 +262,20 @@ pub struct GpuMaxPool2DGradGrad(pub PoolHyper);
 
 impl Op<f32> for GpuMaxPool2D {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let x = ctx.input(0);
+        let x = ctx.dev_in(0);
         let [b, c, h, w] = dims4(x.shape(), "max_pool2d: input")?;
         let (size, pad, stride) = (self.0.size as c_int, self.0.pad as c_int, self.0.stride as c_int);
         let (oh, ow) = unsafe {
             (ffi::ag_pool_out_size(h as c_int, size, pad, stride) as usize, ffi::ag_pool_out_size(w as c_int, size, pad, stride) as usize)
         };
-        let dx = DeviceBuf::upload(&x);
         let (dy, dam) = (DeviceBuf::<f32>::alloc(b * c * oh * ow), DeviceBuf::<f32>::alloc(b * c * oh * ow));
         // taps = NULL: this wrapper keeps to the reference's two outputs (exact while x has <= 2^24 elements)
         ffi::check(unsafe {
-            ffi::ag_maxpool2d_fwd_f32(stream(), dx.ptr(), dy.ptr_mut(), dam.ptr_mut(), std::ptr::null_mut(), b as c_int, c as c_int,
+            ffi::ag_maxpool2d_fwd_f32(stream(), x.ptr(), dy.ptr_mut(), dam.ptr_mut(), std::ptr::null_mut(), b as c_int, c as c_int,
                                       h as c_int, w as c_int, size, pad, stride)
         })?;
-        ctx.append_output(dy.download(&[b, c, oh, ow]));
-        ctx.append_output(dam.download(&[b, c, oh, ow]));
+        ctx.dev_out(dy, &[b, c, oh, ow]);
+        ctx.dev_out(dam, &[b, c, oh, ow]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -290,20 +288,19 @@ impl Op<f32> for GpuMaxPool2D {
 
 impl Op<f32> for GpuMaxPool2DGrad {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (gy, argmax) = (ctx.input(0), ctx.input(1));
+        let (gy, argmax) = (ctx.dev_in(0), ctx.dev_in(1));
         let [b, c, yh, yw] = dims4(gy.shape(), "max_pool2d_grad: gradient")?;
         let (size, pad, stride) = (self.0.size as c_int, self.0.pad as c_int, self.0.stride as c_int);
         // the input extent the reference reconstructs (max_pool2d.rs:263-264)
         let (xh, xw) = unsafe {
             (ffi::ag_pool_grad_in_size(yh as c_int, size, pad, stride) as usize, ffi::ag_pool_grad_in_size(yw as c_int, size, pad, stride) as usize)
         };
-        let (dgy, dam) = (DeviceBuf::upload(&gy), DeviceBuf::upload(&argmax));
         let dgx = DeviceBuf::<f32>::alloc(b * c * xh * xw);
         ffi::check(unsafe {
-            ffi::ag_maxpool2d_bwd_f32(stream(), dgy.ptr(), dam.ptr(), std::ptr::null(), dgx.ptr_mut(), b as c_int, c as c_int,
+            ffi::ag_maxpool2d_bwd_f32(stream(), gy.ptr(), argmax.ptr(), std::ptr::null(), dgx.ptr_mut(), b as c_int, c as c_int,
                                       xh as c_int, xw as c_int, size, pad, stride)
         })?;
-        ctx.append_output(dgx.download(&[b, c, xh, xw]));
+        ctx.dev_out(dgx, &[b, c, xh, xw]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -316,17 +313,16 @@ impl Op<f32> for GpuMaxPool2DGrad {
 
 impl Op<f32> for GpuMaxPool2DGradGrad {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (ggx, argmax) = (ctx.input(0), ctx.input(1));
+        let (ggx, argmax) = (ctx.dev_in(0), ctx.dev_in(1));
         let [b, c, h, w] = dims4(ggx.shape(), "max_pool2d_grad_grad: input")?;
         let out: Vec<usize> = argmax.shape().to_vec();
         let (size, pad, stride) = (self.0.size as c_int, self.0.pad as c_int, self.0.stride as c_int);
-        let (dggx, dam) = (DeviceBuf::upload(&ggx), DeviceBuf::upload(&argmax));
         let dggy = DeviceBuf::<f32>::alloc(out.iter().product());
         ffi::check(unsafe {
-            ffi::ag_maxpool2d_gradgrad_f32(stream(), dggx.ptr(), dam.ptr(), std::ptr::null(), dggy.ptr_mut(), b as c_int, c as c_int,
+            ffi::ag_maxpool2d_gradgrad_f32(stream(), ggx.ptr(), argmax.ptr(), std::ptr::null(), dggy.ptr_mut(), b as c_int, c as c_int,
                                            h as c_int, w as c_int, size, pad, stride)
         })?;
-        ctx.append_output(dggy.download(&out));
+        ctx.dev_out(dggy, &out);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -352,7 +348,7 @@ pub struct GpuBatchMatMul {
 
 impl Op<f32> for GpuMatMul {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (a, b) = (ctx.input(0), ctx.input(1));
+        let (a, b) = (ctx.dev_in(0), ctx.dev_in(1));
         if a.ndim() != 2 {
             return Err(bad_shape("lhs input for MatMul must be 2D".into())); // dot_ops.rs:566-569
         }
@@ -365,15 +361,14 @@ impl Op<f32> for GpuMatMul {
         if k != k2 {
             return Err(bad_shape(format!("ndarray: inputs {m} × {k} and {k2} × {n} are not compatible for matrix multiplication")));
         }
-        let (da, db) = (DeviceBuf::upload(&a), DeviceBuf::upload(&b)); // contiguous copies: the transposes are flags
         let dc = DeviceBuf::<f32>::alloc(m * n);
         let ws = DeviceBuf::<u8>::alloc(unsafe { ffi::ag_matmul_f32_workspace(m as c_int, n as c_int, k as c_int) });
         ffi::check(unsafe {
             ffi::ag_matmul_f32(stream(), self.transpose_a as c_int, self.transpose_b as c_int, m as c_int, n as c_int, k as c_int,
-                               da.ptr(), ac.max(1) as c_int, db.ptr(), bc.max(1) as c_int, dc.ptr_mut(), n.max(1) as c_int,
+                               a.ptr(), ac.max(1) as c_int, b.ptr(), bc.max(1) as c_int, dc.ptr_mut(), n.max(1) as c_int,
                                ws.void(), ws.bytes())
         })?;
-        ctx.append_output(dc.download(&[m, n]));
+        ctx.dev_out(dc, &[m, n]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -388,7 +383,7 @@ impl Op<f32> for GpuMatMul {
 
 impl Op<f32> for GpuBatchMatMul {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let (a, b) = (ctx.input(0), ctx.input(1));
+        let (a, b) = (ctx.dev_in(0), ctx.dev_in(1));
         let (ra, rb) = (a.ndim(), b.ndim());
         if ra < 2 {
             return Err(bad_shape(format!("BatchMatMul: Left-hand-side input's ndim must be >= 2, actual: {ra}")));
@@ -410,17 +405,16 @@ impl Op<f32> for GpuBatchMatMul {
         let (m, k, n) = (sa[ra - 2], sa[ra - 1], sb[rb - 1]);
         let batch: usize = sa[..ra - 2].iter().product();
         let (lda, ldb) = (a.shape()[ra - 1].max(1), b.shape()[rb - 1].max(1));
-        let (da, db) = (DeviceBuf::upload(&a), DeviceBuf::upload(&b));
         let dc = DeviceBuf::<f32>::alloc(batch * m * n);
         ffi::check(unsafe {
             ffi::ag_gemm_f32(stream(), self.transpose_a as c_int, self.transpose_b as c_int, m as c_int, n as c_int, k as c_int, 1.0,
-                             da.ptr(), lda as c_int, (a.shape()[ra - 2] * a.shape()[ra - 1]) as i64, db.ptr(), ldb as c_int,
+                             a.ptr(), lda as c_int, (a.shape()[ra - 2] * a.shape()[ra - 1]) as i64, b.ptr(), ldb as c_int,
                              (b.shape()[rb - 2] * b.shape()[rb - 1]) as i64, 0.0, dc.ptr_mut(), n.max(1) as c_int, (m * n) as i64,
                              batch as c_int)
         })?;
         let mut out = sa[..ra - 2].to_vec();
         out.extend([m, n]);
-        ctx.append_output(dc.download(&out));
+        ctx.dev_out(dc, &out);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -462,37 +456,35 @@ fn axes_of(x_rank: usize, axes: &crate::ndarray_ext::NdArrayView<f32>, sparse: b
 }
 
 fn reduce(ctx: &mut ComputeContext<f32>, keep_dims: bool, sparse: bool, mean: bool) -> R {
-    let x = ctx.input(0);
-    let axes = axes_of(x.ndim(), &ctx.input(1), sparse);
+    let x = ctx.dev_in(0);
+    let axes = axes_of(x.ndim(), &ctx.input(1), sparse); // a handful of indices: read on the host
     if x.ndim() == 0 || axes.is_empty() {
-        ctx.append_output_view(x); // reduction_ops.rs:63-70, 192-195
+        ctx.dev_out_shared(x); // reduction_ops.rs:63-70, 192-195
         return Ok(());
     }
     let dims: Vec<c_int> = x.shape().iter().map(|&d| d as c_int).collect();
     let out_shape: Vec<usize> = x.shape().iter().enumerate()
         .filter_map(|(i, &d)| if axes.contains(&(i as c_int)) { if keep_dims { Some(1) } else { None } } else { Some(d) })
         .collect();
-    let dx = DeviceBuf::upload(&x);
     let dout = DeviceBuf::<f32>::alloc(out_shape.iter().product());
     let ws = DeviceBuf::<u8>::alloc(unsafe {
         ffi::ag_reduce_sum_f32_workspace(dims.as_ptr(), dims.len() as c_int, axes.as_ptr(), axes.len() as c_int)
     });
     ffi::check(unsafe {
-        ffi::ag_reduce_sum_f32(stream(), dx.ptr(), dout.ptr_mut(), dims.as_ptr(), dims.len() as c_int, axes.as_ptr(),
+        ffi::ag_reduce_sum_f32(stream(), x.ptr(), dout.ptr_mut(), dims.as_ptr(), dims.len() as c_int, axes.as_ptr(),
                                axes.len() as c_int, mean as c_int, ws.void(), ws.bytes())
     })?;
-    ctx.append_output(dout.download(&out_shape));
+    ctx.dev_out(dout, &out_shape);
     Ok(())
 }
 
 impl Op<f32> for GpuReduceSumToScalar {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let x = ctx.input(0);
-        let dx = DeviceBuf::upload(&x);
+        let x = ctx.dev_in(0);
         let dout = DeviceBuf::<f32>::alloc(1);
         let ws = DeviceBuf::<u8>::alloc(unsafe { ffi::ag_sum_all_f32_workspace(x.len()) });
-        ffi::check(unsafe { ffi::ag_sum_all_f32(stream(), dx.ptr(), x.len(), dout.ptr_mut(), ws.void(), ws.bytes()) })?;
-        ctx.append_output(dout.download(&[]));
+        ffi::check(unsafe { ffi::ag_sum_all_f32(stream(), x.ptr(), x.len(), dout.ptr_mut(), ws.void(), ws.bytes()) })?;
+        ctx.dev_out(dout, &[]);
         Ok(())
     }
     fn grad(&self, ctx: &mut GradientContext<f32>) {
@@ -560,21 +552,23 @@ pub struct GpuAdamOp {
 
 impl Op<f32> for GpuAdamOp {
     fn compute(&self, ctx: &mut ComputeContext<f32>) -> R {
-        let g = ctx.input(1);
+        let g = ctx.dev_in(1);
         let n = g.len();
-        let dg = DeviceBuf::upload(&g);
         // one fused pass in place on param, m, v; t is read by the update and incremented after it
-        let (mut p, mut m, mut v, mut t) = (ctx.input_mut(0), ctx.input_mut(2), ctx.input_mut(3), ctx.input_mut(4));
-        let (dp, dm, dv, dt) = (DeviceBuf::upload(&p.view()), DeviceBuf::upload(&m.view()), DeviceBuf::upload(&v.view()),
-                                DeviceBuf::upload(&t.view()));
-        ffi::check(unsafe {
-            ffi::ag_adam_update_f32(stream(), dp.ptr_mut(), dg.ptr(), dm.ptr_mut(), dv.ptr_mut(), dt.ptr_mut(), n, self.alpha,
-                                    self.eps, self.b1, self.b2)
-        })?;
-        p.assign(&dp.download(p.shape()));
-        m.assign(&dm.download(m.shape()));
-        v.assign(&dv.download(v.shape()));
-        t.assign(&dt.download(t.shape()));
+        let (p, m, v, t) = (ctx.dev_in_mut(0), ctx.dev_in_mut(2), ctx.dev_in_mut(3), ctx.dev_in_mut(4));
+        if p.len() != n || m.len() != n || v.len() != n || t.len() != 1 {
+            return Err(bad_shape(format!("adam: param {:?}, grad {:?}, m {:?}, v {:?}, t {:?}", p.shape(), g.shape(), m.shape(), v.shape(), t.shape())));
+        }
+        let status = unsafe {
+            ffi::ag_adam_update_f32(stream(), p.ptr_mut(), g.ptr(), m.ptr_mut(), v.ptr_mut(), t.ptr_mut(), n, self.alpha, self.eps,
+                                    self.b1, self.b2)
+        };
+        // hand every array back before reporting: with host storage this is where they are written back
+        ctx.dev_commit(0, p);
+        ctx.dev_commit(2, m);
+        ctx.dev_commit(3, v);
+        ctx.dev_commit(4, t);
+        ffi::check(status)?;
         ctx.append_empty_output();
         Ok(())
     }

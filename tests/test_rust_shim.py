@@ -136,3 +136,157 @@ def test_gpu_ops_implements_every_operator_and_calls_only_declared_functions():
             i += 1
         n_args = n_args + 1 if seen else 0
         assert n_args == len(r[name][1]), f"{name}: called with {n_args} arguments, declared with {len(r[name][1])}"
+
+
+# What each operator's `grad` builds in the reference: (node built, its inputs, its back-prop inputs)
+# in order, then which input gradients are Some.  Read off the reference's sources at the lines cited;
+# the names are the reference's (the GPU twin of `X` is `GpuX`), the input expressions are normalised
+# (`&`, whitespace and `ctx.` dropped).
+REFERENCE_GRADS = {
+    # conv_ops/conv2d.rs:556-586
+    "Conv2D": ([("Conv2DTranspose", ["gy", "w"], []),
+                ("Conv2DFilterGrad", ["cols", "gy", "w"], ["x", "gy"])], [True, True]),
+    # conv_ops/conv2d.rs:599-628
+    "Conv2DWithCols": ([("Conv2DTranspose", ["gy", "w"], []),
+                        ("Conv2DFilterGrad", ["cols", "gy", "w"], ["y.get_backprop_input(0)", "gy"])], [True, True]),
+    # conv_ops/conv2d.rs:746-775
+    "Conv2DFilterGrad": ([("Conv2DTranspose", ["gy", "ggw"], []),
+                          ("Conv2DWithCols", ["cols", "ggw"], ["y.get_backprop_input(0)", "ggw"])], [True, True]),
+    # conv_ops/conv2d_transpose.rs:274-300
+    "Conv2DTranspose": ([("Conv2D", ["gy", "w"], []),
+                         ("Conv2DTransposeFilterGrad", ["gy", "x", "stop_gradient(w)"], [])], [True, True]),
+    # conv_ops/conv2d_transpose.rs:453-479
+    "Conv2DTransposeFilterGrad": ([("Conv2DTranspose", ["x", "gw"], []),
+                                   ("Conv2D", ["gy", "gw"], [])], [True, True, False]),
+    # conv_ops/max_pool2d.rs:229-242, :281-294, :333-336
+    "MaxPool2D": ([("MaxPool2DGrad", ["gy", "indices"], [])], [True]),
+    "MaxPool2DGrad": ([("MaxPool2DGradGrad", ["ggx", "argmax"], [])], [True, False]),
+    "MaxPool2DGradGrad": ([], [False, False]),
+    # dot_ops.rs:608-628, :697-717 (flags false/true then true/false, whatever the op's own flags)
+    "MatMul": ([("MatMul{transpose_a:false,transpose_b:true}", ["gy", "input(1)"], []),
+                ("MatMul{transpose_a:true,transpose_b:false}", ["input(0)", "gy"], [])], [True, True]),
+    "BatchMatMul": ([("BatchMatMul{transpose_a:false,transpose_b:true}", ["gy", "input(1)"], []),
+                     ("BatchMatMul{transpose_a:true,transpose_b:false}", ["input(0)", "gy"], [])], [True, True]),
+    # reduction_ops.rs:130-136, :172-184, :217-238 (the CPU gradient ops serve: they are fills and broadcasts)
+    "ReduceSumToScalar": ([("ReduceSumToScalarGrad", ["output_grad()", "shape(input(0))"], [])], [True]),
+    "ReduceSum": ([("ReduceGradCommon", ["output_grad()", "shape(input(0))", "input(1)"], [])], [True, False]),
+    "ReduceMean": ([("ReduceGradCommon", ["output_grad()", "shape(x)", "axes"], [])], [True, False]),
+    # gradient_descent_ops/adam.rs:60-66
+    "AdamOp": ([], [False] * 5),
+}
+
+
+def _grad_body(text, name):
+    body = text[text.index(f"impl Op<f32> for {name} {{"):]
+    body = body[:body.index("\n}\n")]
+    return body[body.index("fn grad("):]
+
+
+def _split_top(s):
+    out, depth, cur = [], 0, ""
+    for ch in s:
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        if ch == "," and depth == 0:
+            out.append(cur)
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        out.append(cur)
+    return out
+
+
+def _norm_expr(e):
+    return re.sub(r"\s+", "", e).replace("&", "").replace("ctx.", "")
+
+
+def _norm_op(op):
+    op = re.sub(r"\s+", "", op)
+    op = re.sub(r"^crate::tensor_ops::reduction_ops::", "", op)
+    op = re.sub(r"\(self\.0\)$", "", op)           # the hyper-parameters travel unchanged
+    if op.startswith("ReduceGradCommon"):
+        assert "should_make_broadcast_dims:!self.keep_dims" in op and "sparse_axes:self.sparse_axes" in op
+        op = "ReduceGradCommon"
+    return re.sub(r"^Gpu", "", op)
+
+
+def _built_nodes(body):
+    """The nodes a `grad` body builds, in source order, from both spellings: `node(ctx, &[..], Op)` and
+    `Tensor::builder(..).append_input(..)...build(Op)`."""
+    found = []
+    for m in re.finditer(r"\bnode\(ctx,\s*&\[([^\]]*)\],\s*", body):
+        depth, i = 1, m.end()
+        while depth:
+            depth += {"(": 1, "{": 1, ")": -1, "}": -1}.get(body[i], 0)
+            i += 1
+        found.append((m.start(), _norm_op(body[m.end():i - 1]), [_norm_expr(e) for e in _split_top(m.group(1))], []))
+    for m in re.finditer(r"Tensor::builder\(ctx\.graph\(\)\)", body):
+        chain = body[m.end():]
+        ins, bps, pos = [], [], 0
+        while True:
+            c = re.match(r"\s*\.(append_input|append_backprop_input|build)\(", chain[pos:])
+            assert c, chain[pos:pos + 60]
+            depth, i = 1, pos + c.end()
+            while depth:
+                depth += {"(": 1, "{": 1, ")": -1, "}": -1}.get(chain[i], 0)
+                i += 1
+            arg = chain[pos + c.end():i - 1]
+            pos = i
+            if c.group(1) == "append_input":
+                expr, flag = _split_top(arg)
+                assert flag.strip() == "false"
+                ins.append(_norm_expr(expr))
+            elif c.group(1) == "append_backprop_input":
+                bps.append(_norm_expr(arg))
+            else:
+                found.append((m.start(), _norm_op(arg), ins, bps))
+                break
+    return [f[1:] for f in sorted(found)]
+
+
+def test_every_gpu_grad_builds_the_nodes_the_reference_builds():
+    text = open(os.path.join(ROOT, "rust", "src", "gpu_ops.rs")).read()
+    for ref_name, (nodes, some) in REFERENCE_GRADS.items():
+        body = _grad_body(text, "Gpu" + ref_name)
+        got = [(op, ins, bps) for op, ins, bps in _built_nodes(body)]
+        assert got == [(op, ins, bps) for op, ins, bps in nodes], f"Gpu{ref_name}::grad builds {got}"
+        grads = re.findall(r"append_input_grad\((Some|None)", body)
+        if ref_name == "AdamOp":
+            assert "for _ in 0..5" in body and grads == ["None"]
+        else:
+            assert [g == "Some" for g in grads] == some, f"Gpu{ref_name}::grad returns {grads}"
+    # the mean's gradient divides the broadcast by the product of the reduced extents (reduction_ops.rs:231-236)
+    mean = _grad_body(text, "GpuReduceMean")
+    assert "gather_common(shape(&x), &axes, 0)" in mean and "reduce_prod(reduced, &[0], false)" in mean and "broadcast / len" in mean
+    assert set(REFERENCE_GRADS) == {n[3:] for n in re.findall(r"impl Op<f32> for (\w+)", text)}
+
+
+def test_compute_bodies_move_arrays_only_through_device_io():
+    """With device-resident storage the ops must not stage anything themselves: every input and output
+    of every `compute` goes through the DeviceIo calls, whose two implementations (staging, resident)
+    live in device.rs; the resident one relies on functions device_storage.rs defines."""
+    ops = open(os.path.join(ROOT, "rust", "src", "gpu_ops.rs")).read()
+    assert "upload(" not in ops and "download(" not in ops and ".assign(" not in ops and "input_mut(" not in ops
+    for m in re.finditer(r"ctx\.input\((\d)\)", ops):
+        line = ops[ops.rfind("\n", 0, m.start()):ops.find("\n", m.end())]
+        fn = ops[:m.start()].rfind("fn ")
+        in_grad = ops[fn:fn + 8] == "fn grad("
+        assert in_grad or "axes_of(" in line, f"host read outside the axes list: {line.strip()}"
+    dev = open(os.path.join(ROOT, "rust", "src", "device.rs")).read()
+    trait = dev[dev.index("pub trait DeviceIo"):]
+    trait = trait[:trait.index("\n}\n")]
+    methods = re.findall(r"fn (\w+)\(", trait)
+    assert methods == ["dev_in", "dev_in_mut", "dev_commit", "dev_out", "dev_out_shared"]
+    assert dev.count("impl<'v> DeviceIo for ComputeContext<'v, f32>") == 2
+    assert '#[cfg(not(feature = "device_storage"))]\nimpl<\'v> DeviceIo' in dev and '#[cfg(feature = "device_storage")]\nimpl<\'v> DeviceIo' in dev
+    for used in set(re.findall(r"ctx\.(dev_\w+)\(", ops)):
+        assert used in methods
+    store = open(os.path.join(ROOT, "rust", "src", "device_storage.rs")).read()
+    resident = dev[dev.rindex("impl<'v> DeviceIo for ComputeContext"):]
+    for called in set(re.findall(r"self\.(\w+)\(", resident)):
+        assert re.search(rf"pub fn {called}\(", store), f"device.rs relies on ComputeContext::{called}, which device_storage.rs does not define"
+    for f in ("device_view", "device_view_mut", "sync_host_one", "take_to_host", "sync_host", "storage_get", "storage_take", "gather"):
+        assert re.search(rf"fn {f}[<(]", store), f
