@@ -188,10 +188,23 @@ class Timer:
         return {k: sorted(v)[len(v) // 2] for k, v in per.items()}
 
 
-def time_events(torch, fn, iters, warm=3):
+WARM_MS = float(os.environ.get("AG_BENCH_WARM_MS", "40"))
+
+
+def time_events(torch, fn, iters, warm=3, warm_ms=WARM_MS):
+    """Median duration of `fn` over `iters` calls between event pairs, enqueued behind about `warm_ms` milliseconds of
+    the same call back to back with no host wait in between: the GPU raises its clocks over tens of milliseconds of
+    load, and a leg of a few short calls after an idle gap is otherwise timed part-way up that ramp."""
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
     for _ in range(warm):
         fn()
-    torch.cuda.synchronize()
+    b.record()
+    b.synchronize()
+    per = max(a.elapsed_time(b) / warm, 1e-3)
+    for _ in range(min(4000, int(warm_ms / per))):
+        fn()
     evs = []
     for _ in range(iters):
         a = torch.cuda.Event(enable_timing=True)

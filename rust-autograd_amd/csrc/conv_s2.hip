@@ -243,8 +243,10 @@ static bool s2_pair(const S2Geom &g, int B, int C, int K, int W, S2Pair *pr)
 // 32 * b + c % 32) instead of interleaved (row = 2c + b).
 __global__ __launch_bounds__(256) void s2_filter_pair_kernel(const float *__restrict__ w, float *__restrict__ wp, int K, int C,
                                                              int kh, int kw, int pad, int smax, int kwp, int size0, int total,
-                                                             int grouped0, int grouped1)
+                                                             int grouped0, int grouped1, float *__restrict__ slack, int n_slack)
 {
+    // (also zeroes the slack behind the bordered gradient, so that the preparation needs no launch for that)
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < n_slack; e += gridDim.x * 256) slack[e] = 0.f;
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int a = e >= size0, rest = a ? e - size0 : e;
         const int alpha_a = (a + pad) & 1, kha = (kh - alpha_a + 1) / 2;
@@ -333,13 +335,15 @@ ag_status_t s2_igrad_prepare(hipStream_t st, const float *gy, const float *w, fl
                              int kh, int kw, int pad)
 {
     launch_pad_border(st, gy, scratch, B, K, g.OH, g.OW, g.Hp, g.Wc, g.T, g.L);
-    hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, scratch + (long long)B * K * g.Hp * g.Wc, (int)kS2Slack);
+    float *slack = scratch + (long long)B * K * g.Hp * g.Wc;
     S2Pair pr;
     if (s2_pair(g, B, C, K, g.W_b[0] + g.W_b[1], &pr)) {
         const int total = (int)(pr.floats[0] + pr.floats[1]);
         hipLaunchKernelGGL(s2_filter_pair_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, scratch + g.gyp_floats,
-                           K, C, kh, kw, pad, pr.smax, pr.kwp, (int)pr.floats[0], total, pr.grouped[0], pr.grouped[1]);
+                           K, C, kh, kw, pad, pr.smax, pr.kwp, (int)pr.floats[0], total, pr.grouped[0], pr.grouped[1], slack,
+                           (int)kS2Slack);
     } else {
+        hipLaunchKernelGGL(s2_zero_kernel, dim3(4), dim3(256), 0, st, slack, (int)kS2Slack);
         hipLaunchKernelGGL(s2_filter_parity_kernel, dim3((unsigned)((g.wf_floats + 255) / 256)), dim3(256), 0, st, w,
                            scratch + g.gyp_floats, K, C, kh, kw, pad);
     }
@@ -355,6 +359,14 @@ ag_status_t s2_igrad_gemm(hipStream_t st, float *scratch, float *gx, const S2Geo
         // (the prepare step has written the merged filters, so there is no falling back to the parity form here)
         AG_REQUIRE((reinterpret_cast<uintptr_t>(gx) & 7) == 0, AG_ERR_INVALID_DIMS,
                    "conv2d_transpose (column-free, stride 2): the output must be 8-byte aligned");
+        if (g.H_a[0] > 0 && g.H_a[1] > 0 && pr.grouped[0] && pr.grouped[1]) {
+            const float *wrs[2] = {wr, wr + pr.floats[0]}, *origins[2];
+            const unsigned *skips[2] = {pr.skip[0], pr.skip[1]};
+            for (int a = 0; a < 2; ++a)
+                origins[a] = gyp + (long long)(g.T - (g.kh_a[a] - 1 - g.d_a[a])) * g.Wc + (g.L + pr.smax - (pr.kwp - 1));
+            return gemm_conv_input_grad_pair_both(st, wrs, origins, gx, B, C, K, g.H_a, g.W_b[0], g.kh_a, pr.kwp, g.Hp, g.Wc, H, W,
+                                                  skips);
+        }
         for (int a = 0; a < 2; ++a) {
             if (g.H_a[a] > 0) {
                 const int top = g.kh_a[a] - 1 - g.d_a[a];

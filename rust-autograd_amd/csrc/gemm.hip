@@ -952,10 +952,18 @@ struct ImplicitPlan {
 };
 static ImplicitPlan implicit_plan(int B, int C, int Kf, int H, int Wp, int taps, unsigned phase, int pair_w, bool may_split);
 
+// What conv_implicit_gemm launches: a product on tile `cfg`, then, if tail_cfg >= 0, its last columns on a narrower one.
+struct ImplicitLaunch {
+    GemmParams p, tail;
+    int cfg, tail_cfg;
+};
+
+// `plan_only` != null: nothing is launched, the launches are described there instead (for a caller that merges two
+// products into one launch).
 static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const float *gyp, float *gx, int B, int C, int Kf,
                                       int H, int W, int kh, int kw, int Hp, int Wp, unsigned phase, int pair_w = 0,
                                       int pair_a = 0, int pair_h = 0, int dil = 1, float *ws = nullptr, size_t ws_floats = 0,
-                                      const unsigned *pair_skip = nullptr)
+                                      const unsigned *pair_skip = nullptr, ImplicitLaunch *plan_only = nullptr)
 {
     GemmParams p;
     p.A = wr; p.B = gyp; p.C = gx;
@@ -1033,6 +1041,14 @@ static ag_status_t conv_implicit_gemm(hipStream_t st, const float *wr, const flo
                 p.total_blocks = (unsigned)p.tiles_n;
             }
         }
+    }
+    if (plan_only != nullptr) {
+        AG_REQUIRE(p.splits == 1, AG_ERR_INVALID_DIMS, "conv2d_transpose: a merged launch of a sliced product");
+        plan_only->p = p;
+        plan_only->tail = tail;
+        plan_only->cfg = cfg;
+        plan_only->tail_cfg = tail_cfg;
+        return AG_OK;
     }
     launch_direct(st, cfg, true, false, p, num_cus(), g_grid_scale);
     if (ag_status_t s = check_launch("conv2d_transpose")) return s;
@@ -1128,6 +1144,40 @@ ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const flo
                                       int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout, const unsigned *skip)
 {
     return conv_implicit_gemm(st, wr, gyp, gx, B, 2 * C, Kf, Ha, Wb, kh, kw, Hp, Wp, 0, Wout, a, Hout, 1, nullptr, 0, skip);
+}
+
+// Both row parities of the grouped pair form.  Where the two products run on the same tiles they share their launches
+// (launch_direct's `second`): a CU that has finished its tiles of parity 0 goes on with parity 1 instead of waiting for
+// the other CUs, and the two narrow tails fill one round together.
+ag_status_t gemm_conv_input_grad_pair_both(hipStream_t st, const float *const wr[2], const float *const gyp[2], float *gx, int B,
+                                           int C, int Kf, const int Ha[2], int Wb, const int kh[2], int kw, int Hp, int Wp,
+                                           int Hout, int Wout, const unsigned *const skip[2])
+{
+    ImplicitLaunch L[2];
+    for (int a = 0; a < 2; ++a)
+        if (ag_status_t s = conv_implicit_gemm(st, wr[a], gyp[a], gx, B, 2 * C, Kf, Ha[a], Wb, kh[a], kw, Hp, Wp, 0, Wout, a, Hout,
+                                               1, nullptr, 0, skip[a], &L[a]))
+            return s;
+    const bool merge = L[0].cfg == L[1].cfg && L[0].tail_cfg == L[1].tail_cfg && g_grid_scale <= 0 &&
+                       ((L[0].cfg >= 13 && L[0].cfg <= 15) || L[0].cfg == 18) && (L[0].tail_cfg < 0 || L[0].tail_cfg == 13 || L[0].tail_cfg == 18);
+    if (merge) {
+        launch_direct(st, L[0].cfg, true, false, L[0].p, num_cus(), g_grid_scale, &L[1].p);
+        if (ag_status_t s = check_launch("conv2d_transpose")) return s;
+        if (L[0].tail_cfg >= 0) {
+            launch_direct(st, L[0].tail_cfg, true, false, L[0].tail, num_cus(), g_grid_scale, &L[1].tail);
+            return check_launch("conv2d_transpose");
+        }
+        return AG_OK;
+    }
+    for (int a = 0; a < 2; ++a) {
+        launch_direct(st, L[a].cfg, true, false, L[a].p, num_cus(), g_grid_scale);
+        if (ag_status_t s = check_launch("conv2d_transpose")) return s;
+        if (L[a].tail_cfg >= 0) {
+            launch_direct(st, L[a].tail_cfg, true, false, L[a].tail, num_cus(), g_grid_scale);
+            if (ag_status_t s = check_launch("conv2d_transpose")) return s;
+        }
+    }
+    return AG_OK;
 }
 
 // The tiles whose waves hold 64 rows (two 32-row blocks, one per parity): 128 x 128, 128 x 256, 256 x 128, 128 x 64.

@@ -186,8 +186,10 @@ struct DirectTile {
 // "is this a convolution / a phase walk" decided at compile time it takes 0.905 ms, the input gradient 0.937
 // instead of 0.964, the filter gradient 0.868 instead of 0.906 and the 4096^3 NT / TN products 0.965 / 0.971
 // instead of 0.994 / 0.996 ms; the stride-2 forward over phase planes 0.291 instead of 0.300 ms.
+// `bid` / `gdim`: this block's index and the number of blocks that share the product's work items (the whole grid,
+// or one of the two parts of a grid that carries two products).
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
+__device__ __forceinline__ void gemm_dl_body(const GemmParams &p, const unsigned bid, const unsigned gdim)
 {
     // CONV 1 / 2: the tap walk of the implicit convolution (conv_wp != 0, no phase planes), without / with
     // dilation; 3: an ordinary product; 4: the stride-2 forward, whose taps walk the four phase planes; 5: the walk
@@ -248,11 +250,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     };
     Cursor step, first;
     {
-        const unsigned stride = gridDim.x / kXcds;
+        const unsigned stride = gdim / kXcds;
         step.tm = (int)(stride % (unsigned)p.tiles_m);
         step.tn = (int)(stride / (unsigned)p.tiles_m % (unsigned)p.tiles_n);
         step.z = (int)(stride / tiles);
-        unsigned g = xcd_remap(blockIdx.x, total);
+        unsigned g = xcd_remap(bid, total);
         first.tm = (int)(g % (unsigned)p.tiles_m);
         g /= (unsigned)p.tiles_m;
         first.tn = (int)(g % (unsigned)p.tiles_n);
@@ -295,7 +297,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     };
 
     // ---- fetch stream ----
-    unsigned fw = blockIdx.x;
+    unsigned fw = bid;
     bool f_valid = fw < total;
     if (!f_valid) return;
     LoadA ldr_a;
@@ -344,7 +346,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     auto fetch_advance = [&]() {
         if (!f_valid) return;
         if (--f_left == 0) {
-            fw += gridDim.x;
+            fw += gdim;
             f_valid = fw < total;
             if (f_valid) {
                 cursor_next(fcur);
@@ -676,7 +678,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
     }
     wait_loads_then_barrier<(STAGES - 2) * L>();
 
-    unsigned cw = blockIdx.x;
+    unsigned cw = bid;
     Cursor ccur = first;
     Item ci = item_of(ccur);
     const float *cur = lds;  // ring slot being multiplied
@@ -690,7 +692,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
         const bool chained = ci.nt > CHAIN + CHAIN / 4;  // more than one chain: their sums meet in `tot`
         if (chained) zero_tot();
         int chain_left = CHAIN;
-        const bool last_item = cw + gridDim.x >= total;
+        const bool last_item = cw + gdim >= total;
         int c_tap = 0;  // (grouped pair form) tap slot of the k tile being multiplied; an item starts at slot 0
         do {  // k tiles of the item: within a chain the accumulators are touched by MFMAs only
             const bool last = c_left == 1 && last_item;  // nothing follows in the stream
@@ -742,16 +744,59 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(
             break;
         }
         after_epilogue = counted;
-        cw += gridDim.x;
+        cw += gdim;
         cursor_next(ccur);
         ci = item_of(ccur);
     }
 }
 
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_kernel(GemmParams p)
+{
+    gemm_dl_body<BM, BN, BK, WM, WN, STAGES, KA, KB, CONV>(p, blockIdx.x, gridDim.x);
+}
+
+// Two products of one tile shape in one launch: blocks [0, grid0) work through the items of the first, the others
+// through those of the second.  A CU whose block of the first product has run out of items takes a block of the second
+// at once, where two launches leave it idle until the first has drained everywhere (the two row parities of the
+// stride-2 input gradient: two or three rounds of tiles each).
+struct DualParams {
+    GemmParams q[2];
+    unsigned grid0;
+};
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool KA, bool KB, int CONV>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 1) void gemm_dl_dual_kernel(DualParams d)
+{
+    const bool second = blockIdx.x >= d.grid0;
+    gemm_dl_body<BM, BN, BK, WM, WN, STAGES, KA, KB, CONV>(d.q[second ? 1 : 0], blockIdx.x - (second ? d.grid0 : 0u),
+                                                           second ? gridDim.x - d.grid0 : d.grid0);
+}
+
+static long long dl_grid(const GemmParams &p, int cus, int blocks_per_cu)
+{
+    long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);
+    if (g >= p.total_blocks) g = p.total_blocks;        // one item per block
+    else g = g >= kXcds ? g - g % kXcds : kXcds;         // the kernel steps items by grid / 8
+    return g;
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int STAGES>
-static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu)
+static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu, const GemmParams *second)
 {
     constexpr int NT = (BM / WM) * (BN / WN) * 64;
+    if (second != nullptr) {
+        // two grouped pair-form products in one launch (the caller has checked that the tile is one of those)
+        if constexpr (WM == 64 && BM % 64 == 0) {
+            DualParams d;
+            d.q[0] = p;
+            d.q[1] = *second;
+            const long long g0 = dl_grid(p, cus, blocks_per_cu), g1 = dl_grid(*second, cus, blocks_per_cu);
+            d.grid0 = (unsigned)g0;
+            hipLaunchKernelGGL((gemm_dl_dual_kernel<BM, BN, BK, WM, WN, STAGES, true, false, 5>), dim3((unsigned)(g0 + g1)), dim3(NT), 0,
+                               st, d);
+        }
+        return;
+    }
 #define AG_GEMM_DL_CASE(KA_, KB_)                                                                     \
     if constexpr ((KA_ || BM % 64 == 0) && (KB_ || BN % 64 == 0)) if (ka == KA_ && kb == KB_) {      \
         auto kern = gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 3>;                              \
@@ -762,10 +807,7 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
             } else if (p.conv_wp != 0)                                                                \
                 kern = p.conv_dil != 1 ? gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 2>         \
                                        : gemm_dl_kernel<BM, BN, BK, WM, WN, STAGES, KA_, KB_, 1>;        \
-        long long g = (long long)cus * (blocks_per_cu > 0 ? blocks_per_cu : 1);                   \
-        if (g >= p.total_blocks) g = p.total_blocks;        /* one item per block */                 \
-        else g = g >= kXcds ? g - g % kXcds : kXcds;         /* the kernel steps items by grid / 8 */ \
-        hipLaunchKernelGGL(kern, dim3((unsigned)g), dim3(NT), 0, st, p);                              \
+        hipLaunchKernelGGL(kern, dim3((unsigned)dl_grid(p, cus, blocks_per_cu)), dim3(NT), 0, st, p);  \
         return;                                                                                       \
     }
     AG_GEMM_DL_CASE(true, true)
@@ -775,21 +817,24 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
 #undef AG_GEMM_DL_CASE
 }
 
-void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu)
+// `second` != null: a second grouped pair-form product (GemmParams::conv_pair_grouped) of the same tile, carried by the
+// same launch; only for the tiles whose waves hold 64 rows (configurations 13, 14, 15 and 18).
+void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu,
+                   const GemmParams *second)
 {
     switch (cfg) {
         //                BM   BN  BK   WM  WN STAGES
-        case 13: launch_dl<128, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        case 14: launch_dl<128, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        case 15: launch_dl<256, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
-        case 18: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu); break;
+        case 13: launch_dl<128, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu, second); break;
+        case 14: launch_dl<128, 256, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu, second); break;
+        case 15: launch_dl<256, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu, second); break;
+        case 16: launch_dl<192, 128, 32, 96, 32, 3>(st, ka, kb, p, cus, blocks_per_cu, nullptr); break;
+        case 17: launch_dl<128, 192, 32, 32, 96, 3>(st, ka, kb, p, cus, blocks_per_cu, nullptr); break;
+        case 18: launch_dl<128, 64, 32, 64, 32, 3>(st, ka, kb, p, cus, blocks_per_cu, second); break;
         // small problems: tiles that still give every CU a block or two
         // (32 rows only with a k-contiguous A: an m-contiguous tile is swizzled in groups of 64 rows)
-        case 20: launch_dl<32, 128, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
-        case 21: launch_dl<64, 64, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
-        default: launch_dl<64, 128, 32, 32, 64, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2); break;
+        case 20: launch_dl<32, 128, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2, nullptr); break;
+        case 21: launch_dl<64, 64, 32, 32, 32, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2, nullptr); break;
+        default: launch_dl<64, 128, 32, 32, 64, 3>(st, ka, kb, p, cus, blocks_per_cu > 0 ? blocks_per_cu : 2, nullptr); break;
     }
 }
 

@@ -73,7 +73,9 @@ constexpr int kChainK = 512;
 // Launches direct-to-LDS configuration `cfg` (kFirstDirectCfg ..); `ka` / `kb`: the operand is
 // k-contiguous.  `blocks_per_cu` > 0 overrides the persistent grid size.
 constexpr int kFirstDirectCfg = 13;
-void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu);
+// `second`: see gemm_dl.hip (two grouped pair-form products in one launch).
+void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu,
+                   const GemmParams *second = nullptr);
 // Implicit filter gradient: gw[k][c][tap] = sum over images and positions q, counted from the first
 // gradient value of a plane, of gyp[b][k][q + pad * Wp + pad] * xp[b][c][q + ky * Wp + kx].  gyp, xp:
 // zero-bordered [B][.][Hp][Wp] with the same border `pad`; `kq` (a multiple of 32) positions cover
@@ -100,6 +102,11 @@ ag_status_t gemm_conv_input_grad_pair(hipStream_t st, const float *wr, const flo
                                       int Wb, int kh, int kw, int Hp, int Wp, int a, int Hout, int Wout,
                                       const unsigned *skip = nullptr);
 bool gemm_conv_input_grad_pair_grouped(int B, int C, int Kf, int Ha, int Wp, int taps);
+// Both row parities of the grouped pair form (skip[a] non-null for both), merged into shared launches where their tiles
+// agree; arguments indexed by the row parity a are those of two gemm_conv_input_grad_pair calls.
+ag_status_t gemm_conv_input_grad_pair_both(hipStream_t st, const float *const wr[2], const float *const gyp[2], float *gx, int B,
+                                           int C, int Kf, const int Ha[2], int Wb, const int kh[2], int kw, int Hp, int Wp,
+                                           int Hout, int Wout, const unsigned *const skip[2]);
 ag_status_t gemm_conv_fwd_stride2(hipStream_t st, const float *wf, const float *xph, float *y, int B, int K, int C,
                                   int OH, int OW, int kh, int kw, int Hpp, int Wpp);
 // Stride-2 filter gradient: gw[k][c][ky][kx] = sum over images and positions q of
