@@ -144,7 +144,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the per-kernel microbenchmarks")
     ap.add_argument("--cpu-images", type=int, default=B, help="images per step of the CPU baseline (default: the whole batch)")
-    ap.add_argument("--only", choices=("pool", "columns", "config1", "config2", "stride2", "config5", "config3", "reduce", "adam",
+    ap.add_argument("--only", choices=("pool", "columns", "chain", "config1", "config2", "stride2", "config5", "config3", "reduce", "adam",
                                        "elementwise"),
                     help="run only one part of the per-kernel section (for profiler passes): the two pooling kernels, "
                          "the column-materialising convolution kernels, the steps of configuration 1 / 2 through the host "
@@ -757,6 +757,8 @@ def graph_steps(which=None):
         grads = c.grad([loss], [v[k] for k in names])
         adam.update([v[k] for k in names], grads, c, {"x": x2, "y": y2})
 
+    if which in (None, "chain"):
+        out.update(chain_step(G, np, rng, glorot, time, gc))
     for name, step, images in (("config1_conv_block_step", c1_step, 64), ("config2_cnn_adam_step", c2_step, 128)):
         if which is not None and not name.startswith(which):
             continue
@@ -782,6 +784,52 @@ def graph_steps(which=None):
         out[name] = {"ms": round(ms, 3), "images/s": round(images / ms * 1e3, 1),
                      "note": "graph build + host feeds + evaluation through libag_host.so, wall clock per step over 200 consecutive steps after 50 warm-up steps"}
     return out
+
+
+def chain_step(G, np, rng, glorot, time, gc):
+    """conv(64->128, 3x3) -> ReLU -> max_pool 2x2 -> conv(128->128, 3x3) at the headline's input [256,64,56,56], forward and
+    the gradients w.r.t. the input and both filters, through the host operator layer with everything resident on the
+    device -- once with the evaluator's shortcuts (the ReLU inside the pooling's launch, one bordered copy of gy for both
+    gradients of a convolution) and once node by node."""
+    env = G.VariableEnvironment()
+    xid = env.set("x", rng.standard_normal((256, 64, 56, 56), dtype=np.float32))
+    w1, w2 = env.set("w1", glorot((128, 64, 3, 3))), env.set("w2", glorot((128, 128, 3, 3)))
+    flop = 3 * 2.0 * 256 * 128 * 576 * 56 * 56 + 3 * 2.0 * 256 * 128 * 1152 * 28 * 28
+
+    def step():
+        c = env.context()
+        x, a, b = c.variable(xid), c.variable(w1), c.variable(w2)
+        y = c.conv2d(c.max_pool2d(c.relu(c.conv2d(x, a, 1, 1)), 2, 0, 2), b, 1, 1)
+        gx, ga, gb = c.grad([c.reduce_sum(y, [0, 1, 2, 3])], [x, a, b])
+        c.eval([c.reduce_sum(gx, [0, 1, 2, 3]), ga, gb])   # (the input gradient is summed so that 205 MB need not come back)
+
+    res = {}
+    for key, on in (("", True), ("_node_by_node", False)):
+        G.set_shortcuts(on)
+        try:
+            for _ in range(5):
+                step()
+            G.synchronize()
+            gc.collect()
+            gc.disable()
+            try:
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    step()
+                G.synchronize()
+                ms = (time.perf_counter() - t0) * 1e3 / 20
+            finally:
+                gc.enable()
+        finally:
+            G.set_shortcuts(True)
+        res["ms" + key] = round(ms, 3)
+    ms = res["ms"]
+    return {"chain_conv_relu_pool_conv_B256_56x56": {
+        **res, "images/s": round(256 / ms * 1e3, 1), "TFLOP/s": round(flop / ms / 1e9, 2),
+        "frac_mfma": round(flop / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+        "note": "graph build + evaluation through libag_host.so of conv(64->128) -> ReLU -> max_pool 2x2 -> conv(128->128), forward and "
+                "gradients w.r.t. input and filters (0.533 TFLOP of contractions), wall clock per step over 20 steps; ms_node_by_node: "
+                "the same with the evaluator's shortcuts off (every node on its own, a bordered copy of gy per gradient)"}}
 
 
 if __name__ == "__main__":

@@ -91,6 +91,12 @@ int agh_num_nodes(agh_ctx *ctx);
 /* Pairs of nodes that the evaluations of this context so far ran as one launch (a ReLU, or the ReLU of a sum, with the
  * 2 x 2 max pooling behind it); the results are those of the nodes evaluated in turn. */
 int agh_fused_pairs(agh_ctx *ctx);
+/* How often an op of the calling thread found the rearranged copy it needed already made by an earlier op (the
+ * zero-bordered upstream gradient that the two gradients of a column-free convolution share), since the thread began. */
+long long agh_reused_copies(void);
+/* Switches the evaluator's shortcuts (the fused pairs and the reused copies above) off or on for the whole process; on
+ * by default.  The results are the same bits either way: the switch exists to show that, and to time the difference. */
+void agh_set_shortcuts(int on);
 const char *agh_op_name(agh_ctx *ctx, int tensor);
 int agh_topo_rank(agh_ctx *ctx, int tensor);
 int agh_num_inputs(agh_ctx *ctx, int tensor);

@@ -67,6 +67,8 @@ class NdArray {
     // A 0-dimensional 0.0 that every caller shares (the reference's NdArray::zeros(vec![]) of an op
     // without a result, src/op.rs:290-294); nothing writes to it.
     static NdArray shared_zero();
+    // Extents without elements: shape() and ndim() answer, there is no storage behind them (ptr() is null).
+    static NdArray extents_only(const Shape &shape);
     // Identity of the allocation behind the array (views of one allocation compare equal).
     const void *allocation() const { return block_.get(); }
 
@@ -83,12 +85,27 @@ class NdArray {
     // stream used the array last, the caller's stream is ordered after it (a no-op for a thread's own arrays).
     void will_read() const;
     void will_write() const;
+    // A rearranged copy of the elements that one op made for its kernels and a later op can use again instead of making
+    // its own (the zero-bordered upstream gradient, which both gradients of a column-free convolution read).  One slot
+    // per allocation, found again by `key` (whatever identifies the arrangement and anything else it was made from);
+    // dropped when the array is overwritten (will_write) or freed.  `derived` returns an undefined array when the slot
+    // holds nothing for the key.
+    NdArray derived(const std::vector<int64_t> &key) const;
+    void set_derived(std::vector<int64_t> key, const NdArray &copy) const;
+    // Counts the in-place overwrites of the allocation (a key component for copies derived from a second array).
+    int64_t version() const;
 
   private:
     Shape shape_;
     std::shared_ptr<DeviceBlock> block_;
 };
 
+int64_t reused_copies();  // NdArray::derived hits of the calling thread so far
+// The evaluator's shortcuts -- a node evaluated in its producer's launch (Op::fuses_with_producer), a rearranged copy
+// found again (NdArray::derived) -- can be switched off, process-wide, to compare against the plain node-by-node
+// evaluation; results are the same bits either way.  On by default.
+void set_shortcuts(bool on);
+bool shortcuts_enabled();
 void *current_stream();  // hipStream_t of the calling thread: every op it evaluates is ordered on it
 void synchronize();
 

@@ -253,6 +253,8 @@ int agh_grad_helper(agh_ctx *c, const int *losses, int n, const char *ns, int *v
 
 int agh_num_nodes(agh_ctx *c) { return (int)c->ctx.num_nodes(); }
 int agh_fused_pairs(agh_ctx *c) { return (int)c->ctx.fused_pairs(); }
+long long agh_reused_copies(void) { return (long long)reused_copies(); }
+void agh_set_shortcuts(int on) { set_shortcuts(on != 0); }
 
 const char *agh_op_name(agh_ctx *c, int t)
 {

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -99,6 +100,10 @@ struct DeviceBlock {
     hipStream_t writer = nullptr;
     std::vector<hipStream_t> readers;
     bool constant = false;
+    // NdArray::derived / set_derived / version
+    std::vector<int64_t> derived_key;
+    NdArray derived;
+    int64_t version = 0;
     ~DeviceBlock();
 };
 
@@ -216,8 +221,12 @@ void NdArray::will_write() const
     if (!block_ || block_->constant) return;
     hipStream_t mine = t_stream.get();
     std::vector<hipStream_t> before;
+    NdArray dropped;  // (released outside the lock)
     {
         std::lock_guard<std::mutex> lk(block_->mu);
+        ++block_->version;
+        std::swap(dropped, block_->derived);
+        block_->derived_key.clear();
         if (block_->writer == mine && block_->readers.empty()) return;
         if (block_->writer && block_->writer != mine) before.push_back(block_->writer);
         for (hipStream_t r : block_->readers)
@@ -228,9 +237,55 @@ void NdArray::will_write() const
     for (hipStream_t o : before) wait_for_stream(o);
 }
 
+static thread_local int64_t t_reused_copies = 0;
+
+static std::atomic<bool> g_shortcuts{true};
+void set_shortcuts(bool on) { g_shortcuts.store(on); }
+bool shortcuts_enabled() { return g_shortcuts.load(std::memory_order_relaxed); }
+
+NdArray NdArray::derived(const std::vector<int64_t> &key) const
+{
+    NdArray d;
+    if (!block_ || !shortcuts_enabled()) return d;
+    {
+        std::lock_guard<std::mutex> lk(block_->mu);
+        if (block_->derived.defined() && block_->derived_key == key) d = block_->derived;
+    }
+    if (d.defined()) {
+        d.will_read();
+        ++t_reused_copies;
+    }
+    return d;
+}
+
+int64_t reused_copies() { return t_reused_copies; }
+
+void NdArray::set_derived(std::vector<int64_t> key, const NdArray &copy) const
+{
+    if (!block_ || block_->constant) return;
+    NdArray old = copy;  // (the previous occupant is released outside the lock)
+    std::lock_guard<std::mutex> lk(block_->mu);
+    std::swap(block_->derived, old);
+    block_->derived_key = std::move(key);
+}
+
+int64_t NdArray::version() const
+{
+    if (!block_) return 0;
+    std::lock_guard<std::mutex> lk(block_->mu);
+    return block_->version;
+}
+
 size_t NdArray::len() const { return product(shape_); }
 
 float *NdArray::ptr() const { return block_ ? static_cast<float *>(block_->ptr) : nullptr; }
+
+NdArray NdArray::extents_only(const Shape &shape)
+{
+    NdArray a;
+    a.shape_ = shape;
+    return a;
+}
 
 NdArray NdArray::empty(const Shape &shape)
 {
@@ -382,6 +437,7 @@ NdArray NdArray::deep_copy() const
 
 std::vector<float> NdArray::to_host() const
 {
+    if (!block_ && len()) throw Panic("NdArray::to_host: extents without elements");
     std::vector<float> out(len());
     will_read();
     if (len()) staging().download(out.data(), ptr(), len() * sizeof(float));
@@ -729,6 +785,7 @@ std::vector<EvalResult> Context::eval(const std::vector<Tensor> &tensors,
     };
     // The producer of a node's first input when the two can be evaluated in one pass (Op::fuses_with_producer).
     auto fusable_producer = [&](const TensorInternal &n) -> const TensorInternal * {
+        if (!shortcuts_enabled()) return nullptr;
         if (n.incoming_nodes.empty() || n.incoming_nodes[0].array_selector != 0 || n.incoming_nodes[0].allow_mut) return nullptr;
         const TensorInternal &p = node(n.incoming_nodes[0].id);
         if (p.is_placeholder || p.is_variable() || !p.op || !n.op->fuses_with_producer(*p.op)) return nullptr;

@@ -61,6 +61,8 @@ PROTOTYPES = {
     "agh_grad_helper": (_i, [_p, _ip, _i, _s, _ip, _ip, _i]),
     "agh_num_nodes": (_i, [_p]),
     "agh_fused_pairs": (_i, [_p]),
+    "agh_reused_copies": (C.c_longlong, []),
+    "agh_set_shortcuts": (None, [_i]),
     "agh_op_name": (_s, [_p, _i]),
     "agh_topo_rank": (_i, [_p, _i]),
     "agh_num_inputs": (_i, [_p, _i]),
@@ -387,6 +389,16 @@ class Context:
             st = lib().agh_result_status(self._h, i)
             out.append(OpError(st, lib().agh_result_message(self._h, i).decode()) if st != 0 else None)
         return out
+
+
+def reused_copies():
+    """How often an op of this thread found a rearranged copy it needed already made by an earlier op."""
+    return lib().agh_reused_copies()
+
+
+def set_shortcuts(on):
+    """Evaluation-time shortcuts (fused pairs, reused copies) on or off, process-wide; same results either way."""
+    lib().agh_set_shortcuts(int(bool(on)))
 
 
 def synchronize():

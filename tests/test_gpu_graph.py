@@ -1211,6 +1211,81 @@ def test_conv2d_stride2_column_free_through_the_graph_and_the_column_switch(G, o
         assert_close(gxv, ogx, "gx", scale=np.abs(ogx).max())
 
 
+@pytest.mark.parametrize("stride,H", [(1, 32), (2, 64)])
+def test_both_gradients_of_a_column_free_conv_share_the_bordered_gradient(G, rng, stride, H):
+    # the filter gradient and the input gradient read the same zero-bordered copy of gy: evaluated together, the second
+    # of them finds the copy the first one made; evaluated apart, each makes its own -- same bits either way.  A filter
+    # that Adam has rewritten in between is not served from a copy made for its old values.
+    B, Cin, Cout, k, pad = 64, 32, 64, 3, 1
+    xv = rng.standard_normal((B, Cin, H, H)).astype(np.float32)
+    env = G.VariableEnvironment()
+    wid = env.set("w", glorot(rng, (Cout, Cin, k, k)))
+    adam = G.Adam(env, [wid], alpha=1e-2)
+
+    def graph():
+        c = env.context()
+        x, w = c.placeholder("x", list(xv.shape)), c.variable(wid)
+        y = c.conv2d(x, w, pad, stride)
+        gx, gw = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+        return c, w, y, gx, gw
+
+    for step in range(2):
+        say(f"shared bordered gradient stride={stride} step={step}")
+        c, w, y, gx, gw = graph()
+        before = G.reused_copies()
+        gxv, gwv, kept = c.eval([gx, gw, c.nth_tensor(y, 1)], {"x": xv})
+        assert kept.ndim == 1, "the convolution is expected to run column-free at this size"
+        assert G.reused_copies() == before + 1
+        c1, _, _, gx1, _ = graph()
+        c2, _, _, _, gw2 = graph()
+        before = G.reused_copies()
+        assert np.array_equal(c1.eval([gx1], {"x": xv})[0], gxv)
+        assert np.array_equal(c2.eval([gw2], {"x": xv})[0], gwv)
+        assert G.reused_copies() == before
+        # one Adam step on the filter, then everything again with the new values
+        c3, w3, _, _, gw3 = graph()
+        adam.update([w3], [gw3], c3, {"x": xv})
+
+
+def test_a_conv_relu_pool_conv_chain_has_the_same_bits_with_and_without_the_evaluators_shortcuts(G, rng):
+    # conv -> ReLU(+bias) -> 2x2 pooling -> conv, both convolutions column-free, loss = sum of squares: the evaluator runs
+    # each ReLU inside its pooling's launch and each convolution's two gradients off one bordered copy of gy; with the
+    # shortcuts switched off every node runs on its own.  Values, gradients and an Adam step: the same bits.
+    B, C1, C2, H = 32, 32, 64, 64
+    xv = rng.standard_normal((B, C1, H, H)).astype(np.float32)
+    w1v, w2v = glorot(rng, (C2, C1, 3, 3)), glorot(rng, (C2, C2, 3, 3))
+    bv = (0.1 * rng.standard_normal((1, C2, 1, 1))).astype(np.float32)
+    results = []
+    for on in (True, False):
+        G.set_shortcuts(on)
+        try:
+            env = G.VariableEnvironment()
+            ids = [env.set("w1", w1v), env.set("w2", w2v), env.set("b", bv)]
+            adam = G.Adam(env, ids, alpha=1e-2)
+            c = env.context()
+            x = c.placeholder("x", list(xv.shape))
+            w1, w2, b = (c.variable(i) for i in ids)
+            z = c.max_pool2d(c.relu(c.conv2d(x, w1, 1, 1) + b), 2, 0, 2)
+            y = c.conv2d(z, w2, 1, 1)
+            loss = c.sum_all(c.mul(y, y))
+            grads = c.grad([loss], [x, w1, w2, b])
+            say(f"conv-relu-pool-conv chain, shortcuts {'on' if on else 'off'}")
+            reused = G.reused_copies()
+            vals = c.eval([y, z] + grads, {"x": xv})
+            assert (c.fused_pairs, G.reused_copies() - reused) == ((1, 2) if on else (0, 0))
+            c2 = env.context()
+            x = c2.placeholder("x", list(xv.shape))
+            w1, w2, b = (c2.variable(i) for i in ids)
+            y = c2.conv2d(c2.max_pool2d(c2.relu(c2.conv2d(x, w1, 1, 1) + b), 2, 0, 2), w2, 1, 1)
+            adam.update([w1, w2, b], c2.grad([c2.sum_all(c2.mul(y, y))], [w1, w2, b]), c2, {"x": xv})
+            vals += [env.array(i) for i in ids]
+            results.append(vals)
+        finally:
+            G.set_shortcuts(True)
+    for a, b_ in zip(*results):
+        assert np.array_equal(a, b_)
+
+
 def test_conv2d_column_free_second_order(G, orc, rng):
     # the gradient of the filter gradient: w.r.t. x (Conv2DTranspose of the incoming gradient) and
     # w.r.t. gy (Conv2DWithCols, here over the bordered input)
