@@ -294,6 +294,11 @@ __device__ inline float filter_tap_fwd(const float *__restrict__ w, int e, int C
     return w[((long long)k * C + c) * taps + (taps - 1 - tap)];
 }
 
+// Four floats at an address that is only 4-byte aligned.
+struct __attribute__((packed, aligned(4))) Unaligned4 {
+    float x, y, z, w;
+};
+
 // The small jobs that accompany a bordered copy (see pad_border_fast_kernel).
 struct PrepareExtras {
     float *lead;     // n_lead floats to zero before the planes
@@ -349,12 +354,22 @@ __global__ __launch_bounds__(256) void pad_border_fast_kernel(const float *__res
             ++r;
         }
     }
+    // Four elements that lie side by side inside one row of the image are one 16-byte load (aligned to 4 bytes only: the
+    // border shifts the copy against the source); the quads that touch a border or run over a row's end load what
+    // they have of the image one element at a time.
+    const bool whole = oy[3] == oy[0] && (unsigned)oy[0] < (unsigned)OH && ox[0] >= 0 && ox[3] < OW;
+    const int first = oy[0] * OW + ox[0];
     for (int b = blockIdx.y; b < B; b += ny) {
         const float *src = gy + ((long long)b * planes + pl) * (long long)OH * OW;
         float v[4];
+        if (whole) {
+            const Unaligned4 q = *reinterpret_cast<const Unaligned4 *>(src + first);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            v[t] = ((unsigned)oy[t] < (unsigned)OH && (unsigned)ox[t] < (unsigned)OW) ? src[oy[t] * OW + ox[t]] : 0.f;
+            for (int t = 0; t < 4; ++t)
+                v[t] = ((unsigned)oy[t] < (unsigned)OH && (unsigned)ox[t] < (unsigned)OW) ? src[oy[t] * OW + ox[t]] : 0.f;
+        }
         st_stream(reinterpret_cast<float4 *>(gyp) + ((long long)b * quads_img + qi), make_float4(v[0], v[1], v[2], v[3]));
     }
 }
