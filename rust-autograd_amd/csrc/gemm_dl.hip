@@ -822,6 +822,13 @@ static void launch_dl(hipStream_t st, bool ka, bool kb, const GemmParams &p, int
 void launch_direct(hipStream_t st, int cfg, bool ka, bool kb, const GemmParams &p, int cus, int blocks_per_cu,
                    const GemmParams *second)
 {
+    if (second != nullptr && !(ka && !kb && p.conv_pair_grouped != 0 && second->conv_pair_grouped != 0 &&
+                               ((cfg >= 13 && cfg <= 15) || cfg == 18))) {
+        // not a pair of products that one launch can carry: one after the other
+        launch_direct(st, cfg, ka, kb, p, cus, blocks_per_cu, nullptr);
+        launch_direct(st, cfg, ka, kb, *second, cus, blocks_per_cu, nullptr);
+        return;
+    }
     switch (cfg) {
         //                BM   BN  BK   WM  WN STAGES
         case 13: launch_dl<128, 128, 32, 64, 64, 3>(st, ka, kb, p, cus, blocks_per_cu, second); break;

@@ -1109,6 +1109,30 @@ def test_conv2d_stride2_column_free_random_geometries_exact(K):
     assert min(ran) >= 30, ran
 
 
+@pytest.mark.parametrize("B,k,p", [(128, 3, 1), (96, 4, 1), (72, 5, 2)])
+def test_conv2d_stride2_input_gradient_with_both_row_parities_in_one_launch(K, hooked, B, k, p):
+    # 64 -> 128 channels at 56 x 56: the pair form runs on 128 x 256 tiles with its rows grouped by column parity, and the
+    # two row parities (and their narrow tails) share their launches.  With a forced grid size the library launches them
+    # one after the other instead: the same bits, and on integer data those of the column path.
+    L = hooked
+    C, Kc, H = 64, 128, 56
+    r = np.random.default_rng(7 + k)
+    OH = (H + 2 * p - k) // 2 + 1
+    w = r.integers(-2, 3, (Kc, C, k, k)).astype(np.float32)
+    gy = r.integers(-2, 3, (B, Kc, OH, OH)).astype(np.float32)
+    say(f"stride-2 input gradient, merged launches B={B} k={k} pad={p}")
+    merged = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, H), 2, 1)
+    assert merged is not None
+    L.ag_test_gemm_force_grid(1)
+    try:
+        apart = K.conv_input_grad_staged(dev(gy), dev(w), p, (H, H), 2, 1)
+    finally:
+        L.ag_test_gemm_force_grid(0)
+    assert np.array_equal(host(merged[0]), host(apart[0]))
+    cols = K.conv2d_transpose(dev(gy), dev(w), p, 2, 1, out_hw=(H, H), return_cols=True)[0]
+    assert np.array_equal(host(merged[0]), host(cols))
+
+
 def test_conv2d_stride2_filter_grad_keeps_a_nan_inside_its_channel(K, rng):
     B, C, Kc, H, W, k, p = 2, 64, 64, 28, 28, 3, 1
     x = rng.standard_normal((B, C, H, W)).astype(np.float32)
