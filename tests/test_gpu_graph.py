@@ -1247,6 +1247,30 @@ def test_both_gradients_of_a_column_free_conv_share_the_bordered_gradient(G, rng
         adam.update([w3], [gw3], c3, {"x": xv})
 
 
+@pytest.mark.parametrize("B", [4, 64])
+def test_a_convolution_over_a_variable_equals_one_over_a_fed_array(G, rng, B):
+    # the gradients of conv -> 2x2 pooling take their output extents from the forward inputs through ExtentsOf nodes
+    # (an array with a shape and no elements); over a variable that must neither copy the variable nor change a bit
+    # (B = 4: over columns; B = 64: column-free)
+    C, K, H = 32, 32, 32
+    xv = rng.standard_normal((B, C, H, H)).astype(np.float32)
+    wv = glorot(rng, (K, C, 3, 3))
+    got = []
+    for as_variable in (False, True):
+        env = G.VariableEnvironment()
+        wid = env.set("w", wv)
+        c = env.context()
+        x = c.variable(env.set("x", xv)) if as_variable else c.placeholder("x", list(xv.shape))
+        w = c.variable(wid)
+        y = c.max_pool2d(c.conv2d(x, w, 1, 1), 2, 0, 2)
+        grads = c.grad([c.sum_all(c.mul(y, y))], [x, w])
+        say(f"convolution over a {'variable' if as_variable else 'fed array'}, B={B}")
+        got.append(c.eval([y] + grads, None if as_variable else {"x": xv}))
+        assert np.array_equal(env.array(wid), wv)
+    for a, b in zip(*got):
+        assert np.array_equal(a, b)
+
+
 def test_a_conv_relu_pool_conv_chain_has_the_same_bits_with_and_without_the_evaluators_shortcuts(G, rng):
     # conv -> ReLU(+bias) -> 2x2 pooling -> conv, both convolutions column-free, loss = sum of squares: the evaluator runs
     # each ReLU inside its pooling's launch and each convolution's two gradients off one bordered copy of gy; with the
